@@ -1,0 +1,142 @@
+/*
+ * vllm_amd_qlinear.h -- C ABI of the MI355X (gfx950) quantized-linear library
+ * (GPTQ W4A16 + FP8 W8A8).  One shared object: vllm_amd/libvllm_amd_qlinear.so.
+ *
+ * Conventions
+ *  - every pointer is a DEVICE pointer unless the name ends in _host;
+ *  - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *  - the library never allocates device memory, never synchronises the device
+ *    and throws nothing: each call validates its arguments on the host,
+ *    enqueues work on `stream` and returns VAQ_OK or a negative status, the
+ *    text for which is returned by vaq_last_error() (thread local);
+ *  - dtype tags: VAQ_F16 / VAQ_BF16 for 16-bit activations and outputs.
+ *
+ * Every entry point cites the reference interface it stands in for
+ * (paths relative to the reference tree).
+ */
+#ifndef VLLM_AMD_QLINEAR_H_
+#define VLLM_AMD_QLINEAR_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VAQ_OK 0
+#define VAQ_ERR_INVALID_ARG (-1)   /* shape / stride / alignment / enum check failed (TORCH_CHECK analogue)   */
+#define VAQ_ERR_UNSUPPORTED (-2)   /* valid request outside what is built (TORCH_CHECK_NOT_IMPLEMENTED analogue) */
+#define VAQ_ERR_LAUNCH (-3)        /* the HIP runtime refused the launch                                       */
+
+#define VAQ_F16 0
+#define VAQ_BF16 1
+#define VAQ_F32 2
+
+/* Weight layouts produced by vaq_w4a16_repack (both are int32 [K/16, 2N], same bytes). */
+#define VAQ_LAYOUT_MARLIN 0 /* the reference's Marlin tile order, bit-exact with gptq_marlin_repack   */
+#define VAQ_LAYOUT_NATIVE 1 /* wavefront tile order consumed by vaq_w4a16_gemm (K % 128 == 0 needed) */
+
+/* Weight code types (what b_q_type.id selects in the reference, vllm/scalar_type.py:327-351). */
+#define VAQ_WTYPE_U4B8 0 /* symmetric: code - 8            */
+#define VAQ_WTYPE_U4 1   /* asymmetric: code - zeros[g][n] */
+
+/* Text of the last error on the calling thread ("" if none). */
+const char* vaq_last_error(void);
+
+/* Library / device facts.  vaq_num_cus: compute units of `device` (>0) or a negative status. */
+int vaq_abi_version(void);
+int vaq_num_cus(int device);
+
+/*
+ * GPTQ int4 repack.  Replaces `gptq_marlin_repack(Tensor b_q_weight, Tensor perm, SymInt size_k,
+ * SymInt size_n, int num_bits) -> Tensor` (csrc/torch_bindings.cpp:320-321; device code
+ * csrc/quantization/gptq_marlin/gptq_marlin_repack.cu:7-322).
+ *   qweight  int32 [size_k/8, size_n] contiguous (8 nibbles along K per word)
+ *   perm     int32 [size_k] act_order sort indices (output row r takes input row perm[r]) or NULL
+ *   out      int32 [size_k/16, 2*size_n]
+ * num_bits must be 4.  size_k % 16 == 0, size_n % 64 == 0 (NATIVE additionally size_k % 128 == 0).
+ */
+int vaq_w4a16_repack(const int32_t* qweight, const int32_t* perm, int32_t* out, int64_t size_k, int64_t size_n,
+                     int num_bits, int layout, void* stream);
+
+/*
+ * Zero-point repack for the NATIVE layout: GPTQ/compressed-tensors `qzeros` values, packed 8 per int32 along N
+ * in natural order, are what vaq_w4a16_gemm reads, so no device work is needed and no entry point exists for
+ * it; the reference's marlin_zero_points (marlin_utils.py:326-346) is reproduced on the host side only.
+ */
+
+/*
+ * Scratch the caller must hand to vaq_w4a16_gemm for a given problem, in bytes:
+ *   *c_tmp_bytes   fp32 split-K partials   (reference: c_tmp, gptq_marlin.cu:752-763)
+ *   *a_tmp_bytes   permuted activations    (reference: a_tmp, gptq_marlin.cu:799); 0 when has_perm == 0
+ *   *counter_ints  int32 arrival counters that must be ZERO on entry and are left zero
+ *                  (reference: `workspace`, marlin_utils.py:237-245, marlin_template.h:225-271)
+ */
+int vaq_w4a16_gemm_workspace(int64_t size_m, int64_t size_n, int64_t size_k, int has_perm, int device,
+                             size_t* c_tmp_bytes, size_t* a_tmp_bytes, size_t* counter_ints);
+
+/*
+ * W4A16 GEMM  C[M,N] = A[:, perm] . dequant(B) (+ bias), fp32 accumulation, one rounding to the 16-bit dtype.
+ * Replaces `gptq_marlin_gemm(...)` (csrc/torch_bindings.cpp:309-315; csrc/quantization/gptq_marlin/gptq_marlin.cu:674-959).
+ *   a        [M, K] 16-bit, row stride lda elements (lda % 8 == 0, base 16-byte aligned), unit column stride
+ *   b        NATIVE-layout weights from vaq_w4a16_repack
+ *   scales   [K/group_size, N] in the activation dtype, contiguous
+ *   zeros    int32 [K/group_size, N/8] natural nibble order (wtype U4) or NULL (wtype U4B8)
+ *   perm     int32 [K] act_order sort indices or NULL  (is_k_full semantics: group of sorted row r is r / group_size)
+ *   bias     [N] activation dtype or NULL
+ *   c        [M, N] activation dtype, contiguous
+ *   group_size  128 (the only size built; others return VAQ_ERR_UNSUPPORTED)
+ * M == 0 is a no-op.  Kernel choice (decode: M <= 32, MFMA GEMV with in-register dequant; prefill: LDS-staged MFMA)
+ * is internal; `force_path` = 0 auto, 1 decode, 2 prefill (tests / benchmarks).
+ */
+int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
+                   const int32_t* perm, const void* bias, void* c, float* c_tmp, void* a_tmp, int32_t* counters,
+                   int64_t counter_ints, int64_t size_m, int64_t size_n, int64_t size_k, int group_size, int dtype,
+                   int wtype, int force_path, void* stream);
+
+/*
+ * out[m, k] = a[m, perm[k]] for 16-bit elements.  Replaces `permute_cols(Tensor A, Tensor perm) -> Tensor`
+ * (csrc/torch_bindings.cpp:304; csrc/permute_cols.cu:13-87).
+ */
+int vaq_permute_cols(const void* a, int64_t lda, const int32_t* perm, void* out, int64_t size_m, int64_t size_k,
+                     void* stream);
+
+/*
+ * FP8 (OCP e4m3fn) activation quantisation.  `in` is [rows, hidden] F16/BF16/F32 with unit column stride and
+ * row stride in_row_stride (elements); `out` is uint8 codes with row stride out_row_stride.
+ *
+ * vaq_fp8_quant_per_token  replaces `dynamic_per_token_scaled_fp8_quant(Tensor! result, Tensor input, Tensor! scale,
+ *     Tensor? scale_ub)` (csrc/torch_bindings.cpp:585-587; csrc/quantization/w8a8/fp8/common.cu:91-131, :213-247):
+ *     scales[r] = max(min(amax_r, *scale_ub) / 448, 1/(448*512));  out = cvt(clamp(x / scales[r], +-448))  (true division)
+ * vaq_fp8_quant_static     replaces `static_scaled_fp8_quant(Tensor! result, Tensor input, Tensor scale)` (:572; common.cu:11-30, :136-170):
+ *     out = cvt(clamp(x * (1 / *scale), +-448))
+ * vaq_fp8_quant_dynamic    replaces `dynamic_scaled_fp8_quant(Tensor! result, Tensor input, Tensor! scale)` (:578; common.cu:32-89, :172-211):
+ *     *scale = max_all|x| / 448 (written by the call), then as static.
+ */
+int vaq_fp8_quant_per_token(const void* in, int in_dtype, int64_t in_row_stride, uint8_t* out, int64_t out_row_stride,
+                            float* scales, const float* scale_ub, int64_t rows, int64_t hidden, void* stream);
+int vaq_fp8_quant_static(const void* in, int in_dtype, int64_t in_row_stride, uint8_t* out, int64_t out_row_stride,
+                         const float* scale, int64_t rows, int64_t hidden, void* stream);
+int vaq_fp8_quant_dynamic(const void* in, int in_dtype, int64_t in_row_stride, uint8_t* out, int64_t out_row_stride,
+                          float* scale, int64_t rows, int64_t hidden, void* stream);
+
+/*
+ * FP8 scaled GEMM  out[m,n] = round(sa[m] * (sb[n] * sum_k a[m,k] b[k,n]) + bias[n]).
+ * Replaces `cutlass_scaled_mm(Tensor! out, Tensor a, Tensor b, Tensor a_scales, Tensor b_scales, Tensor? bias)`
+ * (csrc/torch_bindings.cpp:412-414; csrc/quantization/w8a8/cutlass/scaled_mm_entry.cu:175-245; epilogue
+ * csrc/cutlass_extensions/epilogue/scaled_mm_epilogues_c3x.hpp:136-216).
+ *   a     e4m3fn [M, K] row-major, row stride lda bytes (lda % 16 == 0)
+ *   b     e4m3fn [K, N] COLUMN-major: element (k, n) at b[n * ldb + k]   (ldb % 16 == 0; ldb may exceed K)
+ *   sa    fp32, sa_count == 1 (per tensor) or M (per token);  sb fp32, sb_count == 1 or N (per channel)
+ *   bias  [N] of out dtype or NULL;  out [M, N] F16/BF16, row stride ldc elements (ldc % 8 == 0)
+ * K % 16 == 0 and N % 16 == 0 required (as the reference's cutlass path, vllm/_custom_ops.py:790-791).
+ */
+int vaq_fp8_scaled_mm(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t ldb, const float* sa, int64_t sa_count,
+                      const float* sb, int64_t sb_count, const void* bias, void* out, int64_t ldc, int out_dtype,
+                      int64_t size_m, int64_t size_n, int64_t size_k, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VLLM_AMD_QLINEAR_H_ */

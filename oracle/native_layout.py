@@ -1,0 +1,50 @@
+"""CPU statement of this build's own NATIVE weight order (no reference counterpart: the reference treats the
+repacked tensor as opaque, marlin.py:85-91 / :153-166).  TEST INFRASTRUCTURE ONLY.
+
+Tile (kt, nt) = rows 128*kt.., columns 16*nt.. is the 256-word block number kt*(N/16)+nt.  Word 4*L + j of a tile,
+L = 16*o + r, holds the codes of rows 128*kt + 32*j + 8*o + e (e = 0..7) of column 16*nt + r; code e sits in nibble
+position p with {0,2,4,6,1,3,5,7}[p] == e.  The inverse (`native_unpack`) is the documented map back to the logical
+[K, N] code matrix.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+_POS_TO_E = np.array([0, 2, 4, 6, 1, 3, 5, 7])
+
+
+def _index_maps(size_k: int, size_n: int):
+    """For every output word (flat index) the row index of its 8 codes (in nibble-position order) and its column."""
+    assert size_k % 128 == 0 and size_n % 16 == 0
+    n_tiles = size_n // 16
+    idx = np.arange(size_k * size_n // 8, dtype=np.int64)
+    j = idx & 3
+    lane = (idx >> 2) & 63
+    tile = idx >> 8
+    kt, nt = tile // n_tiles, tile % n_tiles
+    o, r = lane >> 4, lane & 15
+    k0 = kt * 128 + j * 32 + o * 8
+    n = nt * 16 + r
+    rows = k0[:, None] + _POS_TO_E[None, :]          # [words, 8] row of the code in nibble position p
+    return rows, n
+
+
+def native_pack(q: np.ndarray) -> np.ndarray:
+    """Logical codes int[K, N] (rows already in sorted order for act_order) -> int32 [K/16, 2N]."""
+    size_k, size_n = q.shape
+    rows, n = _index_maps(size_k, size_n)
+    codes = np.asarray(q).astype(np.uint32)[rows, n[:, None]]                 # [words, 8]
+    shifts = (np.arange(8, dtype=np.uint32) * 4)[None, :]
+    words = np.bitwise_or.reduce(codes << shifts, axis=1).astype(np.uint32)
+    return words.view(np.int32).reshape(size_k // 16, 2 * size_n)
+
+
+def native_unpack(packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    """Inverse of :func:`native_pack`."""
+    words = np.asarray(packed).reshape(-1).view(np.uint32)
+    rows, n = _index_maps(size_k, size_n)
+    shifts = (np.arange(8, dtype=np.uint32) * 4)[None, :]
+    codes = (words[:, None] >> shifts) & np.uint32(0xF)
+    q = np.zeros((size_k, size_n), dtype=np.int32)
+    q[rows, n[:, None]] = codes.astype(np.int32)
+    return q

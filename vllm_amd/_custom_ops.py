@@ -1,0 +1,462 @@
+"""Python op surface of the quantized-linear path, same names and call signatures as the reference's
+``vllm/_custom_ops.py`` (gptq_marlin_repack :1134-1141, gptq_marlin_gemm :1193-1232, scaled_fp8_quant :1456-1513,
+cutlass_scaled_mm :754-802, permute_cols), registered as PyTorch custom ops in the ``vllm_amd`` namespace with the
+schemas of ``csrc/torch_bindings.cpp`` (:304, :309-321, :412-414, :572-589) and fake (meta) implementations, and
+implemented by the gfx950 library through its C ABI.
+
+Argument validation repeats the reference's host checks (gptq_marlin.cu:689-902, gptq_marlin_repack.cu:255-280,
+scaled_mm_entry.cu:179-193, common.cu:217-220) and raises ``RuntimeError`` / ``NotImplementedError`` where the
+reference raises through ``TORCH_CHECK`` / ``TORCH_CHECK_NOT_IMPLEMENTED``.  There is no fallback: tensors that are
+not on a GPU are rejected.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _lib
+from .scalar_type import ScalarType, scalar_types
+
+FP8_DTYPE = torch.float8_e4m3fn        # gfx950 is an OCP part (reference: vllm/platforms/rocm.py:447-452)
+GPTQ_MARLIN_TILE = 16
+GPTQ_MARLIN_MIN_THREAD_N = 64
+GPTQ_MARLIN_MIN_THREAD_K = 128
+
+_LAYOUTS = {"marlin": _lib.VAQ_LAYOUT_MARLIN, "native": _lib.VAQ_LAYOUT_NATIVE}
+
+
+def _check(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _ptr(t: torch.Tensor | None):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(device: torch.device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _dtype_tag(dt: torch.dtype) -> int:
+    if dt == torch.float16:
+        return _lib.VAQ_F16
+    if dt == torch.bfloat16:
+        return _lib.VAQ_BF16
+    if dt == torch.float32:
+        return _lib.VAQ_F32
+    raise RuntimeError(f"unsupported dtype {dt}")
+
+
+def _is_gpu(t: torch.Tensor) -> bool:
+    return t.device.type == "cuda"
+
+
+# ============================================================================ repack
+
+def _check_repack_args(b_q_weight, perm, size_k, size_n, num_bits) -> None:
+    """Host checks of gptq_marlin_repack.cu:255-280, same order."""
+    _check(size_k % GPTQ_MARLIN_TILE == 0, f"size_k = {size_k} is not divisible by tile_k_size = {GPTQ_MARLIN_TILE}")
+    _check(size_n % GPTQ_MARLIN_MIN_THREAD_N == 0,
+           f"size_n = {size_n} is not divisible by tile_n_size = {GPTQ_MARLIN_MIN_THREAD_N}")
+    _check(num_bits in (4, 8), f"num_bits must be 4 or 8. Got = {num_bits}")
+    pack_factor = 32 // num_bits
+    _check(b_q_weight.dim() == 2 and size_k // pack_factor == b_q_weight.size(0),
+           f"Shape mismatch: b_q_weight.size(0) = {b_q_weight.size(0) if b_q_weight.dim() else None}, "
+           f"size_k = {size_k}, pack_factor = {pack_factor}")
+    _check(b_q_weight.size(1) == size_n, f"b_q_weight.size(1) = {b_q_weight.size(1)} is not size_n = {size_n}")
+    _check(_is_gpu(b_q_weight), "b_q_weight is not on GPU")
+    _check(b_q_weight.is_contiguous(), "b_q_weight is not contiguous")
+    _check(b_q_weight.dtype == torch.int32, "b_q_weight type is not kInt")
+    _check(_is_gpu(perm), "perm is not on GPU")
+    _check(perm.is_contiguous(), "perm is not contiguous")
+    _check(perm.dtype == torch.int32, "perm type is not at::kInt")
+    _check(perm.numel() in (0, size_k), f"perm.numel() = {perm.numel()} must be 0 or size_k = {size_k}")
+    if num_bits != 4:
+        raise NotImplementedError("gptq_marlin_repack: only num_bits = 4 is built for gfx950")
+
+
+def _repack_impl(b_q_weight: torch.Tensor, perm: torch.Tensor, size_k: int, size_n: int, num_bits: int,
+                 layout: int) -> torch.Tensor:
+    _check_repack_args(b_q_weight, perm, size_k, size_n, num_bits)
+    lib = _lib.load()
+    pack_factor = 32 // num_bits
+    with torch.cuda.device(b_q_weight.device):
+        out = torch.empty((size_k // GPTQ_MARLIN_TILE, size_n * GPTQ_MARLIN_TILE // pack_factor),
+                          dtype=torch.int32, device=b_q_weight.device)
+        _lib.check(lib.vaq_w4a16_repack(_ptr(b_q_weight), _ptr(perm) if perm.numel() else None, _ptr(out), size_k,
+                                        size_n, num_bits, layout, _stream(b_q_weight.device)))
+    return out
+
+
+def _repack_fake(b_q_weight, perm, size_k, size_n, num_bits, layout=0):
+    pack_factor = 32 // num_bits
+    return torch.empty((size_k // GPTQ_MARLIN_TILE, size_n * GPTQ_MARLIN_TILE // pack_factor),
+                       dtype=b_q_weight.dtype, device=b_q_weight.device)
+
+
+# ============================================================================ W4A16 GEMM
+
+def _opt(t: torch.Tensor | None) -> torch.Tensor | None:
+    """The reference passes 'absent' tensors as empty tensors (marlin_utils.py:261-270); presence is size(-1) > 0."""
+    if t is None or t.numel() == 0:
+        return None
+    return t
+
+
+def _check_gemm_args(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, g_idx, perm, workspace, b_q_type_id,
+                     size_m, size_n, size_k, is_k_full, is_zp_float):
+    """Host checks of gptq_marlin.cu:689-902 in the same order.  Returns (group_size, has_act_order, has_zp, wtype)."""
+    b_q_type = ScalarType.from_id(b_q_type_id)
+    _check(b_q_type.size_bits in (4, 8), f"unsupported weight type {b_q_type}")
+    pack_factor = 32 // b_q_type.size_bits
+    _check(a.dim() == 2 and a.size(0) == size_m, f"Shape mismatch: a.size(0) = {a.size(0)}, size_m = {size_m}")
+    _check(a.size(1) == size_k, f"Shape mismatch: a.size(1) = {a.size(1)}, size_k = {size_k}")
+    _check(size_k % GPTQ_MARLIN_TILE == 0, f"size_k = {size_k} is not divisible by tile_size = {GPTQ_MARLIN_TILE}")
+    _check(b_q_weight.dim() == 2 and size_k // GPTQ_MARLIN_TILE == b_q_weight.size(0),
+           f"Shape mismatch: b_q_weight.size(0) = {b_q_weight.size(0)}, size_k = {size_k}, tile_size = {GPTQ_MARLIN_TILE}")
+    _check(b_q_weight.size(1) % GPTQ_MARLIN_TILE == 0,
+           f"b_q_weight.size(1) = {b_q_weight.size(1)} is not divisible by tile_size = {GPTQ_MARLIN_TILE}")
+    actual_size_n = (b_q_weight.size(1) // GPTQ_MARLIN_TILE) * pack_factor
+    _check(size_n == actual_size_n, f"size_n = {size_n}, actual_size_n = {actual_size_n}")
+    _check(_is_gpu(a), "A is not on GPU")
+    _check(a.stride(1) == 1, "A.stride(1) is not 1")
+    _check(a.stride(0) % 8 == 0, "A.stride(0) must divisible by 8")
+    _check(a.data_ptr() % 16 == 0, "A must aligned to 16 bytes")
+    _check(_is_gpu(b_q_weight), "b_q_weight is not on GPU")
+    _check(b_q_weight.is_contiguous(), "b_q_weight is not contiguous")
+    _check(_is_gpu(b_scales), "b_scales is not on GPU")
+    _check(b_scales.is_contiguous(), "b_scales is not contiguous")
+    if c is not None:
+        _check(_is_gpu(c), "c is not on GPU")
+        _check(c.is_contiguous(), "c is not contiguous")
+        _check(c.size(0) == size_m, f"Shape mismatch: c.size(0) = {c.size(0)}, size_m = {size_m}")
+        _check(c.size(1) == size_n, f"Shape mismatch: c.size(1) = {c.size(1)}, size_n = {size_n}")
+    _check(b_scales.dim() == 2, f"b_scales rank = {b_scales.dim()} is not 2")
+    _check(b_scales.size(1) == size_n, f"b_scales dim 1 = {b_scales.size(1)} is not size_n = {size_n}")
+    num_groups = b_scales.size(0)
+
+    has_act_order = False
+    if g_idx is not None and perm is not None:
+        _check(_is_gpu(g_idx), "g_idx is not on GPU")
+        _check(g_idx.is_contiguous(), "g_idx is not contiguous")
+        _check(_is_gpu(perm), "perm is not on GPU")
+        _check(perm.is_contiguous(), "perm is not contiguous")
+        _check((g_idx.size(-1) == 0 and perm.size(-1) == 0) or (g_idx.size(-1) == size_k and perm.size(-1) == size_k),
+               f"Unexpected g_idx.size(-1) = {g_idx.size(-1)} and perm.size(-1) = {perm.size(-1)}, where size_k = {size_k}")
+        has_act_order = g_idx.size(-1) > 0 and perm.size(-1) > 0
+    if has_act_order:
+        if is_k_full:
+            _check(num_groups > 1, "For act_order, num_groups must be > 1")
+            _check(size_k % num_groups == 0, f"size_k = {size_k}, is not divisible by num_groups = {num_groups}")
+            group_size = size_k // num_groups
+        else:
+            group_size = 0
+    elif num_groups > 1:
+        _check(size_k % num_groups == 0, f"size_k = {size_k}, is not divisible by b_scales.size(0) = {b_scales.size(0)}")
+        group_size = size_k // num_groups
+    else:
+        group_size = -1
+
+    _check(global_scale is None, "global_scale can only be used for nvfp4 format.")
+    if b_bias is not None:
+        _check(_is_gpu(b_bias), "b_bias is not on GPU")
+        _check(b_bias.is_contiguous(), "b_bias is not contiguous")
+        _check(b_bias.size(0) == size_n, "b_bias.size(0) != size_n")
+        _check(b_bias.stride(0) == 1, "b_bias.stride(0) != 1")
+    has_zp = b_zeros is not None and b_zeros.size(-1) > 0
+    if b_zeros is not None:
+        _check(_is_gpu(b_zeros), "b_zeros is not on GPU")
+        _check(b_zeros.is_contiguous(), "b_zeros is not contiguous")
+    if has_zp:
+        _check(b_q_type in (scalar_types.uint4, scalar_types.uint8),
+               f"b_q_type must be u4 or u8 when has_zp = True. Got = {b_q_type}")
+    else:
+        _check(b_q_type in (scalar_types.uint4b8, scalar_types.uint8b128, scalar_types.float8_e4m3fn),
+               "b_q_type must be uint4b8, uint8b128, float8_e4m3fn or float4_e2m1f when has_zp = False. "
+               f"Got = {b_q_type}")
+    if has_zp and is_zp_float:
+        _check(a.dtype == torch.float16, "Computation type must be float16 (half) when using float zero points.")
+    if has_zp:
+        _check(b_zeros.dim() == 2, f"b_zeros rank = {b_zeros.dim()} is not 2")
+        if is_zp_float:
+            _check(b_zeros.size(1) == size_n, f"b_zeros dim 1 = {b_zeros.size(1)} is not size_n = {size_n}")
+            _check(num_groups == b_zeros.size(0), f"b_zeros dim 0 = {b_zeros.size(0)} is not num_groups = {num_groups}")
+        else:
+            _check(b_zeros.size(0) == num_groups, f"b_zeros dim 0 = {b_zeros.size(0)} is not num_groups = {num_groups}")
+            _check(b_zeros.size(1) == size_n // pack_factor,
+                   f"b_zeros dim 1 = {b_zeros.size(1)} is not size_n / pack_factor = {size_n // pack_factor}")
+    _check(size_n % GPTQ_MARLIN_MIN_THREAD_N == 0,
+           f"size_n = {size_n}, is not divisible by min_thread_n = {GPTQ_MARLIN_MIN_THREAD_N}")
+    _check(_is_gpu(workspace) and workspace.dtype == torch.int32, "workspace must be an int32 tensor on GPU")
+    _check(a.dtype in (torch.float16, torch.bfloat16), "gpt_marlin_gemm only supports bfloat16 and float16")
+    _check(b_scales.dtype == a.dtype, f"b_scales dtype {b_scales.dtype} must equal the activation dtype {a.dtype}")
+
+    # what this build implements out of everything the reference accepts
+    if b_q_type.size_bits != 4 or b_q_type not in (scalar_types.uint4, scalar_types.uint4b8):
+        raise NotImplementedError(f"gptq_marlin_gemm: weight type {b_q_type} is not built for gfx950 (uint4b8 / uint4)")
+    if is_zp_float:
+        raise NotImplementedError("gptq_marlin_gemm: float zero points (is_zp_float) are not built for gfx950")
+    if has_act_order and not is_k_full:
+        raise NotImplementedError("gptq_marlin_gemm: is_k_full = False (act_order x row-parallel shard) is not built; "
+                                  "one-GPU layers always have is_k_full = True")
+    if group_size != 128:
+        raise NotImplementedError(f"gptq_marlin_gemm: group_size = {group_size} is not built for gfx950 (only 128)")
+    _check(size_k % GPTQ_MARLIN_MIN_THREAD_K == 0,
+           f"size_k = {size_k}, is not divisible by min_thread_k = {GPTQ_MARLIN_MIN_THREAD_K}")
+    wtype = _lib.VAQ_WTYPE_U4 if has_zp else _lib.VAQ_WTYPE_U4B8
+    return group_size, has_act_order, has_zp, wtype
+
+
+def _gemm_impl(a: torch.Tensor, c_or_none: torch.Tensor | None, b_q_weight: torch.Tensor,
+               b_bias_or_none: torch.Tensor | None, b_scales: torch.Tensor, global_scale: torch.Tensor | None,
+               b_zeros_or_none: torch.Tensor | None, g_idx_or_none: torch.Tensor | None,
+               perm_or_none: torch.Tensor | None, workspace: torch.Tensor, b_q_type: int, size_m: int, size_n: int,
+               size_k: int, is_k_full: bool = True, use_atomic_add: bool = False, use_fp32_reduce: bool = False,
+               is_zp_float: bool = False) -> torch.Tensor:
+    # use_atomic_add / use_fp32_reduce select Marlin reduction variants; this build always reduces in fp32.
+    group_size, has_act_order, has_zp, wtype = _check_gemm_args(
+        a, c_or_none, b_q_weight, b_bias_or_none, b_scales, global_scale, b_zeros_or_none, g_idx_or_none, perm_or_none,
+        workspace, b_q_type, size_m, size_n, size_k, is_k_full, is_zp_float)
+    lib = _lib.load()
+    dev = a.device
+    with torch.cuda.device(dev):
+        c = c_or_none if c_or_none is not None else torch.empty((size_m, size_n), dtype=a.dtype, device=dev)
+        if size_m == 0:
+            return c
+        n_ctmp, n_atmp, n_cnt = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+        _lib.check(lib.vaq_w4a16_gemm_workspace(size_m, size_n, size_k, int(has_act_order), dev.index or 0,
+                                                ctypes.byref(n_ctmp), ctypes.byref(n_atmp), ctypes.byref(n_cnt)))
+        _check(workspace.numel() >= n_cnt.value,
+               f"workspace.numel = {workspace.numel()} is below min_workspace_size = {n_cnt.value}")
+        c_tmp = torch.empty((n_ctmp.value // 4,), dtype=torch.float32, device=dev) if n_ctmp.value else None
+        a_tmp = torch.empty((n_atmp.value // 2,), dtype=a.dtype, device=dev) if n_atmp.value else None
+        _lib.check(lib.vaq_w4a16_gemm(
+            _ptr(a), a.stride(0), _ptr(b_q_weight), _ptr(b_scales), _ptr(b_zeros_or_none) if has_zp else None,
+            _ptr(perm_or_none) if has_act_order else None, _ptr(b_bias_or_none), _ptr(c), _ptr(c_tmp), _ptr(a_tmp),
+            _ptr(workspace), workspace.numel(), size_m, size_n, size_k, group_size, _dtype_tag(a.dtype), wtype, 0,
+            _stream(dev)))
+    return c
+
+
+def _gemm_fake(a, c_or_none, b_q_weight, b_bias_or_none, b_scales, global_scale, b_zeros_or_none, g_idx_or_none,
+               perm_or_none, workspace, b_q_type, size_m, size_n, size_k, is_k_full=True, use_atomic_add=False,
+               use_fp32_reduce=False, is_zp_float=False):
+    return torch.empty((size_m, size_n), device=a.device, dtype=a.dtype)
+
+
+# ============================================================================ permute_cols
+
+def _permute_cols_impl(A: torch.Tensor, perm: torch.Tensor) -> torch.Tensor:
+    _check(_is_gpu(A) and _is_gpu(perm), "A and perm must be on GPU")
+    _check(A.dtype in (torch.float16, torch.bfloat16), "Currently only 16bit types are supported")
+    _check(A.dim() == 2 and A.stride(1) == 1, "A must be a 2-D tensor with unit column stride")
+    _check(perm.dtype == torch.int32 and perm.is_contiguous() and perm.numel() == A.size(1),
+           "perm must be a contiguous int32 tensor of A.size(1) entries")
+    _check(A.size(1) % 8 == 0, "A columns must be a multiple of 8")
+    lib = _lib.load()
+    with torch.cuda.device(A.device):
+        out = torch.empty((A.size(0), A.size(1)), dtype=A.dtype, device=A.device)
+        _lib.check(lib.vaq_permute_cols(_ptr(A), A.stride(0), _ptr(perm), _ptr(out), A.size(0), A.size(1),
+                                        _stream(A.device)))
+    return out
+
+
+def _permute_cols_fake(A, perm):
+    return torch.empty_like(A, memory_format=torch.contiguous_format)
+
+
+# ============================================================================ FP8 activation quantisation
+
+def _check_quant_io(result: torch.Tensor, input: torch.Tensor) -> tuple[int, int]:
+    """common.cu:139-142 / :217-220 checks; returns (num_tokens, hidden)."""
+    _check(_is_gpu(input) and _is_gpu(result), "input and result must be on GPU")
+    _check(input.dim() >= 1 and input.stride(-1) == 1, "last dimension of input must be contiguous")
+    _check(result.stride(-1) == 1, "last dimension of output must be contiguous")
+    _check(result.dtype == FP8_DTYPE, f"result must be {FP8_DTYPE}")
+    _check(input.dtype in (torch.float16, torch.bfloat16, torch.float32), f"unsupported input dtype {input.dtype}")
+    _check(input.dim() == 2 and result.dim() == 2, "input and result must be 2-D")
+    hidden = input.size(-1)
+    tokens = input.numel() // hidden if hidden else 0
+    _check(result.size(-1) == hidden and result.size(0) >= tokens, "result shape does not cover input")
+    return tokens, hidden
+
+
+def _static_quant_impl(result: torch.Tensor, input: torch.Tensor, scale: torch.Tensor) -> None:
+    tokens, hidden = _check_quant_io(result, input)
+    _check(_is_gpu(scale) and scale.dtype == torch.float32 and scale.numel() == 1, "scale must be one fp32 on GPU")
+    if tokens == 0:
+        return
+    lib = _lib.load()
+    with torch.cuda.device(input.device):
+        _lib.check(lib.vaq_fp8_quant_static(_ptr(input), _dtype_tag(input.dtype), input.stride(0), _ptr(result),
+                                            result.stride(0), _ptr(scale), tokens, hidden, _stream(input.device)))
+
+
+def _dynamic_quant_impl(result: torch.Tensor, input: torch.Tensor, scale: torch.Tensor) -> None:
+    tokens, hidden = _check_quant_io(result, input)
+    _check(_is_gpu(scale) and scale.dtype == torch.float32 and scale.numel() == 1, "scale must be one fp32 on GPU")
+    if tokens == 0:
+        return
+    lib = _lib.load()
+    with torch.cuda.device(input.device):
+        _lib.check(lib.vaq_fp8_quant_dynamic(_ptr(input), _dtype_tag(input.dtype), input.stride(0), _ptr(result),
+                                             result.stride(0), _ptr(scale), tokens, hidden, _stream(input.device)))
+
+
+def _per_token_quant_impl(result: torch.Tensor, input: torch.Tensor, scale: torch.Tensor,
+                          scale_ub: torch.Tensor | None) -> None:
+    tokens, hidden = _check_quant_io(result, input)
+    _check(_is_gpu(scale) and scale.dtype == torch.float32 and scale.is_contiguous() and scale.numel() >= tokens,
+           "scale must be a contiguous fp32 tensor with one entry per token")
+    if scale_ub is not None:
+        _check(_is_gpu(scale_ub) and scale_ub.dtype == torch.float32 and scale_ub.numel() == 1,
+               "scale_ub must be one fp32 on GPU")
+    if tokens == 0:
+        return
+    lib = _lib.load()
+    with torch.cuda.device(input.device):
+        _lib.check(lib.vaq_fp8_quant_per_token(_ptr(input), _dtype_tag(input.dtype), input.stride(0), _ptr(result),
+                                               result.stride(0), _ptr(scale), _ptr(scale_ub), tokens, hidden,
+                                               _stream(input.device)))
+
+
+# ============================================================================ FP8 scaled GEMM
+
+def _check_scaled_mm_args(out, a, b, a_scales, b_scales, bias) -> None:
+    """scaled_mm_entry.cu:179-193 plus the scale-shape rules of c3x/scaled_mm_helper.hpp:5-52."""
+    _check(a.dim() == 2 and b.dim() == 2 and out.dim() == 2, "a, b and out must be 2-D")
+    _check(out.size(0) == a.size(0) and a.size(1) == b.size(0) and b.size(1) == out.size(1),
+           f"shape mismatch: a {tuple(a.shape)}, b {tuple(b.shape)}, out {tuple(out.shape)}")
+    _check(a.stride(1) == 1 and out.stride(1) == 1, "a and out must be row-major")
+    _check(b.stride(0) == 1, "b must be column-major")
+    _check(out.stride(0) % 16 == 0 and b.stride(1) % 16 == 0, "out.stride(0) and b.stride(1) must be multiples of 16")
+    if bias is not None:
+        _check(bias.numel() == b.size(1) and bias.is_contiguous() and bias.dim() == 1, "bias must be contiguous [N]")
+        _check(bias.dtype == out.dtype, "bias dtype must equal the output dtype")
+    _check(all(_is_gpu(t) for t in (out, a, b, a_scales, b_scales)), "all tensors must be on GPU")
+    _check(a_scales.dtype == torch.float32 and b_scales.dtype == torch.float32, "scales must be fp32")
+    _check(a_scales.is_contiguous() and b_scales.is_contiguous(), "scales must be contiguous")
+    _check(a_scales.numel() in (1, a.size(0)), f"a_scales.numel() = {a_scales.numel()} must be 1 or M = {a.size(0)}")
+    _check(b_scales.numel() in (1, b.size(1)), f"b_scales.numel() = {b_scales.numel()} must be 1 or N = {b.size(1)}")
+    _check(out.dtype in (torch.float16, torch.bfloat16), "out must be float16 or bfloat16")
+    if a.dtype != FP8_DTYPE or b.dtype != FP8_DTYPE:
+        raise NotImplementedError(f"cutlass_scaled_mm: only {FP8_DTYPE} x {FP8_DTYPE} is built for gfx950 "
+                                  f"(got {a.dtype} x {b.dtype})")
+    _check(a.stride(0) % 16 == 0, "a.stride(0) must be a multiple of 16")
+    _check(b.size(0) % 16 == 0 and b.size(1) % 16 == 0, "K and N must be multiples of 16")
+
+
+def _scaled_mm_impl(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor, a_scales: torch.Tensor,
+                    b_scales: torch.Tensor, bias: torch.Tensor | None) -> None:
+    _check_scaled_mm_args(out, a, b, a_scales, b_scales, bias)
+    if a.size(0) == 0:
+        return
+    lib = _lib.load()
+    with torch.cuda.device(a.device):
+        _lib.check(lib.vaq_fp8_scaled_mm(_ptr(a), a.stride(0), _ptr(b), b.stride(1), _ptr(a_scales), a_scales.numel(),
+                                         _ptr(b_scales), b_scales.numel(), _ptr(bias), _ptr(out), out.stride(0),
+                                         _dtype_tag(out.dtype), a.size(0), b.size(1), a.size(1), _stream(a.device)))
+
+
+# ============================================================================ registration
+
+_NS = "vllm_amd"
+_library = torch.library.Library(_NS, "FRAGMENT")
+
+
+def _register(name: str, schema: str, impl, fake=None) -> None:
+    _library.define(f"{name}{schema}")
+    _library.impl(name, impl, "CUDA")
+    if fake is not None:
+        torch.library.register_fake(f"{_NS}::{name}", fake, lib=_library)
+
+
+_register("gptq_marlin_repack",
+          "(Tensor b_q_weight, Tensor perm, SymInt size_k, SymInt size_n, int num_bits, int layout=1) -> Tensor",
+          _repack_impl, _repack_fake)
+_register("gptq_marlin_gemm",
+          "(Tensor a, Tensor? c_or_none, Tensor b_q_weight, Tensor? b_bias_or_none, Tensor b_scales, "
+          "Tensor? global_scale, Tensor? b_zeros_or_none, Tensor? g_idx_or_none, Tensor? perm_or_none, "
+          "Tensor workspace, int b_q_type, SymInt size_m, SymInt size_n, SymInt size_k, bool is_k_full=True, "
+          "bool use_atomic_add=False, bool use_fp32_reduce=False, bool is_zp_float=False) -> Tensor",
+          _gemm_impl, _gemm_fake)
+_register("permute_cols", "(Tensor A, Tensor perm) -> Tensor", _permute_cols_impl, _permute_cols_fake)
+_register("static_scaled_fp8_quant", "(Tensor! result, Tensor input, Tensor scale) -> ()", _static_quant_impl,
+          lambda result, input, scale: None)
+_register("dynamic_scaled_fp8_quant", "(Tensor! result, Tensor input, Tensor! scale) -> ()", _dynamic_quant_impl,
+          lambda result, input, scale: None)
+_register("dynamic_per_token_scaled_fp8_quant", "(Tensor! result, Tensor input, Tensor! scale, Tensor? scale_ub) -> ()",
+          _per_token_quant_impl, lambda result, input, scale, scale_ub: None)
+_register("cutlass_scaled_mm", "(Tensor! out, Tensor a, Tensor b, Tensor a_scales, Tensor b_scales, Tensor? bias) -> ()",
+          _scaled_mm_impl, lambda out, a, b, a_scales, b_scales, bias: None)
+
+_ops = getattr(torch.ops, _NS)
+
+
+# ============================================================================ public wrappers (reference signatures)
+
+def gptq_marlin_repack(b_q_weight: torch.Tensor, perm: torch.Tensor, size_k: int, size_n: int, num_bits: int, *,
+                       layout: str = "native") -> torch.Tensor:
+    """GPTQ int32[K/8, N] -> repacked int32[K/16, 2N].
+
+    ``layout="native"`` (default) is the wavefront tile order ``gptq_marlin_gemm`` consumes; ``layout="marlin"``
+    reproduces the reference's Marlin order bit-for-bit.  Callers treat the result as opaque either way.
+    """
+    return _ops.gptq_marlin_repack(b_q_weight, perm, size_k, size_n, num_bits, _LAYOUTS[layout])
+
+
+def gptq_marlin_gemm(a: torch.Tensor, c: torch.Tensor | None, b_q_weight: torch.Tensor, b_bias: torch.Tensor | None,
+                     b_scales: torch.Tensor, global_scale: torch.Tensor | None, b_zeros: torch.Tensor | None,
+                     g_idx: torch.Tensor | None, perm: torch.Tensor | None, workspace: torch.Tensor,
+                     b_q_type: ScalarType, size_m: int, size_n: int, size_k: int, is_k_full: bool = True,
+                     use_atomic_add: bool = False, use_fp32_reduce: bool = False,
+                     is_zp_float: bool = False) -> torch.Tensor:
+    return _ops.gptq_marlin_gemm(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, g_idx, perm, workspace,
+                                 b_q_type.id, size_m, size_n, size_k, is_k_full, use_atomic_add, use_fp32_reduce,
+                                 is_zp_float)
+
+
+def permute_cols(a: torch.Tensor, perm: torch.Tensor) -> torch.Tensor:
+    return _ops.permute_cols(a, perm)
+
+
+def scaled_fp8_quant(input: torch.Tensor, scale: torch.Tensor | None = None, num_token_padding: int | None = None,
+                     scale_ub: torch.Tensor | None = None, use_per_token_if_dynamic: bool = False,
+                     output: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """Quantise ``input`` [tokens, hidden] to FP8 (e4m3fn); static if ``scale`` is given, else dynamic per tensor or,
+    with ``use_per_token_if_dynamic``, per token.  Rows beyond ``input.shape[0]`` of a padded output are left
+    uninitialised, as in the reference."""
+    assert input.ndim == 2
+    shape = tuple(input.shape)
+    if num_token_padding:
+        shape = (max(num_token_padding, input.shape[0]), shape[1])
+    if output is None:
+        output = torch.empty(shape, device=input.device, dtype=FP8_DTYPE)
+    else:
+        assert num_token_padding is None, "padding not supported if output passed in"
+        assert output.dtype == FP8_DTYPE
+    if scale is None:
+        if use_per_token_if_dynamic:
+            scale = torch.empty((shape[0], 1), device=input.device, dtype=torch.float32)
+            _ops.dynamic_per_token_scaled_fp8_quant(output, input, scale, scale_ub)
+        else:
+            scale = torch.empty((1, 1), device=input.device, dtype=torch.float32)
+            _ops.dynamic_scaled_fp8_quant(output, input, scale)
+    else:
+        assert scale.numel() == 1, f"{scale.shape}"
+        _ops.static_scaled_fp8_quant(output, input, scale)
+    return output, scale
+
+
+def cutlass_scaled_mm(a: torch.Tensor, b: torch.Tensor, scale_a: torch.Tensor, scale_b: torch.Tensor,
+                      out_dtype: torch.dtype, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """``(scale_a * a) @ (scale_b * b) + bias`` with fp8 ``a`` [M,K] row-major, ``b`` [K,N] column-major, fused."""
+    assert out_dtype is torch.bfloat16 or out_dtype is torch.float16
+    assert bias is None or bias.numel() == b.shape[1] and bias.dtype == out_dtype
+    target_shape = (*a.shape[:-1], b.shape[1])
+    a = a.view(-1, a.shape[-1])
+    out = torch.empty((a.shape[0], b.shape[1]), dtype=out_dtype, device=a.device)
+    _ops.cutlass_scaled_mm(out, a, b, scale_a, scale_b, bias)
+    return out.view(*target_shape)

@@ -1,0 +1,87 @@
+"""ctypes binding of ``libvllm_amd_qlinear.so`` (the C ABI in ``include/vllm_amd_qlinear.h``).
+
+Loading is lazy and loud: if the shared object is missing the first op call raises ``RuntimeError`` -- there is no
+fallback implementation.  Build it with ``python -m vllm_amd.build``.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p, POINTER
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libvllm_amd_qlinear.so"
+
+VAQ_OK = 0
+VAQ_ERR_INVALID_ARG = -1
+VAQ_ERR_UNSUPPORTED = -2
+VAQ_ERR_LAUNCH = -3
+
+VAQ_F16, VAQ_BF16, VAQ_F32 = 0, 1, 2
+VAQ_LAYOUT_MARLIN, VAQ_LAYOUT_NATIVE = 0, 1
+VAQ_WTYPE_U4B8, VAQ_WTYPE_U4 = 0, 1
+
+# name -> (restype, argtypes); must list every symbol the header declares (tests check this against the header)
+_SIGNATURES = {
+    "vaq_last_error": (c_char_p, []),
+    "vaq_abi_version": (c_int, []),
+    "vaq_num_cus": (c_int, [c_int]),
+    "vaq_w4a16_repack": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_int, c_void_p]),
+    "vaq_w4a16_gemm_workspace": (c_int, [c_int64, c_int64, c_int64, c_int, c_int, POINTER(c_size_t), POINTER(c_size_t),
+                                         POINTER(c_size_t)]),
+    "vaq_w4a16_gemm": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int,
+                               c_void_p]),
+    "vaq_permute_cols": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
+    "vaq_fp8_quant_per_token": (c_int, [c_void_p, c_int, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
+                                        c_int64, c_void_p]),
+    "vaq_fp8_quant_static": (c_int, [c_void_p, c_int, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p]),
+    "vaq_fp8_quant_dynamic": (c_int, [c_void_p, c_int, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64,
+                                      c_void_p]),
+    "vaq_fp8_scaled_mm": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
+                                  c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p]),
+}
+# tuning aids exported by the library but not part of the drop-in header
+_DEBUG_SIGNATURES = {
+    "vaq_debug_set_decode_config": (None, [c_int, c_int, c_int]),
+    "vaq_debug_set_prefill_tile": (None, [c_int]),
+    "vaq_debug_set_fp8_config": (None, [c_int, c_int]),
+}
+
+_lib = None
+
+
+def exported_symbols() -> list[str]:
+    return sorted(_SIGNATURES)
+
+
+def load() -> ctypes.CDLL:
+    """Return the loaded library, loading it on first use.  Raises RuntimeError if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: the gfx950 kernels are not built (run `python -m vllm_amd.build`). "
+            "vllm_amd has no fallback path.")
+    lib = ctypes.CDLL(str(LIB_PATH))
+    for name, (res, args) in {**_SIGNATURES, **_DEBUG_SIGNATURES}.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError:
+            if name in _DEBUG_SIGNATURES:
+                continue
+            raise RuntimeError(f"{LIB_PATH} does not export {name}; rebuild it") from None
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(status: int) -> None:
+    """Translate a C-ABI status into the exception the reference would raise for the same condition."""
+    if status == VAQ_OK:
+        return
+    msg = load().vaq_last_error().decode("utf-8", "replace")
+    if status == VAQ_ERR_UNSUPPORTED:
+        raise NotImplementedError(msg)
+    raise RuntimeError(msg)

@@ -1,0 +1,234 @@
+// FP8 (OCP e4m3fn) activation quantisation for gfx950: per-token dynamic, per-tensor dynamic, per-tensor static.
+//
+// Bit-exactness contract (codes AND scales) with the reference kernels:
+//   per token : amax = max|float(x)| ; s = max(min(amax, ub) / 448, 1/(448*512)) ; q = cvt(clamp(float(x) / s, +-448))
+//               -- a true IEEE fp32 division per element, not a reciprocal multiply;
+//   per tensor: s = amax_all / 448 ; q = cvt(clamp(float(x) * (1 / s), +-448))   (reciprocal multiply);
+//   static    : q = cvt(clamp(float(x) * (1 / scale), +-448)).
+// cvt is the hardware v_cvt_pk_fp8_f32 (round-to-nearest-even; inputs are already clamped, NaN stays NaN).
+// The file is compiled without fast-math, so `/` is the correctly rounded division.
+//
+// HBM-bound: each row is read ONCE -- a workgroup keeps its whole row in registers between the absmax pass and the
+// convert pass whenever the row has at most 256 threads x 8 vectors x 8 elements = 16384 elements and is 16-byte
+// aligned; other rows take a two-pass scalar path.
+#include "vaq_common.h"
+
+namespace vaq {
+
+constexpr float FP8_MAX = 448.0f;
+constexpr int QT = 256;         // threads per workgroup
+constexpr int QV = 8;           // cached 8-element vectors per thread
+
+template <typename T>
+__device__ inline float load_as_float(const T* p);
+template <>
+__device__ inline float load_as_float<float>(const float* p) { return *p; }
+struct bf16_t { uint16_t v; };
+struct f16_t { uint16_t v; };
+template <>
+__device__ inline float load_as_float<bf16_t>(const bf16_t* p) { return F16Traits<true>::to_float(p->v); }
+template <>
+__device__ inline float load_as_float<f16_t>(const f16_t* p) { return F16Traits<false>::to_float(p->v); }
+
+__device__ inline float clamp448(float x) { return fmaxf(-FP8_MAX, fminf(x, FP8_MAX)); }
+
+// two fp32 -> two e4m3fn codes in the low 16 bits
+__device__ inline uint32_t cvt2(float a, float b) { return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xffffu; }
+__device__ inline uint8_t cvt1(float a) { return (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(a, a, 0, false) & 0xff); }
+
+// 8 consecutive elements of a row as floats
+template <typename T>
+struct Vec8 {
+  float f[8];
+  __device__ inline void load(const T* p) {
+    if constexpr (sizeof(T) == 2) {
+      const v4u r = *reinterpret_cast<const v4u*>(p);
+      const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        T lo, hi;
+        lo.v = (uint16_t)(w[i] & 0xffffu);
+        hi.v = (uint16_t)(w[i] >> 16);
+        f[2 * i] = load_as_float<T>(&lo);
+        f[2 * i + 1] = load_as_float<T>(&hi);
+      }
+    } else {
+      const v4f a = *reinterpret_cast<const v4f*>(p);
+      const v4f b = *reinterpret_cast<const v4f*>(p + 4);
+      f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w;
+      f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+    }
+  }
+};
+
+__device__ inline float block_max(float v, float* smem) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0) smem[wave] = v;
+  __syncthreads();
+  float r = smem[0];
+#pragma unroll
+  for (int i = 1; i < QT / 64; ++i) r = fmaxf(r, smem[i]);
+  __syncthreads();
+  return r;
+}
+
+// MODE 0: dynamic per token (divide by row scale, scale written per row)
+// MODE 1: per tensor with a given scale (multiply by reciprocal) -- static, and pass 2 of dynamic per tensor
+// MODE 2: absmax only: atomic max of rowmax/448 into *scale (pass 1 of dynamic per tensor)
+template <typename T, int MODE>
+__global__ __launch_bounds__(QT) void fp8_quant_kernel(const T* __restrict__ in, int64_t in_stride,
+                                                        uint8_t* __restrict__ out, int64_t out_stride,
+                                                        float* __restrict__ scales, const float* __restrict__ scale_ub,
+                                                        int hidden) {
+  __shared__ float smem[QT / 64];
+  const int64_t row = blockIdx.x;
+  const T* x = in + row * in_stride;
+  uint8_t* y = out + row * out_stride;
+  const int tid = threadIdx.x;
+
+  const bool vec_ok = (hidden % 8 == 0) && (((uintptr_t)x % 16) == 0) && (((uintptr_t)y % 8) == 0) &&
+                      (hidden <= QT * QV * 8);
+  Vec8<T> cache[QV];
+  const int nvec = hidden / 8;
+
+  float scale_or_inv;
+  if constexpr (MODE != 1) {
+    float amax = 0.f;
+    if (vec_ok) {
+#pragma unroll
+      for (int i = 0; i < QV; ++i) {
+        const int v = tid + i * QT;
+        if (v < nvec) {
+          cache[i].load(x + (int64_t)v * 8);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(cache[i].f[e]));
+        }
+      }
+    } else {
+      for (int e = tid; e < hidden; e += QT) amax = fmaxf(amax, fabsf(load_as_float<T>(x + e)));
+    }
+    amax = block_max(amax, smem);
+    if constexpr (MODE == 2) {
+      // non-negative floats order like their bit patterns
+      if (tid == 0) atomicMax(reinterpret_cast<int*>(scales), __float_as_int(amax / FP8_MAX));
+      return;
+    } else {
+      float s = scale_ub ? fminf(amax, *scale_ub) : amax;
+      s = fmaxf(s / FP8_MAX, 1.0f / (FP8_MAX * 512.0f));
+      if (tid == 0) scales[row] = s;
+      scale_or_inv = s;
+    }
+  } else {
+    scale_or_inv = 1.0f / (*scales);
+    if (vec_ok) {
+#pragma unroll
+      for (int i = 0; i < QV; ++i) {
+        const int v = tid + i * QT;
+        if (v < nvec) cache[i].load(x + (int64_t)v * 8);
+      }
+    }
+  }
+
+  auto conv = [&](float v) -> float {
+    if constexpr (MODE == 0) return clamp448(v / scale_or_inv);
+    else return clamp448(v * scale_or_inv);
+  };
+
+  if (vec_ok) {
+#pragma unroll
+    for (int i = 0; i < QV; ++i) {
+      const int v = tid + i * QT;
+      if (v < nvec) {
+        v2u o;
+        o.x = cvt2(conv(cache[i].f[0]), conv(cache[i].f[1])) | (cvt2(conv(cache[i].f[2]), conv(cache[i].f[3])) << 16);
+        o.y = cvt2(conv(cache[i].f[4]), conv(cache[i].f[5])) | (cvt2(conv(cache[i].f[6]), conv(cache[i].f[7])) << 16);
+        *reinterpret_cast<v2u*>(y + (int64_t)v * 8) = o;
+      }
+    }
+  } else {
+    for (int e = tid; e < hidden; e += QT) y[e] = cvt1(conv(load_as_float<T>(x + e)));
+  }
+}
+
+__global__ void fill_zero_kernel(float* p) { *p = 0.f; }
+
+template <int MODE>
+static int launch_quant(const void* in, int in_dtype, int64_t in_stride, uint8_t* out, int64_t out_stride,
+                        float* scales, const float* ub, int64_t rows, int64_t hidden, hipStream_t s) {
+  const dim3 grid((unsigned)rows), block(QT);
+  switch (in_dtype) {
+    case VAQ_BF16:
+      hipLaunchKernelGGL((fp8_quant_kernel<bf16_t, MODE>), grid, block, 0, s, (const bf16_t*)in, in_stride, out,
+                         out_stride, scales, ub, (int)hidden);
+      break;
+    case VAQ_F16:
+      hipLaunchKernelGGL((fp8_quant_kernel<f16_t, MODE>), grid, block, 0, s, (const f16_t*)in, in_stride, out,
+                         out_stride, scales, ub, (int)hidden);
+      break;
+    case VAQ_F32:
+      hipLaunchKernelGGL((fp8_quant_kernel<float, MODE>), grid, block, 0, s, (const float*)in, in_stride, out,
+                         out_stride, scales, ub, (int)hidden);
+      break;
+    default:
+      set_error("fp8_quant: unsupported input dtype tag %d", in_dtype);
+      return VAQ_ERR_INVALID_ARG;
+  }
+  return VAQ_OK;
+}
+
+static int check_quant(const char* who, const void* in, int64_t in_stride, const uint8_t* out, int64_t out_stride,
+                       const float* scale, int64_t rows, int64_t hidden) {
+  VAQ_CHECK_ARG(rows >= 0 && hidden > 0, "%s: bad shape [%lld, %lld]", who, (long long)rows, (long long)hidden);
+  VAQ_CHECK_ARG(rows < (1ll << 31) && hidden < (1ll << 31), "%s: shape too large", who);
+  VAQ_CHECK_ARG(in_stride >= hidden && out_stride >= hidden, "%s: row strides (%lld, %lld) smaller than hidden = %lld",
+                who, (long long)in_stride, (long long)out_stride, (long long)hidden);
+  if (rows > 0) VAQ_CHECK_ARG(in && out && scale, "%s: null pointer", who);
+  return VAQ_OK;
+}
+
+}  // namespace vaq
+
+extern "C" int vaq_fp8_quant_per_token(const void* in, int in_dtype, int64_t in_row_stride, uint8_t* out,
+                                       int64_t out_row_stride, float* scales, const float* scale_ub, int64_t rows,
+                                       int64_t hidden, void* stream) {
+  using namespace vaq;
+  int rc = check_quant("fp8_quant_per_token", in, in_row_stride, out, out_row_stride, scales, rows, hidden);
+  if (rc != VAQ_OK || rows == 0) return rc;
+  rc = launch_quant<0>(in, in_dtype, in_row_stride, out, out_row_stride, scales, scale_ub, rows, hidden,
+                       (hipStream_t)stream);
+  if (rc != VAQ_OK) return rc;
+  VAQ_CHECK_LAUNCH("fp8_quant_per_token");
+  return VAQ_OK;
+}
+
+extern "C" int vaq_fp8_quant_static(const void* in, int in_dtype, int64_t in_row_stride, uint8_t* out,
+                                    int64_t out_row_stride, const float* scale, int64_t rows, int64_t hidden,
+                                    void* stream) {
+  using namespace vaq;
+  int rc = check_quant("fp8_quant_static", in, in_row_stride, out, out_row_stride, scale, rows, hidden);
+  if (rc != VAQ_OK || rows == 0) return rc;
+  rc = launch_quant<1>(in, in_dtype, in_row_stride, out, out_row_stride, const_cast<float*>(scale), nullptr, rows,
+                       hidden, (hipStream_t)stream);
+  if (rc != VAQ_OK) return rc;
+  VAQ_CHECK_LAUNCH("fp8_quant_static");
+  return VAQ_OK;
+}
+
+extern "C" int vaq_fp8_quant_dynamic(const void* in, int in_dtype, int64_t in_row_stride, uint8_t* out,
+                                     int64_t out_row_stride, float* scale, int64_t rows, int64_t hidden,
+                                     void* stream) {
+  using namespace vaq;
+  int rc = check_quant("fp8_quant_dynamic", in, in_row_stride, out, out_row_stride, scale, rows, hidden);
+  if (rc != VAQ_OK || rows == 0) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  // the running maximum starts from zero; a one-thread kernel rather than a memset node keeps the call graph-capturable
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(1), 0, s, scale);
+  rc = launch_quant<2>(in, in_dtype, in_row_stride, out, out_row_stride, scale, nullptr, rows, hidden, s);
+  if (rc != VAQ_OK) return rc;
+  rc = launch_quant<1>(in, in_dtype, in_row_stride, out, out_row_stride, scale, nullptr, rows, hidden, s);
+  if (rc != VAQ_OK) return rc;
+  VAQ_CHECK_LAUNCH("fp8_quant_dynamic");
+  return VAQ_OK;
+}

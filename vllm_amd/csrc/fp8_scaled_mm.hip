@@ -1,0 +1,384 @@
+// FP8 (e4m3fn x e4m3fn) scaled GEMM for gfx950:
+//     out[m,n] = round( sa[m] * ( sb[n] * sum_k a[m,k] b[k,n] ) + bias[n] ),   fp32 accumulation and epilogue.
+// a is [M,K] row-major, b is [K,N] column-major (= weight [N,K] row-major with row pitch ldb), so both operands are
+// k-contiguous and go to the matrix cores without any data re-arrangement.
+//
+// Two kernels:
+//  * tile kernel (any M): one workgroup of 4 wavefronts (2 x 2) per BM x BN output tile, K walked in steps of 128
+//    bytes through double-buffered, padded LDS (pitch 144 B), v_mfma_f32_32x32x64_f8f6f4 (the full-rate gfx950 FP8
+//    instruction, 32 bytes per lane per operand);
+//  * stream kernel (M <= 32): weight-streaming GEMV-like kernel, weights are the A operand of
+//    v_mfma_f32_16x16x128_f8f6f4 straight from global memory, activations stay in registers, the wavefronts of a
+//    workgroup split K and reduce through LDS.
+//
+// The per-lane byte -> k assignment inside an MFMA operand is the same function for A and B, so any consistent choice
+// of which 32 bytes a lane supplies yields the exact dot product; both kernels give lane (row, q) the bytes
+// k0 + 32*q .. k0 + 32*q + 31 of its row.
+#include "vaq_common.h"
+
+namespace vaq {
+
+struct Fp8MMParams {
+  const uint8_t* a;
+  int64_t lda;
+  const uint8_t* b;
+  int64_t ldb;
+  const float* sa;
+  int sa_per_row;   // 1: sa[m], 0: sa[0]
+  const float* sb;
+  int sb_per_col;
+  const uint16_t* bias;
+  uint16_t* out;
+  int64_t ldc;
+  int M, N, K;
+};
+
+__device__ inline v16f mfma_fp8_32(v8i a, v8i b, v16f c) {
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+__device__ inline v4f mfma_fp8_16(v8i a, v8i b, v4f c) {
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
+constexpr int F8_BK = 128;       // bytes of K per step
+constexpr int F8_PITCH = 144;    // LDS row pitch in bytes
+
+// ----------------------------------------------------------------------------- tile kernel
+template <bool BF16_OUT, int WMB, int WNB>
+__global__ __launch_bounds__(256) void fp8_mm_tile_kernel(const Fp8MMParams p) {
+  using T = F16Traits<BF16_OUT>;
+  constexpr int BM = 64 * WMB, BN = 64 * WNB;
+  constexpr int A_CH = BM / 32, B_CH = BN / 32;   // 16-byte chunks per thread per step
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds8[];
+  uint8_t* As = lds8;                         // [2][BM][PITCH]
+  uint8_t* Bs = lds8 + 2 * BM * F8_PITCH;     // [2][BN][PITCH]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  const int total = tiles_m * tiles_n;
+  int bid = blockIdx.x;
+  if (total % 8 == 0) bid = (bid & 7) * (total / 8) + (bid >> 3);   // one contiguous band of tiles per XCD
+  const int tm = bid % tiles_m, tn = bid / tiles_m;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  v4u areg[A_CH], breg[B_CH];
+  auto load_g = [&](int step) {
+    const int kb = step * F8_BK;
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c >> 3, ch = c & 7;
+      const int m = m0 + row, k = kb + ch * 16;
+      v4u v = {0u, 0u, 0u, 0u};
+      if (m < p.M && k < p.K) v = *reinterpret_cast<const v4u*>(p.a + (int64_t)m * p.lda + k);
+      areg[i] = v;
+    }
+#pragma unroll
+    for (int i = 0; i < B_CH; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c >> 3, ch = c & 7;
+      const int n = n0 + row, k = kb + ch * 16;
+      v4u v = {0u, 0u, 0u, 0u};
+      if (n < p.N && k < p.K) v = *reinterpret_cast<const v4u*>(p.b + (int64_t)n * p.ldb + k);
+      breg[i] = v;
+    }
+  };
+  auto store_l = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) {
+      const int c = tid + 256 * i;
+      *reinterpret_cast<v4u*>(As + ((size_t)buf * BM + (c >> 3)) * F8_PITCH + (c & 7) * 16) = areg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < B_CH; ++i) {
+      const int c = tid + 256 * i;
+      *reinterpret_cast<v4u*>(Bs + ((size_t)buf * BN + (c >> 3)) * F8_PITCH + (c & 7) * 16) = breg[i];
+    }
+  };
+
+  v16f acc[WMB][WNB];
+#pragma unroll
+  for (int i = 0; i < WMB; ++i)
+#pragma unroll
+    for (int j = 0; j < WNB; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const int steps = (p.K + F8_BK - 1) / F8_BK;
+  load_g(0);
+  store_l(0);
+  if (steps > 1) load_g(1);
+  __syncthreads();
+
+  for (int step = 0; step < steps; ++step) {
+    const int cur = step & 1;
+    if (step + 1 < steps) {
+      store_l(cur ^ 1);
+      if (step + 2 < steps) load_g(step + 2);
+    }
+    const uint8_t* Ab = As + ((size_t)cur * BM + wm * 32 * WMB + (lane & 31)) * F8_PITCH + (lane >> 5) * 32;
+    const uint8_t* Bb = Bs + ((size_t)cur * BN + wn * 32 * WNB + (lane & 31)) * F8_PITCH + (lane >> 5) * 32;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      v8i af[WMB], bf[WNB];
+#pragma unroll
+      for (int i = 0; i < WMB; ++i) {
+        const v4i lo = *reinterpret_cast<const v4i*>(Ab + (size_t)i * 32 * F8_PITCH + kk * 64);
+        const v4i hi = *reinterpret_cast<const v4i*>(Ab + (size_t)i * 32 * F8_PITCH + kk * 64 + 16);
+        af[i] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      }
+#pragma unroll
+      for (int j = 0; j < WNB; ++j) {
+        const v4i lo = *reinterpret_cast<const v4i*>(Bb + (size_t)j * 32 * F8_PITCH + kk * 64);
+        const v4i hi = *reinterpret_cast<const v4i*>(Bb + (size_t)j * 32 * F8_PITCH + kk * 64 + 16);
+        bf[j] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      }
+#pragma unroll
+      for (int i = 0; i < WMB; ++i)
+#pragma unroll
+        for (int j = 0; j < WNB; ++j) acc[i][j] = mfma_fp8_32(af[i], bf[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+
+  // epilogue: lane holds column n = lane%32, rows 8*(e/4) + 4*(lane/32) + e%4 of each 32x32 block
+#pragma unroll
+  for (int j = 0; j < WNB; ++j) {
+    const int n = n0 + wn * 32 * WNB + j * 32 + (lane & 31);
+    if (n >= p.N) continue;
+    const float sbn = p.sb[p.sb_per_col ? n : 0];
+    const bool hb = p.bias != nullptr;
+    const float bv = hb ? T::to_float(p.bias[n]) : 0.f;
+#pragma unroll
+    for (int i = 0; i < WMB; ++i) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = m0 + wm * 32 * WMB + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+        if (m < p.M) {
+          const float sam = p.sa[p.sa_per_row ? m : 0];
+          float v = sam * (sbn * acc[i][j][e]);
+          if (hb) v += bv;
+          p.out[(int64_t)m * p.ldc + n] = T::from_float(v);
+        }
+      }
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------- stream kernel (M <= 32)
+// blockDim = (64, WK).  Wavefront w owns K steps [w*KS, (w+1)*KS) of 128 bytes; activations of that slab live in
+// registers for the whole kernel; the workgroup walks a contiguous range of 16-row weight tiles.
+template <bool BF16_OUT, int KS, int MB>
+__global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p, int WK) {
+  using T = F16Traits<BF16_OUT>;
+  extern __shared__ v4f red[];   // [2][WK][MB][64]
+  const int lane = threadIdx.x, w = threadIdx.y;
+  const int q = lane >> 4, r16 = lane & 15;
+  const int kbase = w * KS * 128 + q * 32;
+
+  v8i breg[KS][MB];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int m = mb * 16 + r16;
+      const int k = kbase + s * 128;
+      v4i lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+      if (m < p.M) {
+        const uint8_t* row = p.a + (int64_t)m * p.lda;
+        if (k < p.K) lo = *reinterpret_cast<const v4i*>(row + k);
+        if (k + 16 < p.K) hi = *reinterpret_cast<const v4i*>(row + k + 16);
+      }
+      breg[s][mb] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
+  }
+
+  const int NT = p.N / 16;
+  const int nt0 = (int)(((int64_t)NT * blockIdx.x) / gridDim.x);
+  const int nt1 = (int)(((int64_t)NT * (blockIdx.x + 1)) / gridDim.x);
+
+  v4i wlo[KS], whi[KS];
+  auto issue = [&](int nt, int s) {
+    const int k = kbase + s * 128;
+    const uint8_t* row = p.b + (int64_t)(nt * 16 + r16) * p.ldb;
+    wlo[s] = v4i{0, 0, 0, 0};
+    whi[s] = v4i{0, 0, 0, 0};
+    if (k < p.K) wlo[s] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(row + k));
+    if (k + 16 < p.K) whi[s] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(row + k + 16));
+  };
+  if (nt0 < nt1) {
+#pragma unroll
+    for (int s = 0; s < KS; ++s) issue(nt0, s);
+  }
+
+  int parity = 0;
+  for (int nt = nt0; nt < nt1; ++nt) {
+    v4f acc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const v8i aop = v8i{wlo[s].x, wlo[s].y, wlo[s].z, wlo[s].w, whi[s].x, whi[s].y, whi[s].z, whi[s].w};
+      if (nt + 1 < nt1) issue(nt + 1, s);
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) acc[mb] = mfma_fp8_16(aop, breg[s][mb], acc[mb]);
+    }
+
+    v4f tot = v4f{0.f, 0.f, 0.f, 0.f};
+    bool reducer = w < MB;
+    if (WK > 1) {
+      v4f* buf = red + (size_t)parity * WK * MB * 64;
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) buf[(w * MB + mb) * 64 + lane] = acc[mb];
+      __syncthreads();
+      if (reducer)
+        for (int ww = 0; ww < WK; ++ww) tot += buf[(ww * MB + w) * 64 + lane];
+      parity ^= 1;
+    } else {
+      reducer = true;
+    }
+    if (reducer) {
+      const int mb_lo = (WK > 1) ? w : 0, mb_hi = (WK > 1) ? w + 1 : MB;
+      for (int mb = mb_lo; mb < mb_hi; ++mb) {
+        const v4f val = (WK > 1) ? tot : acc[mb];
+        const int m = mb * 16 + r16;
+        if (m < p.M) {
+          const int n = nt * 16 + q * 4;
+          const float sam = p.sa[p.sa_per_row ? m : 0];
+          float o[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float sbn = p.sb[p.sb_per_col ? n + r : 0];
+            o[r] = sam * (sbn * val[r]);
+            if (p.bias) o[r] += T::to_float(p.bias[n + r]);
+          }
+          v2u ov;
+          ov.x = (uint32_t)T::from_float(o[0]) | ((uint32_t)T::from_float(o[1]) << 16);
+          ov.y = (uint32_t)T::from_float(o[2]) | ((uint32_t)T::from_float(o[3]) << 16);
+          *reinterpret_cast<v2u*>(p.out + (int64_t)m * p.ldc + n) = ov;
+        }
+      }
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------- host side
+
+static int g_force_fp8_path = 0;   // 0 auto, 1 stream, 2 tile
+static int g_force_fp8_gx = 0;
+
+template <bool BF16_OUT, int WMB, int WNB>
+static int launch_tile(const Fp8MMParams& p, hipStream_t s) {
+  constexpr int BM = 64 * WMB, BN = 64 * WNB;
+  const size_t lds = (size_t)2 * (BM + BN) * F8_PITCH;
+  auto kern = fp8_mm_tile_kernel<BF16_OUT, WMB, WNB>;
+  static bool attr_done = false;
+  if (!attr_done) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
+        hipSuccess) {
+      set_error("fp8_scaled_mm: cannot reserve %zu bytes of LDS", lds);
+      (void)hipGetLastError();
+      return VAQ_ERR_LAUNCH;
+    }
+    attr_done = true;
+  }
+  const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(256), lds, s, p);
+  return VAQ_OK;
+}
+
+template <bool BF16_OUT>
+static int dispatch_tile(const Fp8MMParams& p, hipStream_t s) {
+  const int cus = num_cus_current_device();
+  auto tiles = [&](int bm, int bn) { return (int64_t)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
+  if (tiles(256, 256) >= cus) return launch_tile<BF16_OUT, 4, 4>(p, s);
+  if (tiles(128, 128) >= cus) return launch_tile<BF16_OUT, 2, 2>(p, s);
+  return launch_tile<BF16_OUT, 1, 2>(p, s);
+}
+
+template <bool BF16_OUT, int KS, int MB>
+static void launch_stream(const Fp8MMParams& p, int wk, int gx, hipStream_t s) {
+  const size_t lds = wk > 1 ? (size_t)2 * wk * MB * 64 * sizeof(v4f) : 0;
+  hipLaunchKernelGGL((fp8_mm_stream_kernel<BF16_OUT, KS, MB>), dim3(gx), dim3(64, wk), lds, s, p, wk);
+}
+
+template <bool BF16_OUT>
+static bool dispatch_stream(const Fp8MMParams& p, hipStream_t s) {
+  const int steps = (p.K + 127) / 128;
+  const int MB = p.M <= 16 ? 1 : 2;
+  // wavefronts along K: at most 8; per-wave slab of KS steps
+  int ks;
+  if (steps <= 8 * 4) ks = 4;
+  else if (steps <= 8 * 8) ks = 8;
+  else if (steps <= 8 * 14 && MB == 1) ks = 14;
+  else return false;
+  const int wk = (steps + ks - 1) / ks;
+  const int NT = p.N / 16;
+  int gx = g_force_fp8_gx > 0 ? g_force_fp8_gx : 2 * num_cus_current_device();
+  if (gx > NT) gx = NT;
+  if (MB == 1) {
+    if (ks == 4) launch_stream<BF16_OUT, 4, 1>(p, wk, gx, s);
+    else if (ks == 8) launch_stream<BF16_OUT, 8, 1>(p, wk, gx, s);
+    else launch_stream<BF16_OUT, 14, 1>(p, wk, gx, s);
+  } else {
+    if (ks == 4) launch_stream<BF16_OUT, 4, 2>(p, wk, gx, s);
+    else launch_stream<BF16_OUT, 8, 2>(p, wk, gx, s);
+  }
+  return true;
+}
+
+}  // namespace vaq
+
+extern "C" int vaq_fp8_scaled_mm(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t ldb, const float* sa,
+                                 int64_t sa_count, const float* sb, int64_t sb_count, const void* bias, void* out,
+                                 int64_t ldc, int out_dtype, int64_t size_m, int64_t size_n, int64_t size_k,
+                                 void* stream) {
+  using namespace vaq;
+  VAQ_CHECK_ARG(size_m >= 0 && size_n > 0 && size_k > 0, "fp8_scaled_mm: bad shape M=%lld N=%lld K=%lld",
+                (long long)size_m, (long long)size_n, (long long)size_k);
+  VAQ_CHECK_ARG(size_m < (1ll << 31) && size_n < (1ll << 31) && size_k < (1ll << 31), "fp8_scaled_mm: shape too large");
+  VAQ_CHECK_ARG(size_k % 16 == 0 && size_n % 16 == 0, "fp8_scaled_mm: K = %lld and N = %lld must be multiples of 16",
+                (long long)size_k, (long long)size_n);
+  VAQ_CHECK_ARG(lda >= size_k && lda % 16 == 0, "fp8_scaled_mm: a row stride %lld must be >= K and a multiple of 16",
+                (long long)lda);
+  VAQ_CHECK_ARG(ldb >= size_k && ldb % 16 == 0, "fp8_scaled_mm: b column stride %lld must be >= K and a multiple of 16",
+                (long long)ldb);
+  VAQ_CHECK_ARG(ldc >= size_n && ldc % 8 == 0, "fp8_scaled_mm: out row stride %lld must be >= N and a multiple of 8",
+                (long long)ldc);
+  VAQ_CHECK_ARG(sa_count == 1 || sa_count == size_m, "fp8_scaled_mm: a_scales count %lld must be 1 or M",
+                (long long)sa_count);
+  VAQ_CHECK_ARG(sb_count == 1 || sb_count == size_n, "fp8_scaled_mm: b_scales count %lld must be 1 or N",
+                (long long)sb_count);
+  VAQ_CHECK_ARG(out_dtype == VAQ_F16 || out_dtype == VAQ_BF16, "fp8_scaled_mm: out dtype tag %d", out_dtype);
+  if (size_m == 0) return VAQ_OK;
+  VAQ_CHECK_ARG(a && b && sa && sb && out, "fp8_scaled_mm: null pointer");
+  VAQ_CHECK_ARG(((uintptr_t)a % 16) == 0 && ((uintptr_t)b % 16) == 0 && ((uintptr_t)out % 8) == 0,
+                "fp8_scaled_mm: a and b must be 16-byte aligned, out 8-byte aligned");
+  Fp8MMParams p;
+  p.a = a; p.lda = lda; p.b = b; p.ldb = ldb;
+  p.sa = sa; p.sa_per_row = (sa_count > 1 || size_m == 1) ? 1 : 0;
+  p.sb = sb; p.sb_per_col = (sb_count > 1 || size_n == 1) ? 1 : 0;
+  p.bias = (const uint16_t*)bias;
+  p.out = (uint16_t*)out; p.ldc = ldc;
+  p.M = (int)size_m; p.N = (int)size_n; p.K = (int)size_k;
+  hipStream_t s = (hipStream_t)stream;
+  const bool bf16 = out_dtype == VAQ_BF16;
+  bool done = false;
+  const bool want_stream = g_force_fp8_path == 1 || (g_force_fp8_path == 0 && size_m <= 32);
+  if (want_stream && size_m <= 32) done = bf16 ? dispatch_stream<true>(p, s) : dispatch_stream<false>(p, s);
+  if (!done) {
+    int rc = bf16 ? dispatch_tile<true>(p, s) : dispatch_tile<false>(p, s);
+    if (rc != VAQ_OK) return rc;
+  }
+  VAQ_CHECK_LAUNCH("fp8_scaled_mm");
+  return VAQ_OK;
+}
+
+// Benchmark / tuning aid, not part of the drop-in surface.  path: 0 auto, 1 stream, 2 tile; gx: stream-kernel grid.
+extern "C" void vaq_debug_set_fp8_config(int path, int gx) {
+  vaq::g_force_fp8_path = path;
+  vaq::g_force_fp8_gx = gx;
+}

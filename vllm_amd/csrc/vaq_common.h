@@ -1,0 +1,113 @@
+// Shared host/device helpers for the gfx950 quantized-linear kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/vllm_amd_qlinear.h"
+
+namespace vaq {
+
+// ----------------------------------------------------------------------------- host: error reporting
+void set_error(const char* fmt, ...);   // defined in api.hip (thread-local buffer)
+
+#define VAQ_CHECK_ARG(cond, ...)            \
+  do {                                      \
+    if (!(cond)) {                          \
+      ::vaq::set_error(__VA_ARGS__);        \
+      return VAQ_ERR_INVALID_ARG;           \
+    }                                       \
+  } while (0)
+
+#define VAQ_CHECK_SUPPORTED(cond, ...)      \
+  do {                                      \
+    if (!(cond)) {                          \
+      ::vaq::set_error(__VA_ARGS__);        \
+      return VAQ_ERR_UNSUPPORTED;           \
+    }                                       \
+  } while (0)
+
+#define VAQ_CHECK_LAUNCH(what)                                                     \
+  do {                                                                             \
+    hipError_t e__ = hipGetLastError();                                            \
+    if (e__ != hipSuccess) {                                                       \
+      ::vaq::set_error("%s: launch failed: %s", what, hipGetErrorString(e__));     \
+      return VAQ_ERR_LAUNCH;                                                       \
+    }                                                                              \
+  } while (0)
+
+int num_cus_current_device();   // cached per device, api.hip
+
+// ----------------------------------------------------------------------------- device: vector types
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+
+// 16-bit float handling is done on raw bit patterns so that bf16 and fp16 share one code path.
+template <bool BF16>
+struct F16Traits;
+
+template <>
+struct F16Traits<true> {
+  // (code & 0xF) | EX is the bf16 number 128 + code (7 mantissa bits, exponent 2^7).
+  static constexpr uint32_t EX = 0x43004300u;
+  static constexpr float CODE_BIAS = 128.0f;
+  __device__ static inline float to_float(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+  __device__ static inline uint16_t from_float(float f) {   // round-to-nearest-even, NaN preserved
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+  }
+  __device__ static inline v4f mfma16(v4u a, v4u b, v4f c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+  }
+  __device__ static inline v16f mfma32(v4u a, v4u b, v16f c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+  }
+  static constexpr uint32_t ONE2 = 0x3f803f80u;   // packed (1.0, 1.0)
+};
+
+template <>
+struct F16Traits<false> {
+  // (code & 0xF) | EX is the fp16 number 1024 + code (10 mantissa bits, exponent 2^10).
+  static constexpr uint32_t EX = 0x64006400u;
+  static constexpr float CODE_BIAS = 1024.0f;
+  __device__ static inline float to_float(uint16_t h) {
+    _Float16 x = __builtin_bit_cast(_Float16, h);
+    return (float)x;
+  }
+  __device__ static inline uint16_t from_float(float f) {
+    _Float16 x = (_Float16)f;   // v_cvt_f16_f32: round-to-nearest-even
+    return __builtin_bit_cast(uint16_t, x);
+  }
+  __device__ static inline v4f mfma16(v4u a, v4u b, v4f c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+  __device__ static inline v16f mfma32(v4u a, v4u b, v16f c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+  static constexpr uint32_t ONE2 = 0x3c003c00u;
+};
+
+// One native-layout weight word (8 codes, nibble p holds element {0,2,4,6,1,3,5,7}[p]) -> 8 consecutive 16-bit
+// numbers CODE_BIAS + code, i.e. one 16x16x32 MFMA operand register quad.
+template <bool BF16>
+__device__ inline v4u dequant_biased(uint32_t w) {
+  constexpr uint32_t M = 0x000f000fu, EX = F16Traits<BF16>::EX;
+  v4u r;
+  r.x = (w & M) | EX;
+  r.y = ((w >> 4) & M) | EX;
+  r.z = ((w >> 8) & M) | EX;
+  r.w = ((w >> 12) & M) | EX;
+  return r;
+}
+
+}  // namespace vaq

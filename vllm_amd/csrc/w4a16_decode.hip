@@ -1,0 +1,332 @@
+// W4A16 decode-shaped GEMM (M <= 32) for gfx950: C[M,N] = A[M,K] . dequant(B[K,N]) (+bias).
+//
+// Memory-bound: the job is to stream K*N/2 bytes of packed int4 once, at HBM speed, with as little VALU work per
+// byte as possible.  Design:
+//
+//  * Weights arrive in the NATIVE tile order (see w4a16_repack.hip): one 16-byte load per lane = one 1 KiB
+//    wavefront load = a 16(n) x 128(k) tile = the A operands of four v_mfma_f32_16x16x32 and exactly one
+//    quantisation group.
+//  * The weights are the MFMA *A* operand (rows = n), the activations the *B* operand (columns = m), so the cost per
+//    weight byte does not depend on M (up to 16 per m-block) and the matrix pipe does all multiply-adds.
+//  * Dequantisation is 7 VALU ops per 8 codes: `(w >> 4i) & 0x000f000f | EX` yields the 16-bit numbers BIAS + code
+//    (BIAS = 128 for bf16, 1024 for fp16).  The "- BIAS - zero" and the group scale are NOT applied per element:
+//        C[m,n] = sum_g s[g,n] * ( P_g[m,n] - (BIAS + z[g,n]) * S_g[m] ),
+//        P_g[m,n] = sum_{k in g} a[m,k] * (BIAS + code[k,n])      (4 MFMAs, fp32)
+//        S_g[m]   = sum_{k in g} a[m,k]                           (MFMA against an all-ones operand, once per wave)
+//    which costs two fp32 FMAs per output per group.  The products a*(BIAS+code) are exact in fp32 and the group
+//    scale is applied in fp32, so the result is at least as accurate as scaling every weight in 16 bits first.
+//  * Each wavefront owns a fixed slab of TG groups along K, keeps the matching activations in registers for the
+//    whole kernel (loaded once; act_order gathers through `perm` here, so no permuted copy of A is needed) and walks
+//    a contiguous range of n-tiles, prefetching the next TG tiles while the current ones are consumed.
+//  * The WK wavefronts of a workgroup cover WK*TG groups of the same n-tile and reduce through LDS (one barrier per
+//    n-tile, double-buffered).  If K needs more than one workgroup (SK > 1) the partial tiles go to `c_tmp` and the
+//    last workgroup to arrive at a per-tile counter sums them in a fixed order (deterministic) and resets the counter.
+#include "vaq_common.h"
+
+namespace vaq {
+
+struct DecodeParams {
+  const uint16_t* a;
+  int64_t lda;
+  const v4u* b;
+  const uint16_t* scales;
+  const uint32_t* zeros;
+  const int32_t* perm;
+  const uint16_t* bias;
+  uint16_t* c;
+  v4f* c_tmp;
+  int32_t* counters;
+  int M, N, K, G, NT, SK, WK;
+};
+
+// Workgroups are at most 8 wavefronts, i.e. two per SIMD, which leaves 256 registers per lane.
+template <bool BF16, int TG, int MB, bool HAS_ZP>
+__global__ __launch_bounds__(512) void w4a16_decode_kernel(const DecodeParams p) {
+  using T = F16Traits<BF16>;
+  extern __shared__ v4f red[];   // [2][WK][MB][64]
+
+  const int lane = threadIdx.x, w = threadIdx.y;
+  const int o = lane >> 4, r16 = lane & 15;
+  const int sk = blockIdx.y;
+  const int g0 = (sk * p.WK + w) * TG;
+
+  // ---- activations of this wave's K slab, as MFMA B operands (column = m, 8 consecutive k per lane) ----
+  v4u breg[TG][4][MB];
+  float S[TG][MB];
+#pragma unroll
+  for (int t = 0; t < TG; ++t) {
+    const int g = g0 + t;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int m = mb * 16 + r16;
+      const bool ok = (g < p.G) && (m < p.M);
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const int k = g * 128 + jj * 32 + o * 8;
+        v4u v = {0u, 0u, 0u, 0u};
+        if (ok) {
+          const uint16_t* row = p.a + (int64_t)m * p.lda;
+          if (p.perm) {
+            const v4i p0 = *reinterpret_cast<const v4i*>(p.perm + k);
+            const v4i p1 = *reinterpret_cast<const v4i*>(p.perm + k + 4);
+            v.x = (uint32_t)row[p0.x] | ((uint32_t)row[p0.y] << 16);
+            v.y = (uint32_t)row[p0.z] | ((uint32_t)row[p0.w] << 16);
+            v.z = (uint32_t)row[p1.x] | ((uint32_t)row[p1.y] << 16);
+            v.w = (uint32_t)row[p1.z] | ((uint32_t)row[p1.w] << 16);
+          } else {
+            v = *reinterpret_cast<const v4u*>(row + k);
+          }
+        }
+        breg[t][jj][mb] = v;
+      }
+      const v4u ones = {T::ONE2, T::ONE2, T::ONE2, T::ONE2};
+      v4f s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) s4 = T::mfma16(ones, breg[t][jj][mb], s4);
+      S[t][mb] = s4.x;
+    }
+  }
+
+  // ---- contiguous range of n-tiles for this workgroup ----
+  const int nt0 = (int)(((int64_t)p.NT * blockIdx.x) / gridDim.x);
+  const int nt1 = (int)(((int64_t)p.NT * (blockIdx.x + 1)) / gridDim.x);
+
+  v4u wq[TG];
+  v2u sc[TG];
+  uint32_t zq[TG];
+  // Slot t is refilled for the next n-tile as soon as it has been consumed, so TG tile loads stay in flight per
+  // wavefront with a single set of registers.
+  auto issue_load = [&](int nt, int t) {
+    const int g = g0 + t;
+    if (g < p.G) {
+      wq[t] = __builtin_nontemporal_load(&p.b[((int64_t)g * p.NT + nt) * 64 + lane]);
+      sc[t] = *reinterpret_cast<const v2u*>(p.scales + (int64_t)g * p.N + nt * 16 + o * 4);
+      if constexpr (HAS_ZP) zq[t] = p.zeros[(int64_t)g * (p.N >> 3) + nt * 2 + (o >> 1)];
+    }
+  };
+#pragma unroll
+  for (int t = 0; t < TG; ++t) {
+    wq[t] = v4u{0u, 0u, 0u, 0u};
+    sc[t] = v2u{0u, 0u};
+    zq[t] = 0u;
+    if (nt0 < nt1) issue_load(nt0, t);
+  }
+
+  int parity = 0;
+  for (int nt = nt0; nt < nt1; ++nt) {
+    v4f acc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb] = v4f{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+    for (int t = 0; t < TG; ++t) {
+      v4f P[MB];
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) P[mb] = v4f{0.f, 0.f, 0.f, 0.f};
+      const uint32_t wj[4] = {wq[t].x, wq[t].y, wq[t].z, wq[t].w};
+      const v2u sct = sc[t];
+      const uint32_t zqt = zq[t];
+      if (nt + 1 < nt1) issue_load(nt + 1, t);
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const v4u aop = dequant_biased<BF16>(wj[jj]);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) P[mb] = T::mfma16(aop, breg[t][jj][mb], P[mb]);
+      }
+      // group epilogue: acc += s * (P - (BIAS + z) * S)
+      float s[4], zc[4];
+      s[0] = T::to_float((uint16_t)(sct.x & 0xffffu));
+      s[1] = T::to_float((uint16_t)(sct.x >> 16));
+      s[2] = T::to_float((uint16_t)(sct.y & 0xffffu));
+      s[3] = T::to_float((uint16_t)(sct.y >> 16));
+      if constexpr (HAS_ZP) {
+        const uint32_t z4 = zqt >> ((o & 1) * 16);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) zc[r] = T::CODE_BIAS + (float)((z4 >> (4 * r)) & 0xFu);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) zc[r] = T::CODE_BIAS + 8.0f;
+      }
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const float Sg = S[t][mb];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[mb][r] = fmaf(s[r], fmaf(-zc[r], Sg, P[mb][r]), acc[mb][r]);
+      }
+    }
+
+    // ---- reduce the WK partial tiles of this workgroup through LDS ----
+    v4f tot = v4f{0.f, 0.f, 0.f, 0.f};
+    bool reducer = w < MB;
+    if (p.WK > 1) {
+      v4f* buf = red + (size_t)parity * p.WK * MB * 64;
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) buf[(w * MB + mb) * 64 + lane] = acc[mb];
+      __syncthreads();
+      if (reducer) {
+        for (int ww = 0; ww < p.WK; ++ww) {
+          const v4f v = buf[(ww * MB + w) * 64 + lane];
+          tot += v;
+        }
+      }
+      parity ^= 1;
+    } else {
+      // single wave per workgroup: it owns every m-block itself
+      reducer = true;
+    }
+
+    if (reducer) {
+      const int mb_lo = (p.WK > 1) ? w : 0;
+      const int mb_hi = (p.WK > 1) ? w + 1 : MB;
+      for (int mb = mb_lo; mb < mb_hi; ++mb) {
+        v4f val = (p.WK > 1) ? tot : acc[mb];
+        bool write_out = true;
+        if (p.SK > 1) {
+          const int64_t slot = ((int64_t)nt * MB + mb) * 64 + lane;
+          const int64_t sk_stride = (int64_t)p.NT * MB * 64;
+          p.c_tmp[sk * sk_stride + slot] = val;
+          __threadfence();
+          int old = 0;
+          if (lane == 0) old = __hip_atomic_fetch_add(&p.counters[nt * MB + mb], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          old = __shfl(old, 0);
+          write_out = (old == p.SK - 1);
+          if (write_out) {
+            __threadfence();
+            val = v4f{0.f, 0.f, 0.f, 0.f};
+            for (int s2 = 0; s2 < p.SK; ++s2) {
+              const v4f v = __builtin_nontemporal_load(&p.c_tmp[s2 * sk_stride + slot]);
+              val += v;
+            }
+            if (lane == 0) __hip_atomic_store(&p.counters[nt * MB + mb], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+        }
+        const int m = mb * 16 + r16;
+        if (write_out && m < p.M) {
+          const int n = nt * 16 + o * 4;
+          if (p.bias) {
+            const v2u bb = *reinterpret_cast<const v2u*>(p.bias + n);
+            val[0] += T::to_float((uint16_t)(bb.x & 0xffffu));
+            val[1] += T::to_float((uint16_t)(bb.x >> 16));
+            val[2] += T::to_float((uint16_t)(bb.y & 0xffffu));
+            val[3] += T::to_float((uint16_t)(bb.y >> 16));
+          }
+          v2u outv;
+          outv.x = (uint32_t)T::from_float(val[0]) | ((uint32_t)T::from_float(val[1]) << 16);
+          outv.y = (uint32_t)T::from_float(val[2]) | ((uint32_t)T::from_float(val[3]) << 16);
+          *reinterpret_cast<v2u*>(p.c + (int64_t)m * p.N + n) = outv;
+        }
+      }
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------- host side
+
+struct DecodeConfig {
+  int tg, wk, sk, gx;
+};
+
+static int g_force_tg = 0, g_force_wk = 0, g_force_gx = 0;
+
+static DecodeConfig pick_decode_config(int M, int N, int K) {
+  const int G = K / 128, NT = N / 16;
+  const int MB = M <= 16 ? 1 : 2;
+  DecodeConfig c;
+  if (g_force_tg > 0) c.tg = g_force_tg;
+  else if (MB == 2) c.tg = G >= 2 ? 2 : 1;
+  else if (G >= 8) c.tg = 4;
+  else if (G >= 2) c.tg = 2;
+  else c.tg = 1;
+  const int kw = (G + c.tg - 1) / c.tg;          // wavefronts needed along K
+  int wk_max = 8;
+  if (g_force_wk > 0 && g_force_wk < wk_max) wk_max = g_force_wk;
+  c.sk = (kw + wk_max - 1) / wk_max;
+  c.wk = (kw + c.sk - 1) / c.sk;
+  const int cus = num_cus_current_device();
+  int gx = g_force_gx > 0 ? g_force_gx : (2 * cus) / c.sk;
+  if (gx < 1) gx = 1;
+  if (gx > NT) gx = NT;
+  c.gx = gx;
+  return c;
+}
+
+template <bool BF16, int TG, int MB, bool HAS_ZP>
+static void launch_decode(const DecodeParams& p, int gx, hipStream_t s) {
+  const size_t lds = p.WK > 1 ? (size_t)2 * p.WK * MB * 64 * sizeof(v4f) : 0;
+  hipLaunchKernelGGL((w4a16_decode_kernel<BF16, TG, MB, HAS_ZP>), dim3(gx, p.SK), dim3(64, p.WK), lds, s, p);
+}
+
+template <bool BF16, int MB, bool HAS_ZP>
+static int dispatch_tg(const DecodeParams& p, int tg, int gx, hipStream_t s) {
+  switch (tg) {
+    case 1: launch_decode<BF16, 1, MB, HAS_ZP>(p, gx, s); return VAQ_OK;
+    case 2: launch_decode<BF16, 2, MB, HAS_ZP>(p, gx, s); return VAQ_OK;
+    case 4:
+      if constexpr (MB == 1) { launch_decode<BF16, 4, MB, HAS_ZP>(p, gx, s); return VAQ_OK; }
+      break;
+    default: break;
+  }
+  set_error("w4a16_gemm(decode): unsupported TG=%d for MB=%d", tg, MB);
+  return VAQ_ERR_UNSUPPORTED;
+}
+
+// Called from vaq_w4a16_gemm (w4a16_gemm.hip) after argument validation.
+int w4a16_decode_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* counter_ints) {
+  const DecodeConfig c = pick_decode_config(M, N, K);
+  const int MB = M <= 16 ? 1 : 2;
+  const int NT = N / 16;
+  *c_tmp_bytes = c.sk > 1 ? (size_t)c.sk * NT * MB * 64 * sizeof(v4f) : 0;
+  *counter_ints = c.sk > 1 ? (size_t)NT * MB : 0;
+  return VAQ_OK;
+}
+
+int w4a16_decode_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
+                        const int32_t* perm, const void* bias, void* c, float* c_tmp, int32_t* counters,
+                        int64_t counter_ints, int M, int N, int K, int dtype, hipStream_t s) {
+  DecodeParams p;
+  p.a = (const uint16_t*)a;
+  p.lda = lda;
+  p.b = (const v4u*)b;
+  p.scales = (const uint16_t*)scales;
+  p.zeros = (const uint32_t*)zeros;
+  p.perm = perm;
+  p.bias = (const uint16_t*)bias;
+  p.c = (uint16_t*)c;
+  p.c_tmp = (v4f*)c_tmp;
+  p.counters = counters;
+  p.M = M; p.N = N; p.K = K;
+  p.G = K / 128;
+  p.NT = N / 16;
+  const DecodeConfig cfg = pick_decode_config(M, N, K);
+  p.SK = cfg.sk;
+  p.WK = cfg.wk;
+  const int MB = M <= 16 ? 1 : 2;
+  if (cfg.sk > 1) {
+    VAQ_CHECK_ARG(c_tmp != nullptr && counters != nullptr, "w4a16_gemm: split-K needs c_tmp and counters");
+    VAQ_CHECK_ARG(counter_ints >= (int64_t)p.NT * MB,
+                  "w4a16_gemm: workspace.numel = %lld is below min_workspace_size = %lld", (long long)counter_ints,
+                  (long long)p.NT * MB);
+  }
+  const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
+  int rc;
+  if (MB == 1) {
+    if (bf16) rc = zp ? dispatch_tg<true, 1, true>(p, cfg.tg, cfg.gx, s) : dispatch_tg<true, 1, false>(p, cfg.tg, cfg.gx, s);
+    else rc = zp ? dispatch_tg<false, 1, true>(p, cfg.tg, cfg.gx, s) : dispatch_tg<false, 1, false>(p, cfg.tg, cfg.gx, s);
+  } else {
+    if (bf16) rc = zp ? dispatch_tg<true, 2, true>(p, cfg.tg, cfg.gx, s) : dispatch_tg<true, 2, false>(p, cfg.tg, cfg.gx, s);
+    else rc = zp ? dispatch_tg<false, 2, true>(p, cfg.tg, cfg.gx, s) : dispatch_tg<false, 2, false>(p, cfg.tg, cfg.gx, s);
+  }
+  if (rc != VAQ_OK) return rc;
+  VAQ_CHECK_LAUNCH("w4a16_gemm(decode)");
+  return VAQ_OK;
+}
+
+}  // namespace vaq
+
+// Benchmark / tuning aid, not part of the drop-in surface: override the decode launch shape
+// (0 = automatic).  Process-global and not thread-safe.
+extern "C" void vaq_debug_set_decode_config(int tg, int wk, int gx) {
+  vaq::g_force_tg = tg;
+  vaq::g_force_wk = wk;
+  vaq::g_force_gx = gx;
+}

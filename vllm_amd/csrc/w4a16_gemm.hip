@@ -1,0 +1,91 @@
+// C-ABI entry of the W4A16 GEMM: argument validation and the decode / prefill dispatch.
+#include "vaq_common.h"
+
+namespace vaq {
+int w4a16_decode_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* counter_ints);
+int w4a16_decode_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
+                        const int32_t* perm, const void* bias, void* c, float* c_tmp, int32_t* counters,
+                        int64_t counter_ints, int M, int N, int K, int dtype, hipStream_t s);
+int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
+                         const void* bias, void* c, int M, int N, int K, int dtype, hipStream_t s);
+
+constexpr int64_t DECODE_MAX_M = 32;
+
+static int check_shape(int64_t size_m, int64_t size_n, int64_t size_k) {
+  VAQ_CHECK_ARG(size_m >= 0, "w4a16_gemm: size_m = %lld is negative", (long long)size_m);
+  VAQ_CHECK_ARG(size_n > 0 && size_n % 64 == 0, "w4a16_gemm: size_n = %lld, is not divisible by min_thread_n = 64",
+                (long long)size_n);
+  VAQ_CHECK_ARG(size_k > 0 && size_k % 128 == 0, "w4a16_gemm: size_k = %lld, is not divisible by min_thread_k = 128",
+                (long long)size_k);
+  VAQ_CHECK_ARG(size_m < (1ll << 31) && size_n < (1ll << 31) && size_k < (1ll << 31) &&
+                    size_k * size_n / 8 < (1ll << 40),
+                "w4a16_gemm: problem too large");
+  return VAQ_OK;
+}
+}  // namespace vaq
+
+extern "C" int vaq_w4a16_gemm_workspace(int64_t size_m, int64_t size_n, int64_t size_k, int has_perm, int device,
+                                        size_t* c_tmp_bytes, size_t* a_tmp_bytes, size_t* counter_ints) {
+  using namespace vaq;
+  (void)device;
+  VAQ_CHECK_ARG(c_tmp_bytes && a_tmp_bytes && counter_ints, "w4a16_gemm_workspace: null output pointer");
+  int rc = check_shape(size_m, size_n, size_k);
+  if (rc != VAQ_OK) return rc;
+  *c_tmp_bytes = 0;
+  *a_tmp_bytes = 0;
+  *counter_ints = 0;
+  if (size_m == 0) return VAQ_OK;
+  if (size_m <= DECODE_MAX_M) return w4a16_decode_workspace((int)size_m, (int)size_n, (int)size_k, c_tmp_bytes, counter_ints);
+  if (has_perm) *a_tmp_bytes = (size_t)size_m * (size_t)size_k * 2;
+  return VAQ_OK;
+}
+
+extern "C" int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
+                              const int32_t* perm, const void* bias, void* c, float* c_tmp, void* a_tmp,
+                              int32_t* counters, int64_t counter_ints, int64_t size_m, int64_t size_n, int64_t size_k,
+                              int group_size, int dtype, int wtype, int force_path, void* stream) {
+  using namespace vaq;
+  int rc = check_shape(size_m, size_n, size_k);
+  if (rc != VAQ_OK) return rc;
+  VAQ_CHECK_ARG(dtype == VAQ_F16 || dtype == VAQ_BF16, "w4a16_gemm: only supports bfloat16 and float16 (dtype tag %d)",
+                dtype);
+  VAQ_CHECK_ARG(wtype == VAQ_WTYPE_U4B8 || wtype == VAQ_WTYPE_U4, "w4a16_gemm: unknown weight type tag %d", wtype);
+  VAQ_CHECK_ARG((wtype == VAQ_WTYPE_U4) == (zeros != nullptr),
+                "w4a16_gemm: b_q_type must be uint4 when has_zp = True and uint4b8 when has_zp = False");
+  VAQ_CHECK_SUPPORTED(group_size == 128, "w4a16_gemm: group_size = %d is not built (only 128)", group_size);
+  VAQ_CHECK_ARG(force_path >= 0 && force_path <= 2, "w4a16_gemm: force_path = %d", force_path);
+  if (size_m == 0) return VAQ_OK;
+  VAQ_CHECK_ARG(a && b && scales && c, "w4a16_gemm: null pointer");
+  VAQ_CHECK_ARG(lda >= size_k && lda % 8 == 0, "w4a16_gemm: A.stride(0) = %lld must be >= size_k and divisible by 8",
+                (long long)lda);
+  VAQ_CHECK_ARG(((uintptr_t)a % 16) == 0, "w4a16_gemm: A must aligned to 16 bytes");
+  VAQ_CHECK_ARG(((uintptr_t)b % 16) == 0 && ((uintptr_t)scales % 8) == 0 && ((uintptr_t)c % 8) == 0,
+                "w4a16_gemm: b_q_weight must be 16-byte, b_scales and c 8-byte aligned");
+  VAQ_CHECK_ARG(!perm || ((uintptr_t)perm % 16) == 0, "w4a16_gemm: perm must be 16-byte aligned");
+  VAQ_CHECK_ARG(!bias || ((uintptr_t)bias % 8) == 0, "w4a16_gemm: bias must be 8-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+
+  bool decode = size_m <= DECODE_MAX_M;
+  if (force_path == 1) {
+    VAQ_CHECK_ARG(size_m <= DECODE_MAX_M, "w4a16_gemm: decode path forced with size_m = %lld > %lld", (long long)size_m,
+                  (long long)DECODE_MAX_M);
+    decode = true;
+  } else if (force_path == 2) {
+    decode = false;
+  }
+  if (decode)
+    return w4a16_decode_launch(a, lda, b, scales, zeros, perm, bias, c, c_tmp, counters, counter_ints, (int)size_m,
+                               (int)size_n, (int)size_k, dtype, s);
+
+  const void* a_eff = a;
+  int64_t lda_eff = lda;
+  if (perm) {
+    VAQ_CHECK_ARG(a_tmp != nullptr, "w4a16_gemm: act_order on the prefill path needs a_tmp [size_m, size_k]");
+    VAQ_CHECK_ARG(((uintptr_t)a_tmp % 16) == 0, "w4a16_gemm: a_tmp must be 16-byte aligned");
+    rc = vaq_permute_cols(a, lda, perm, a_tmp, size_m, size_k, stream);
+    if (rc != VAQ_OK) return rc;
+    a_eff = a_tmp;
+    lda_eff = size_k;
+  }
+  return w4a16_prefill_launch(a_eff, lda_eff, b, scales, zeros, bias, c, (int)size_m, (int)size_n, (int)size_k, dtype, s);
+}

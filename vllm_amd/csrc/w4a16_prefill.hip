@@ -1,0 +1,293 @@
+// W4A16 prefill-shaped GEMM (M > 32) for gfx950: C[M,N] = A[M,K] . dequant(B[K,N]) (+bias).
+//
+// MFMA-bound.  One workgroup (4 wavefronts, 2 x 2) computes a BM x BN output tile with v_mfma_f32_32x32x16;
+// each wavefront owns (BM/2) x (BN/2) of it as WMB x WNB accumulator blocks of 32 x 32 fp32.
+//
+//  * K is walked in steps of 64.  A[BM x 64] goes global -> registers -> LDS unchanged.  The weight tile is read
+//    in the NATIVE order (one 16-byte load per lane covers 128 k of one column, i.e. two K steps), dequantised
+//    *with* its group scale and zero point to the 16-bit activation type and written to LDS as [n][k] so that both
+//    MFMA operands are 16-byte, k-contiguous LDS reads.
+//  * Dequantisation is exact: code -> fp32 (v_cvt_f32_ubyte), w = fma(code, s, -(z*s)) is the exact real number
+//    (code - z) * s (<= 16 significant bits), then one round-to-nearest-even to bf16/fp16.  That is bit-for-bit the
+//    weight `(q - z).to(dtype) * s` of the reference's dequantise-then-matmul path.
+//  * LDS rows are padded to 72 elements (144 B): 16-byte accesses by 8 consecutive rows hit 8 disjoint bank groups.
+//  * LDS is double buffered: while the MFMAs of step i run from buffer i&1, step i+1 is staged into the other
+//    buffer; one barrier per step.  Global loads for step i+2 are issued right after the registers are drained.
+//  * act_order: the caller passes activations already gathered through `perm` (vaq_permute_cols).
+#include "vaq_common.h"
+
+namespace vaq {
+
+struct PrefillParams {
+  const uint16_t* a;
+  int64_t lda;
+  const v4u* b;
+  const uint16_t* scales;
+  const uint32_t* zeros;
+  const uint16_t* bias;
+  uint16_t* c;
+  int M, N, K, G, NT;
+};
+
+constexpr int PF_BK = 64;
+constexpr int PF_PITCH = 72;   // LDS row pitch in 16-bit elements
+
+template <bool BF16>
+__device__ inline uint32_t pack2(float lo, float hi) {
+  if constexpr (BF16) {
+    typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+    v2bf r = {(__bf16)lo, (__bf16)hi};   // v_cvt_pk_bf16_f32, round-to-nearest-even
+    return __builtin_bit_cast(uint32_t, r);
+  } else {
+    return (uint32_t)F16Traits<false>::from_float(lo) | ((uint32_t)F16Traits<false>::from_float(hi) << 16);
+  }
+}
+
+// One native weight word (8 codes of 8 consecutive k) -> 8 scaled 16-bit weights in k order.
+template <bool BF16>
+__device__ inline v4u dequant_scaled(uint32_t w, float s, float neg_zs) {
+  const uint32_t t = w & 0x0f0f0f0fu;          // nibble positions 0,2,4,6 -> elements 0,4,1,5
+  const uint32_t u = (w >> 4) & 0x0f0f0f0fu;   // nibble positions 1,3,5,7 -> elements 2,6,3,7
+  const float e0 = fmaf((float)(t & 0xffu), s, neg_zs);
+  const float e4 = fmaf((float)((t >> 8) & 0xffu), s, neg_zs);
+  const float e1 = fmaf((float)((t >> 16) & 0xffu), s, neg_zs);
+  const float e5 = fmaf((float)(t >> 24), s, neg_zs);
+  const float e2 = fmaf((float)(u & 0xffu), s, neg_zs);
+  const float e6 = fmaf((float)((u >> 8) & 0xffu), s, neg_zs);
+  const float e3 = fmaf((float)((u >> 16) & 0xffu), s, neg_zs);
+  const float e7 = fmaf((float)(u >> 24), s, neg_zs);
+  v4u r;
+  r.x = pack2<BF16>(e0, e1);
+  r.y = pack2<BF16>(e2, e3);
+  r.z = pack2<BF16>(e4, e5);
+  r.w = pack2<BF16>(e6, e7);
+  return r;
+}
+
+template <bool BF16, int WMB, int WNB, bool HAS_ZP>
+__global__ __launch_bounds__(256) void w4a16_prefill_kernel(const PrefillParams p) {
+  using T = F16Traits<BF16>;
+  constexpr int BM = 64 * WMB, BN = 64 * WNB;
+  constexpr int A_CH = BM / 32;    // 16-byte chunks of A per thread per step
+  constexpr int W_LD = BN / 64;    // 16-byte weight loads per thread per group
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  uint16_t* As = lds;                           // [2][BM][PITCH]
+  uint16_t* Bs = lds + 2 * BM * PF_PITCH;       // [2][BN][PITCH]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // XCD-aware tile order: consecutive workgroup ids land on different XCDs (round-robin over 8), so give each XCD a
+  // contiguous band of tile ids; tiles in a band share A rows / W columns in that XCD's L2.
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  const int total = tiles_m * tiles_n;
+  int bid = blockIdx.x;
+  {
+    const int per = (total + 7) / 8;
+    const int xcd = bid & 7, idx = bid >> 3;
+    const int remapped = xcd * per + idx;
+    // only valid as a bijection when total % 8 == 0; otherwise keep the plain order
+    if (total % 8 == 0) bid = remapped;
+  }
+  // walk tiles column-band-major in groups of 8 m-tiles so that neighbours share weights
+  const int tm = bid % tiles_m, tn = bid / tiles_m;
+  const int m0 = tm * BM, n0 = tn * BN, nt0 = n0 / 16;
+
+  // ---- per-thread staging state ----
+  v4u areg[A_CH];
+  v4u wreg[W_LD];
+  float ws[W_LD], wnz[W_LD];     // scale and -(zero*scale) of the current group, per owned column
+
+  auto load_a = [&](int step) {
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c >> 3, ch = c & 7;
+      const int m = m0 + row;
+      v4u v = {0u, 0u, 0u, 0u};
+      if (m < p.M) v = *reinterpret_cast<const v4u*>(p.a + (int64_t)m * p.lda + step * PF_BK + ch * 8);
+      areg[i] = v;
+    }
+  };
+  auto store_a = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c >> 3, ch = c & 7;
+      *reinterpret_cast<v4u*>(As + ((size_t)buf * BM + row) * PF_PITCH + ch * 8) = areg[i];
+    }
+  };
+  auto load_w = [&](int g) {
+#pragma unroll
+    for (int i = 0; i < W_LD; ++i) {
+      const int ntl = i * 4 + wave;
+      const int nt = nt0 + ntl;
+      v4u v = {0u, 0u, 0u, 0u};
+      float s = 0.f, z = 8.f;
+      if (nt < p.NT) {
+        v = p.b[((int64_t)g * p.NT + nt) * 64 + lane];
+        const int n = nt * 16 + (lane & 15);
+        s = T::to_float(p.scales[(int64_t)g * p.N + n]);
+        if constexpr (HAS_ZP) {
+          const uint32_t zw = p.zeros[(int64_t)g * (p.N >> 3) + (n >> 3)];
+          z = (float)((zw >> ((n & 7) * 4)) & 0xFu);
+        }
+      }
+      wreg[i] = v;
+      ws[i] = s;
+      wnz[i] = -(z * s);   // exact: <= 4 + 11 significant bits
+    }
+  };
+  auto store_w = [&](int buf, int half) {
+    const int o = lane >> 4, r = lane & 15;
+#pragma unroll
+    for (int i = 0; i < W_LD; ++i) {
+      const int ntl = i * 4 + wave;
+      const uint32_t w0 = half ? wreg[i].z : wreg[i].x;
+      const uint32_t w1 = half ? wreg[i].w : wreg[i].y;
+      uint16_t* rowp = Bs + ((size_t)buf * BN + ntl * 16 + r) * PF_PITCH + o * 8;
+      *reinterpret_cast<v4u*>(rowp) = dequant_scaled<BF16>(w0, ws[i], wnz[i]);
+      *reinterpret_cast<v4u*>(rowp + 32) = dequant_scaled<BF16>(w1, ws[i], wnz[i]);
+    }
+  };
+
+  v16f acc[WMB][WNB];
+#pragma unroll
+  for (int i = 0; i < WMB; ++i)
+#pragma unroll
+    for (int j = 0; j < WNB; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const int steps = p.K / PF_BK;
+
+  // ---- prologue: stage step 0, issue loads for step 1 ----
+  load_a(0);
+  load_w(0);
+  store_a(0);
+  store_w(0, 0);
+  if (steps > 1) load_a(1);
+  __syncthreads();
+
+  for (int step = 0; step < steps; ++step) {
+    const int cur = step & 1;
+    // stage step+1 into the other buffer
+    if (step + 1 < steps) {
+      const int nstep = step + 1;
+      store_a(cur ^ 1);
+      store_w(cur ^ 1, nstep & 1);
+      if (nstep + 1 < steps) {
+        load_a(nstep + 1);
+        if (nstep & 1) load_w((nstep + 1) >> 1);   // both halves of the group consumed: fetch the next group
+      }
+    }
+    // MFMAs of this step
+    const uint16_t* Ab = As + ((size_t)cur * BM + wm * 32 * WMB + (lane & 31)) * PF_PITCH + (lane >> 5) * 8;
+    const uint16_t* Bb = Bs + ((size_t)cur * BN + wn * 32 * WNB + (lane & 31)) * PF_PITCH + (lane >> 5) * 8;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      v4u af[WMB], bf[WNB];
+#pragma unroll
+      for (int i = 0; i < WMB; ++i) af[i] = *reinterpret_cast<const v4u*>(Ab + (size_t)i * 32 * PF_PITCH + kk * 16);
+#pragma unroll
+      for (int j = 0; j < WNB; ++j) bf[j] = *reinterpret_cast<const v4u*>(Bb + (size_t)j * 32 * PF_PITCH + kk * 16);
+#pragma unroll
+      for (int i = 0; i < WMB; ++i)
+#pragma unroll
+        for (int j = 0; j < WNB; ++j) acc[i][j] = T::mfma32(af[i], bf[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane holds column n = lane%32, rows 8*(e/4) + 4*(lane/32) + e%4 of each 32x32 block ----
+#pragma unroll
+  for (int j = 0; j < WNB; ++j) {
+    const int n = n0 + wn * 32 * WNB + j * 32 + (lane & 31);
+    if (n >= p.N) continue;
+    float bv = 0.f;
+    if (p.bias) bv = T::to_float(p.bias[n]);
+#pragma unroll
+    for (int i = 0; i < WMB; ++i) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = m0 + wm * 32 * WMB + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+        if (m < p.M) p.c[(int64_t)m * p.N + n] = T::from_float(acc[i][j][e] + bv);
+      }
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------- host side
+
+template <bool BF16, int WMB, int WNB, bool HAS_ZP>
+static int launch_prefill(const PrefillParams& p, hipStream_t s) {
+  constexpr int BM = 64 * WMB, BN = 64 * WNB;
+  const size_t lds = (size_t)2 * (BM + BN) * PF_PITCH * sizeof(uint16_t);
+  auto kern = w4a16_prefill_kernel<BF16, WMB, WNB, HAS_ZP>;
+  static bool attr_done = false;   // idempotent attribute; a benign race sets it twice
+  if (!attr_done) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
+        hipSuccess) {
+      set_error("w4a16_gemm(prefill): cannot reserve %zu bytes of LDS", lds);
+      (void)hipGetLastError();
+      return VAQ_ERR_LAUNCH;
+    }
+    attr_done = true;
+  }
+  const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(256), lds, s, p);
+  return VAQ_OK;
+}
+
+template <bool BF16, bool HAS_ZP>
+static int dispatch_tile(const PrefillParams& p, int tile, hipStream_t s) {
+  switch (tile) {
+    case 0: return launch_prefill<BF16, 4, 4, HAS_ZP>(p, s);   // 256 x 256
+    case 1: return launch_prefill<BF16, 2, 2, HAS_ZP>(p, s);   // 128 x 128
+    case 2: return launch_prefill<BF16, 1, 2, HAS_ZP>(p, s);   //  64 x 128
+    default: break;
+  }
+  set_error("w4a16_gemm(prefill): unknown tile id %d", tile);
+  return VAQ_ERR_UNSUPPORTED;
+}
+
+static int g_force_tile = -1;
+
+static int pick_tile(int M, int N) {
+  if (g_force_tile >= 0) return g_force_tile;
+  const int cus = num_cus_current_device();
+  auto tiles = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+  if (tiles(256, 256) >= cus) return 0;
+  if (tiles(128, 128) >= cus) return 1;
+  return 2;
+}
+
+int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
+                         const void* bias, void* c, int M, int N, int K, int dtype, hipStream_t s) {
+  PrefillParams p;
+  p.a = (const uint16_t*)a;
+  p.lda = lda;
+  p.b = (const v4u*)b;
+  p.scales = (const uint16_t*)scales;
+  p.zeros = (const uint32_t*)zeros;
+  p.bias = (const uint16_t*)bias;
+  p.c = (uint16_t*)c;
+  p.M = M; p.N = N; p.K = K;
+  p.G = K / 128;
+  p.NT = N / 16;
+  const int tile = pick_tile(M, N);
+  const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
+  int rc;
+  if (bf16) rc = zp ? dispatch_tile<true, true>(p, tile, s) : dispatch_tile<true, false>(p, tile, s);
+  else rc = zp ? dispatch_tile<false, true>(p, tile, s) : dispatch_tile<false, false>(p, tile, s);
+  if (rc != VAQ_OK) return rc;
+  VAQ_CHECK_LAUNCH("w4a16_gemm(prefill)");
+  return VAQ_OK;
+}
+
+}  // namespace vaq
+
+// Benchmark / tuning aid, not part of the drop-in surface: force the prefill tile (-1 = automatic,
+// 0 = 256x256, 1 = 128x128, 2 = 64x128).  Process-global and not thread-safe.
+extern "C" void vaq_debug_set_prefill_tile(int tile) { vaq::g_force_tile = tile; }
