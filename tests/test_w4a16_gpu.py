@@ -1,0 +1,189 @@
+"""GPU parity tests of the W4A16 path (repack, decode GEMM, prefill GEMM) against the CPU oracle, through the op
+surface that sits on the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import native_layout as nl
+from oracle import w4a16 as o
+from tests.helpers import W4A16Layer, check_gemm_close, to_dev
+
+pytestmark = pytest.mark.gpu
+
+LLAMA_SHAPES = [(4096, 6144), (4096, 4096), (4096, 28672), (14336, 4096)]
+
+
+def _acts(m, k, device, dtype=torch.bfloat16, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(m, k, generator=g).to(dtype).to(device)
+
+
+# ------------------------------------------------------------------------------------------------ repack
+
+@pytest.mark.parametrize("k,n", [(128, 64), (128, 256), (1024, 256), (128 * 13, 64 * 37), (128 * 11, 64 * 13), (4096, 4096)])
+@pytest.mark.parametrize("act_order", [False, True])
+def test_repack_bit_exact_both_layouts(device, k, n, act_order):
+    import vllm_amd._custom_ops as ops
+    rng = np.random.default_rng(k + n)
+    q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    qw = to_dev(o.gptq_pack(q, 4), device)
+    if act_order:
+        perm_np = rng.permutation(k).astype(np.int32)
+        perm = to_dev(perm_np, device)
+        q_sorted = q[perm_np]
+    else:
+        perm = torch.empty(0, dtype=torch.int32, device=device)
+        q_sorted = q
+    marlin = ops.gptq_marlin_repack(qw, perm, k, n, 4, layout="marlin")
+    native = ops.gptq_marlin_repack(qw, perm, k, n, 4)
+    assert marlin.shape == native.shape == (k // 16, 2 * n) and marlin.dtype == torch.int32
+    assert np.array_equal(marlin.cpu().numpy(), o.marlin_weights(q_sorted)), "marlin order differs from the oracle"
+    assert np.array_equal(native.cpu().numpy(), nl.native_pack(q_sorted)), "native order differs from its spec"
+    assert np.array_equal(nl.native_unpack(native.cpu().numpy(), k, n), q_sorted)
+
+
+# ------------------------------------------------------------------------------------------------ GEMM, small shapes
+
+SMALL = [(128, 64), (512, 256), (1024, 192), (2048, 576), (14336 // 4, 128)]
+
+
+@pytest.mark.parametrize("k,n", SMALL)
+@pytest.mark.parametrize("m", [1, 4, 16, 17, 32])
+@pytest.mark.parametrize("asym,act_order", [(False, False), (True, False), (False, True), (True, True)])
+def test_decode_gemm_small(device, k, n, m, asym, act_order):
+    if act_order and k == 128:
+        pytest.skip("act_order needs more than one group (gptq_marlin.cu:805)")
+    case = o.make_w4a16_case(k, n, 128, asym=asym, act_order=act_order, seed=k + n + m)
+    layer = W4A16Layer(case, device)
+    a = _acts(m, k, device, seed=m)
+    out = layer(a)
+    assert out.shape == (m, n) and out.dtype == torch.bfloat16
+    check_gemm_close(out, o.gemm_ref(a.cpu(), o.case_w_ref(case)), f"decode k={k} n={n} m={m}")
+    assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
+
+
+@pytest.mark.parametrize("k,n", SMALL)
+@pytest.mark.parametrize("m", [33, 64, 200, 257])
+@pytest.mark.parametrize("asym,act_order", [(False, False), (True, True)])
+def test_prefill_gemm_small(device, k, n, m, asym, act_order):
+    if act_order and k == 128:
+        pytest.skip("act_order needs more than one group (gptq_marlin.cu:805)")
+    case = o.make_w4a16_case(k, n, 128, asym=asym, act_order=act_order, seed=k + n + m)
+    layer = W4A16Layer(case, device)
+    a = _acts(m, k, device, seed=m)
+    out = layer(a)
+    check_gemm_close(out, o.gemm_ref(a.cpu(), o.case_w_ref(case)), f"prefill k={k} n={n} m={m}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m", [3, 16, 96])
+def test_gemm_fp16_and_bias(device, dtype, m):
+    k, n = 1024, 256
+    case = o.make_w4a16_case(k, n, 128, asym=True, dtype=dtype, seed=5)
+    layer = W4A16Layer(case, device, dtype)
+    a = _acts(m, k, device, dtype, seed=2)
+    bias = (torch.randn(n, generator=torch.Generator().manual_seed(3)) * 0.5).to(dtype)
+    out = layer(a, bias.to(device))
+    assert out.dtype == dtype
+    check_gemm_close(out, o.gemm_ref(a.cpu(), o.case_w_ref(case), bias), f"{dtype} m={m} bias")
+
+
+@pytest.mark.parametrize("m", [1, 48])
+def test_one_hot_activation_returns_dequantised_rows_exactly(device, m):
+    """A one-hot row of A selects one dequantised weight row: the GEMM must return rn16((q - z) * s) bit-for-bit."""
+    k, n = 512, 128
+    case = o.make_w4a16_case(k, n, 128, asym=True, seed=11)
+    layer = W4A16Layer(case, device)
+    rows = [(37 * i + 5) % k for i in range(m)]
+    a = torch.zeros(m, k, dtype=torch.bfloat16)
+    for i, r in enumerate(rows):
+        a[i, r] = 1
+    out = layer(a.to(device)).cpu()
+    w = o.case_w_ref(case)
+    assert torch.equal(out, w[rows])
+
+
+@pytest.mark.parametrize("m", [8, 40])
+def test_unit_weights_give_row_sums(device, m):
+    k, n = 1024, 128
+    q = np.full((k, n), 9, dtype=np.int32)
+    case = dict(q=q, qweight=o.gptq_pack(q, 4), scales=torch.ones(k // 128, n, dtype=torch.bfloat16), zp_vals=None,
+                qzeros=None, g_idx=None, group_size=128)
+    layer = W4A16Layer(case, device)
+    a = _acts(m, k, device, seed=9)
+    out = layer(a).cpu().double()
+    expect = a.cpu().double().sum(dim=1, keepdim=True)
+    assert (out - expect).abs().max() <= expect.abs().max() * 2.0 ** -7
+
+
+def test_zero_point_eight_equals_symmetric(device):
+    k, n, m = 512, 128, 5
+    case = o.make_w4a16_case(k, n, 128, seed=4)
+    sym = W4A16Layer(case, device)
+    case_asym = dict(case, zp_vals=np.full((k // 128, n), 8, dtype=np.int32))
+    asym = W4A16Layer(case_asym, device)
+    a = _acts(m, k, device)
+    assert torch.equal(sym(a), asym(a))
+
+
+def test_strided_activations(device):
+    """Rows of A may be a strided view (reference: test_marlin_gemm_subset_input, test_marlin_gemm.py:537-581)."""
+    k, n = 512, 128
+    case = o.make_w4a16_case(k, n, 128, seed=6)
+    layer = W4A16Layer(case, device)
+    for m in (7, 70):
+        big = _acts(m, k + 128, device, seed=m)
+        a = big[:, 64:64 + k]
+        check_gemm_close(layer(a), o.gemm_ref(a.cpu(), o.case_w_ref(case)), f"strided m={m}")
+
+
+def test_m_zero_returns_empty(device):
+    case = o.make_w4a16_case(128, 64, 128)
+    layer = W4A16Layer(case, device)
+    out = layer(torch.empty(0, 128, dtype=torch.bfloat16, device=device))
+    assert out.shape == (0, 64)
+
+
+# ------------------------------------------------------------------------------------------------ BASELINE sizes
+
+def test_config1_reference_cpu_case(device):
+    """BASELINE config 1: M=16, K=N=4096, g=128, symmetric: bit-exact repack + output tolerance."""
+    k = n = 4096
+    case = o.make_w4a16_case(k, n, 128, seed=0)
+    layer = W4A16Layer(case, device)
+    assert np.array_equal(nl.native_unpack(layer.w.cpu().numpy(), k, n), case["q"])
+    a = _acts(16, k, device)
+    check_gemm_close(layer(a), o.gemm_ref(a.cpu(), o.case_w_ref(case)), "config 1")
+
+
+@pytest.mark.parametrize("k,n", LLAMA_SHAPES)
+def test_config2_decode_llama_shapes(device, k, n):
+    case = o.make_w4a16_case(k, n, 128, seed=1)
+    layer = W4A16Layer(case, device)
+    w_ref = o.case_w_ref(case)
+    for m in (1, 4, 16):
+        a = _acts(m, k, device, seed=m)
+        out = layer(a)
+        check_gemm_close(out, o.gemm_ref(a.cpu(), w_ref), f"config 2 k={k} n={n} m={m}")
+        assert torch.equal(out, layer(a)), "decode GEMM is not deterministic run to run"
+
+
+@pytest.mark.parametrize("k,n", LLAMA_SHAPES)
+@pytest.mark.parametrize("group_level", [False, True])
+def test_config3_prefill_llama_shapes_sampled(device, k, n, group_level):
+    """Asymmetric + act_order at M=4096 (also 512): the oracle is evaluated on 24 sampled rows (the full fp64 GEMM
+    would take minutes on the CPU); rows are independent in a GEMM, so a wrong tile shows up in its rows."""
+    case = o.make_w4a16_case(k, n, 128, asym=True, act_order=True, group_level_perm=group_level, seed=2)
+    layer = W4A16Layer(case, device)
+    w_ref = o.case_w_ref(case)
+    for m in (512, 4096):
+        a = _acts(m, k, device, seed=m)
+        out = layer(a)
+        rows = np.random.default_rng(m).choice(m, size=24, replace=False)
+        rows = np.concatenate([rows, [0, m - 1]])
+        ref = o.gemm_ref(a.cpu()[rows], w_ref)
+        check_gemm_close(out[rows], ref, f"config 3 k={k} n={n} m={m}")
+        # every row must be finite and of plausible magnitude (catches tiles that were never written)
+        assert torch.isfinite(out).all()
+        col_norm = out.float().norm(dim=1)
+        assert bool((col_norm > 0).all())

@@ -78,7 +78,7 @@ def _check_repack_args(b_q_weight, perm, size_k, size_n, num_bits) -> None:
 
 
 def _repack_impl(b_q_weight: torch.Tensor, perm: torch.Tensor, size_k: int, size_n: int, num_bits: int,
-                 layout: int) -> torch.Tensor:
+                 layout: int = _lib.VAQ_LAYOUT_NATIVE) -> torch.Tensor:
     _check_repack_args(b_q_weight, perm, size_k, size_n, num_bits)
     lib = _lib.load()
     pack_factor = 32 // num_bits
@@ -90,7 +90,7 @@ def _repack_impl(b_q_weight: torch.Tensor, perm: torch.Tensor, size_k: int, size
     return out
 
 
-def _repack_fake(b_q_weight, perm, size_k, size_n, num_bits, layout=0):
+def _repack_fake(b_q_weight, perm, size_k, size_n, num_bits, layout=1):
     pack_factor = 32 // num_bits
     return torch.empty((size_k // GPTQ_MARLIN_TILE, size_n * GPTQ_MARLIN_TILE // pack_factor),
                        dtype=b_q_weight.dtype, device=b_q_weight.device)
@@ -201,6 +201,8 @@ def _check_gemm_args(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, 
     if has_act_order and not is_k_full:
         raise NotImplementedError("gptq_marlin_gemm: is_k_full = False (act_order x row-parallel shard) is not built; "
                                   "one-GPU layers always have is_k_full = True")
+    if group_size == -1 and size_k == 128:
+        group_size = 128          # one group spanning K = 128 rows is the same thing as group_size 128
     if group_size != 128:
         raise NotImplementedError(f"gptq_marlin_gemm: group_size = {group_size} is not built for gfx950 (only 128)")
     _check(size_k % GPTQ_MARLIN_MIN_THREAD_K == 0,
