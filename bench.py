@@ -1,0 +1,319 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+Headline workload (``config.workload``): BASELINE config 2 -- decode-shaped W4A16 GEMMs, the four Llama-3-8B
+projection shapes (K,N) x M in {1,4,16}, group 128, symmetric int4, bf16 activations.  One *step* is one pass over
+those 12 GEMMs, launched through the public op surface (``vllm_amd._custom_ops.gptq_marlin_gemm`` -> C ABI) and
+replayed as a HIP graph, as a serving loop would run them.  Every GEMM of a step reads its own copy of the weights and
+two full sets alternate between steps, so ~650 MB of distinct weights cycle through the 256 MB Infinity Cache: the
+figure is an HBM figure, not a cache figure.
+
+``value`` = algorithmic bytes of one step / time of one step (GB/s); inputs are resident in HBM before the timed
+region.  ``roofline`` prices the dominant kernel (the decode GEMM) against the 8 TB/s HBM peak; ``cpu_baseline`` times
+the CPU oracle (torch dequantise + matmul, the reference's CPU-runnable path) on a bounded sample on the host cores.
+Extra sections (prefill W4A16, FP8 GEMM and FP8 activation quant, each against its own roofline) are reported under
+``extra`` and on stderr; they are measured outside the timed region.
+
+One GPU only: ``--gpus N`` with N > 1 exits with a message.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+LLAMA_SHAPES = [(4096, 6144), (4096, 4096), (4096, 28672), (14336, 4096)]   # (K, N): qkv, o, gate_up, down
+DECODE_MS = (1, 4, 16)
+HBM_PEAK_GBS = 8000.0
+BF16_PEAK_TFLOPS = 2500.0
+FP8_PEAK_TFLOPS = 5000.0
+GROUP = 128
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def w4a16_bytes(m, k, n, asym_act=False):
+    b = k * n // 2 + (k // GROUP) * n * 2 + m * k * 2 + m * n * 2
+    if asym_act:
+        b += (k // GROUP) * n // 2 + 4 * k
+    return b
+
+
+def fp8_mm_bytes(m, k, n, bias=True):
+    return k * n + 4 * n + m * k + 4 * m + 2 * m * n + (2 * n if bias else 0)
+
+
+# --------------------------------------------------------------------------------------------- device-side workload
+
+class W4Layer:
+    """Synthetic GPTQ layer already in the GEMM's native layout (random bits == uniform int4 codes)."""
+
+    def __init__(self, k, n, dev, gen, asym=False, act_order=False):
+        from vllm_amd.layers.quantization.utils.marlin_utils import marlin_make_workspace_new
+        from vllm_amd.scalar_type import scalar_types
+        self.k, self.n = k, n
+        self.w = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 16, 2 * n), dtype=torch.int32, device=dev, generator=gen)
+        self.s = (torch.randn(k // GROUP, n, device=dev, generator=gen).abs() * 0.01 + 1e-3).to(torch.float16).to(torch.bfloat16)
+        self.empty = torch.empty(0, dtype=torch.int32, device=dev)
+        self.zp = self.empty
+        self.wtype = scalar_types.uint4b8
+        if asym:
+            self.zp = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // GROUP, n // 8), dtype=torch.int32, device=dev, generator=gen)
+            self.wtype = scalar_types.uint4
+        self.g_idx = self.perm = self.empty
+        if act_order:
+            self.perm = torch.randperm(k, device=dev, generator=gen).to(torch.int32)
+            self.g_idx = (torch.arange(k, device=dev) // GROUP).to(torch.int32)
+        self.ws = marlin_make_workspace_new(dev)
+
+    def __call__(self, a):
+        import vllm_amd._custom_ops as ops
+        return ops.gptq_marlin_gemm(a, None, self.w, None, self.s, None, self.zp, self.g_idx, self.perm, self.ws,
+                                    self.wtype, a.shape[0], self.n, self.k, is_k_full=True, use_fp32_reduce=True)
+
+
+def time_graph(fn, iters, warmup, inner=1):
+    """Capture ``fn`` (a sequence of launches) into a HIP graph, replay; returns seconds per replay."""
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        fn()
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        fn()
+    for _ in range(warmup):
+        g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / iters / inner
+
+
+def headline(dev, steps, warmup):
+    gen = torch.Generator(device=dev).manual_seed(0)
+    sets = []
+    for _ in range(2):          # two full weight sets alternate between steps
+        layers = [(W4Layer(k, n, dev, gen), m) for (k, n) in LLAMA_SHAPES for m in DECODE_MS]
+        sets.append(layers)
+    acts = {(k, m): torch.randn(m, k, device=dev, generator=gen).to(torch.bfloat16) for (k, _) in LLAMA_SHAPES for m in DECODE_MS}
+    step_bytes = sum(w4a16_bytes(m, k, n) for (k, n) in LLAMA_SHAPES for m in DECODE_MS)
+    weight_bytes = sum(l.w.numel() * 4 for layers in sets for l, _ in layers)
+    log(f"[headline] 12 GEMMs/step, {step_bytes / 1e6:.1f} MB algorithmic per step, {weight_bytes / 1e6:.0f} MB of distinct weights cycling")
+
+    def run_set(i):
+        for layer, m in sets[i]:
+            layer(acts[(layer.k, m)])
+
+    graphs = []
+    for i in range(2):
+        run_set(i)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            run_set(i)
+        graphs.append(g)
+    for w in range(warmup):
+        graphs[w & 1].replay()
+    torch.cuda.synchronize()
+    # timed region: exactly `steps` steps, events on the stream the kernels run on, synchronised on both sides
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for st in range(steps):
+        graphs[st & 1].replay()
+    e1.record()
+    torch.cuda.synchronize()
+    sec = e0.elapsed_time(e1) * 1e-3 / steps
+    return sec, step_bytes, sets, acts
+
+
+def per_shape_decode(dev, sets, acts):
+    """Each decode GEMM on its own: graph of its launches over both weight copies plus enough extra copies to stay
+    cold would need more memory than is useful; instead alternate the two copies interleaved with the other layers'
+    launches removed -- i.e. warm-ish for small layers.  Reported as 'cache-resident unless noted'."""
+    rows = []
+    gen = torch.Generator(device=dev).manual_seed(1)
+    for (k, n) in LLAMA_SHAPES:
+        copies = max(2, int(600e6 // (k * n // 2)))
+        layers = [W4Layer(k, n, dev, gen) for _ in range(copies)]
+        for m in DECODE_MS:
+            a = acts[(k, m)]
+
+            def fn():
+                for l in layers:
+                    l(a)
+            t = time_graph(fn, iters=10, warmup=3, inner=copies)
+            b = w4a16_bytes(m, k, n)
+            rows.append(dict(kind="w4a16_decode", K=k, N=n, M=m, us=t * 1e6, GBps=b / t / 1e9, hbm_frac=b / t / 1e9 / HBM_PEAK_GBS,
+                             TFLOPs=2 * m * n * k / t / 1e12, cold=True))
+            log(f"[decode  cold] K={k:5d} N={n:5d} M={m:2d}: {t * 1e6:7.2f} us  {b / t / 1e9:7.0f} GB/s ({100 * b / t / 1e9 / HBM_PEAK_GBS:4.1f}% of 8 TB/s)")
+        del layers
+    return rows
+
+
+def prefill_section(dev):
+    rows = []
+    gen = torch.Generator(device=dev).manual_seed(2)
+    for (k, n) in LLAMA_SHAPES:
+        layer = W4Layer(k, n, dev, gen, asym=True, act_order=True)
+        for m in (512, 2048, 4096):
+            a = torch.randn(m, k, device=dev, generator=gen).to(torch.bfloat16)
+            inner = 4 if m <= 512 else 1
+            t = time_graph(lambda: [layer(a) for _ in range(inner)], iters=5, warmup=2, inner=inner)
+            fl = 2.0 * m * n * k
+            rows.append(dict(kind="w4a16_prefill_asym_actorder", K=k, N=n, M=m, us=t * 1e6, TFLOPs=fl / t / 1e12,
+                             mfma_frac=fl / t / 1e12 / BF16_PEAK_TFLOPS, GBps=w4a16_bytes(m, k, n, True) / t / 1e9))
+            log(f"[prefill     ] K={k:5d} N={n:5d} M={m:4d}: {t * 1e6:8.1f} us  {fl / t / 1e12:7.1f} TFLOP/s ({100 * fl / t / 1e12 / BF16_PEAK_TFLOPS:4.1f}% of 2.5 PF)")
+        del layer
+    return rows
+
+
+def fp8_section(dev):
+    import vllm_amd._custom_ops as ops
+    rows = []
+    gen = torch.Generator(device=dev).manual_seed(3)
+    for (k, n) in LLAMA_SHAPES:
+        w = (torch.randn(n, k, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+        wq, ws = ops.scaled_fp8_quant(w, use_per_token_if_dynamic=True)
+        del w
+        bias = (torch.randn(n, device=dev, generator=gen) * 0.01).to(torch.bfloat16)
+        wt = wq.t()
+        for m in (1, 16, 256, 4096):
+            a = torch.randn(m, k, device=dev, generator=gen).to(torch.bfloat16)
+            aq, sa = ops.scaled_fp8_quant(a, use_per_token_if_dynamic=True)
+            inner = 20 if m <= 256 else 2
+            t = time_graph(lambda: [ops.cutlass_scaled_mm(aq, wt, sa, ws, torch.bfloat16, bias) for _ in range(inner)],
+                           iters=5, warmup=2, inner=inner)
+            tq = time_graph(lambda: [ops.scaled_fp8_quant(a, use_per_token_if_dynamic=True) for _ in range(20)],
+                            iters=5, warmup=2, inner=20)
+            fl = 2.0 * m * n * k
+            b = fp8_mm_bytes(m, k, n)
+            qb = 3 * m * k + 4 * m
+            rows.append(dict(kind="fp8_scaled_mm", K=k, N=n, M=m, us=t * 1e6, TFLOPs=fl / t / 1e12, mfma_frac=fl / t / 1e12 / FP8_PEAK_TFLOPS,
+                             GBps=b / t / 1e9, hbm_frac=b / t / 1e9 / HBM_PEAK_GBS, quant_us=tq * 1e6, quant_GBps=qb / tq / 1e9,
+                             cold=False))
+            log(f"[fp8 mm  warm] K={k:5d} N={n:5d} M={m:4d}: {t * 1e6:8.1f} us  {fl / t / 1e12:7.1f} TFLOP/s ({100 * fl / t / 1e12 / FP8_PEAK_TFLOPS:4.1f}% of 5 PF)  "
+                f"{b / t / 1e9:6.0f} GB/s | quant {tq * 1e6:6.1f} us {qb / tq / 1e9:6.0f} GB/s")
+        del wq, wt
+    return rows
+
+
+# --------------------------------------------------------------------------------------------- CPU baseline
+
+def cpu_baseline(budget_s: float = 15.0):
+    """The reference's CPU-runnable path, restated by the oracle: unpack int4 -> (q - 8).to(bf16) * s -> torch.matmul,
+    dequantisation included in every call (the reference path dequantises per call).  Bounded sample of the headline
+    workload: whole steps (the 12 GEMMs) are repeated until about `budget_s` seconds of CPU work have been timed."""
+    from oracle import w4a16 as o
+    threads = torch.get_num_threads()
+    rng = np.random.default_rng(0)
+    layers = []
+    for (k, n) in LLAMA_SHAPES:
+        qweight = rng.integers(-2 ** 31, 2 ** 31 - 1, size=(k // 8, n), dtype=np.int64).astype(np.int32)
+        scales = (torch.randn(k // GROUP, n).abs() * 0.01 + 1e-3).to(torch.bfloat16)
+        layers.append((k, n, qweight, scales))
+    total_b, total_t, steps_done = 0, 0.0, 0
+    while total_t < budget_s and steps_done < 50:
+        for (k, n, qweight, scales) in layers:
+            for m in DECODE_MS:
+                a = torch.randn(m, k).to(torch.bfloat16)
+                t0 = time.perf_counter()
+                w = o.dequantize(o.unpack_rows(qweight, 4), scales, 8, GROUP)
+                out = o.gemm_ref_like_reference(a, w)
+                total_t += time.perf_counter() - t0
+                total_b += w4a16_bytes(m, k, n)
+                assert out.shape == (m, n)
+        steps_done += 1
+    log(f"[cpu baseline] {steps_done} step(s) of 12 GEMMs in {total_t:.1f} s on {threads} threads: {total_b / total_t / 1e9:.3f} GB/s")
+    return dict(value=round(total_b / total_t / 1e9, 4), unit="GB/s", cores=threads, kind="port",
+                sample=f"{steps_done} full step(s) of the headline workload (12 GEMMs each) through the oracle: unpack + "
+                       f"dequantise (bf16) + torch.matmul per call, {total_t:.1f} s of CPU time")
+
+
+# --------------------------------------------------------------------------------------------- main
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--no-extra", action="store_true", help="skip the prefill / FP8 sections")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures ONE GPU (the quantized-linear path has no cross-GPU step); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    from vllm_amd import _lib
+    _lib.load()      # fail loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    sec, step_bytes, sets, acts = headline(dev, args.steps, args.warmup)
+    value = step_bytes / sec / 1e9
+    launches = len(LLAMA_SHAPES) * len(DECODE_MS)
+    log(f"[headline] {sec * 1e6:.1f} us/step, {value:.0f} GB/s = {100 * value / HBM_PEAK_GBS:.1f}% of HBM peak")
+    extra = {}
+    try:
+        extra["decode_per_shape"] = per_shape_decode(dev, sets, acts)
+    except Exception as e:   # extras never invalidate the headline
+        log(f"[decode per shape] failed: {e}")
+    del sets
+    torch.cuda.empty_cache()
+    if not args.no_extra:
+        for name, fn in (("prefill", prefill_section), ("fp8", fp8_section)):
+            try:
+                extra[name] = fn(dev)
+            except Exception as e:
+                log(f"[{name}] failed: {e}")
+            torch.cuda.empty_cache()
+    cpu = None if args.no_cpu else cpu_baseline()
+
+    out = {
+        "metric": "W4A16 decode GEMM effective HBM bandwidth (Llama-3-8B shapes, M in {1,4,16})",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE configs[1]: decode W4A16 GEMMs, (K,N) in {(4096,6144),(4096,4096),(4096,28672),"
+                               "(14336,4096)} x M in {1,4,16}, group 128, symmetric int4, bf16 act, fp32 acc; one step = "
+                               "12 GEMMs in a HIP graph, weights cold (650 MB cycling)",
+                   "launches_per_step": launches},
+        "roofline": {"bound": "hbm", "kernel": "vaq::w4a16_decode_kernel", "achieved": round(value, 2), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(value / HBM_PEAK_GBS, 4), "traffic": None,
+                     "avg_launch_us": round(sec * 1e6 / launches, 3),
+                     "algorithmic_bytes_per_launch": step_bytes // launches},
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

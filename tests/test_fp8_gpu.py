@@ -1,0 +1,219 @@
+"""GPU parity tests of the FP8 path: activation quantisation (bit-exact codes and scales) and the scaled GEMM,
+through the op surface that sits on the C ABI."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8 as f
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+LLAMA_SHAPES = [(4096, 6144), (4096, 4096), (4096, 28672), (14336, 4096)]
+
+
+def _codes(t: torch.Tensor) -> np.ndarray:
+    return t.detach().cpu().view(torch.uint8).numpy()
+
+
+# ------------------------------------------------------------------------------------------------ quantisation
+
+def test_quant_every_bf16_value_bit_exact(device):
+    """All 65 280 finite bf16 inputs in one row block, at several row scales: codes and scales equal the oracle."""
+    import vllm_amd._custom_ops as ops
+    bits = torch.arange(65536, dtype=torch.int32)
+    vals = (bits << 16).view(torch.float32)
+    vals = vals[torch.isfinite(vals)]
+    finite = vals.to(torch.bfloat16)
+    rows = []
+    for cap in (3.0e38, 1.0e4, 448.0, 1.0, 1.0e-3, 1.0e-30):
+        rows.append(torch.where(finite.float().abs() <= cap, finite, torch.zeros_like(finite)))
+    x = torch.stack(rows)                      # [6, 65280]; every row has a different amax, hence a different scale
+    q_ref, s_ref = f.ref_dynamic_per_token_quant(x)
+    q, s = ops.scaled_fp8_quant(x.to(device), use_per_token_if_dynamic=True)
+    assert np.array_equal(s.cpu().numpy(), s_ref.numpy())
+    assert np.array_equal(_codes(q), _codes(q_ref))
+
+
+# hidden sizes / token counts / dtypes of the reference's own test grid (tests/kernels/quantization/test_fp8_quant.py:15-21)
+@pytest.mark.parametrize("hidden", [17, 1024, 1025, 1026, 5137, 8193, 4096, 14336, 16384, 16392])
+@pytest.mark.parametrize("tokens", [1, 7, 257])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("use_ub", [False, True])
+def test_per_token_quant_bit_exact(device, hidden, tokens, dtype, use_ub):
+    import vllm_amd._custom_ops as ops
+    torch.manual_seed(0)
+    x = (torch.rand(tokens, hidden) + 1e-6).to(dtype)            # reference test input: rand + 1e-6, seed 0
+    x[::2] *= -1.7
+    ub = torch.tensor([x.float().abs().mean().item()], dtype=torch.float32) if use_ub else None
+    q_ref, s_ref = f.ref_dynamic_per_token_quant(x, ub)
+    q, s = ops.scaled_fp8_quant(x.to(device), scale_ub=None if ub is None else ub.to(device), use_per_token_if_dynamic=True)
+    assert q.dtype == torch.float8_e4m3fn and s.shape == (tokens, 1) and s.dtype == torch.float32
+    assert np.array_equal(s.cpu().numpy(), s_ref.numpy())
+    assert np.array_equal(_codes(q), _codes(q_ref))
+
+
+def test_per_token_quant_edge_rows_and_golden(device):
+    import vllm_amd._custom_ops as ops
+    gd = np.load(os.path.join(GOLDEN, "fp8_quant_small.npz"))
+    x = torch.from_numpy(gd["x_bits"]).view(torch.bfloat16)
+    q, s = ops.scaled_fp8_quant(x.to(device), use_per_token_if_dynamic=True)
+    assert np.array_equal(_codes(q), gd["codes"]) and np.array_equal(s.cpu().numpy(), gd["scales"])
+    assert s[4, 0].item() == float(np.float32(1.0) / (np.float32(448.0) * np.float32(512.0)))     # all-zero row
+    q, s = ops.scaled_fp8_quant(x.to(device), scale_ub=torch.from_numpy(gd["ub"]).to(device), use_per_token_if_dynamic=True)
+    assert np.array_equal(_codes(q), gd["codes_ub"]) and np.array_equal(s.cpu().numpy(), gd["scales_ub"])
+    q, s = ops.scaled_fp8_quant(x.to(device))
+    assert np.array_equal(_codes(q), gd["codes_tensor"]) and np.array_equal(s.cpu().numpy(), gd["scale_tensor"])
+
+
+def test_per_token_quant_strided_rows_and_padding(device):
+    import vllm_amd._custom_ops as ops
+    torch.manual_seed(1)
+    big = torch.randn(9, 3000).to(torch.bfloat16)
+    big_dev = big.to(device)
+    x = big[:, 8:8 + 2048]                                       # row stride 3000 elements, 16-byte aligned rows
+    for lo, hi in ((8, 8 + 2048), (3, 3 + 1000)):                # second slice: unaligned rows -> scalar path
+        q_ref, s_ref = f.ref_dynamic_per_token_quant(big[:, lo:hi])
+        view = big_dev[:, lo:hi]
+        assert view.stride() == (3000, 1)
+        q, s = ops.scaled_fp8_quant(view, use_per_token_if_dynamic=True)
+        assert np.array_equal(_codes(q), _codes(q_ref)) and np.array_equal(s.cpu().numpy(), s_ref.numpy())
+    # padded output: rows beyond the input are allocated but not written
+    q, s = ops.scaled_fp8_quant(x.contiguous().to(device), num_token_padding=17, use_per_token_if_dynamic=True)
+    assert q.shape == (17, 2048) and s.shape == (17, 1)
+    q_ref, s_ref = f.ref_dynamic_per_token_quant(x)
+    assert np.array_equal(_codes(q[:9]), _codes(q_ref)) and np.array_equal(s[:9].cpu().numpy(), s_ref.numpy())
+
+
+@pytest.mark.parametrize("hidden", [17, 1024, 5137, 14336])
+@pytest.mark.parametrize("tokens", [1, 7, 300])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_per_tensor_quant_bit_exact(device, hidden, tokens, dtype):
+    import vllm_amd._custom_ops as ops
+    torch.manual_seed(0)
+    x = (torch.rand(tokens, hidden) + 1e-6).to(dtype) * 3 - 1
+    q_ref, s_ref = f.ref_dynamic_per_tensor_quant(x)
+    q, s = ops.scaled_fp8_quant(x.to(device))
+    assert s.shape == (1, 1) and np.array_equal(s.cpu().numpy(), s_ref.numpy())
+    assert np.array_equal(_codes(q), _codes(q_ref))
+    # static quantisation with the scale just computed reproduces the same codes
+    q2, s2 = ops.scaled_fp8_quant(x.to(device), scale=s.reshape(1))
+    assert np.array_equal(_codes(q2), _codes(q_ref))
+
+
+def test_quant_large_row_count(device):
+    """Many rows (the reference's int64-indexing case, test_fp8_quant.py:99-120, scaled to stay quick)."""
+    import vllm_amd._custom_ops as ops
+    torch.manual_seed(2)
+    x = torch.randn(70000, 1152).to(torch.bfloat16)
+    q_ref, s_ref = f.ref_dynamic_per_token_quant(x)
+    q, s = ops.scaled_fp8_quant(x.to(device), use_per_token_if_dynamic=True)
+    assert np.array_equal(s.cpu().numpy(), s_ref.numpy()) and np.array_equal(_codes(q), _codes(q_ref))
+
+
+# ------------------------------------------------------------------------------------------------ scaled GEMM
+
+def _mm_case(m, k, n, seed, per_token=True, per_channel=True, bias=True, out_dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    a_q, sa = f.ref_dynamic_per_token_quant(a)
+    if not per_token:
+        a_q, sa = f.ref_dynamic_per_tensor_quant(a)
+        sa = sa.reshape(1)
+    w_q, sb = f.make_fp8_weight(n, k, seed=seed + 1)
+    if not per_channel:
+        w = (torch.randn(n, k, generator=g) * 0.02).to(torch.bfloat16)
+        w_q, sb = f.ref_dynamic_per_tensor_quant(w)
+        sb = sb.reshape(1)
+    b = (torch.randn(n, generator=g) * 0.01).to(out_dtype) if bias else None
+    return a_q, sa, w_q, sb, b
+
+
+def _check_mm(out, ref, what):
+    """Tolerance: the reference's own test uses rtol 0.5 / atol 0.15 (test_cutlass_scaled_mm.py:96); the products of
+    fp8 numbers are exact and accumulation is fp32, so this build holds one output rounding:
+    |out - ref| <= 2 ulp(out dtype) of max(|ref|, tiny) plus 1e-3 of the row-independent magnitude."""
+    o64, r64 = out.detach().cpu().double(), ref.double()
+    assert torch.isfinite(o64).all(), what
+    eps = 2.0 ** -7 if out.dtype == torch.bfloat16 else 2.0 ** -10
+    tol = 2 * eps * r64.abs() + 2e-3 * r64.abs().mean()
+    bad = (o64 - r64).abs() > tol
+    assert not bool(bad.any()), f"{what}: {int(bad.sum())} of {bad.numel()} outside tolerance, max err {(o64 - r64).abs().max():.4e}"
+
+
+MNK = [(1, 256, 128), (1, 16384, 1024), (1, 24576, 496), (16, 256, 496), (16, 16384, 128), (16, 24576, 4096),
+       (32, 8192, 4096), (32, 16384, 4096), (33, 1024, 1024), (33, 8192, 128), (64, 2048, 496), (64, 16384, 1024),
+       (100, 8192, 496), (128, 32768, 4096), (256, 4096, 4096), (512, 256, 1024), (512, 8192, 4096),
+       (512, 16384, 128), (512, 24576, 128)]   # (M, N, K) grid of the reference's test (test_cutlass_scaled_mm.py:18-38)
+
+
+@pytest.mark.parametrize("m,n,k", MNK)
+@pytest.mark.parametrize("per_token,per_channel", [(True, True), (False, False)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_scaled_mm_reference_grid(device, m, n, k, per_token, per_channel, bias):
+    import vllm_amd._custom_ops as ops
+    if n * k > 64 * 2 ** 20 and not (per_token and bias):
+        pytest.skip("largest shapes only in the headline configuration (keeps the CPU oracle time down)")
+    a_q, sa, w_q, sb, b = _mm_case(m, k, n, seed=m + n + k, per_token=per_token, per_channel=per_channel, bias=bias)
+    ref = f.scaled_mm_ref(a_q, w_q.t(), sa, sb, torch.bfloat16, b)
+    out = ops.cutlass_scaled_mm(a_q.to(device), w_q.to(device).t(), sa.to(device), sb.to(device), torch.bfloat16,
+                                None if b is None else b.to(device))
+    assert out.shape == (m, n) and out.dtype == torch.bfloat16
+    _check_mm(out, ref, f"scaled_mm m={m} n={n} k={k}")
+
+
+@pytest.mark.parametrize("m", [1, 16, 256])
+def test_scaled_mm_mixed_scales_fp16_and_padded_weight(device, m):
+    """per-token x per-tensor, per-tensor x per-channel, fp16 output, and a weight whose rows are padded by 256 bytes
+    (b.stride(1) = K + 256, as the reference pads FP8 weights on ROCm, fp8_utils.py:952-966)."""
+    import vllm_amd._custom_ops as ops
+    n, k = 512, 1024
+    a_q, sa, w_q, sb, b = _mm_case(m, k, n, seed=5, out_dtype=torch.float16)
+    for sa_, sb_ in ((sa, sb[:1].reshape(1)), (sa[:1].reshape(1), sb)):
+        ref = f.scaled_mm_ref(a_q, w_q.t(), sa_, sb_, torch.float16, b)
+        out = ops.cutlass_scaled_mm(a_q.to(device), w_q.to(device).t(), sa_.to(device), sb_.to(device), torch.float16, b.to(device))
+        _check_mm(out, ref, f"mixed scales m={m}")
+    padded = torch.zeros(n, k + 256, dtype=torch.uint8, device=device)
+    padded[:, :k] = w_q.view(torch.uint8).to(device)
+    w_view = padded.view(torch.float8_e4m3fn)[:, :k].t()
+    assert w_view.stride() == (1, k + 256)
+    ref = f.scaled_mm_ref(a_q, w_q.t(), sa, sb, torch.float16, b)
+    out = ops.cutlass_scaled_mm(a_q.to(device), w_view, sa.to(device), sb.to(device), torch.float16, b.to(device))
+    _check_mm(out, ref, f"padded weight m={m}")
+
+
+def test_scaled_mm_exact_small_integers(device):
+    """With scales 1 and small-integer operands every partial sum is an exactly representable integer, so any
+    dropped / duplicated k or transposed operand changes the result: the output must equal the integer GEMM."""
+    import vllm_amd._custom_ops as ops
+    g = torch.Generator().manual_seed(0)
+    for m, n, k in ((5, 64, 272), (40, 48, 1040), (300, 320, 144)):
+        a = torch.randint(-3, 4, (m, k), generator=g).float()
+        w = torch.randint(-2, 3, (n, k), generator=g).float()
+        one_m, one_n = torch.ones(m, 1), torch.ones(n, 1)
+        out = ops.cutlass_scaled_mm(a.to(torch.float8_e4m3fn).to(device), w.to(torch.float8_e4m3fn).to(device).t(),
+                                    one_m.to(device), one_n.to(device), torch.float16)
+        assert torch.equal(out.cpu().float(), a @ w.t()), (m, n, k)
+
+
+@pytest.mark.parametrize("k,n", LLAMA_SHAPES)
+def test_config4_llama_shapes(device, k, n):
+    """BASELINE config 4: M in {1, 16, 256, 4096}, per-token x per-channel (+bias); activations quantised on the GPU
+    (bit-exact with the oracle), M = 4096 checked on sampled rows."""
+    import vllm_amd._custom_ops as ops
+    w_q, sb = f.make_fp8_weight(n, k, seed=1)
+    w_dev = w_q.to(device).t()
+    g = torch.Generator().manual_seed(2)
+    bias = (torch.randn(n, generator=g) * 0.01).to(torch.bfloat16)
+    for m in (1, 16, 256, 4096):
+        a = torch.randn(m, k, generator=g).to(torch.bfloat16)
+        a_q, sa = ops.scaled_fp8_quant(a.to(device), use_per_token_if_dynamic=True)
+        rows = np.arange(m) if m <= 256 else np.concatenate([np.random.default_rng(m).choice(m, 30, replace=False), [0, m - 1]])
+        a_ref, sa_ref = f.ref_dynamic_per_token_quant(a[rows])
+        assert np.array_equal(_codes(a_q[rows]), _codes(a_ref)) and np.array_equal(sa[rows].cpu().numpy(), sa_ref.numpy())
+        out = ops.cutlass_scaled_mm(a_q, w_dev, sa, sb.to(device), torch.bfloat16, bias.to(device))
+        ref = f.scaled_mm_ref(a_ref, w_q.t(), sa_ref, sb, torch.bfloat16, bias)
+        _check_mm(out[rows], ref, f"config 4 k={k} n={n} m={m}")
+        assert torch.isfinite(out.float()).all()

@@ -39,53 +39,35 @@ struct DecodeParams {
   int M, N, K, G, NT, SK, WK;
 };
 
-// Workgroups are at most 8 wavefronts, i.e. two per SIMD, which leaves 256 registers per lane.
-template <bool BF16, int TG, int MB, bool HAS_ZP>
-__global__ __launch_bounds__(512) void w4a16_decode_kernel(const DecodeParams p) {
+// Split-K partial tiles cross workgroups (and therefore XCDs, whose L2 caches are not coherent with each other)
+// through device-scope write-through stores and loads: no L2 write-back / invalidate is needed, only a wait for the
+// stores to be acknowledged before the arrival counter is bumped.
+__device__ inline void store_partial(float* dst, v4f v) {
+  __hip_atomic_store(dst + 0, v.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(dst + 1, v.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(dst + 2, v.z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(dst + 3, v.w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ inline v4f load_partial(const float* src) {
+  v4f v;
+  v.x = __hip_atomic_load(src + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  v.y = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  v.z = __hip_atomic_load(src + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  v.w = __hip_atomic_load(src + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return v;
+}
+
+// MAXW = upper bound on wavefronts per workgroup (8 leaves 256 registers per lane, 16 leaves 128).
+template <bool BF16, int TG, int MB, bool HAS_ZP, int MAXW>
+__global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodeParams p) {
   using T = F16Traits<BF16>;
   extern __shared__ v4f red[];   // [2][WK][MB][64]
 
-  const int lane = threadIdx.x, w = threadIdx.y;
+  const int lane = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(threadIdx.y);   // wave-uniform: keeps tile addresses in scalar registers
   const int o = lane >> 4, r16 = lane & 15;
   const int sk = blockIdx.y;
   const int g0 = (sk * p.WK + w) * TG;
-
-  // ---- activations of this wave's K slab, as MFMA B operands (column = m, 8 consecutive k per lane) ----
-  v4u breg[TG][4][MB];
-  float S[TG][MB];
-#pragma unroll
-  for (int t = 0; t < TG; ++t) {
-    const int g = g0 + t;
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      const int m = mb * 16 + r16;
-      const bool ok = (g < p.G) && (m < p.M);
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const int k = g * 128 + jj * 32 + o * 8;
-        v4u v = {0u, 0u, 0u, 0u};
-        if (ok) {
-          const uint16_t* row = p.a + (int64_t)m * p.lda;
-          if (p.perm) {
-            const v4i p0 = *reinterpret_cast<const v4i*>(p.perm + k);
-            const v4i p1 = *reinterpret_cast<const v4i*>(p.perm + k + 4);
-            v.x = (uint32_t)row[p0.x] | ((uint32_t)row[p0.y] << 16);
-            v.y = (uint32_t)row[p0.z] | ((uint32_t)row[p0.w] << 16);
-            v.z = (uint32_t)row[p1.x] | ((uint32_t)row[p1.y] << 16);
-            v.w = (uint32_t)row[p1.z] | ((uint32_t)row[p1.w] << 16);
-          } else {
-            v = *reinterpret_cast<const v4u*>(row + k);
-          }
-        }
-        breg[t][jj][mb] = v;
-      }
-      const v4u ones = {T::ONE2, T::ONE2, T::ONE2, T::ONE2};
-      v4f s4 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) s4 = T::mfma16(ones, breg[t][jj][mb], s4);
-      S[t][mb] = s4.x;
-    }
-  }
 
   // ---- contiguous range of n-tiles for this workgroup ----
   const int nt0 = (int)(((int64_t)p.NT * blockIdx.x) / gridDim.x);
@@ -96,20 +78,84 @@ __global__ __launch_bounds__(512) void w4a16_decode_kernel(const DecodeParams p)
   uint32_t zq[TG];
   // Slot t is refilled for the next n-tile as soon as it has been consumed, so TG tile loads stay in flight per
   // wavefront with a single set of registers.
+  // Groups past the end of K (ragged last wavefront) are clamped for addressing; their activations are zero, so they
+  // contribute nothing.  No branches: every load of a wavefront is issued back to back.
   auto issue_load = [&](int nt, int t) {
-    const int g = g0 + t;
-    if (g < p.G) {
-      wq[t] = __builtin_nontemporal_load(&p.b[((int64_t)g * p.NT + nt) * 64 + lane]);
-      sc[t] = *reinterpret_cast<const v2u*>(p.scales + (int64_t)g * p.N + nt * 16 + o * 4);
-      if constexpr (HAS_ZP) zq[t] = p.zeros[(int64_t)g * (p.N >> 3) + nt * 2 + (o >> 1)];
-    }
+    const int g = min(g0 + t, p.G - 1);
+    const v4u* tile = p.b + ((size_t)g * p.NT + nt) * 64;                 // scalar
+    wq[t] = __builtin_nontemporal_load(tile + lane);
+    const uint16_t* srow = p.scales + (size_t)g * p.N + nt * 16;          // scalar
+    sc[t] = *reinterpret_cast<const v2u*>(srow + o * 4);
+    if constexpr (HAS_ZP) zq[t] = (p.zeros + (size_t)g * (p.N >> 3) + nt * 2)[o >> 1];
   };
+  // The first weight tiles are requested before anything else so that their latency overlaps the activation loads.
 #pragma unroll
   for (int t = 0; t < TG; ++t) {
     wq[t] = v4u{0u, 0u, 0u, 0u};
     sc[t] = v2u{0u, 0u};
     zq[t] = 0u;
     if (nt0 < nt1) issue_load(nt0, t);
+  }
+
+  // ---- activations of this wave's K slab, as MFMA B operands (column = m, 8 consecutive k per lane) ----
+  // Loaded unconditionally from clamped addresses and zeroed afterwards, so that all loads are in flight together.
+  v4u breg[TG][4][MB];
+  float S[TG][MB];
+  if (p.perm == nullptr) {
+#pragma unroll
+    for (int t = 0; t < TG; ++t) {
+      const int g = min(g0 + t, p.G - 1);
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const int m = min(mb * 16 + r16, p.M - 1);
+        const uint16_t* row = p.a + (int64_t)m * p.lda + g * 128 + o * 8;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) breg[t][jj][mb] = *reinterpret_cast<const v4u*>(row + jj * 32);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int t = 0; t < TG; ++t) {
+      const int g = min(g0 + t, p.G - 1);
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const int m = min(mb * 16 + r16, p.M - 1);
+        const uint16_t* row = p.a + (int64_t)m * p.lda;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          const int k = g * 128 + jj * 32 + o * 8;
+          const v4i p0 = *reinterpret_cast<const v4i*>(p.perm + k);
+          const v4i p1 = *reinterpret_cast<const v4i*>(p.perm + k + 4);
+          v4u v;
+          v.x = (uint32_t)row[p0.x] | ((uint32_t)row[p0.y] << 16);
+          v.y = (uint32_t)row[p0.z] | ((uint32_t)row[p0.w] << 16);
+          v.z = (uint32_t)row[p1.x] | ((uint32_t)row[p1.y] << 16);
+          v.w = (uint32_t)row[p1.z] | ((uint32_t)row[p1.w] << 16);
+          breg[t][jj][mb] = v;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < TG; ++t) {
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const bool ok = (g0 + t < p.G) && (mb * 16 + r16 < p.M);
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj)
+        if (!ok) breg[t][jj][mb] = v4u{0u, 0u, 0u, 0u};
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < TG; ++t) {
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const v4u ones = {T::ONE2, T::ONE2, T::ONE2, T::ONE2};
+      v4f s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) s4 = T::mfma16(ones, breg[t][jj][mb], s4);
+      S[t][mb] = s4.x;
+    }
   }
 
   int parity = 0;
@@ -182,21 +228,18 @@ __global__ __launch_bounds__(512) void w4a16_decode_kernel(const DecodeParams p)
         v4f val = (p.WK > 1) ? tot : acc[mb];
         bool write_out = true;
         if (p.SK > 1) {
-          const int64_t slot = ((int64_t)nt * MB + mb) * 64 + lane;
-          const int64_t sk_stride = (int64_t)p.NT * MB * 64;
-          p.c_tmp[sk * sk_stride + slot] = val;
-          __threadfence();
+          const int64_t slot = (((int64_t)nt * MB + mb) * 64 + lane) * 4;
+          const int64_t sk_stride = (int64_t)p.NT * MB * 64 * 4;
+          float* part = reinterpret_cast<float*>(p.c_tmp);
+          store_partial(part + sk * sk_stride + slot, val);
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // partial tile acknowledged before the counter moves
           int old = 0;
           if (lane == 0) old = __hip_atomic_fetch_add(&p.counters[nt * MB + mb], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           old = __shfl(old, 0);
           write_out = (old == p.SK - 1);
           if (write_out) {
-            __threadfence();
             val = v4f{0.f, 0.f, 0.f, 0.f};
-            for (int s2 = 0; s2 < p.SK; ++s2) {
-              const v4f v = __builtin_nontemporal_load(&p.c_tmp[s2 * sk_stride + slot]);
-              val += v;
-            }
+            for (int s2 = 0; s2 < p.SK; ++s2) val += load_partial(part + s2 * sk_stride + slot);   // fixed order
             if (lane == 0) __hip_atomic_store(&p.counters[nt * MB + mb], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
         }
@@ -223,25 +266,31 @@ __global__ __launch_bounds__(512) void w4a16_decode_kernel(const DecodeParams p)
 // ----------------------------------------------------------------------------- host side
 
 struct DecodeConfig {
-  int tg, wk, sk, gx;
+  int tg, wk, sk, gx, maxw;
 };
 
 static int g_force_tg = 0, g_force_wk = 0, g_force_gx = 0;
 
+// Launch shapes that are instantiated: (TG, MAXW) in {(1,16), (2,16), (4,8), (4,16), (7,8)} for one m-block and
+// {(1,16), (2,16), (2,8)... } for two.  `wk` wavefronts of a workgroup x `sk` workgroups cover the K/128 groups.
 static DecodeConfig pick_decode_config(int M, int N, int K) {
   const int G = K / 128, NT = N / 16;
   const int MB = M <= 16 ? 1 : 2;
   DecodeConfig c;
   if (g_force_tg > 0) c.tg = g_force_tg;
   else if (MB == 2) c.tg = G >= 2 ? 2 : 1;
+  else if (G % 7 == 0 && G >= 56) c.tg = 7;
   else if (G >= 8) c.tg = 4;
   else if (G >= 2) c.tg = 2;
   else c.tg = 1;
   const int kw = (G + c.tg - 1) / c.tg;          // wavefronts needed along K
-  int wk_max = 8;
-  if (g_force_wk > 0 && g_force_wk < wk_max) wk_max = g_force_wk;
+  int wk_max = (c.tg == 7) ? 8 : ((MB == 1 && c.tg == 4) ? 8 : 16);
+  if (g_force_wk > 0) wk_max = g_force_wk;
+  if (c.tg == 7 && wk_max > 8) wk_max = 8;
+  if (wk_max > 16) wk_max = 16;
   c.sk = (kw + wk_max - 1) / wk_max;
   c.wk = (kw + c.sk - 1) / c.sk;
+  c.maxw = c.wk > 8 ? 16 : 8;
   const int cus = num_cus_current_device();
   int gx = g_force_gx > 0 ? g_force_gx : (2 * cus) / c.sk;
   if (gx < 1) gx = 1;
@@ -250,23 +299,38 @@ static DecodeConfig pick_decode_config(int M, int N, int K) {
   return c;
 }
 
-template <bool BF16, int TG, int MB, bool HAS_ZP>
+template <bool BF16, int TG, int MB, bool HAS_ZP, int MAXW>
 static void launch_decode(const DecodeParams& p, int gx, hipStream_t s) {
   const size_t lds = p.WK > 1 ? (size_t)2 * p.WK * MB * 64 * sizeof(v4f) : 0;
-  hipLaunchKernelGGL((w4a16_decode_kernel<BF16, TG, MB, HAS_ZP>), dim3(gx, p.SK), dim3(64, p.WK), lds, s, p);
+  hipLaunchKernelGGL((w4a16_decode_kernel<BF16, TG, MB, HAS_ZP, MAXW>), dim3(gx, p.SK), dim3(64, p.WK), lds, s, p);
 }
 
 template <bool BF16, int MB, bool HAS_ZP>
-static int dispatch_tg(const DecodeParams& p, int tg, int gx, hipStream_t s) {
-  switch (tg) {
-    case 1: launch_decode<BF16, 1, MB, HAS_ZP>(p, gx, s); return VAQ_OK;
-    case 2: launch_decode<BF16, 2, MB, HAS_ZP>(p, gx, s); return VAQ_OK;
-    case 4:
-      if constexpr (MB == 1) { launch_decode<BF16, 4, MB, HAS_ZP>(p, gx, s); return VAQ_OK; }
-      break;
-    default: break;
+static int dispatch_tg(const DecodeParams& p, const DecodeConfig& c, hipStream_t s) {
+  const int gx = c.gx;
+  if (c.maxw == 16) {
+    switch (c.tg) {
+      case 1: launch_decode<BF16, 1, MB, HAS_ZP, 16>(p, gx, s); return VAQ_OK;
+      case 2: launch_decode<BF16, 2, MB, HAS_ZP, 16>(p, gx, s); return VAQ_OK;
+      case 4:
+        if constexpr (MB == 1) { launch_decode<BF16, 4, MB, HAS_ZP, 16>(p, gx, s); return VAQ_OK; }
+        break;
+      default: break;
+    }
+  } else {
+    switch (c.tg) {
+      case 1: launch_decode<BF16, 1, MB, HAS_ZP, 8>(p, gx, s); return VAQ_OK;
+      case 2: launch_decode<BF16, 2, MB, HAS_ZP, 8>(p, gx, s); return VAQ_OK;
+      case 4:
+        if constexpr (MB == 1) { launch_decode<BF16, 4, MB, HAS_ZP, 8>(p, gx, s); return VAQ_OK; }
+        break;
+      case 7:
+        if constexpr (MB == 1) { launch_decode<BF16, 7, MB, HAS_ZP, 8>(p, gx, s); return VAQ_OK; }
+        break;
+      default: break;
+    }
   }
-  set_error("w4a16_gemm(decode): unsupported TG=%d for MB=%d", tg, MB);
+  set_error("w4a16_gemm(decode): unsupported launch shape TG=%d MAXW=%d for MB=%d", c.tg, c.maxw, MB);
   return VAQ_ERR_UNSUPPORTED;
 }
 
@@ -310,11 +374,11 @@ int w4a16_decode_launch(const void* a, int64_t lda, const int32_t* b, const void
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
   if (MB == 1) {
-    if (bf16) rc = zp ? dispatch_tg<true, 1, true>(p, cfg.tg, cfg.gx, s) : dispatch_tg<true, 1, false>(p, cfg.tg, cfg.gx, s);
-    else rc = zp ? dispatch_tg<false, 1, true>(p, cfg.tg, cfg.gx, s) : dispatch_tg<false, 1, false>(p, cfg.tg, cfg.gx, s);
+    if (bf16) rc = zp ? dispatch_tg<true, 1, true>(p, cfg, s) : dispatch_tg<true, 1, false>(p, cfg, s);
+    else rc = zp ? dispatch_tg<false, 1, true>(p, cfg, s) : dispatch_tg<false, 1, false>(p, cfg, s);
   } else {
-    if (bf16) rc = zp ? dispatch_tg<true, 2, true>(p, cfg.tg, cfg.gx, s) : dispatch_tg<true, 2, false>(p, cfg.tg, cfg.gx, s);
-    else rc = zp ? dispatch_tg<false, 2, true>(p, cfg.tg, cfg.gx, s) : dispatch_tg<false, 2, false>(p, cfg.tg, cfg.gx, s);
+    if (bf16) rc = zp ? dispatch_tg<true, 2, true>(p, cfg, s) : dispatch_tg<true, 2, false>(p, cfg, s);
+    else rc = zp ? dispatch_tg<false, 2, true>(p, cfg, s) : dispatch_tg<false, 2, false>(p, cfg, s);
   }
   if (rc != VAQ_OK) return rc;
   VAQ_CHECK_LAUNCH("w4a16_gemm(decode)");
