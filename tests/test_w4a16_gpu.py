@@ -123,7 +123,11 @@ def test_zero_point_eight_equals_symmetric(device):
     case_asym = dict(case, zp_vals=np.full((k // 128, n), 8, dtype=np.int32))
     asym = W4A16Layer(case_asym, device)
     a = _acts(m, k, device)
-    assert torch.equal(sym(a), asym(a))
+    # the two kernels order their fp32 operations differently (the symmetric one folds the zero point into the MFMA
+    # chain), so the results agree to an output ulp, not necessarily bit for bit
+    o_sym, o_asym = sym(a).float(), asym(a).float()
+    assert (o_sym - o_asym).abs().max() <= 2.0 ** -7 * o_sym.abs().max()
+    check_gemm_close(asym(a), o.gemm_ref(a.cpu(), o.case_w_ref(case)), "uint4 with zero point 8")
 
 
 def test_strided_activations(device):

@@ -57,14 +57,39 @@ __device__ inline v4f load_partial(const float* src) {
   return v;
 }
 
+// (x & mask) | ex in one VALU op (mask from a scalar register, ex from a vector register: a VOP3 instruction of this
+// architecture cannot carry two literals, and the compiler otherwise emits two instructions).
+__device__ inline uint32_t and_or(uint32_t x, uint32_t mask, uint32_t ex) {
+  uint32_t d;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(x), "s"(mask), "v"(ex));
+  return d;
+}
+
+template <bool BF16>
+__device__ inline v4u dequant_biased_fast(uint32_t w, uint32_t ex) {
+  constexpr uint32_t M = 0x000f000fu;
+  v4u r;
+  r.x = and_or(w, M, ex);
+  r.y = and_or(w >> 4, M, ex);
+  r.z = and_or(w >> 8, M, ex);
+  r.w = and_or(w >> 12, M, ex);
+  return r;
+}
+
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint64_t bytes) {
+  const uint32_t n = bytes > 0xffffffffull ? 0xffffffffu : (uint32_t)bytes;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)n, 0x00020000);
+}
+
 // MAXW = upper bound on wavefronts per workgroup (8 leaves 256 registers per lane, 16 leaves 128).
-template <bool BF16, int TG, int MB, bool HAS_ZP, int MAXW>
+// D    = n-tiles kept in flight per wavefront (prefetch depth of the register ring).
+template <bool BF16, int TG, int MB, bool HAS_ZP, int MAXW, int D>
 __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodeParams p) {
   using T = F16Traits<BF16>;
   extern __shared__ v4f red[];   // [2][WK][MB][64]
 
   const int lane = threadIdx.x;
-  const int w = __builtin_amdgcn_readfirstlane(threadIdx.y);   // wave-uniform: keeps tile addresses in scalar registers
+  const int w = __builtin_amdgcn_readfirstlane(threadIdx.y);   // wave-uniform: tile offsets stay in scalar registers
   const int o = lane >> 4, r16 = lane & 15;
   const int sk = blockIdx.y;
   const int g0 = (sk * p.WK + w) * TG;
@@ -73,34 +98,43 @@ __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodePar
   const int nt0 = (int)(((int64_t)p.NT * blockIdx.x) / gridDim.x);
   const int nt1 = (int)(((int64_t)p.NT * (blockIdx.x + 1)) / gridDim.x);
 
-  v4u wq[TG];
-  v2u sc[TG];
-  uint32_t zq[TG];
-  // Slot t is refilled for the next n-tile as soon as it has been consumed, so TG tile loads stay in flight per
-  // wavefront with a single set of registers.
+  // Weights, scales and zero points are read through buffer descriptors: the per-tile part of the address is a
+  // scalar offset, the per-lane part a constant, so a load costs no vector ALU work.
+  const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b, (uint64_t)p.K * p.N / 2);
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(p.scales, (uint64_t)p.G * p.N * 2);
+  const __amdgpu_buffer_rsrc_t rz = make_rsrc(HAS_ZP ? (const void*)p.zeros : (const void*)p.scales, (uint64_t)p.G * (p.N / 8) * 4);
+  const int vo_b = lane * 16, vo_s = o * 8, vo_z = (o >> 1) * 4;
+
+  v4u wq[D][TG];
+  v2u sc[D][TG];
+  uint32_t zq[D][TG];
   // Groups past the end of K (ragged last wavefront) are clamped for addressing; their activations are zero, so they
-  // contribute nothing.  No branches: every load of a wavefront is issued back to back.
-  auto issue_load = [&](int nt, int t) {
-    const int g = min(g0 + t, p.G - 1);
-    const v4u* tile = p.b + ((size_t)g * p.NT + nt) * 64;                 // scalar
-    wq[t] = __builtin_nontemporal_load(tile + lane);
-    const uint16_t* srow = p.scales + (size_t)g * p.N + nt * 16;          // scalar
-    sc[t] = *reinterpret_cast<const v2u*>(srow + o * 4);
-    if constexpr (HAS_ZP) zq[t] = (p.zeros + (size_t)g * (p.N >> 3) + nt * 2)[o >> 1];
+  // contribute nothing.
+  auto issue_load = [&](int u, int nt, int t) {
+    const uint32_t g = (uint32_t)min(g0 + t, p.G - 1);
+    wq[u][t] = __builtin_amdgcn_raw_buffer_load_b128(rb, vo_b, (int)((g * (uint32_t)p.NT + (uint32_t)nt) * 1024u), 2);
+    sc[u][t] = __builtin_amdgcn_raw_buffer_load_b64(rs, vo_s, (int)((g * (uint32_t)p.N + (uint32_t)nt * 16u) * 2u), 0);
+    if constexpr (HAS_ZP)
+      zq[u][t] = __builtin_amdgcn_raw_buffer_load_b32(rz, vo_z, (int)((g * (uint32_t)(p.N >> 3) + (uint32_t)nt * 2u) * 4u), 0);
   };
   // The first weight tiles are requested before anything else so that their latency overlaps the activation loads.
 #pragma unroll
-  for (int t = 0; t < TG; ++t) {
-    wq[t] = v4u{0u, 0u, 0u, 0u};
-    sc[t] = v2u{0u, 0u};
-    zq[t] = 0u;
-    if (nt0 < nt1) issue_load(nt0, t);
+  for (int u = 0; u < D; ++u) {
+#pragma unroll
+    for (int t = 0; t < TG; ++t) {
+      wq[u][t] = v4u{0u, 0u, 0u, 0u};
+      sc[u][t] = v2u{0u, 0u};
+      zq[u][t] = 0u;
+    }
+    if (nt0 + u < nt1) {
+#pragma unroll
+      for (int t = 0; t < TG; ++t) issue_load(u, nt0 + u, t);
+    }
   }
 
   // ---- activations of this wave's K slab, as MFMA B operands (column = m, 8 consecutive k per lane) ----
   // Loaded unconditionally from clamped addresses and zeroed afterwards, so that all loads are in flight together.
   v4u breg[TG][4][MB];
-  float S[TG][MB];
   if (p.perm == nullptr) {
 #pragma unroll
     for (int t = 0; t < TG; ++t) {
@@ -136,6 +170,9 @@ __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodePar
       }
     }
   }
+  // S[t][mb] = sum of the group's activations per column m (identical in the 4 accumulator registers).  For the
+  // symmetric type the whole correction -(BIAS + 8) * S is the starting value of the group's MFMA chain.
+  v4f Sv[TG][MB];
 #pragma unroll
   for (int t = 0; t < TG; ++t) {
 #pragma unroll
@@ -144,119 +181,127 @@ __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodePar
 #pragma unroll
       for (int jj = 0; jj < 4; ++jj)
         if (!ok) breg[t][jj][mb] = v4u{0u, 0u, 0u, 0u};
-    }
-  }
-#pragma unroll
-  for (int t = 0; t < TG; ++t) {
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
       const v4u ones = {T::ONE2, T::ONE2, T::ONE2, T::ONE2};
       v4f s4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int jj = 0; jj < 4; ++jj) s4 = T::mfma16(ones, breg[t][jj][mb], s4);
-      S[t][mb] = s4.x;
+      if constexpr (!HAS_ZP) s4 *= -(T::CODE_BIAS + 8.0f);
+      Sv[t][mb] = s4;
     }
   }
 
+  const uint32_t ex = T::EX;
   int parity = 0;
-  for (int nt = nt0; nt < nt1; ++nt) {
-    v4f acc[MB];
+  for (int base = nt0; base < nt1; base += D) {
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) acc[mb] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int u = 0; u < D; ++u) {
+      const int nt = base + u;
+      if (nt >= nt1) break;
+
+      v4f acc[MB];
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) acc[mb] = v4f{0.f, 0.f, 0.f, 0.f};
 
 #pragma unroll
-    for (int t = 0; t < TG; ++t) {
-      v4f P[MB];
+      for (int t = 0; t < TG; ++t) {
+        const uint32_t wj[4] = {wq[u][t].x, wq[u][t].y, wq[u][t].z, wq[u][t].w};
+        const v2u sct = sc[u][t];
+        const uint32_t zqt = zq[u][t];
+        if (nt + D < nt1) issue_load(u, nt + D, t);      // refill this ring slot D n-tiles ahead
+        v4f P[MB];
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) P[mb] = v4f{0.f, 0.f, 0.f, 0.f};
-      const uint32_t wj[4] = {wq[t].x, wq[t].y, wq[t].z, wq[t].w};
-      const v2u sct = sc[t];
-      const uint32_t zqt = zq[t];
-      if (nt + 1 < nt1) issue_load(nt + 1, t);
+        for (int mb = 0; mb < MB; ++mb) P[mb] = HAS_ZP ? v4f{0.f, 0.f, 0.f, 0.f} : Sv[t][mb];
 #pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const v4u aop = dequant_biased<BF16>(wj[jj]);
+        for (int jj = 0; jj < 4; ++jj) {
+          const v4u aop = dequant_biased_fast<BF16>(wj[jj], ex);
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) P[mb] = T::mfma16(aop, breg[t][jj][mb], P[mb]);
-      }
-      // group epilogue: acc += s * (P - (BIAS + z) * S)
-      float s[4], zc[4];
-      s[0] = T::to_float((uint16_t)(sct.x & 0xffffu));
-      s[1] = T::to_float((uint16_t)(sct.x >> 16));
-      s[2] = T::to_float((uint16_t)(sct.y & 0xffffu));
-      s[3] = T::to_float((uint16_t)(sct.y >> 16));
-      if constexpr (HAS_ZP) {
-        const uint32_t z4 = zqt >> ((o & 1) * 16);
+          for (int mb = 0; mb < MB; ++mb) P[mb] = T::mfma16(aop, breg[t][jj][mb], P[mb]);
+        }
+        // group epilogue: acc += s * (P - (BIAS + z) * S)   (the subtraction is already inside P when symmetric)
+        float s[4];
+        if constexpr (BF16) {
+          s[0] = __uint_as_float(sct.x << 16);
+          s[1] = __uint_as_float(sct.x & 0xffff0000u);
+          s[2] = __uint_as_float(sct.y << 16);
+          s[3] = __uint_as_float(sct.y & 0xffff0000u);
+        } else {
+          s[0] = T::to_float((uint16_t)(sct.x & 0xffffu));
+          s[1] = T::to_float((uint16_t)(sct.x >> 16));
+          s[2] = T::to_float((uint16_t)(sct.y & 0xffffu));
+          s[3] = T::to_float((uint16_t)(sct.y >> 16));
+        }
+        if constexpr (HAS_ZP) {
+          const uint32_t z4 = zqt >> ((o & 1) * 16);
+          float zc[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) zc[r] = T::CODE_BIAS + (float)((z4 >> (4 * r)) & 0xFu);
-      } else {
+          for (int r = 0; r < 4; ++r) zc[r] = T::CODE_BIAS + (float)((z4 >> (4 * r)) & 0xFu);
 #pragma unroll
-        for (int r = 0; r < 4; ++r) zc[r] = T::CODE_BIAS + 8.0f;
-      }
+          for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        const float Sg = S[t][mb];
+            for (int r = 0; r < 4; ++r) acc[mb][r] = fmaf(s[r], fmaf(-zc[r], Sv[t][mb][r], P[mb][r]), acc[mb][r]);
+        } else {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[mb][r] = fmaf(s[r], fmaf(-zc[r], Sg, P[mb][r]), acc[mb][r]);
-      }
-    }
-
-    // ---- reduce the WK partial tiles of this workgroup through LDS ----
-    v4f tot = v4f{0.f, 0.f, 0.f, 0.f};
-    bool reducer = w < MB;
-    if (p.WK > 1) {
-      v4f* buf = red + (size_t)parity * p.WK * MB * 64;
+          for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) buf[(w * MB + mb) * 64 + lane] = acc[mb];
-      __syncthreads();
-      if (reducer) {
-        for (int ww = 0; ww < p.WK; ++ww) {
-          const v4f v = buf[(ww * MB + w) * 64 + lane];
-          tot += v;
+            for (int r = 0; r < 4; ++r) acc[mb][r] = fmaf(s[r], P[mb][r], acc[mb][r]);
         }
       }
-      parity ^= 1;
-    } else {
-      // single wave per workgroup: it owns every m-block itself
-      reducer = true;
-    }
 
-    if (reducer) {
-      const int mb_lo = (p.WK > 1) ? w : 0;
-      const int mb_hi = (p.WK > 1) ? w + 1 : MB;
-      for (int mb = mb_lo; mb < mb_hi; ++mb) {
-        v4f val = (p.WK > 1) ? tot : acc[mb];
-        bool write_out = true;
-        if (p.SK > 1) {
-          const int64_t slot = (((int64_t)nt * MB + mb) * 64 + lane) * 4;
-          const int64_t sk_stride = (int64_t)p.NT * MB * 64 * 4;
-          float* part = reinterpret_cast<float*>(p.c_tmp);
-          store_partial(part + sk * sk_stride + slot, val);
-          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // partial tile acknowledged before the counter moves
-          int old = 0;
-          if (lane == 0) old = __hip_atomic_fetch_add(&p.counters[nt * MB + mb], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          old = __shfl(old, 0);
-          write_out = (old == p.SK - 1);
-          if (write_out) {
-            val = v4f{0.f, 0.f, 0.f, 0.f};
-            for (int s2 = 0; s2 < p.SK; ++s2) val += load_partial(part + s2 * sk_stride + slot);   // fixed order
-            if (lane == 0) __hip_atomic_store(&p.counters[nt * MB + mb], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          }
+      // ---- reduce the WK partial tiles of this workgroup through LDS; the reducing wavefront rotates ----
+      const int it = nt - nt0;
+      int my_mb = -1;
+      v4f tot = v4f{0.f, 0.f, 0.f, 0.f};
+      if (p.WK > 1) {
+        v4f* buf = red + (size_t)parity * p.WK * MB * 64;
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) buf[(w * MB + mb) * 64 + lane] = acc[mb];
+        __syncthreads();
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          if ((it * MB + mb) % p.WK == w) my_mb = mb;
+        if (my_mb >= 0) {
+          for (int ww = 0; ww < p.WK; ++ww) tot += buf[(ww * MB + my_mb) * 64 + lane];
         }
-        const int m = mb * 16 + r16;
-        if (write_out && m < p.M) {
-          const int n = nt * 16 + o * 4;
-          if (p.bias) {
-            const v2u bb = *reinterpret_cast<const v2u*>(p.bias + n);
-            val[0] += T::to_float((uint16_t)(bb.x & 0xffffu));
-            val[1] += T::to_float((uint16_t)(bb.x >> 16));
-            val[2] += T::to_float((uint16_t)(bb.y & 0xffffu));
-            val[3] += T::to_float((uint16_t)(bb.y >> 16));
+        parity ^= 1;
+      }
+
+      const int mb_lo = (p.WK > 1) ? my_mb : 0;
+      const int mb_hi = (p.WK > 1) ? my_mb + 1 : MB;
+      if (p.WK == 1 || my_mb >= 0) {
+        for (int mb = mb_lo; mb < mb_hi; ++mb) {
+          v4f val = (p.WK > 1) ? tot : acc[mb];
+          bool write_out = true;
+          if (p.SK > 1) {
+            const int64_t slot = (((int64_t)nt * MB + mb) * 64 + lane) * 4;
+            const int64_t sk_stride = (int64_t)p.NT * MB * 64 * 4;
+            float* part = reinterpret_cast<float*>(p.c_tmp);
+            store_partial(part + sk * sk_stride + slot, val);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // partial tile acknowledged before the counter moves
+            int old = 0;
+            if (lane == 0) old = __hip_atomic_fetch_add(&p.counters[nt * MB + mb], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            old = __shfl(old, 0);
+            write_out = (old == p.SK - 1);
+            if (write_out) {
+              val = v4f{0.f, 0.f, 0.f, 0.f};
+              for (int s2 = 0; s2 < p.SK; ++s2) val += load_partial(part + s2 * sk_stride + slot);   // fixed order
+              if (lane == 0) __hip_atomic_store(&p.counters[nt * MB + mb], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
           }
-          v2u outv;
-          outv.x = (uint32_t)T::from_float(val[0]) | ((uint32_t)T::from_float(val[1]) << 16);
-          outv.y = (uint32_t)T::from_float(val[2]) | ((uint32_t)T::from_float(val[3]) << 16);
-          *reinterpret_cast<v2u*>(p.c + (int64_t)m * p.N + n) = outv;
+          const int m = mb * 16 + r16;
+          if (write_out && m < p.M) {
+            const int n = nt * 16 + o * 4;
+            if (p.bias) {
+              const v2u bb = *reinterpret_cast<const v2u*>(p.bias + n);
+              val[0] += T::to_float((uint16_t)(bb.x & 0xffffu));
+              val[1] += T::to_float((uint16_t)(bb.x >> 16));
+              val[2] += T::to_float((uint16_t)(bb.y & 0xffffu));
+              val[3] += T::to_float((uint16_t)(bb.y >> 16));
+            }
+            v2u outv;
+            outv.x = (uint32_t)T::from_float(val[0]) | ((uint32_t)T::from_float(val[1]) << 16);
+            outv.y = (uint32_t)T::from_float(val[2]) | ((uint32_t)T::from_float(val[3]) << 16);
+            *reinterpret_cast<v2u*>(p.c + (int64_t)m * p.N + n) = outv;
+          }
         }
       }
     }
@@ -266,69 +311,70 @@ __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodePar
 // ----------------------------------------------------------------------------- host side
 
 struct DecodeConfig {
-  int tg, wk, sk, gx, maxw;
+  int tg, wk, sk, gx, maxw, d;
 };
 
-static int g_force_tg = 0, g_force_wk = 0, g_force_gx = 0;
+static int g_force_tg = 0, g_force_wk = 0, g_force_gx = 0, g_force_d = 0;
 
-// Launch shapes that are instantiated: (TG, MAXW) in {(1,16), (2,16), (4,8), (4,16), (7,8)} for one m-block and
-// {(1,16), (2,16), (2,8)... } for two.  `wk` wavefronts of a workgroup x `sk` workgroups cover the K/128 groups.
+// `wk` wavefronts of a workgroup x `sk` workgroups cover the K/128 groups, TG groups per wavefront.
 static DecodeConfig pick_decode_config(int M, int N, int K) {
   const int G = K / 128, NT = N / 16;
   const int MB = M <= 16 ? 1 : 2;
   DecodeConfig c;
   if (g_force_tg > 0) c.tg = g_force_tg;
-  else if (MB == 2) c.tg = G >= 2 ? 2 : 1;
-  else if (G % 7 == 0 && G >= 56) c.tg = 7;
-  else if (G >= 8) c.tg = 4;
-  else if (G >= 2) c.tg = 2;
-  else c.tg = 1;
+  else if (MB == 2) c.tg = 1;
+  else if (G % 7 == 0 && G >= 56) c.tg = 7;      // K = 14336: 7 groups per wavefront, 8 wavefronts, 2 workgroups
+  else c.tg = G >= 2 ? 2 : 1;
+  if (c.tg != 1 && c.tg != 2 && c.tg != 4 && c.tg != 7) c.tg = 2;
+  if (MB == 2 && c.tg >= 4) c.tg = 2;
   const int kw = (G + c.tg - 1) / c.tg;          // wavefronts needed along K
-  int wk_max = (c.tg == 7) ? 8 : ((MB == 1 && c.tg == 4) ? 8 : 16);
-  if (g_force_wk > 0) wk_max = g_force_wk;
-  if (c.tg == 7 && wk_max > 8) wk_max = 8;
-  if (wk_max > 16) wk_max = 16;
+  int wk_max = (c.tg >= 4 || (MB == 2 && c.tg == 2)) ? 8 : 16;
+  if (g_force_wk > 0 && g_force_wk < wk_max) wk_max = g_force_wk;
   c.sk = (kw + wk_max - 1) / wk_max;
   c.wk = (kw + c.sk - 1) / c.sk;
-  c.maxw = c.wk > 8 ? 16 : 8;
+  c.maxw = wk_max > 8 ? 16 : 8;
   const int cus = num_cus_current_device();
-  int gx = g_force_gx > 0 ? g_force_gx : (2 * cus) / c.sk;
+  int gx = g_force_gx > 0 ? g_force_gx : cus / c.sk;
   if (gx < 1) gx = 1;
   if (gx > NT) gx = NT;
   c.gx = gx;
+  const int per = (NT + gx - 1) / gx;           // n-tiles per workgroup
+  c.d = g_force_d > 0 ? g_force_d : (per >= 2 ? 2 : 1);   // depth 3 spills in the 128-register shapes
+  if (c.tg == 7) c.d = 1;
+  if (c.d > 3) c.d = 3;
+  if (c.d < 1) c.d = 1;
   return c;
 }
 
-template <bool BF16, int TG, int MB, bool HAS_ZP, int MAXW>
+template <bool BF16, int TG, int MB, bool HAS_ZP, int MAXW, int D>
 static void launch_decode(const DecodeParams& p, int gx, hipStream_t s) {
   const size_t lds = p.WK > 1 ? (size_t)2 * p.WK * MB * 64 * sizeof(v4f) : 0;
-  hipLaunchKernelGGL((w4a16_decode_kernel<BF16, TG, MB, HAS_ZP, MAXW>), dim3(gx, p.SK), dim3(64, p.WK), lds, s, p);
+  hipLaunchKernelGGL((w4a16_decode_kernel<BF16, TG, MB, HAS_ZP, MAXW, D>), dim3(gx, p.SK), dim3(64, p.WK), lds, s, p);
 }
 
+template <bool BF16, int TG, int MB, bool HAS_ZP, int MAXW>
+static int dispatch_d(const DecodeParams& p, const DecodeConfig& c, hipStream_t s) {
+  switch (c.d) {
+    case 1: launch_decode<BF16, TG, MB, HAS_ZP, MAXW, 1>(p, c.gx, s); return VAQ_OK;
+    case 2: launch_decode<BF16, TG, MB, HAS_ZP, MAXW, 2>(p, c.gx, s); return VAQ_OK;
+    case 3: launch_decode<BF16, TG, MB, HAS_ZP, MAXW, 3>(p, c.gx, s); return VAQ_OK;
+    default: break;
+  }
+  set_error("w4a16_gemm(decode): unsupported prefetch depth %d", c.d);
+  return VAQ_ERR_UNSUPPORTED;
+}
+
+// Instantiated launch shapes: one m-block: (TG,MAXW) in {(1,16), (2,16), (4,8), (7,8; depth 1)}; two m-blocks: {(1,16), (2,8)}.
 template <bool BF16, int MB, bool HAS_ZP>
 static int dispatch_tg(const DecodeParams& p, const DecodeConfig& c, hipStream_t s) {
-  const int gx = c.gx;
-  if (c.maxw == 16) {
-    switch (c.tg) {
-      case 1: launch_decode<BF16, 1, MB, HAS_ZP, 16>(p, gx, s); return VAQ_OK;
-      case 2: launch_decode<BF16, 2, MB, HAS_ZP, 16>(p, gx, s); return VAQ_OK;
-      case 4:
-        if constexpr (MB == 1) { launch_decode<BF16, 4, MB, HAS_ZP, 16>(p, gx, s); return VAQ_OK; }
-        break;
-      default: break;
-    }
+  if constexpr (MB == 1) {
+    if (c.tg == 1 && c.maxw == 16) return dispatch_d<BF16, 1, 1, HAS_ZP, 16>(p, c, s);
+    if (c.tg == 2 && c.maxw == 16) return dispatch_d<BF16, 2, 1, HAS_ZP, 16>(p, c, s);
+    if (c.tg == 4 && c.maxw == 8) return dispatch_d<BF16, 4, 1, HAS_ZP, 8>(p, c, s);
+    if (c.tg == 7 && c.maxw == 8) { launch_decode<BF16, 7, 1, HAS_ZP, 8, 1>(p, c.gx, s); return VAQ_OK; }
   } else {
-    switch (c.tg) {
-      case 1: launch_decode<BF16, 1, MB, HAS_ZP, 8>(p, gx, s); return VAQ_OK;
-      case 2: launch_decode<BF16, 2, MB, HAS_ZP, 8>(p, gx, s); return VAQ_OK;
-      case 4:
-        if constexpr (MB == 1) { launch_decode<BF16, 4, MB, HAS_ZP, 8>(p, gx, s); return VAQ_OK; }
-        break;
-      case 7:
-        if constexpr (MB == 1) { launch_decode<BF16, 7, MB, HAS_ZP, 8>(p, gx, s); return VAQ_OK; }
-        break;
-      default: break;
-    }
+    if (c.tg == 1 && c.maxw == 16) return dispatch_d<BF16, 1, 2, HAS_ZP, 16>(p, c, s);
+    if (c.tg == 2 && c.maxw == 8) return dispatch_d<BF16, 2, 2, HAS_ZP, 8>(p, c, s);
   }
   set_error("w4a16_gemm(decode): unsupported launch shape TG=%d MAXW=%d for MB=%d", c.tg, c.maxw, MB);
   return VAQ_ERR_UNSUPPORTED;
@@ -392,5 +438,6 @@ int w4a16_decode_launch(const void* a, int64_t lda, const int32_t* b, const void
 extern "C" void vaq_debug_set_decode_config(int tg, int wk, int gx) {
   vaq::g_force_tg = tg;
   vaq::g_force_wk = wk;
-  vaq::g_force_gx = gx;
+  vaq::g_force_gx = gx % 100000;
+  vaq::g_force_d = gx / 100000;     // prefetch depth rides in the upper digits: gx = depth * 100000 + grid
 }

@@ -18,7 +18,7 @@ static int check_shape(int64_t size_m, int64_t size_n, int64_t size_k) {
   VAQ_CHECK_ARG(size_k > 0 && size_k % 128 == 0, "w4a16_gemm: size_k = %lld, is not divisible by min_thread_k = 128",
                 (long long)size_k);
   VAQ_CHECK_ARG(size_m < (1ll << 31) && size_n < (1ll << 31) && size_k < (1ll << 31) &&
-                    size_k * size_n / 8 < (1ll << 40),
+                    size_k * size_n / 2 < (1ll << 32),
                 "w4a16_gemm: problem too large");
   return VAQ_OK;
 }
