@@ -94,16 +94,26 @@ def time_graph(fn, iters, warmup, inner=1):
     g = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g):
         fn()
-    for _ in range(warmup):
+    # warm up for at least ~30 ms of GPU time: the shader clock needs milliseconds to ramp up
+    t_end = time.perf_counter() + 0.03
+    n = 0
+    while n < warmup or time.perf_counter() < t_end:
         g.replay()
+        n += 1
+        if n % 8 == 0:
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(iters):
-        g.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e-3 / iters / inner
+    best = None
+    for _ in range(3):                      # median of three timed bursts
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) * 1e-3 / iters / inner
+        best = [t] if best is None else best + [t]
+    return sorted(best)[1]
 
 
 def headline(dev, steps, warmup):

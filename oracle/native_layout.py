@@ -1,7 +1,8 @@
 """CPU statement of this build's own NATIVE weight order (no reference counterpart: the reference treats the
 repacked tensor as opaque, marlin.py:85-91 / :153-166).  TEST INFRASTRUCTURE ONLY.
 
-Tile (kt, nt) = rows 128*kt.., columns 16*nt.. is the 256-word block number kt*(N/16)+nt.  Word 4*L + j of a tile,
+Tile (kt, nt) = rows 128*kt.., columns 16*nt.. is the 256-word block number nt*(K/128)+kt (the tiles of a
+16-column strip are contiguous along K).  Word 4*L + j of a tile,
 L = 16*o + r, holds the codes of rows 128*kt + 32*j + 8*o + e (e = 0..7) of column 16*nt + r; code e sits in nibble
 position p with {0,2,4,6,1,3,5,7}[p] == e.  The inverse (`native_unpack`) is the documented map back to the logical
 [K, N] code matrix.
@@ -16,12 +17,12 @@ _POS_TO_E = np.array([0, 2, 4, 6, 1, 3, 5, 7])
 def _index_maps(size_k: int, size_n: int):
     """For every output word (flat index) the row index of its 8 codes (in nibble-position order) and its column."""
     assert size_k % 128 == 0 and size_n % 16 == 0
-    n_tiles = size_n // 16
+    k_tiles = size_k // 128
     idx = np.arange(size_k * size_n // 8, dtype=np.int64)
     j = idx & 3
     lane = (idx >> 2) & 63
     tile = idx >> 8
-    kt, nt = tile // n_tiles, tile % n_tiles
+    nt, kt = tile // k_tiles, tile % k_tiles
     o, r = lane >> 4, lane & 15
     k0 = kt * 128 + j * 32 + o * 8
     n = nt * 16 + r

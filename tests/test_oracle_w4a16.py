@@ -99,12 +99,12 @@ def test_native_layout_roundtrip_and_word_content(k, n):
     assert np.array_equal(nl.native_unpack(packed, k, n), q)
     # spot-check the definition by hand for a few words
     words = packed.reshape(-1).view(np.uint32)
-    n_tiles = n // 16
-    for idx in (0, 1, 5, 255, 256, 4 * 64 * (n_tiles + 1) + 4 * 37 + 2, words.size - 1):
+    k_tiles = k // 128
+    for idx in (0, 1, 5, 255, 256, 4 * 64 * (k_tiles + 1) + 4 * 37 + 2, words.size - 1):
         if idx >= words.size:
             continue
         j, lane, tile = idx & 3, (idx >> 2) & 63, idx >> 8
-        kt, nt = divmod(tile, n_tiles)
+        nt, kt = divmod(tile, k_tiles)
         o_, r = lane >> 4, lane & 15
         k0 = 128 * kt + 32 * j + 8 * o_
         col = 16 * nt + r

@@ -44,6 +44,8 @@ _SIGNATURES = {
 _DEBUG_SIGNATURES = {
     "vaq_debug_set_decode_config": (None, [c_int, c_int, c_int]),
     "vaq_debug_set_prefill_tile": (None, [c_int]),
+    "vaq_debug_set_decode_impl": (None, [c_int]),
+    "vaq_debug_set_decode2_config": (None, [c_int, c_int]),
     "vaq_debug_set_fp8_config": (None, [c_int, c_int]),
 }
 

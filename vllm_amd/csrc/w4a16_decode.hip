@@ -37,6 +37,7 @@ struct DecodeParams {
   v4f* c_tmp;
   int32_t* counters;
   int M, N, K, G, NT, SK, WK;
+  uint32_t k_mask, k_ex;   // 0x000f000f and the exponent pattern, passed as run-time values (see and_or)
 };
 
 // Split-K partial tiles cross workgroups (and therefore XCDs, whose L2 caches are not coherent with each other)
@@ -57,17 +58,13 @@ __device__ inline v4f load_partial(const float* src) {
   return v;
 }
 
-// (x & mask) | ex in one VALU op (mask from a scalar register, ex from a vector register: a VOP3 instruction of this
-// architecture cannot carry two literals, and the compiler otherwise emits two instructions).
-__device__ inline uint32_t and_or(uint32_t x, uint32_t mask, uint32_t ex) {
-  uint32_t d;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(x), "s"(mask), "v"(ex));
-  return d;
-}
+// (x & mask) | ex.  mask and ex reach the kernel as run-time arguments: with literal constants the compiler emits two
+// instructions (a VOP3 op of this architecture cannot carry two literals); with register operands it selects the
+// single v_and_or_b32, and unlike inline assembly the instruction stays visible to the MFMA hazard recogniser.
+__device__ inline uint32_t and_or(uint32_t x, uint32_t mask, uint32_t ex) { return (x & mask) | ex; }
 
 template <bool BF16>
-__device__ inline v4u dequant_biased_fast(uint32_t w, uint32_t ex) {
-  constexpr uint32_t M = 0x000f000fu;
+__device__ inline v4u dequant_biased_fast(uint32_t w, uint32_t M, uint32_t ex) {
   v4u r;
   r.x = and_or(w, M, ex);
   r.y = and_or(w >> 4, M, ex);
@@ -110,12 +107,18 @@ __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodePar
   uint32_t zq[D][TG];
   // Groups past the end of K (ragged last wavefront) are clamped for addressing; their activations are zero, so they
   // contribute nothing.
-  auto issue_load = [&](int u, int nt, int t) {
+  uint32_t ob[TG], os_[TG], oz[TG];      // scalar byte offsets of this wavefront's groups at n-tile 0
+#pragma unroll
+  for (int t = 0; t < TG; ++t) {
     const uint32_t g = (uint32_t)min(g0 + t, p.G - 1);
-    wq[u][t] = __builtin_amdgcn_raw_buffer_load_b128(rb, vo_b, (int)((g * (uint32_t)p.NT + (uint32_t)nt) * 1024u), 2);
-    sc[u][t] = __builtin_amdgcn_raw_buffer_load_b64(rs, vo_s, (int)((g * (uint32_t)p.N + (uint32_t)nt * 16u) * 2u), 0);
-    if constexpr (HAS_ZP)
-      zq[u][t] = __builtin_amdgcn_raw_buffer_load_b32(rz, vo_z, (int)((g * (uint32_t)(p.N >> 3) + (uint32_t)nt * 2u) * 4u), 0);
+    ob[t] = g * 1024u;
+    os_[t] = g * (uint32_t)p.N * 2u;
+    oz[t] = g * (uint32_t)(p.N >> 3) * 4u;
+  }
+  auto issue_load = [&](int u, int nt, int t) {
+    wq[u][t] = __builtin_amdgcn_raw_buffer_load_b128(rb, vo_b, (int)(ob[t] + (uint32_t)nt * (uint32_t)p.G * 1024u), 2);
+    sc[u][t] = __builtin_amdgcn_raw_buffer_load_b64(rs, vo_s, (int)(os_[t] + (uint32_t)nt * 32u), 0);
+    if constexpr (HAS_ZP) zq[u][t] = __builtin_amdgcn_raw_buffer_load_b32(rz, vo_z, (int)(oz[t] + (uint32_t)nt * 8u), 0);
   };
   // The first weight tiles are requested before anything else so that their latency overlaps the activation loads.
 #pragma unroll
@@ -190,8 +193,11 @@ __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodePar
     }
   }
 
-  const uint32_t ex = T::EX;
+  uint32_t ex;     // kept in a vector register so that (x & msk) | ex is a legal single VOP3 instruction (one scalar operand)
+  asm volatile("v_mov_b32 %0, %1" : "=v"(ex) : "s"(p.k_ex));
+  const uint32_t msk = p.k_mask;
   int parity = 0;
+  int red_w = 0;      // wavefront that reduces m-block 0 of the current n-tile; advances by MB per n-tile (mod WK)
   for (int base = nt0; base < nt1; base += D) {
 #pragma unroll
     for (int u = 0; u < D; ++u) {
@@ -213,7 +219,7 @@ __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodePar
         for (int mb = 0; mb < MB; ++mb) P[mb] = HAS_ZP ? v4f{0.f, 0.f, 0.f, 0.f} : Sv[t][mb];
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
-          const v4u aop = dequant_biased_fast<BF16>(wj[jj], ex);
+          const v4u aop = dequant_biased_fast<BF16>(wj[jj], msk, ex);
 #pragma unroll
           for (int mb = 0; mb < MB; ++mb) P[mb] = T::mfma16(aop, breg[t][jj][mb], P[mb]);
         }
@@ -248,7 +254,6 @@ __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodePar
       }
 
       // ---- reduce the WK partial tiles of this workgroup through LDS; the reducing wavefront rotates ----
-      const int it = nt - nt0;
       int my_mb = -1;
       v4f tot = v4f{0.f, 0.f, 0.f, 0.f};
       if (p.WK > 1) {
@@ -258,11 +263,17 @@ __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodePar
         __syncthreads();
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          if ((it * MB + mb) % p.WK == w) my_mb = mb;
+        {
+          int cand = red_w + mb;
+          if (cand >= p.WK) cand -= p.WK;
+          if (cand == w) my_mb = mb;
+        }
         if (my_mb >= 0) {
           for (int ww = 0; ww < p.WK; ++ww) tot += buf[(ww * MB + my_mb) * 64 + lane];
         }
         parity ^= 1;
+        red_w += MB;
+        if (red_w >= p.WK) red_w -= p.WK;
       }
 
       const int mb_lo = (p.WK > 1) ? my_mb : 0;
@@ -407,6 +418,8 @@ int w4a16_decode_launch(const void* a, int64_t lda, const int32_t* b, const void
   p.M = M; p.N = N; p.K = K;
   p.G = K / 128;
   p.NT = N / 16;
+  p.k_mask = 0x000f000fu;
+  p.k_ex = dtype == VAQ_BF16 ? 0x43004300u : 0x64006400u;
   const DecodeConfig cfg = pick_decode_config(M, N, K);
   p.SK = cfg.sk;
   p.WK = cfg.wk;

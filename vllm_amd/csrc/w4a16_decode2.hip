@@ -1,0 +1,408 @@
+// W4A16 decode-shaped GEMM (M <= 32), barrier-free variant: activations staged in LDS, one independent task per
+// wavefront.  C[M,N] = A[M,K] . dequant(B[K,N]) (+bias), same arithmetic as w4a16_decode.hip.
+//
+//  * A workgroup is 16 wavefronts = WKS slices of K  x  WN = 16/WKS n-tiles (16 columns each).  Wavefront (wks, wn)
+//    streams the GS consecutive 1 KiB weight tiles (= quantisation groups) of its slice for its n-tile; all its tile
+//    loads are issued up front through a register ring of min(GS, 8) slots, so no wavefront ever waits for another one
+//    inside the K loop.
+//  * The activations of the workgroup's K slab (WKS*GS groups) are written once to LDS in MFMA-B-operand order
+//    ([k-octet][m] 16-byte slots, rows m >= M zero, XOR-swizzled so that both the row-contiguous fill and the
+//    operand reads are bank-conflict free) and read back with one ds_read_b128 per MFMA.  Weight loads are issued
+//    before the fill so that their latency covers it.
+//  * Per tile: 4 x { dequantise one word to 8 biased 16-bit numbers (7 VALU ops), MFMA with the activations, MFMA of
+//    the constant operand -(BIAS + zero) with the same activations }, then acc += scale * P (fp32).  The second MFMA
+//    removes the bias and the zero point exactly as `P - (BIAS+z)*S` would, without keeping S anywhere.
+//  * WKS > 1: one LDS reduction at the end (wavefronts wks == 0 sum their column's slices).  K slabs that do not fit
+//    LDS (SK > 1 workgroups per n-tile) hand partial tiles over through device-scope write-through stores and an
+//    arrival counter, summed in fixed order by the last arriver.
+#include "vaq_common.h"
+
+namespace vaq {
+
+struct Decode2Params {
+  const uint16_t* a;
+  int64_t lda;
+  const v4u* b;
+  const uint16_t* scales;
+  const uint32_t* zeros;
+  const int32_t* perm;
+  const uint16_t* bias;
+  uint16_t* c;
+  float* c_tmp;
+  int32_t* counters;
+  int M, N, K, G, NT, SK, WKS;
+  uint32_t k_mask, k_ex;   // 0x000f000f and the exponent pattern, passed as run-time values (see and_or)
+};
+
+__device__ inline void d2_store_partial(float* dst, v4f v) {
+  __hip_atomic_store(dst + 0, v.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(dst + 1, v.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(dst + 2, v.z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(dst + 3, v.w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ inline v4f d2_load_partial(const float* src) {
+  v4f v;
+  v.x = __hip_atomic_load(src + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  v.y = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  v.z = __hip_atomic_load(src + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  v.w = __hip_atomic_load(src + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return v;
+}
+
+// (x & mask) | ex.  mask and ex reach the kernel as run-time arguments: with literal constants the compiler emits two
+// instructions (a VOP3 op of this architecture cannot carry two literals); with register operands it selects the
+// single v_and_or_b32, and unlike inline assembly the instruction stays visible to the MFMA hazard recogniser.
+__device__ inline uint32_t d2_and_or(uint32_t x, uint32_t mask, uint32_t ex) { return (x & mask) | ex; }
+
+__device__ inline __amdgpu_buffer_rsrc_t d2_rsrc(const void* base, uint64_t bytes) {
+  const uint32_t n = bytes > 0xffffffffull ? 0xffffffffu : (uint32_t)bytes;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)n, 0x00020000);
+}
+
+constexpr int D2_WAVES = 16;
+
+template <bool BF16, int GS, int MB, bool HAS_ZP>
+__global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Decode2Params p) {
+  using T = F16Traits<BF16>;
+  constexpr int R = GS < 8 ? GS : 8;                 // ring slots
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+  const int lane = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(threadIdx.y);
+  const int o = lane >> 4, r16 = lane & 15;
+  const int WKS = p.WKS, WN = D2_WAVES / WKS;
+  const int wks = w / WN, wn = w - wks * WN;
+  const int sk = blockIdx.y;
+  const int slab_groups = WKS * GS;
+  const int slab_g0 = sk * slab_groups;             // first group of this workgroup's K slab
+  const int nt_raw = blockIdx.x * WN + wn;
+  const bool nt_ok = nt_raw < p.NT;
+  const int nt = nt_ok ? nt_raw : p.NT - 1;
+  const int g_first = slab_g0 + wks * GS;           // this wavefront's first group
+
+  // ---- 1. request the first R weight tiles (+ scales, zero points) ----
+  const __amdgpu_buffer_rsrc_t rb = d2_rsrc(p.b, (uint64_t)p.K * p.N / 2);
+  const __amdgpu_buffer_rsrc_t rs = d2_rsrc(p.scales, (uint64_t)p.G * p.N * 2);
+  const __amdgpu_buffer_rsrc_t rz = d2_rsrc(HAS_ZP ? (const void*)p.zeros : (const void*)p.scales, (uint64_t)p.G * (p.N / 8) * 4);
+  const int vo_b = lane * 16, vo_s = o * 8, vo_z = (r16 >> 3) * 4;
+  v4u wq[R];
+  v2u sc[R];
+  uint32_t zq[R];
+  auto issue_load = [&](int slot, int gi) {
+    const uint32_t g = (uint32_t)min(g_first + gi, p.G - 1);     // clamped: activations past K are zero
+    wq[slot] = __builtin_amdgcn_raw_buffer_load_b128(rb, vo_b, (int)(((uint32_t)nt * (uint32_t)p.G + g) * 1024u), 2);
+    sc[slot] = __builtin_amdgcn_raw_buffer_load_b64(rs, vo_s, (int)((g * (uint32_t)p.N + (uint32_t)nt * 16u) * 2u), 0);
+    if constexpr (HAS_ZP)
+      zq[slot] = __builtin_amdgcn_raw_buffer_load_b32(rz, vo_z, (int)((g * (uint32_t)(p.N >> 3) + (uint32_t)nt * 2u) * 4u), 0);
+    else
+      zq[slot] = 0u;
+  };
+#pragma unroll
+  for (int s = 0; s < R; ++s) issue_load(s, s);
+
+  // ---- 2. stage the activations of the K slab in LDS ----
+  // slot (16 bytes) of (m-block mb, row ml, k-octet ko):  mb*KO*16 + ko*16 + (ml ^ (ko & 15))
+  const int KO = slab_groups * 16;                   // k-octets in the slab
+  {
+    // chunk c = m * KO + ko (16 bytes: row m, k-octet ko); thread tid handles c = tid, tid + 1024, ...  The (m, ko)
+    // pair is advanced incrementally: one scalar division per kernel instead of one vector division per chunk.
+    const int tid = w * 64 + lane;
+    const int chunks = KO * 16 * MB;
+    const int64_t k_slab0 = (int64_t)slab_g0 * 128;
+    constexpr int NTHR = D2_WAVES * 64;
+    const int step_m = NTHR / KO, step_ko = NTHR - step_m * KO;     // scalar
+    int m = tid / KO, ko = tid - m * KO;
+    for (int c0 = 0; c0 < chunks; c0 += NTHR * 4) {
+      v4u v[4];
+      int mm[4], kk[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        mm[i] = m;
+        kk[i] = ko;
+        const int64_t k = k_slab0 + (int64_t)ko * 8;
+        v[i] = v4u{0u, 0u, 0u, 0u};
+        if (m < 16 * MB && m < p.M && k < p.K) {
+          const uint16_t* row = p.a + (int64_t)m * p.lda;
+          if (p.perm == nullptr) {
+            v[i] = *reinterpret_cast<const v4u*>(row + k);
+          } else {
+            const v4i p0 = *reinterpret_cast<const v4i*>(p.perm + k);
+            const v4i p1 = *reinterpret_cast<const v4i*>(p.perm + k + 4);
+            v[i].x = (uint32_t)row[p0.x] | ((uint32_t)row[p0.y] << 16);
+            v[i].y = (uint32_t)row[p0.z] | ((uint32_t)row[p0.w] << 16);
+            v[i].z = (uint32_t)row[p1.x] | ((uint32_t)row[p1.y] << 16);
+            v[i].w = (uint32_t)row[p1.z] | ((uint32_t)row[p1.w] << 16);
+          }
+        }
+        m += step_m;
+        ko += step_ko;
+        if (ko >= KO) {
+          ko -= KO;
+          m += 1;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (mm[i] < 16 * MB) {
+          const int mb = mm[i] >> 4, ml = mm[i] & 15;
+          const int slot = mb * KO * 16 + kk[i] * 16 + (ml ^ (kk[i] & 15));
+          *reinterpret_cast<v4u*>(lds + (size_t)slot * 16) = v[i];
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- 3. the K loop of this wavefront: GS tiles, fully unrolled ----
+  // operand read of MFMA jj of local group gl: k-octet = gl*16 + jj*4 + o  ->  (ko & 15) = jj*4 + o
+  uint32_t abase[4];
+#pragma unroll
+  for (int jj = 0; jj < 4; ++jj) {
+    const int kol = jj * 4 + o;
+    abase[jj] = (uint32_t)(((wks * GS * 16 + kol) * 16 + (r16 ^ kol)) * 16);
+  }
+  uint32_t ex;     // kept in a vector register so that (x & MSK) | ex is a legal single VOP3 instruction (one scalar operand)
+  asm volatile("v_mov_b32 %0, %1" : "=v"(ex) : "s"(p.k_ex));
+  const uint32_t MSK = p.k_mask;
+  constexpr uint32_t NEG_BIAS_BITS = BF16 ? 0xC300u : 0xE400u;     // -(BIAS) as a 16-bit pattern; "| z" adds the zero point
+  v4f acc[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) acc[mb] = v4f{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+  for (int gi = 0; gi < GS; ++gi) {
+    const int slot = gi % R;
+    const uint32_t wj[4] = {wq[slot].x, wq[slot].y, wq[slot].z, wq[slot].w};
+    const v2u sct = sc[slot];
+    const uint32_t zqt = zq[slot];
+    if (gi + R < GS) issue_load(slot, gi + R);
+
+    uint32_t zbits;
+    if constexpr (HAS_ZP) zbits = NEG_BIAS_BITS | ((zqt >> ((r16 & 7) * 4)) & 0xFu);
+    else zbits = NEG_BIAS_BITS | 8u;
+    const uint32_t z2 = zbits | (zbits << 16);
+    const v4u zop = {z2, z2, z2, z2};
+
+    v4f P[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) P[mb] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      v4u aop;
+      aop.x = d2_and_or(wj[jj], MSK, ex);
+      aop.y = d2_and_or(wj[jj] >> 4, MSK, ex);
+      aop.z = d2_and_or(wj[jj] >> 8, MSK, ex);
+      aop.w = d2_and_or(wj[jj] >> 12, MSK, ex);
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const v4u bop = *reinterpret_cast<const v4u*>(lds + abase[jj] + (uint32_t)(mb * KO * 256) + (uint32_t)(gi * 4096));
+        P[mb] = T::mfma16(aop, bop, P[mb]);
+        P[mb] = T::mfma16(zop, bop, P[mb]);
+      }
+    }
+    float s[4];
+    if constexpr (BF16) {
+      s[0] = __uint_as_float(sct.x << 16);
+      s[1] = __uint_as_float(sct.x & 0xffff0000u);
+      s[2] = __uint_as_float(sct.y << 16);
+      s[3] = __uint_as_float(sct.y & 0xffff0000u);
+    } else {
+      s[0] = T::to_float((uint16_t)(sct.x & 0xffffu));
+      s[1] = T::to_float((uint16_t)(sct.x >> 16));
+      s[2] = T::to_float((uint16_t)(sct.y & 0xffffu));
+      s[3] = T::to_float((uint16_t)(sct.y >> 16));
+    }
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[mb][r] = fmaf(s[r], P[mb][r], acc[mb][r]);
+  }
+
+  // ---- 4. reduce the K slices of the workgroup ----
+  v4f* red = reinterpret_cast<v4f*>(lds + (size_t)KO * 16 * MB * 16);     // [16 waves][MB][64]
+  if (WKS > 1) {
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) red[(w * MB + mb) * 64 + lane] = acc[mb];
+    __syncthreads();
+    if (wks != 0) return;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      v4f t = acc[mb];
+      for (int s2 = 1; s2 < WKS; ++s2) t += red[((s2 * WN + wn) * MB + mb) * 64 + lane];
+      acc[mb] = t;
+    }
+  }
+  if (!nt_ok) return;
+
+  // ---- 5. hand over across workgroups if K is split, then write the 16-bit outputs ----
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    v4f val = acc[mb];
+    bool write_out = true;
+    if (p.SK > 1) {
+      const int64_t slot = (((int64_t)nt * MB + mb) * 64 + lane) * 4;
+      const int64_t sk_stride = (int64_t)p.NT * MB * 64 * 4;
+      d2_store_partial(p.c_tmp + sk * sk_stride + slot, val);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // partial tile acknowledged before the counter moves
+      int old = 0;
+      if (lane == 0) old = __hip_atomic_fetch_add(&p.counters[nt * MB + mb], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      old = __shfl(old, 0);
+      write_out = (old == p.SK - 1);
+      if (write_out) {
+        val = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int s2 = 0; s2 < p.SK; ++s2) val += d2_load_partial(p.c_tmp + s2 * sk_stride + slot);   // fixed order
+        if (lane == 0) __hip_atomic_store(&p.counters[nt * MB + mb], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    const int m = mb * 16 + r16;
+    if (write_out && m < p.M) {
+      const int n = nt * 16 + o * 4;
+      if (p.bias) {
+        const v2u bb = *reinterpret_cast<const v2u*>(p.bias + n);
+        val[0] += T::to_float((uint16_t)(bb.x & 0xffffu));
+        val[1] += T::to_float((uint16_t)(bb.x >> 16));
+        val[2] += T::to_float((uint16_t)(bb.y & 0xffffu));
+        val[3] += T::to_float((uint16_t)(bb.y >> 16));
+      }
+      v2u outv;
+      outv.x = (uint32_t)T::from_float(val[0]) | ((uint32_t)T::from_float(val[1]) << 16);
+      outv.y = (uint32_t)T::from_float(val[2]) | ((uint32_t)T::from_float(val[3]) << 16);
+      *reinterpret_cast<v2u*>(p.c + (int64_t)m * p.N + n) = outv;
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------- host side
+
+struct Decode2Config {
+  int gs, wks, sk;
+};
+
+static int g2_force_gs = 0, g2_force_wks = 0;
+
+static int round_gs(int x) {
+  const int opts[] = {1, 2, 4, 7, 8, 14, 16};
+  for (int o : opts)
+    if (o >= x) return o;
+  return 16;
+}
+
+// Groups per slab are limited by LDS (128 KiB of activations): 32 groups for one m-block, 16 for two.
+static Decode2Config pick_decode2_config(int M, int N, int K) {
+  const int G = K / 128, NT = N / 16;
+  const int MB = M <= 16 ? 1 : 2;
+  const int slab_max = MB == 1 ? 32 : 16;
+  Decode2Config c;
+  c.sk = (G + slab_max - 1) / slab_max;
+  const int gslab = (G + c.sk - 1) / c.sk;            // groups per slab
+  const int cus = num_cus_current_device();
+  int want = (cus * D2_WAVES) / (NT * c.sk);          // K slices wanted so that NT*SK*WKS ~ one workgroup per CU
+  int wks = 1;
+  while (wks * 2 <= want && wks < 16) wks *= 2;
+  while (wks > 1 && wks > gslab) wks /= 2;
+  if (g2_force_wks > 0) wks = g2_force_wks;
+  int gs = round_gs((gslab + wks - 1) / wks);
+  if (g2_force_gs > 0) gs = g2_force_gs;
+  while (wks * gs > slab_max && wks > 1) wks /= 2;     // respect the LDS limit
+  // the slab is now wks*gs groups; recompute the number of slabs
+  c.sk = (G + wks * gs - 1) / (wks * gs);
+  c.gs = gs;
+  c.wks = wks;
+  return c;
+}
+
+template <bool BF16, int GS, int MB, bool HAS_ZP>
+static int launch_decode2(const Decode2Params& p, hipStream_t s) {
+  const int WN = D2_WAVES / p.WKS;
+  const size_t lds = (size_t)p.WKS * GS * 4096 * MB + (p.WKS > 1 ? (size_t)D2_WAVES * MB * 1024 : 0);
+  auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP>;
+  static size_t attr_lds = 0;
+  if (lds > attr_lds) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
+        hipSuccess) {
+      set_error("w4a16_gemm(decode): cannot reserve %zu bytes of LDS", lds);
+      (void)hipGetLastError();
+      return VAQ_ERR_LAUNCH;
+    }
+    attr_lds = lds;
+  }
+  const int gx = (p.NT + WN - 1) / WN;
+  hipLaunchKernelGGL(kern, dim3(gx, p.SK), dim3(64, D2_WAVES), lds, s, p);
+  return VAQ_OK;
+}
+
+template <bool BF16, int MB, bool HAS_ZP>
+static int dispatch_gs2(const Decode2Params& p, int gs, hipStream_t s) {
+  switch (gs) {
+    case 1: return launch_decode2<BF16, 1, MB, HAS_ZP>(p, s);
+    case 2: return launch_decode2<BF16, 2, MB, HAS_ZP>(p, s);
+    case 4: return launch_decode2<BF16, 4, MB, HAS_ZP>(p, s);
+    case 7: return launch_decode2<BF16, 7, MB, HAS_ZP>(p, s);
+    case 8: return launch_decode2<BF16, 8, MB, HAS_ZP>(p, s);
+    case 14: return launch_decode2<BF16, 14, MB, HAS_ZP>(p, s);
+    case 16: return launch_decode2<BF16, 16, MB, HAS_ZP>(p, s);
+    default: break;
+  }
+  set_error("w4a16_gemm(decode): unsupported groups per wavefront %d", gs);
+  return VAQ_ERR_UNSUPPORTED;
+}
+
+int w4a16_decode2_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* counter_ints) {
+  const Decode2Config c = pick_decode2_config(M, N, K);
+  const int MB = M <= 16 ? 1 : 2;
+  const int NT = N / 16;
+  *c_tmp_bytes = c.sk > 1 ? (size_t)c.sk * NT * MB * 64 * sizeof(v4f) : 0;
+  *counter_ints = c.sk > 1 ? (size_t)NT * MB : 0;
+  return VAQ_OK;
+}
+
+int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
+                         const int32_t* perm, const void* bias, void* c, float* c_tmp, int32_t* counters,
+                         int64_t counter_ints, int M, int N, int K, int dtype, hipStream_t s) {
+  Decode2Params p;
+  p.a = (const uint16_t*)a;
+  p.lda = lda;
+  p.b = (const v4u*)b;
+  p.scales = (const uint16_t*)scales;
+  p.zeros = (const uint32_t*)zeros;
+  p.perm = perm;
+  p.bias = (const uint16_t*)bias;
+  p.c = (uint16_t*)c;
+  p.c_tmp = c_tmp;
+  p.counters = counters;
+  p.M = M; p.N = N; p.K = K;
+  p.G = K / 128;
+  p.NT = N / 16;
+  p.k_mask = 0x000f000fu;
+  p.k_ex = dtype == VAQ_BF16 ? 0x43004300u : 0x64006400u;
+  const Decode2Config cfg = pick_decode2_config(M, N, K);
+  p.SK = cfg.sk;
+  p.WKS = cfg.wks;
+  const int MB = M <= 16 ? 1 : 2;
+  if (cfg.sk > 1) {
+    VAQ_CHECK_ARG(c_tmp != nullptr && counters != nullptr, "w4a16_gemm: split-K needs c_tmp and counters");
+    VAQ_CHECK_ARG(counter_ints >= (int64_t)p.NT * MB,
+                  "w4a16_gemm: workspace.numel = %lld is below min_workspace_size = %lld", (long long)counter_ints,
+                  (long long)p.NT * MB);
+  }
+  const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
+  int rc;
+  if (MB == 1) {
+    if (bf16) rc = zp ? dispatch_gs2<true, 1, true>(p, cfg.gs, s) : dispatch_gs2<true, 1, false>(p, cfg.gs, s);
+    else rc = zp ? dispatch_gs2<false, 1, true>(p, cfg.gs, s) : dispatch_gs2<false, 1, false>(p, cfg.gs, s);
+  } else {
+    if (bf16) rc = zp ? dispatch_gs2<true, 2, true>(p, cfg.gs, s) : dispatch_gs2<true, 2, false>(p, cfg.gs, s);
+    else rc = zp ? dispatch_gs2<false, 2, true>(p, cfg.gs, s) : dispatch_gs2<false, 2, false>(p, cfg.gs, s);
+  }
+  if (rc != VAQ_OK) return rc;
+  VAQ_CHECK_LAUNCH("w4a16_gemm(decode)");
+  return VAQ_OK;
+}
+
+}  // namespace vaq
+
+// Benchmark / tuning aid, not part of the drop-in surface (0 = automatic).  Process-global, not thread-safe.
+extern "C" void vaq_debug_set_decode2_config(int gs, int wks) {
+  vaq::g2_force_gs = gs;
+  vaq::g2_force_wks = wks;
+}

@@ -6,10 +6,23 @@ int w4a16_decode_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* cou
 int w4a16_decode_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
                         const int32_t* perm, const void* bias, void* c, float* c_tmp, int32_t* counters,
                         int64_t counter_ints, int M, int N, int K, int dtype, hipStream_t s);
+int w4a16_decode2_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* counter_ints);
+int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
+                         const int32_t* perm, const void* bias, void* c, float* c_tmp, int32_t* counters,
+                         int64_t counter_ints, int M, int N, int K, int dtype, hipStream_t s);
 int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
                          const void* bias, void* c, int M, int N, int K, int dtype, hipStream_t s);
 
 constexpr int64_t DECODE_MAX_M = 32;
+static int g_decode_impl = -1;  // -1: automatic, 0: LDS-staged activations (w4a16_decode2.hip), 1: register-resident (w4a16_decode.hip)
+
+// Measured on MI355X (Llama-3-8B shapes): keeping the activations in registers wins while they are few (M <= 8:
+// each workgroup pulls M*K*2 bytes of A) and for wide layers; staging them once per workgroup in LDS wins for
+// M > 8 on layers with few n-tiles, where A traffic per compute unit dominates.
+static int decode_impl_for(int64_t size_m, int64_t size_n) {
+  if (g_decode_impl >= 0) return g_decode_impl;
+  return (size_m > 8 && size_n <= 8192) ? 0 : 1;
+}
 
 static int check_shape(int64_t size_m, int64_t size_n, int64_t size_k) {
   VAQ_CHECK_ARG(size_m >= 0, "w4a16_gemm: size_m = %lld is negative", (long long)size_m);
@@ -35,7 +48,9 @@ extern "C" int vaq_w4a16_gemm_workspace(int64_t size_m, int64_t size_n, int64_t 
   *a_tmp_bytes = 0;
   *counter_ints = 0;
   if (size_m == 0) return VAQ_OK;
-  if (size_m <= DECODE_MAX_M) return w4a16_decode_workspace((int)size_m, (int)size_n, (int)size_k, c_tmp_bytes, counter_ints);
+  if (size_m <= DECODE_MAX_M)
+    return decode_impl_for(size_m, size_n) == 0 ? w4a16_decode2_workspace((int)size_m, (int)size_n, (int)size_k, c_tmp_bytes, counter_ints)
+                              : w4a16_decode_workspace((int)size_m, (int)size_n, (int)size_k, c_tmp_bytes, counter_ints);
   if (has_perm) *a_tmp_bytes = (size_t)size_m * (size_t)size_k * 2;
   return VAQ_OK;
 }
@@ -73,6 +88,9 @@ extern "C" int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, cons
   } else if (force_path == 2) {
     decode = false;
   }
+  if (decode && decode_impl_for(size_m, size_n) == 0)
+    return w4a16_decode2_launch(a, lda, b, scales, zeros, perm, bias, c, c_tmp, counters, counter_ints, (int)size_m,
+                                (int)size_n, (int)size_k, dtype, s);
   if (decode)
     return w4a16_decode_launch(a, lda, b, scales, zeros, perm, bias, c, c_tmp, counters, counter_ints, (int)size_m,
                                (int)size_n, (int)size_k, dtype, s);
@@ -89,3 +107,7 @@ extern "C" int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, cons
   }
   return w4a16_prefill_launch(a_eff, lda_eff, b, scales, zeros, bias, c, (int)size_m, (int)size_n, (int)size_k, dtype, s);
 }
+
+// Benchmark / tuning aid, not part of the drop-in surface: choose the decode implementation (-1 = automatic, 0 = LDS-staged
+// activations, 1 = register-resident activations).  Process-global, not thread-safe.
+extern "C" void vaq_debug_set_decode_impl(int impl) { vaq::g_decode_impl = impl; }

@@ -126,7 +126,7 @@ __global__ __launch_bounds__(256) void w4a16_prefill_kernel(const PrefillParams 
       v4u v = {0u, 0u, 0u, 0u};
       float s = 0.f, z = 8.f;
       if (nt < p.NT) {
-        v = p.b[((int64_t)g * p.NT + nt) * 64 + lane];
+        v = p.b[((int64_t)nt * p.G + g) * 64 + lane];
         const int n = nt * 16 + (lane & 15);
         s = T::to_float(p.scales[(int64_t)g * p.N + n]);
         if constexpr (HAS_ZP) {
