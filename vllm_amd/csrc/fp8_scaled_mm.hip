@@ -43,6 +43,51 @@ __device__ inline v4f mfma_fp8_16(v8i a, v8i b, v4f c) {
 constexpr int F8_BK = 128;       // bytes of K per step
 constexpr int F8_PITCH = 144;    // LDS row pitch in bytes
 
+// Epilogue of the tile kernels.  The MFMAs are issued with the weight fragment as the A operand, so a 32x32
+// accumulator block holds D[n_local][m_local]: lane -> column m_local = lane & 31, registers e -> rows
+// n_local = 8*(e/4) + 4*(lane/32) + e%4.  Four consecutive registers are four consecutive n of one output row: one
+// 8-byte store, one scale load per row, one 16-byte load of the channel scales.
+template <bool BF16_OUT, int WMB, int WNB>
+__device__ inline void tile_epilogue(const Fp8MMParams& p, v16f (&acc)[WMB][WNB], int m0, int n0, int wm, int wn, int lane) {
+  using T = F16Traits<BF16_OUT>;
+#pragma unroll
+  for (int i = 0; i < WMB; ++i) {
+    const int m = m0 + wm * 32 * WMB + i * 32 + (lane & 31);
+    if (m >= p.M) continue;
+    const float sam = p.sa[p.sa_per_row ? m : 0];
+    uint16_t* orow = p.out + (int64_t)m * p.ldc;
+#pragma unroll
+    for (int j = 0; j < WNB; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + wn * 32 * WNB + j * 32 + 8 * q + 4 * (lane >> 5);
+        if (n >= p.N) continue;
+        float sb4[4];
+        if (p.sb_per_col) {
+          const v4f t = *reinterpret_cast<const v4f*>(p.sb + n);
+          sb4[0] = t.x; sb4[1] = t.y; sb4[2] = t.z; sb4[3] = t.w;
+        } else {
+          sb4[0] = sb4[1] = sb4[2] = sb4[3] = p.sb[0];
+        }
+        float o[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = sam * (sb4[r] * acc[i][j][4 * q + r]);
+        if (p.bias) {
+          const v2u bb = *reinterpret_cast<const v2u*>(p.bias + n);
+          o[0] += T::to_float((uint16_t)(bb.x & 0xffffu));
+          o[1] += T::to_float((uint16_t)(bb.x >> 16));
+          o[2] += T::to_float((uint16_t)(bb.y & 0xffffu));
+          o[3] += T::to_float((uint16_t)(bb.y >> 16));
+        }
+        v2u ov;
+        ov.x = (uint32_t)T::from_float(o[0]) | ((uint32_t)T::from_float(o[1]) << 16);
+        ov.y = (uint32_t)T::from_float(o[2]) | ((uint32_t)T::from_float(o[3]) << 16);
+        *reinterpret_cast<v2u*>(orow + n) = ov;
+      }
+    }
+  }
+}
+
 // ----------------------------------------------------------------------------- tile kernel
 template <bool BF16_OUT, int WMB, int WNB>
 __global__ __launch_bounds__(256) void fp8_mm_tile_kernel(const Fp8MMParams p) {
@@ -139,33 +184,116 @@ __global__ __launch_bounds__(256) void fp8_mm_tile_kernel(const Fp8MMParams p) {
 #pragma unroll
       for (int i = 0; i < WMB; ++i)
 #pragma unroll
-        for (int j = 0; j < WNB; ++j) acc[i][j] = mfma_fp8_32(af[i], bf[j], acc[i][j]);
+        for (int j = 0; j < WNB; ++j) acc[i][j] = mfma_fp8_32(bf[j], af[i], acc[i][j]);   // rows = n, columns = m
     }
     __syncthreads();
   }
 
-  // epilogue: lane holds column n = lane%32, rows 8*(e/4) + 4*(lane/32) + e%4 of each 32x32 block
+  tile_epilogue<BF16_OUT, WMB, WNB>(p, acc, m0, n0, wm, wn, lane);
+}
+
+// ----------------------------------------------------------------------------- tile kernel, direct-to-LDS variant
+// Same tiling as fp8_mm_tile_kernel, but both operand tiles go global -> LDS with `buffer_load_dwordx4 ... lds`
+// (no registers, no VALU, no ds_write): each wavefront instruction moves 8 rows x 128 bytes.  The LDS tile is
+// unpadded [row][8 chunks of 16 B] with the chunk index XOR-ed by (row & 7), applied on the *global* side (the LDS
+// side of such a load is fixed: lane L writes bytes 16L..16L+15), which keeps the 16-byte operand reads of 8
+// consecutive rows on 8 different bank groups.  Rows beyond M / N fall outside the buffer descriptor and read as zero.
+// Requires K % 128 == 0 (a partial last step would read the neighbouring row instead of zeros).
+template <bool BF16_OUT, int WMB, int WNB>
+__global__ __launch_bounds__(256) void fp8_mm_tile2_kernel(const Fp8MMParams p) {
+  using T = F16Traits<BF16_OUT>;
+  constexpr int BM = 64 * WMB, BN = 64 * WNB;
+  constexpr int STAGE = (BM + BN) * 128;          // bytes per stage
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds8[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  const int total = tiles_m * tiles_n;
+  int bid = blockIdx.x;
+  if (total % 8 == 0) bid = (bid & 7) * (total / 8) + (bid >> 3);   // one contiguous band of tiles per XCD
+  const int tm = bid % tiles_m, tn = bid / tiles_m;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.a), 0, (int)((uint32_t)p.M * (uint32_t)p.lda), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.b), 0, (int)((uint32_t)p.N * (uint32_t)p.ldb), 0x00020000);
+  const int lrow = lane >> 3, lchunk = (lane & 7) ^ lrow;
+  const uint32_t voff_a = (uint32_t)lrow * (uint32_t)p.lda + (uint32_t)lchunk * 16u;
+  const uint32_t voff_b = (uint32_t)lrow * (uint32_t)p.ldb + (uint32_t)lchunk * 16u;
+
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  auto issue_loads = [&](int step, int buf) {
+    uint8_t* Ab = lds8 + (size_t)buf * STAGE;
+    uint8_t* Bb = Ab + BM * 128;
 #pragma unroll
-  for (int j = 0; j < WNB; ++j) {
-    const int n = n0 + wn * 32 * WNB + j * 32 + (lane & 31);
-    if (n >= p.N) continue;
-    const float sbn = p.sb[p.sb_per_col ? n : 0];
-    const bool hb = p.bias != nullptr;
-    const float bv = hb ? T::to_float(p.bias[n]) : 0.f;
-#pragma unroll
-    for (int i = 0; i < WMB; ++i) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int m = m0 + wm * 32 * WMB + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-        if (m < p.M) {
-          const float sam = p.sa[p.sa_per_row ? m : 0];
-          float v = sam * (sbn * acc[i][j][e]);
-          if (hb) v += bv;
-          p.out[(int64_t)m * p.ldc + n] = T::from_float(v);
-        }
-      }
+    for (int i = 0; i < BM / 32; ++i) {
+      const int r0 = wave * (BM / 4) + i * 8;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(Ab + r0 * 128), 16, (int)voff_a,
+                                               (int)((uint32_t)(m0 + r0) * (uint32_t)p.lda + (uint32_t)step * 128u), 0, 0);
     }
+#pragma unroll
+    for (int i = 0; i < BN / 32; ++i) {
+      const int r0 = wave * (BN / 4) + i * 8;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(Bb + r0 * 128), 16, (int)voff_b,
+                                               (int)((uint32_t)(n0 + r0) * (uint32_t)p.ldb + (uint32_t)step * 128u), 0, 0);
+    }
+  };
+
+  v16f acc[WMB][WNB];
+#pragma unroll
+  for (int i = 0; i < WMB; ++i)
+#pragma unroll
+    for (int j = 0; j < WNB; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // operand read offsets: row r = lane&31 of a 32-row block, 32 bytes = chunks (kk*4 + kh*2, +1), swizzled by (r & 7)
+  const int r7 = lane & 7, kh = lane >> 5;
+  uint32_t coff[2][2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) coff[kk][h] = (uint32_t)(((kk * 4 + kh * 2 + h) ^ r7) * 16);
+  const uint32_t arow = (uint32_t)((wm * 32 * WMB + (lane & 31)) * 128);
+  const uint32_t brow = (uint32_t)(BM * 128 + (wn * 32 * WNB + (lane & 31)) * 128);
+
+  const int steps = p.K / F8_BK;
+  issue_loads(0, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  for (int step = 0; step < steps; ++step) {
+    const int cur = step & 1;
+    if (step + 1 < steps) issue_loads(step + 1, cur ^ 1);
+    const uint8_t* base = lds8 + (size_t)cur * STAGE;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      v8i af[WMB], bf[WNB];
+#pragma unroll
+      for (int i = 0; i < WMB; ++i) {
+        const v4i lo = *reinterpret_cast<const v4i*>(base + arow + i * 4096 + coff[kk][0]);
+        const v4i hi = *reinterpret_cast<const v4i*>(base + arow + i * 4096 + coff[kk][1]);
+        af[i] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      }
+#pragma unroll
+      for (int j = 0; j < WNB; ++j) {
+        const v4i lo = *reinterpret_cast<const v4i*>(base + brow + j * 4096 + coff[kk][0]);
+        const v4i hi = *reinterpret_cast<const v4i*>(base + brow + j * 4096 + coff[kk][1]);
+        bf[j] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      }
+#pragma unroll
+      for (int i = 0; i < WMB; ++i)
+#pragma unroll
+        for (int j = 0; j < WNB; ++j) acc[i][j] = mfma_fp8_32(bf[j], af[i], acc[i][j]);   // rows = n, columns = m
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // next stage has landed in LDS
+    __syncthreads();
   }
+
+  tile_epilogue<BF16_OUT, WMB, WNB>(p, acc, m0, n0, wm, wn, lane);
 }
 
 // ----------------------------------------------------------------------------- stream kernel (M <= 32)
@@ -290,8 +418,39 @@ static int launch_tile(const Fp8MMParams& p, hipStream_t s) {
   return VAQ_OK;
 }
 
+template <bool BF16_OUT, int WMB, int WNB>
+static int launch_tile2(const Fp8MMParams& p, hipStream_t s) {
+  constexpr int BM = 64 * WMB, BN = 64 * WNB;
+  const size_t lds = (size_t)2 * (BM + BN) * 128;
+  auto kern = fp8_mm_tile2_kernel<BF16_OUT, WMB, WNB>;
+  static bool attr_done = false;
+  if (!attr_done) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
+        hipSuccess) {
+      set_error("fp8_scaled_mm: cannot reserve %zu bytes of LDS", lds);
+      (void)hipGetLastError();
+      return VAQ_ERR_LAUNCH;
+    }
+    attr_done = true;
+  }
+  const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(256), lds, s, p);
+  return VAQ_OK;
+}
+
+static int g_fp8_tile_impl = 0;   // 0: direct-to-LDS kernel when its preconditions hold, 1: always the register-staged kernel
+
 template <bool BF16_OUT>
 static int dispatch_tile(const Fp8MMParams& p, hipStream_t s) {
+  const bool direct_ok = g_fp8_tile_impl == 0 && p.K % F8_BK == 0 && (uint64_t)p.M * (uint64_t)p.lda < (1ull << 32) &&
+                         (uint64_t)p.N * (uint64_t)p.ldb < (1ull << 32);
+  if (direct_ok) {
+    const int cus2 = num_cus_current_device();
+    auto tiles2 = [&](int bm, int bn) { return (int64_t)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
+    if (tiles2(256, 256) >= cus2) return launch_tile2<BF16_OUT, 4, 4>(p, s);
+    if (tiles2(128, 128) >= cus2) return launch_tile2<BF16_OUT, 2, 2>(p, s);
+    return launch_tile2<BF16_OUT, 1, 2>(p, s);
+  }
   const int cus = num_cus_current_device();
   auto tiles = [&](int bm, int bn) { return (int64_t)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
   if (tiles(256, 256) >= cus) return launch_tile<BF16_OUT, 4, 4>(p, s);
@@ -357,6 +516,8 @@ extern "C" int vaq_fp8_scaled_mm(const uint8_t* a, int64_t lda, const uint8_t* b
   VAQ_CHECK_ARG(a && b && sa && sb && out, "fp8_scaled_mm: null pointer");
   VAQ_CHECK_ARG(((uintptr_t)a % 16) == 0 && ((uintptr_t)b % 16) == 0 && ((uintptr_t)out % 8) == 0,
                 "fp8_scaled_mm: a and b must be 16-byte aligned, out 8-byte aligned");
+  VAQ_CHECK_ARG(((uintptr_t)sb % 16) == 0 && (!bias || ((uintptr_t)bias % 8) == 0),
+                "fp8_scaled_mm: b_scales must be 16-byte aligned, bias 8-byte aligned");
   Fp8MMParams p;
   p.a = a; p.lda = lda; p.b = b; p.ldb = ldb;
   p.sa = sa; p.sa_per_row = (sa_count > 1 || size_m == 1) ? 1 : 0;
@@ -379,6 +540,7 @@ extern "C" int vaq_fp8_scaled_mm(const uint8_t* a, int64_t lda, const uint8_t* b
 
 // Benchmark / tuning aid, not part of the drop-in surface.  path: 0 auto, 1 stream, 2 tile; gx: stream-kernel grid.
 extern "C" void vaq_debug_set_fp8_config(int path, int gx) {
-  vaq::g_force_fp8_path = path;
+  vaq::g_force_fp8_path = path % 10;
+  vaq::g_fp8_tile_impl = path / 10;       // tens digit: 1 = force the register-staged tile kernel
   vaq::g_force_fp8_gx = gx;
 }

@@ -218,6 +218,179 @@ __global__ __launch_bounds__(256) void w4a16_prefill_kernel(const PrefillParams 
   }
 }
 
+// ----------------------------------------------------------------------------- direct-to-LDS variant
+// Same arithmetic, different plumbing:
+//  * the activation tile goes global -> LDS with `buffer_load_dwordx4 ... lds` (no registers, no VALU);
+//  * LDS tiles are unpadded [row][8 chunks of 16 B] with the chunk index XOR-ed by (row & 7) (conflict-free 16-byte
+//    accesses for the DMA layout, the dequantised-weight writes and the operand reads);
+//  * WAVES_M x WAVES_N wavefronts per workgroup (8 = two per SIMD lets one wavefront dequantise while the other one
+//    issues MFMAs);
+//  * the MFMAs take the weight fragment as A operand, so four consecutive accumulator registers are four consecutive
+//    output columns of one row: packed 8-byte stores in the epilogue;
+//  * weight words of group g+1 are requested one K step before they are needed (two register sets, by group parity).
+template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(const PrefillParams p) {
+  using T = F16Traits<BF16>;
+  constexpr int NW = WAVES_M * WAVES_N;
+  constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;
+  constexpr int WMB = TM / 32, WNB = TN / 32;
+  constexpr int W_LD = BN / (16 * NW);            // 16-byte weight loads per thread per group
+  constexpr int A_LD = BM / (8 * NW);             // direct-to-LDS instructions per wavefront per step
+  constexpr int STAGE = (BM + BN) * 128;          // bytes per stage
+  static_assert(W_LD >= 1 && A_LD >= 1, "tile too small for this many wavefronts");
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds8[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  const int total = tiles_m * tiles_n;
+  int bid = blockIdx.x;
+  if (total % 8 == 0) bid = (bid & 7) * (total / 8) + (bid >> 3);   // one contiguous band of tiles per XCD
+  const int tm = bid % tiles_m, tn = bid / tiles_m;
+  const int m0 = tm * BM, n0 = tn * BN, nt0 = n0 / 16;
+
+  // ---- activation tile: direct-to-LDS loads ----
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(p.a), 0, (int)((uint32_t)p.M * (uint32_t)p.lda * 2u), 0x00020000);
+  const int lrow = lane >> 3, lchunk = (lane & 7) ^ lrow;
+  const uint32_t voff_a = ((uint32_t)lrow * (uint32_t)p.lda) * 2u + (uint32_t)lchunk * 16u;
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  auto issue_a = [&](int step, int buf) {
+    uint8_t* Ab = lds8 + (size_t)buf * STAGE;
+#pragma unroll
+    for (int i = 0; i < A_LD; ++i) {
+      const int r0 = (wave * A_LD + i) * 8;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(Ab + r0 * 128), 16, (int)voff_a,
+                                               (int)(((uint32_t)(m0 + r0) * (uint32_t)p.lda + (uint32_t)step * 64u) * 2u), 0, 0);
+    }
+  };
+
+  // ---- weight words: two register sets (group parity) ----
+  v4u wreg[2][W_LD];
+  float ws[2][W_LD], wnz[2][W_LD];
+  const int o = lane >> 4, r = lane & 15;
+  auto load_w = [&](int g, int set) {
+#pragma unroll
+    for (int i = 0; i < W_LD; ++i) {
+      const int ntl = i * NW + wave;
+      const int nt = min(nt0 + ntl, p.NT - 1);          // clamped: columns past N are computed but never stored
+      wreg[set][i] = p.b[((int64_t)nt * p.G + g) * 64 + lane];
+      const int n = nt * 16 + r;
+      const float sv = T::to_float(p.scales[(int64_t)g * p.N + n]);
+      float z = 8.f;
+      if constexpr (HAS_ZP) {
+        const uint32_t zw = p.zeros[(int64_t)g * (p.N >> 3) + (n >> 3)];
+        z = (float)((zw >> ((n & 7) * 4)) & 0xFu);
+      }
+      ws[set][i] = sv;
+      wnz[set][i] = -(z * sv);   // exact: <= 4 + 11 significant bits
+    }
+  };
+  auto store_w = [&](int buf, int half, int set) {
+    uint8_t* Bb = lds8 + (size_t)buf * STAGE + BM * 128;
+#pragma unroll
+    for (int i = 0; i < W_LD; ++i) {
+      const int row = (i * NW + wave) * 16 + r;
+      const uint32_t w0 = half ? wreg[set][i].z : wreg[set][i].x;
+      const uint32_t w1 = half ? wreg[set][i].w : wreg[set][i].y;
+      uint8_t* rowp = Bb + row * 128;
+      *reinterpret_cast<v4u*>(rowp + ((o ^ (row & 7)) * 16)) = dequant_scaled<BF16>(w0, ws[set][i], wnz[set][i]);
+      *reinterpret_cast<v4u*>(rowp + (((4 + o) ^ (row & 7)) * 16)) = dequant_scaled<BF16>(w1, ws[set][i], wnz[set][i]);
+    }
+  };
+
+  v16f acc[WMB][WNB];
+#pragma unroll
+  for (int i = 0; i < WMB; ++i)
+#pragma unroll
+    for (int j = 0; j < WNB; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // operand reads: row = lane & 31 of a 32-row block, chunk c = kk*2 + (lane >> 5), swizzled by (row & 7) = lane & 7
+  const int r7 = lane & 7, kh = lane >> 5;
+  uint32_t coff[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) coff[kk] = (uint32_t)(((kk * 2 + kh) ^ r7) * 16);
+  const uint32_t arow = (uint32_t)((wm * TM + (lane & 31)) * 128);
+  const uint32_t brow = (uint32_t)(BM * 128 + (wn * TN + (lane & 31)) * 128);
+
+  auto compute = [&](int cur) {
+    const uint8_t* base = lds8 + (size_t)cur * STAGE;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      v4u af[WMB], bf[WNB];
+#pragma unroll
+      for (int i = 0; i < WMB; ++i) af[i] = *reinterpret_cast<const v4u*>(base + arow + i * 4096 + coff[kk]);
+#pragma unroll
+      for (int j = 0; j < WNB; ++j) bf[j] = *reinterpret_cast<const v4u*>(base + brow + j * 4096 + coff[kk]);
+#pragma unroll
+      for (int i = 0; i < WMB; ++i)
+#pragma unroll
+        for (int j = 0; j < WNB; ++j) acc[i][j] = T::mfma32(bf[j], af[i], acc[i][j]);   // rows = n, columns = m
+    }
+  };
+
+  // ---- prologue: stage step 0 (group 0, half 0) ----
+  issue_a(0, 0);
+  load_w(0, 0);
+  store_w(0, 0, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  for (int g = 0; g < p.G; ++g) {
+    const int set = g & 1;
+    // even step 2g (buffer 0): stage step 2g+1 = (g, half 1) into buffer 1; request group g+1
+    issue_a(2 * g + 1, 1);
+    if (g + 1 < p.G) load_w(g + 1, set ^ 1);
+    store_w(1, 1, set);
+    compute(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    // odd step 2g+1 (buffer 1): stage step 2g+2 = (g+1, half 0) into buffer 0
+    if (g + 1 < p.G) {
+      issue_a(2 * g + 2, 0);
+      store_w(0, 0, set ^ 1);
+    }
+    compute(1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+
+  // ---- epilogue: four consecutive accumulator registers = four consecutive n of one row ----
+#pragma unroll
+  for (int i = 0; i < WMB; ++i) {
+    const int m = m0 + wm * TM + i * 32 + (lane & 31);
+    if (m >= p.M) continue;
+    uint16_t* orow = p.c + (int64_t)m * p.N;
+#pragma unroll
+    for (int j = 0; j < WNB; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + wn * TN + j * 32 + 8 * q + 4 * (lane >> 5);
+        if (n >= p.N) continue;
+        float ov[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ov[e] = acc[i][j][4 * q + e];
+        if (p.bias) {
+          const v2u bb = *reinterpret_cast<const v2u*>(p.bias + n);
+          ov[0] += T::to_float((uint16_t)(bb.x & 0xffffu));
+          ov[1] += T::to_float((uint16_t)(bb.x >> 16));
+          ov[2] += T::to_float((uint16_t)(bb.y & 0xffffu));
+          ov[3] += T::to_float((uint16_t)(bb.y >> 16));
+        }
+        v2u pk;
+        pk.x = pack2<BF16>(ov[0], ov[1]);
+        pk.y = pack2<BF16>(ov[2], ov[3]);
+        *reinterpret_cast<v2u*>(orow + n) = pk;
+      }
+    }
+  }
+}
+
 // ----------------------------------------------------------------------------- host side
 
 template <bool BF16, int WMB, int WNB, bool HAS_ZP>
@@ -240,9 +413,34 @@ static int launch_prefill(const PrefillParams& p, hipStream_t s) {
   return VAQ_OK;
 }
 
+template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP>
+static int launch_prefill2(const PrefillParams& p, hipStream_t s) {
+  const size_t lds = (size_t)2 * (BM + BN) * 128;
+  auto kern = w4a16_prefill2_kernel<BF16, BM, BN, WAVES_M, WAVES_N, HAS_ZP>;
+  static bool attr_done = false;
+  if (!attr_done) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
+        hipSuccess) {
+      set_error("w4a16_gemm(prefill): cannot reserve %zu bytes of LDS", lds);
+      (void)hipGetLastError();
+      return VAQ_ERR_LAUNCH;
+    }
+    attr_done = true;
+  }
+  const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(WAVES_M * WAVES_N * 64), lds, s, p);
+  return VAQ_OK;
+}
+
+// tile ids: 0..2 = register-staged kernel (256x256, 128x128, 64x128); 10.. = direct-to-LDS kernel
 template <bool BF16, bool HAS_ZP>
 static int dispatch_tile(const PrefillParams& p, int tile, hipStream_t s) {
   switch (tile) {
+    case 10: return launch_prefill2<BF16, 256, 256, 2, 4, HAS_ZP>(p, s);   // 8 wavefronts, 128 x 64 each
+    case 11: return launch_prefill2<BF16, 256, 256, 2, 2, HAS_ZP>(p, s);   // 4 wavefronts, 128 x 128 each
+    case 12: return launch_prefill2<BF16, 128, 128, 2, 2, HAS_ZP>(p, s);   // 4 wavefronts, 64 x 64 each
+    case 13: return launch_prefill2<BF16, 128, 256, 2, 4, HAS_ZP>(p, s);   // 8 wavefronts, 64 x 64 each
+    case 14: return launch_prefill2<BF16, 64, 128, 2, 2, HAS_ZP>(p, s);    // 4 wavefronts, 32 x 64 each
     case 0: return launch_prefill<BF16, 4, 4, HAS_ZP>(p, s);   // 256 x 256
     case 1: return launch_prefill<BF16, 2, 2, HAS_ZP>(p, s);   // 128 x 128
     case 2: return launch_prefill<BF16, 1, 2, HAS_ZP>(p, s);   //  64 x 128
@@ -254,8 +452,17 @@ static int dispatch_tile(const PrefillParams& p, int tile, hipStream_t s) {
 
 static int g_force_tile = -1;
 
-static int pick_tile(int M, int N) {
+static int pick_tile(int M, int N, int64_t lda) {
   if (g_force_tile >= 0) return g_force_tile;
+  const bool direct_ok = (uint64_t)M * (uint64_t)lda * 2 < (1ull << 32);
+  if (direct_ok) {
+    const int cus2 = num_cus_current_device();
+    auto tiles2 = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    // measured: the 256x256 / 8-wavefront tile wins as soon as it fills ~60 % of the compute units
+    if (tiles2(256, 256) * 10 >= cus2 * 6) return 10;
+    if (tiles2(128, 128) * 2 >= cus2) return 12;
+    return 14;
+  }
   const int cus = num_cus_current_device();
   auto tiles = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   if (tiles(256, 256) >= cus) return 0;
@@ -276,7 +483,7 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
   p.M = M; p.N = N; p.K = K;
   p.G = K / 128;
   p.NT = N / 16;
-  const int tile = pick_tile(M, N);
+  const int tile = pick_tile(M, N, lda);
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
   if (bf16) rc = zp ? dispatch_tile<true, true>(p, tile, s) : dispatch_tile<true, false>(p, tile, s);
