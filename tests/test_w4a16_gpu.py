@@ -18,6 +18,17 @@ def _acts(m, k, device, dtype=torch.bfloat16, seed=0):
     return torch.randn(m, k, generator=g).to(dtype).to(device)
 
 
+@pytest.fixture(params=["auto", "lds_staged", "register_resident"])
+def decode_kernel(request):
+    """Runs a test once with the library's own choice of decode kernel and once with each of the two kernels forced, so
+    that both are checked on every shape whichever one the selection rule would pick."""
+    from vllm_amd import _lib
+    lib = _lib.load()
+    lib.vaq_debug_set_decode_impl({"auto": -1, "lds_staged": 0, "register_resident": 1}[request.param])
+    yield request.param
+    lib.vaq_debug_set_decode_impl(-1)
+
+
 # ------------------------------------------------------------------------------------------------ repack
 
 @pytest.mark.parametrize("k,n", [(128, 64), (128, 256), (1024, 256), (128 * 13, 64 * 37), (128 * 11, 64 * 13), (4096, 4096)])
@@ -50,7 +61,7 @@ SMALL = [(128, 64), (512, 256), (1024, 192), (2048, 576), (14336 // 4, 128)]
 @pytest.mark.parametrize("k,n", SMALL)
 @pytest.mark.parametrize("m", [1, 4, 16, 17, 32])
 @pytest.mark.parametrize("asym,act_order", [(False, False), (True, False), (False, True), (True, True)])
-def test_decode_gemm_small(device, k, n, m, asym, act_order):
+def test_decode_gemm_small(device, decode_kernel, k, n, m, asym, act_order):
     if act_order and k == 128:
         pytest.skip("act_order needs more than one group (gptq_marlin.cu:805)")
     case = o.make_w4a16_case(k, n, 128, asym=asym, act_order=act_order, seed=k + n + m)
@@ -76,8 +87,8 @@ def test_prefill_gemm_small(device, k, n, m, asym, act_order):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("m", [3, 16, 96])
-def test_gemm_fp16_and_bias(device, dtype, m):
+@pytest.mark.parametrize("m", [1, 3, 16, 96])
+def test_gemm_fp16_and_bias(device, decode_kernel, dtype, m):
     k, n = 1024, 256
     case = o.make_w4a16_case(k, n, 128, asym=True, dtype=dtype, seed=5)
     layer = W4A16Layer(case, device, dtype)
@@ -161,7 +172,7 @@ def test_config1_reference_cpu_case(device):
 
 
 @pytest.mark.parametrize("k,n", LLAMA_SHAPES)
-def test_config2_decode_llama_shapes(device, k, n):
+def test_config2_decode_llama_shapes(device, decode_kernel, k, n):
     case = o.make_w4a16_case(k, n, 128, seed=1)
     layer = W4A16Layer(case, device)
     w_ref = o.case_w_ref(case)

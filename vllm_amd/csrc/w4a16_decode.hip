@@ -120,21 +120,6 @@ __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodePar
     sc[u][t] = __builtin_amdgcn_raw_buffer_load_b64(rs, vo_s, (int)(os_[t] + (uint32_t)nt * 32u), 0);
     if constexpr (HAS_ZP) zq[u][t] = __builtin_amdgcn_raw_buffer_load_b32(rz, vo_z, (int)(oz[t] + (uint32_t)nt * 8u), 0);
   };
-  // The first weight tiles are requested before anything else so that their latency overlaps the activation loads.
-#pragma unroll
-  for (int u = 0; u < D; ++u) {
-#pragma unroll
-    for (int t = 0; t < TG; ++t) {
-      wq[u][t] = v4u{0u, 0u, 0u, 0u};
-      sc[u][t] = v2u{0u, 0u};
-      zq[u][t] = 0u;
-    }
-    if (nt0 + u < nt1) {
-#pragma unroll
-      for (int t = 0; t < TG; ++t) issue_load(u, nt0 + u, t);
-    }
-  }
-
   // ---- activations of this wave's K slab, as MFMA B operands (column = m, 8 consecutive k per lane) ----
   // Loaded unconditionally from clamped addresses and zeroed afterwards, so that all loads are in flight together.
   v4u breg[TG][4][MB];
@@ -173,6 +158,22 @@ __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodePar
       }
     }
   }
+  // The first weight tiles are requested right after the activation loads: loads retire in issue order as far as the
+  // wait counter is concerned, so this order lets the wait for the activations leave the weight tiles in flight.
+#pragma unroll
+  for (int u = 0; u < D; ++u) {
+#pragma unroll
+    for (int t = 0; t < TG; ++t) {
+      wq[u][t] = v4u{0u, 0u, 0u, 0u};
+      sc[u][t] = v2u{0u, 0u};
+      zq[u][t] = 0u;
+    }
+    if (nt0 + u < nt1) {
+#pragma unroll
+      for (int t = 0; t < TG; ++t) issue_load(u, nt0 + u, t);
+    }
+  }
+
   // S[t][mb] = sum of the group's activations per column m (identical in the 4 accumulator registers).  For the
   // symmetric type the whole correction -(BIAS + 8) * S is the starting value of the group's MFMA chain.
   v4f Sv[TG][MB];

@@ -1,14 +1,17 @@
 // W4A16 decode-shaped GEMM (M <= 32), barrier-free variant: activations staged in LDS, one independent task per
 // wavefront.  C[M,N] = A[M,K] . dequant(B[K,N]) (+bias), same arithmetic as w4a16_decode.hip.
 //
-//  * A workgroup is 16 wavefronts = WKS slices of K  x  WN = 16/WKS n-tiles (16 columns each).  Wavefront (wks, wn)
+//  * A workgroup is WKS slices of K  x  WN n-tiles (16 columns each) = up to 16 wavefronts.  Wavefront (wks, wn)
 //    streams the GS consecutive 1 KiB weight tiles (= quantisation groups) of its slice for its n-tile; all its tile
 //    loads are issued up front through a register ring of min(GS, 8) slots, so no wavefront ever waits for another one
 //    inside the K loop.
 //  * The activations of the workgroup's K slab (WKS*GS groups) are written once to LDS in MFMA-B-operand order
 //    ([k-octet][m] 16-byte slots, rows m >= M zero, XOR-swizzled so that both the row-contiguous fill and the
-//    operand reads are bank-conflict free) and read back with one ds_read_b128 per MFMA.  Weight loads are issued
-//    before the fill so that their latency covers it.
+//    operand reads are bank-conflict free) and read back with one ds_read_b128 per MFMA.  The activation loads are
+//    issued before the first weight loads, in branch-free code (see step 1).  Only MR rows per m-block are staged (MR = 1, 4 or 16, the
+//    smallest that holds M): MFMA columns are independent, so lanes of the columns m >= MR read the slot of row
+//    m mod MR and their results are never stored.  With few rows a whole K = 14336 slab fits LDS and K need not be
+//    split over workgroups.
 //  * Per tile: 4 x { dequantise one word to 8 biased 16-bit numbers (7 VALU ops), MFMA with the activations, MFMA of
 //    the constant operand -(BIAS + zero) with the same activations }, then acc += scale * P (fp32).  The second MFMA
 //    removes the bias and the zero point exactly as `P - (BIAS+z)*S` would, without keeping S anywhere.
@@ -16,6 +19,8 @@
 //    LDS (SK > 1 workgroups per n-tile) hand partial tiles over through device-scope write-through stores and an
 //    arrival counter, summed in fixed order by the last arriver.
 #include "vaq_common.h"
+
+#include <type_traits>
 
 namespace vaq {
 
@@ -30,7 +35,7 @@ struct Decode2Params {
   uint16_t* c;
   float* c_tmp;
   int32_t* counters;
-  int M, N, K, G, NT, SK, WKS;
+  int M, N, K, G, NT, SK, WKS, WN;
   uint32_t k_mask, k_ex;   // 0x000f000f and the exponent pattern, passed as run-time values (see and_or)
 };
 
@@ -61,16 +66,17 @@ __device__ inline __amdgpu_buffer_rsrc_t d2_rsrc(const void* base, uint64_t byte
 
 constexpr int D2_WAVES = 16;
 
-template <bool BF16, int GS, int MB, bool HAS_ZP>
+template <bool BF16, int GS, int MB, bool HAS_ZP, int MR>
 __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Decode2Params p) {
   using T = F16Traits<BF16>;
+  static_assert(MR == 16 || MB == 1, "compact row staging is for a single m-block");
   constexpr int R = GS < 8 ? GS : 8;                 // ring slots
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
   const int lane = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(threadIdx.y);
   const int o = lane >> 4, r16 = lane & 15;
-  const int WKS = p.WKS, WN = D2_WAVES / WKS;
+  const int WKS = p.WKS, WN = p.WN;
   const int wks = w / WN, wn = w - wks * WN;
   const int sk = blockIdx.y;
   const int slab_groups = WKS * GS;
@@ -80,7 +86,10 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   const int nt = nt_ok ? nt_raw : p.NT - 1;
   const int g_first = slab_g0 + wks * GS;           // this wavefront's first group
 
-  // ---- 1. request the first R weight tiles (+ scales, zero points) ----
+  // ---- 1. activations of the K slab -> LDS, with the first R weight tiles requested in between ----
+  // Loads retire in issue order as far as the wait counter is concerned, so the activation loads go out FIRST: the
+  // wait before the LDS writes then leaves the weight tiles in flight instead of draining them.
+  // slot (16 bytes) of (m-block mb, row ml, k-octet ko):  mb*KO*MR + ko*MR + (ml ^ (ko & (MR-1)))
   const __amdgpu_buffer_rsrc_t rb = d2_rsrc(p.b, (uint64_t)p.K * p.N / 2);
   const __amdgpu_buffer_rsrc_t rs = d2_rsrc(p.scales, (uint64_t)p.G * p.N * 2);
   const __amdgpu_buffer_rsrc_t rz = d2_rsrc(HAS_ZP ? (const void*)p.zeros : (const void*)p.scales, (uint64_t)p.G * (p.N / 8) * 4);
@@ -97,35 +106,69 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
     else
       zq[slot] = 0u;
   };
-#pragma unroll
-  for (int s = 0; s < R; ++s) issue_load(s, s);
 
-  // ---- 2. stage the activations of the K slab in LDS ----
-  // slot (16 bytes) of (m-block mb, row ml, k-octet ko):  mb*KO*16 + ko*16 + (ml ^ (ko & 15))
   const int KO = slab_groups * 16;                   // k-octets in the slab
+  // 16 bytes behind the activations for lanes without a chunk (the start of the reduction buffer, unused until the K
+  // loop is over, when there is one)
+  const uint32_t dummy_slot = (uint32_t)(KO * MR * MB);
   {
-    // chunk c = m * KO + ko (16 bytes: row m, k-octet ko); thread tid handles c = tid, tid + 1024, ...  The (m, ko)
+    // chunk c = m * KO + ko (16 bytes: row m, k-octet ko); thread tid handles c = tid, tid + NTHR, ...  The (m, ko)
     // pair is advanced incrementally: one scalar division per kernel instead of one vector division per chunk.
     const int tid = w * 64 + lane;
-    const int chunks = KO * 16 * MB;
+    const int chunks = KO * MR * MB;
     const int64_t k_slab0 = (int64_t)slab_g0 * 128;
-    constexpr int NTHR = D2_WAVES * 64;
+    const int NTHR = WKS * WN * 64;
     const int step_m = NTHR / KO, step_ko = NTHR - step_m * KO;     // scalar
     int m = tid / KO, ko = tid - m * KO;
-    for (int c0 = 0; c0 < chunks; c0 += NTHR * 4) {
-      v4u v[4];
-      int mm[4], kk[4];
+    if (p.perm == nullptr) {
+      // Straight-line code, no branch between the loads and the LDS writes (at a join the compiler's wait-count
+      // bookkeeping falls back to draining every load): the rows are read through a buffer descriptor that ends with
+      // the last valid element, chunks that do not exist get an out-of-range offset and come back as zeros, and
+      // their lanes write to a dummy slot.  FB chunks per thread cover a full-size slab in the first pass.
+      constexpr int FB = MR == 1 ? 2 : 8;
+      const __amdgpu_buffer_rsrc_t ra = d2_rsrc(p.a, ((uint64_t)(p.M - 1) * (uint64_t)p.lda + (uint64_t)p.K) * 2);
+      auto fill_pass = [&](auto first) {
+        v4u v[FB];
+        uint32_t slot[FB];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        mm[i] = m;
-        kk[i] = ko;
-        const int64_t k = k_slab0 + (int64_t)ko * 8;
-        v[i] = v4u{0u, 0u, 0u, 0u};
-        if (m < 16 * MB && m < p.M && k < p.K) {
-          const uint16_t* row = p.a + (int64_t)m * p.lda;
-          if (p.perm == nullptr) {
-            v[i] = *reinterpret_cast<const v4u*>(row + k);
-          } else {
+        for (int i = 0; i < FB; ++i) {
+          const int64_t k = k_slab0 + (int64_t)ko * 8;
+          const bool ok = m < MR * MB && m < p.M && k < p.K;
+          const uint32_t off = ok ? (uint32_t)(((int64_t)m * p.lda + k) * 2) : 0x80000000u;
+          v[i] = __builtin_amdgcn_raw_buffer_load_b128(ra, (int)off, 0, 0);
+          const int mb = m / MR, ml = m % MR;
+          slot[i] = m < MR * MB ? (uint32_t)(mb * KO * MR + ko * MR + (ml ^ (ko & (MR - 1)))) : dummy_slot;
+          m += step_m;
+          ko += step_ko;
+          if (ko >= KO) {
+            ko -= KO;
+            m += 1;
+          }
+        }
+        if constexpr (decltype(first)::value) {
+#pragma unroll
+          for (int s = 0; s < R; ++s) issue_load(s, s);
+        }
+#pragma unroll
+        for (int i = 0; i < FB; ++i) *reinterpret_cast<v4u*>(lds + (size_t)slot[i] * 16) = v[i];
+      };
+      fill_pass(std::true_type{});
+      for (int c0 = NTHR * FB; c0 < chunks; c0 += NTHR * FB) fill_pass(std::false_type{});
+    } else {
+      // act_order: the columns of A are gathered through `perm`; two dependent levels of loads, weights requested first
+#pragma unroll
+      for (int s = 0; s < R; ++s) issue_load(s, s);
+      for (int c0 = 0; c0 < chunks; c0 += NTHR * 4) {
+        v4u v[4];
+        int mm[4], kk[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          mm[i] = m;
+          kk[i] = ko;
+          const int64_t k = k_slab0 + (int64_t)ko * 8;
+          v[i] = v4u{0u, 0u, 0u, 0u};
+          if (m < MR * MB && m < p.M && k < p.K) {
+            const uint16_t* row = p.a + (int64_t)m * p.lda;
             const v4i p0 = *reinterpret_cast<const v4i*>(p.perm + k);
             const v4i p1 = *reinterpret_cast<const v4i*>(p.perm + k + 4);
             v[i].x = (uint32_t)row[p0.x] | ((uint32_t)row[p0.y] << 16);
@@ -133,20 +176,20 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
             v[i].z = (uint32_t)row[p1.x] | ((uint32_t)row[p1.y] << 16);
             v[i].w = (uint32_t)row[p1.z] | ((uint32_t)row[p1.w] << 16);
           }
+          m += step_m;
+          ko += step_ko;
+          if (ko >= KO) {
+            ko -= KO;
+            m += 1;
+          }
         }
-        m += step_m;
-        ko += step_ko;
-        if (ko >= KO) {
-          ko -= KO;
-          m += 1;
-        }
-      }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (mm[i] < 16 * MB) {
-          const int mb = mm[i] >> 4, ml = mm[i] & 15;
-          const int slot = mb * KO * 16 + kk[i] * 16 + (ml ^ (kk[i] & 15));
-          *reinterpret_cast<v4u*>(lds + (size_t)slot * 16) = v[i];
+        for (int i = 0; i < 4; ++i) {
+          if (mm[i] < MR * MB) {
+            const int mb = mm[i] / MR, ml = mm[i] % MR;
+            const int slot = mb * KO * MR + kk[i] * MR + (ml ^ (kk[i] & (MR - 1)));
+            *reinterpret_cast<v4u*>(lds + (size_t)slot * 16) = v[i];
+          }
         }
       }
     }
@@ -159,7 +202,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
 #pragma unroll
   for (int jj = 0; jj < 4; ++jj) {
     const int kol = jj * 4 + o;
-    abase[jj] = (uint32_t)(((wks * GS * 16 + kol) * 16 + (r16 ^ kol)) * 16);
+    abase[jj] = (uint32_t)(((wks * GS * 16 + kol) * MR + ((r16 ^ kol) & (MR - 1))) * 16);
   }
   uint32_t ex;     // kept in a vector register so that (x & MSK) | ex is a legal single VOP3 instruction (one scalar operand)
   asm volatile("v_mov_b32 %0, %1" : "=v"(ex) : "s"(p.k_ex));
@@ -195,7 +238,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
       aop.w = d2_and_or(wj[jj] >> 12, MSK, ex);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        const v4u bop = *reinterpret_cast<const v4u*>(lds + abase[jj] + (uint32_t)(mb * KO * 256) + (uint32_t)(gi * 4096));
+        const v4u bop = *reinterpret_cast<const v4u*>(lds + abase[jj] + (uint32_t)(mb * KO * MR * 16) + (uint32_t)(gi * 256 * MR));
         P[mb] = T::mfma16(aop, bop, P[mb]);
         P[mb] = T::mfma16(zop, bop, P[mb]);
       }
@@ -219,7 +262,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   }
 
   // ---- 4. reduce the K slices of the workgroup ----
-  v4f* red = reinterpret_cast<v4f*>(lds + (size_t)KO * 16 * MB * 16);     // [16 waves][MB][64]
+  v4f* red = reinterpret_cast<v4f*>(lds + (size_t)KO * MR * MB * 16);     // [16 waves][MB][64]
   if (WKS > 1) {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) red[(w * MB + mb) * 64 + lane] = acc[mb];
@@ -275,10 +318,10 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
 // ----------------------------------------------------------------------------- host side
 
 struct Decode2Config {
-  int gs, wks, sk;
+  int gs, wks, wn, sk, mr;
 };
 
-static int g2_force_gs = 0, g2_force_wks = 0;
+static int g2_force_gs = 0, g2_force_wks = 0, g2_force_wn = 0;
 
 static int round_gs(int x) {
   const int opts[] = {1, 2, 4, 7, 8, 14, 16};
@@ -287,16 +330,19 @@ static int round_gs(int x) {
   return 16;
 }
 
-// Groups per slab are limited by LDS (128 KiB of activations): 32 groups for one m-block, 16 for two.
+// Groups per slab are limited by LDS (128 KiB of activations, 256 bytes per group and staged row): 512 / rows.
 static Decode2Config pick_decode2_config(int M, int N, int K) {
   const int G = K / 128, NT = N / 16;
   const int MB = M <= 16 ? 1 : 2;
-  const int slab_max = MB == 1 ? 32 : 16;
   Decode2Config c;
+  c.mr = M == 1 ? 1 : (M <= 4 ? 4 : 16);
+  const int slab_max = 512 / (c.mr * MB);
   c.sk = (G + slab_max - 1) / slab_max;
   const int gslab = (G + c.sk - 1) / c.sk;            // groups per slab
   const int cus = num_cus_current_device();
-  int want = (cus * D2_WAVES) / (NT * c.sk);          // K slices wanted so that NT*SK*WKS ~ one workgroup per CU
+  // K slices wanted: about 16 wavefronts per compute unit, 8 when few rows are staged (measured: with little LDS to
+  // fill, longer per-wavefront tile streams beat more wavefronts)
+  int want = (cus * (c.mr <= 4 ? 8 : D2_WAVES)) / (NT * c.sk);
   int wks = 1;
   while (wks * 2 <= want && wks < 16) wks *= 2;
   while (wks > 1 && wks > gslab) wks /= 2;
@@ -308,14 +354,37 @@ static Decode2Config pick_decode2_config(int M, int N, int K) {
   c.sk = (G + wks * gs - 1) / (wks * gs);
   c.gs = gs;
   c.wks = wks;
+  // n-tiles per workgroup (at most 16 / wks).  A compute unit holds 16 of these wavefronts and as many workgroups as
+  // its LDS allows.  First the fewest rounds of workgroups per compute unit, then the fewest wavefronts on the busiest
+  // compute unit (i.e. spread over the device), then the smaller workgroup.
+  int best_wn = 1;
+  long best_rounds = -1, best_waves = -1;
+  const size_t lds_wg = (size_t)wks * gs * 256 * c.mr * MB + (wks > 1 ? (size_t)D2_WAVES * MB * 1024 : 16);
+  for (int wn = 1; wn <= D2_WAVES / wks; ++wn) {
+    long slots = D2_WAVES / (wks * wn);
+    const long lds_slots = (long)((size_t)(160 * 1024) / lds_wg);
+    if (slots > lds_slots) slots = lds_slots;
+    if (slots < 1) slots = 1;
+    const long wgs = (long)((NT + wn - 1) / wn) * c.sk;
+    const long per_cu = (wgs + cus - 1) / cus;
+    const long rounds = (per_cu + slots - 1) / slots;
+    const long waves = (per_cu < slots ? per_cu : slots) * wn * wks;
+    if (best_rounds < 0 || rounds < best_rounds || (rounds == best_rounds && waves < best_waves)) {
+      best_rounds = rounds;
+      best_waves = waves;
+      best_wn = wn;
+    }
+  }
+  c.wn = g2_force_wn > 0 ? g2_force_wn : best_wn;
+  if (c.wn * wks > D2_WAVES) c.wn = D2_WAVES / wks;
   return c;
 }
 
-template <bool BF16, int GS, int MB, bool HAS_ZP>
+template <bool BF16, int GS, int MB, bool HAS_ZP, int MR>
 static int launch_decode2(const Decode2Params& p, hipStream_t s) {
-  const int WN = D2_WAVES / p.WKS;
-  const size_t lds = (size_t)p.WKS * GS * 4096 * MB + (p.WKS > 1 ? (size_t)D2_WAVES * MB * 1024 : 0);
-  auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP>;
+  const int WN = p.WN;
+  const size_t lds = (size_t)p.WKS * GS * 256 * MR * MB + (p.WKS > 1 ? (size_t)D2_WAVES * MB * 1024 : 16);
+  auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP, MR>;
   static size_t attr_lds = 0;
   if (lds > attr_lds) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
@@ -327,24 +396,39 @@ static int launch_decode2(const Decode2Params& p, hipStream_t s) {
     attr_lds = lds;
   }
   const int gx = (p.NT + WN - 1) / WN;
-  hipLaunchKernelGGL(kern, dim3(gx, p.SK), dim3(64, D2_WAVES), lds, s, p);
+  hipLaunchKernelGGL(kern, dim3(gx, p.SK), dim3(64, p.WKS * WN), lds, s, p);
   return VAQ_OK;
 }
 
-template <bool BF16, int MB, bool HAS_ZP>
+template <bool BF16, int MB, bool HAS_ZP, int MR>
 static int dispatch_gs2(const Decode2Params& p, int gs, hipStream_t s) {
   switch (gs) {
-    case 1: return launch_decode2<BF16, 1, MB, HAS_ZP>(p, s);
-    case 2: return launch_decode2<BF16, 2, MB, HAS_ZP>(p, s);
-    case 4: return launch_decode2<BF16, 4, MB, HAS_ZP>(p, s);
-    case 7: return launch_decode2<BF16, 7, MB, HAS_ZP>(p, s);
-    case 8: return launch_decode2<BF16, 8, MB, HAS_ZP>(p, s);
-    case 14: return launch_decode2<BF16, 14, MB, HAS_ZP>(p, s);
-    case 16: return launch_decode2<BF16, 16, MB, HAS_ZP>(p, s);
+    case 1: return launch_decode2<BF16, 1, MB, HAS_ZP, MR>(p, s);
+    case 2: return launch_decode2<BF16, 2, MB, HAS_ZP, MR>(p, s);
+    case 4: return launch_decode2<BF16, 4, MB, HAS_ZP, MR>(p, s);
+    case 7: return launch_decode2<BF16, 7, MB, HAS_ZP, MR>(p, s);
+    case 8: return launch_decode2<BF16, 8, MB, HAS_ZP, MR>(p, s);
+    case 14: return launch_decode2<BF16, 14, MB, HAS_ZP, MR>(p, s);
+    case 16: return launch_decode2<BF16, 16, MB, HAS_ZP, MR>(p, s);
     default: break;
   }
   set_error("w4a16_gemm(decode): unsupported groups per wavefront %d", gs);
   return VAQ_ERR_UNSUPPORTED;
+}
+
+template <int MB, int MR>
+static int dispatch_types2(const Decode2Params& p, int gs, bool bf16, bool zp, hipStream_t s) {
+  if (bf16) return zp ? dispatch_gs2<true, MB, true, MR>(p, gs, s) : dispatch_gs2<true, MB, false, MR>(p, gs, s);
+  return zp ? dispatch_gs2<false, MB, true, MR>(p, gs, s) : dispatch_gs2<false, MB, false, MR>(p, gs, s);
+}
+
+template <int MB>
+static int dispatch_mr2(const Decode2Params& p, const Decode2Config& c, bool bf16, bool zp, hipStream_t s) {
+  switch (c.mr) {
+    case 1: return dispatch_types2<MB, 1>(p, c.gs, bf16, zp, s);
+    case 4: return dispatch_types2<MB, 4>(p, c.gs, bf16, zp, s);
+    default: return dispatch_types2<MB, 16>(p, c.gs, bf16, zp, s);
+  }
 }
 
 int w4a16_decode2_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* counter_ints) {
@@ -378,6 +462,7 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
   const Decode2Config cfg = pick_decode2_config(M, N, K);
   p.SK = cfg.sk;
   p.WKS = cfg.wks;
+  p.WN = cfg.wn;
   const int MB = M <= 16 ? 1 : 2;
   if (cfg.sk > 1) {
     VAQ_CHECK_ARG(c_tmp != nullptr && counters != nullptr, "w4a16_gemm: split-K needs c_tmp and counters");
@@ -387,13 +472,8 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
   }
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
-  if (MB == 1) {
-    if (bf16) rc = zp ? dispatch_gs2<true, 1, true>(p, cfg.gs, s) : dispatch_gs2<true, 1, false>(p, cfg.gs, s);
-    else rc = zp ? dispatch_gs2<false, 1, true>(p, cfg.gs, s) : dispatch_gs2<false, 1, false>(p, cfg.gs, s);
-  } else {
-    if (bf16) rc = zp ? dispatch_gs2<true, 2, true>(p, cfg.gs, s) : dispatch_gs2<true, 2, false>(p, cfg.gs, s);
-    else rc = zp ? dispatch_gs2<false, 2, true>(p, cfg.gs, s) : dispatch_gs2<false, 2, false>(p, cfg.gs, s);
-  }
+  if (MB == 1) rc = dispatch_mr2<1>(p, cfg, bf16, zp, s);
+  else rc = dispatch_types2<2, 16>(p, cfg.gs, bf16, zp, s);
   if (rc != VAQ_OK) return rc;
   VAQ_CHECK_LAUNCH("w4a16_gemm(decode)");
   return VAQ_OK;
@@ -404,5 +484,6 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
 // Benchmark / tuning aid, not part of the drop-in surface (0 = automatic).  Process-global, not thread-safe.
 extern "C" void vaq_debug_set_decode2_config(int gs, int wks) {
   vaq::g2_force_gs = gs;
-  vaq::g2_force_wks = wks;
+  vaq::g2_force_wks = wks % 100;      // wks + 100 * (n-tiles per workgroup)
+  vaq::g2_force_wn = wks / 100;
 }

@@ -16,12 +16,15 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
 constexpr int64_t DECODE_MAX_M = 32;
 static int g_decode_impl = -1;  // -1: automatic, 0: LDS-staged activations (w4a16_decode2.hip), 1: register-resident (w4a16_decode.hip)
 
-// Measured on MI355X (Llama-3-8B shapes): keeping the activations in registers wins while they are few (M <= 8:
-// each workgroup pulls M*K*2 bytes of A) and for wide layers; staging them once per workgroup in LDS wins for
-// M > 8 on layers with few n-tiles, where A traffic per compute unit dominates.
-static int decode_impl_for(int64_t size_m, int64_t size_n) {
+// Measured on MI355X (Llama-3-8B shapes): staging the activations once per workgroup in LDS (one independent task
+// per wavefront, no barrier in the K loop) wins on layers with few n-tiles per compute unit at every M; on wide layers
+// (many n-tiles per compute unit) the register-resident kernel, whose wavefronts walk over n-tiles with their slice of
+// the activations held in registers, is ahead.
+static int decode_impl_for(int64_t size_m, int64_t size_n, int64_t lda) {
+  // the LDS-staged kernel addresses A through a 32-bit buffer offset
+  if (size_m * lda * 2 >= (1ll << 31)) return 1;
   if (g_decode_impl >= 0) return g_decode_impl;
-  return (size_m > 8 && size_n <= 8192) ? 0 : 1;
+  return size_n <= 8192 ? 0 : 1;
 }
 
 static int check_shape(int64_t size_m, int64_t size_n, int64_t size_k) {
@@ -48,9 +51,17 @@ extern "C" int vaq_w4a16_gemm_workspace(int64_t size_m, int64_t size_n, int64_t 
   *a_tmp_bytes = 0;
   *counter_ints = 0;
   if (size_m == 0) return VAQ_OK;
-  if (size_m <= DECODE_MAX_M)
-    return decode_impl_for(size_m, size_n) == 0 ? w4a16_decode2_workspace((int)size_m, (int)size_n, (int)size_k, c_tmp_bytes, counter_ints)
-                              : w4a16_decode_workspace((int)size_m, (int)size_n, (int)size_k, c_tmp_bytes, counter_ints);
+  if (size_m <= DECODE_MAX_M) {
+    // enough for either decode kernel: which one runs also depends on the row stride of A, unknown here
+    size_t t1 = 0, n1 = 0, t2 = 0, n2 = 0;
+    rc = w4a16_decode_workspace((int)size_m, (int)size_n, (int)size_k, &t1, &n1);
+    if (rc != VAQ_OK) return rc;
+    rc = w4a16_decode2_workspace((int)size_m, (int)size_n, (int)size_k, &t2, &n2);
+    if (rc != VAQ_OK) return rc;
+    *c_tmp_bytes = t1 > t2 ? t1 : t2;
+    *counter_ints = n1 > n2 ? n1 : n2;
+    return VAQ_OK;
+  }
   if (has_perm) *a_tmp_bytes = (size_t)size_m * (size_t)size_k * 2;
   return VAQ_OK;
 }
@@ -88,7 +99,7 @@ extern "C" int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, cons
   } else if (force_path == 2) {
     decode = false;
   }
-  if (decode && decode_impl_for(size_m, size_n) == 0)
+  if (decode && decode_impl_for(size_m, size_n, lda) == 0)
     return w4a16_decode2_launch(a, lda, b, scales, zeros, perm, bias, c, c_tmp, counters, counter_ints, (int)size_m,
                                 (int)size_n, (int)size_k, dtype, s);
   if (decode)
