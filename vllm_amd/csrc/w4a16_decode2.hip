@@ -2,16 +2,15 @@
 // wavefront.  C[M,N] = A[M,K] . dequant(B[K,N]) (+bias), same arithmetic as w4a16_decode.hip.
 //
 //  * A workgroup is WKS slices of K  x  WN n-tiles (16 columns each) = up to 16 wavefronts.  Wavefront (wks, wn)
-//    streams the GS consecutive 1 KiB weight tiles (= quantisation groups) of its slice for its n-tile; all its tile
-//    loads are issued up front through a register ring of min(GS, 8) slots, so no wavefront ever waits for another one
-//    inside the K loop.
+//    streams the GS consecutive 1 KiB weight tiles (= quantisation groups) of its slice for its n-tile through a
+//    register ring of min(GS, 2) slots; no wavefront ever waits for another one inside the K loop.
 //  * The activations of the workgroup's K slab (WKS*GS groups) are written once to LDS in MFMA-B-operand order
 //    ([k-octet][m] 16-byte slots, rows m >= M zero, XOR-swizzled so that both the row-contiguous fill and the
 //    operand reads are bank-conflict free) and read back with one ds_read_b128 per MFMA.  The activation loads are
-//    issued before the first weight loads, in branch-free code (see step 1).  Only MR rows per m-block are staged (MR = 1, 4 or 16, the
-//    smallest that holds M): MFMA columns are independent, so lanes of the columns m >= MR read the slot of row
-//    m mod MR and their results are never stored.  With few rows a whole K = 14336 slab fits LDS and K need not be
-//    split over workgroups.
+//    issued before the first weight loads, in branch-free code (see step 1).  Only MR rows per m-block are staged
+//    (MR = 1, 4 or 16, the smallest that holds M): MFMA columns are independent, so lanes of the columns m >= MR read
+//    the slot of row m mod MR and their results are never stored.  With few rows a whole K = 14336 slab fits LDS and
+//    K need not be split over workgroups.
 //  * Per tile: 4 x { dequantise one word to 8 biased 16-bit numbers (7 VALU ops), MFMA with the activations, MFMA of
 //    the constant operand -(BIAS + zero) with the same activations }, then acc += scale * P (fp32).  The second MFMA
 //    removes the bias and the zero point exactly as `P - (BIAS+z)*S` would, without keeping S anywhere.
@@ -70,7 +69,11 @@ template <bool BF16, int GS, int MB, bool HAS_ZP, int MR>
 __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Decode2Params p) {
   using T = F16Traits<BF16>;
   static_assert(MR == 16 || MB == 1, "compact row staging is for a single m-block");
-  constexpr int R = GS < 8 ? GS : 8;                 // ring slots
+  // Ring slots.  Two tiles in flight per wavefront measured best: a wavefront does not get past its load instructions
+  // until the memory pipeline has accepted them, and with deeper rings (every wavefront of the device asking for
+  // 7-8 KiB at once) the first MFMA of each wavefront starts when most of the stream has already been served, so the
+  // arithmetic no longer overlaps it.
+  constexpr int R = GS < 2 ? GS : 2;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
   const int lane = threadIdx.x;
@@ -212,13 +215,12 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) acc[mb] = v4f{0.f, 0.f, 0.f, 0.f};
 
-#pragma unroll
-  for (int gi = 0; gi < GS; ++gi) {
-    const int slot = gi % R;
+  // One tile: `slot` is a compile-time constant wherever this is expanded; `reissue` refills the slot R tiles ahead.
+  auto do_tile = [&](int gi, int slot, bool reissue) {
     const uint32_t wj[4] = {wq[slot].x, wq[slot].y, wq[slot].z, wq[slot].w};
     const v2u sct = sc[slot];
     const uint32_t zqt = zq[slot];
-    if (gi + R < GS) issue_load(slot, gi + R);
+    if (reissue) issue_load(slot, gi + R);
 
     uint32_t zbits;
     if constexpr (HAS_ZP) zbits = NEG_BIAS_BITS | ((zqt >> ((r16 & 7) * 4)) & 0xFu);
@@ -259,6 +261,22 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int r = 0; r < 4; ++r) acc[mb][r] = fmaf(s[r], P[mb][r], acc[mb][r]);
+  };
+  if constexpr (GS <= 4) {
+#pragma unroll
+    for (int gi = 0; gi < GS; ++gi) do_tile(gi, gi % R, gi + R < GS);
+  } else {
+    // Long streams run as a rolled loop of R tiles per trip (short code: these kernels alternate with others and
+    // start with a cold instruction cache).  Every trip of the loop refills its slots unconditionally -- a branch
+    // around a load would make the compiler's wait counts drain the ring -- and the last tiles are peeled.
+    constexpr int MAIN = ((GS - R) / R) * R;      // tiles consumed inside the loop
+#pragma unroll 1
+    for (int g0 = 0; g0 < MAIN; g0 += R) {
+#pragma unroll
+      for (int u = 0; u < R; ++u) do_tile(g0 + u, u, true);
+    }
+#pragma unroll
+    for (int gi = MAIN; gi < GS; ++gi) do_tile(gi, gi % R, gi + R < GS);
   }
 
   // ---- 4. reduce the K slices of the workgroup ----
@@ -341,8 +359,8 @@ static Decode2Config pick_decode2_config(int M, int N, int K) {
   const int gslab = (G + c.sk - 1) / c.sk;            // groups per slab
   const int cus = num_cus_current_device();
   // K slices wanted: about 16 wavefronts per compute unit, 8 when few rows are staged (measured: with little LDS to
-  // fill, longer per-wavefront tile streams beat more wavefronts)
-  int want = (cus * (c.mr <= 4 ? 8 : D2_WAVES)) / (NT * c.sk);
+  // fill, longer per-wavefront tile streams beat more wavefronts on layers with few n-tiles)
+  int want = (cus * (c.mr <= 4 && NT <= 2 * cus ? 8 : D2_WAVES)) / (NT * c.sk);
   int wks = 1;
   while (wks * 2 <= want && wks < 16) wks *= 2;
   while (wks > 1 && wks > gslab) wks /= 2;

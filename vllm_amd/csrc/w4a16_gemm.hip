@@ -17,14 +17,14 @@ constexpr int64_t DECODE_MAX_M = 32;
 static int g_decode_impl = -1;  // -1: automatic, 0: LDS-staged activations (w4a16_decode2.hip), 1: register-resident (w4a16_decode.hip)
 
 // Measured on MI355X (Llama-3-8B shapes): staging the activations once per workgroup in LDS (one independent task
-// per wavefront, no barrier in the K loop) wins on layers with few n-tiles per compute unit at every M; on wide layers
-// (many n-tiles per compute unit) the register-resident kernel, whose wavefronts walk over n-tiles with their slice of
-// the activations held in registers, is ahead.
+// per wavefront, no barrier in the K loop) wins everywhere except for M > 2 on wide layers (many n-tiles per compute
+// unit), where the register-resident kernel, whose wavefronts walk over n-tiles with their slice of the activations
+// held in registers, is slightly ahead.
 static int decode_impl_for(int64_t size_m, int64_t size_n, int64_t lda) {
   // the LDS-staged kernel addresses A through a 32-bit buffer offset
   if (size_m * lda * 2 >= (1ll << 31)) return 1;
   if (g_decode_impl >= 0) return g_decode_impl;
-  return size_n <= 8192 ? 0 : 1;
+  return (size_n <= 8192 || size_m <= 2) ? 0 : 1;
 }
 
 static int check_shape(int64_t size_m, int64_t size_n, int64_t size_k) {
