@@ -16,6 +16,8 @@
 //  * act_order: the caller passes activations already gathered through `perm` (vaq_permute_cols).
 #include "vaq_common.h"
 
+#include <type_traits>
+
 namespace vaq {
 
 struct PrefillParams {
@@ -62,6 +64,16 @@ __device__ inline v4u dequant_scaled(uint32_t w, float s, float neg_zs) {
   r.z = pack2<BF16>(e4, e5);
   r.w = pack2<BF16>(e6, e7);
   return r;
+}
+
+// Quarter t of dequant_scaled: register t of its result (elements 2t and 2t+1).
+template <bool BF16>
+__device__ inline uint32_t dequant_part(uint32_t w, float s, float neg_zs, int t) {
+  const uint32_t x = ((t & 1) ? (w >> 4) : w) & 0x0f0f0f0fu;
+  const int sh = (t >> 1) * 8;
+  const float lo = fmaf((float)((x >> sh) & 0xffu), s, neg_zs);
+  const float hi = fmaf((float)((x >> (sh + 16)) & 0xffu), s, neg_zs);
+  return pack2<BF16>(lo, hi);
 }
 
 template <bool BF16, int WMB, int WNB, bool HAS_ZP>
@@ -221,8 +233,10 @@ __global__ __launch_bounds__(256) void w4a16_prefill_kernel(const PrefillParams 
 // ----------------------------------------------------------------------------- direct-to-LDS variant
 // Same arithmetic, different plumbing:
 //  * the activation tile goes global -> LDS with `buffer_load_dwordx4 ... lds` (no registers, no VALU);
-//  * LDS tiles are unpadded [row][8 chunks of 16 B] with the chunk index XOR-ed by (row & 7) (conflict-free 16-byte
-//    accesses for the DMA layout, the dequantised-weight writes and the operand reads);
+//  * LDS tiles are unpadded: a pair of 128-byte rows is one 256-byte line of 16 chunks (16 B each, chunk index
+//    (row & 1) * 8 + c), and the chunk index is XOR-ed with (row >> 1) & 15.  The LDS of this architecture has 64 banks
+//    (256 bytes per cycle): 16 lanes that touch 16 consecutive rows at the same k chunk -- the operand reads and the
+//    dequantised-weight writes -- then hit 16 different 16-byte bank groups, and so do the 16 lanes of a DMA line;
 //  * WAVES_M x WAVES_N wavefronts per workgroup (8 = two per SIMD lets one wavefront dequantise while the other one
 //    issues MFMAs);
 //  * the MFMAs take the weight fragment as A operand, so four consecutive accumulator registers are four consecutive
@@ -236,7 +250,9 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
   constexpr int WMB = TM / 32, WNB = TN / 32;
   constexpr int W_LD = BN / (16 * NW);            // 16-byte weight loads per thread per group
   constexpr int A_LD = BM / (8 * NW);             // direct-to-LDS instructions per wavefront per step
-  constexpr int STAGE = (BM + BN) * 128;          // bytes per stage
+  constexpr int A_ST = BM * 128, W_ST = BN * 128; // bytes per activation / weight stage
+  constexpr int W_BASE = 3 * A_ST;                // three activation stages, then two weight stages
+  constexpr int KW = W_LD * (HAS_ZP ? 3 : 2);     // vector-memory instructions of one load_w
   static_assert(W_LD >= 1 && A_LD >= 1, "tile too small for this many wavefronts");
   extern __shared__ __attribute__((aligned(16))) uint8_t lds8[];
 
@@ -255,29 +271,40 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
   // ---- activation tile: direct-to-LDS loads ----
   const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint16_t*>(p.a), 0, (int)((uint32_t)p.M * (uint32_t)p.lda * 2u), 0x00020000);
-  const int lrow = lane >> 3, lchunk = (lane & 7) ^ lrow;
-  const uint32_t voff_a = ((uint32_t)lrow * (uint32_t)p.lda) * 2u + (uint32_t)lchunk * 16u;
+  // DMA instruction i of this wavefront fills rows r0 .. r0+7 (r0 = (wave*A_LD + i) * 8): lane l lands in LDS slot
+  // r0*8 + l, i.e. row pair j = r0/2 + (l >> 4), swizzled chunk l & 15; it must therefore fetch the element that
+  // belongs there: c16 = (l & 15) ^ (j & 15), row = 2j + (c16 >> 3), chunk = c16 & 7.
+  uint32_t voff_a[A_LD];
+#pragma unroll
+  for (int i = 0; i < A_LD; ++i) {
+    const int j = (wave * A_LD + i) * 4 + (lane >> 4);
+    const int c16 = (lane & 15) ^ (j & 15);
+    const int lrow = 2 * (lane >> 4) + (c16 >> 3);
+    voff_a[i] = ((uint32_t)lrow * (uint32_t)p.lda) * 2u + (uint32_t)(c16 & 7) * 16u;
+  }
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
   auto issue_a = [&](int step, int buf) {
-    uint8_t* Ab = lds8 + (size_t)buf * STAGE;
+    uint8_t* Ab = lds8 + (size_t)buf * A_ST;
 #pragma unroll
     for (int i = 0; i < A_LD; ++i) {
       const int r0 = (wave * A_LD + i) * 8;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(Ab + r0 * 128), 16, (int)voff_a,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(Ab + r0 * 128), 16, (int)voff_a[i],
                                                (int)(((uint32_t)(m0 + r0) * (uint32_t)p.lda + (uint32_t)step * 64u) * 2u), 0, 0);
     }
   };
 
-  // ---- weight words: two register sets (group parity) ----
-  v4u wreg[2][W_LD];
-  float ws[2][W_LD], wnz[2][W_LD];
+  // ---- weight words: the group being dequantised (cur) and the next one in flight (nxt).  Two named sets with a
+  // register copy per group, not one array indexed by the group's parity: a run-time index into a register array turns
+  // every access into a select chain, and the loads would have to be waited for as soon as they are issued. ----
+  v4u wcur[W_LD], wnxt[W_LD];
+  float scur[W_LD], zcur[W_LD], snxt[W_LD], znxt[W_LD];      // scale and -(zero * scale)
   const int o = lane >> 4, r = lane & 15;
-  auto load_w = [&](int g, int set) {
+  auto load_w = [&](int g) {
 #pragma unroll
     for (int i = 0; i < W_LD; ++i) {
       const int ntl = i * NW + wave;
       const int nt = min(nt0 + ntl, p.NT - 1);          // clamped: columns past N are computed but never stored
-      wreg[set][i] = p.b[((int64_t)nt * p.G + g) * 64 + lane];
+      wnxt[i] = p.b[((int64_t)nt * p.G + g) * 64 + lane];
       const int n = nt * 16 + r;
       const float sv = T::to_float(p.scales[(int64_t)g * p.N + n]);
       float z = 8.f;
@@ -285,21 +312,35 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
         const uint32_t zw = p.zeros[(int64_t)g * (p.N >> 3) + (n >> 3)];
         z = (float)((zw >> ((n & 7) * 4)) & 0xFu);
       }
-      ws[set][i] = sv;
-      wnz[set][i] = -(z * sv);   // exact: <= 4 + 11 significant bits
+      snxt[i] = sv;
+      znxt[i] = -(z * sv);   // exact: <= 4 + 11 significant bits
     }
   };
-  auto store_w = [&](int buf, int half, int set) {
-    uint8_t* Bb = lds8 + (size_t)buf * STAGE + BM * 128;
+  auto advance_w = [&]() {
 #pragma unroll
     for (int i = 0; i < W_LD; ++i) {
-      const int row = (i * NW + wave) * 16 + r;
-      const uint32_t w0 = half ? wreg[set][i].z : wreg[set][i].x;
-      const uint32_t w1 = half ? wreg[set][i].w : wreg[set][i].y;
-      uint8_t* rowp = Bb + row * 128;
-      *reinterpret_cast<v4u*>(rowp + ((o ^ (row & 7)) * 16)) = dequant_scaled<BF16>(w0, ws[set][i], wnz[set][i]);
-      *reinterpret_cast<v4u*>(rowp + (((4 + o) ^ (row & 7)) * 16)) = dequant_scaled<BF16>(w1, ws[set][i], wnz[set][i]);
+      wcur[i] = wnxt[i];
+      scur[i] = snxt[i];
+      zcur[i] = znxt[i];
     }
+  };
+  // Prologue only: dequantise half 0 of the current group into weight stage 0.
+  auto store_w0 = [&]() {
+    uint8_t* Bb = lds8 + W_BASE;
+#pragma unroll
+    for (int pc = 0; pc < 2 * W_LD; ++pc) {
+      const int i = pc >> 1, which = pc & 1;
+      const int row = (i * NW + wave) * 16 + r;
+      const uint32_t wsel = which ? wcur[i].y : wcur[i].x;
+      const int c0 = (row & 1) * 8 + o + which * 4, sw = (row >> 1) & 15;
+      *reinterpret_cast<v4u*>(Bb + (row >> 1) * 256 + ((c0 ^ sw) * 16)) = dequant_scaled<BF16>(wsel, scur[i], zcur[i]);
+    }
+  };
+  auto issue_a_one = [&](int step, int buf, int i) {
+    uint8_t* Ab = lds8 + (size_t)buf * A_ST;
+    const int r0 = (wave * A_LD + i) * 8;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(Ab + r0 * 128), 16, (int)voff_a[i],
+                                             (int)(((uint32_t)(m0 + r0) * (uint32_t)p.lda + (uint32_t)step * 64u) * 2u), 0, 0);
   };
 
   v16f acc[WMB][WNB];
@@ -310,55 +351,127 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  // operand reads: row = lane & 31 of a 32-row block, chunk c = kk*2 + (lane >> 5), swizzled by (row & 7) = lane & 7
-  const int r7 = lane & 7, kh = lane >> 5;
+  // operand reads: row = lane & 31 of a 32-row block (blocks start at multiples of 32 rows), chunk kk*2 + (lane >> 5)
+  const int kh = lane >> 5;
   uint32_t coff[4];
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) coff[kk] = (uint32_t)(((kk * 2 + kh) ^ r7) * 16);
-  const uint32_t arow = (uint32_t)((wm * TM + (lane & 31)) * 128);
-  const uint32_t brow = (uint32_t)(BM * 128 + (wn * TN + (lane & 31)) * 128);
+  for (int kk = 0; kk < 4; ++kk)
+    coff[kk] = (uint32_t)(((lane & 31) >> 1) * 256 + ((((lane & 1) * 8 + kk * 2 + kh) ^ ((lane >> 1) & 15)) * 16));
+  const uint32_t arow = (uint32_t)(wm * TM * 128);
+  const uint32_t brow = (uint32_t)(wn * TN * 128);
 
-  auto compute = [&](int cur) {
-    const uint8_t* base = lds8 + (size_t)cur * STAGE;
+  // One K step (64 wide = 4 MFMA k-slices) on activation stage `a_cur` and weight stage `w_cur`, fused with the staging
+  // work for later steps: the DMA requests of the activation tile two steps ahead (into stage `a_dst`), and the
+  // dequantisation of the next step's weights into the other weight stage.  The fragments of slice kk+1 are read
+  // while the MFMAs of slice kk run; the staging work is cut into sub-steps that alternate with shares of the MFMAs
+  // (sched_barrier keeps the compiler from regrouping them).
+  auto fused_step = [&](int a_cur, int w_cur, auto stage_c, auto dma_c, int a_dst, int a_step, int half) {
+    constexpr bool stage_on = decltype(stage_c)::value;
+    constexpr bool dma_on = decltype(dma_c)::value;
+    constexpr int NM = WMB * WNB;                    // MFMAs per slice
+    constexpr int SUB = (NM % 4 == 0) ? 4 : 1;       // sub-steps per slice
+    constexpr int PPS = (2 * W_LD + 3) / 4;          // dequantisation pieces per slice (at most)
+    const uint8_t* base_a = lds8 + (size_t)a_cur * A_ST;
+    const uint8_t* base_b = lds8 + W_BASE + (size_t)w_cur * W_ST;
+    uint8_t* Bn = lds8 + W_BASE + (size_t)(w_cur ^ 1) * W_ST;
+    if constexpr (dma_on) {
+#pragma unroll
+      for (int i = 0; i < A_LD; ++i) issue_a_one(a_step, a_dst, i);
+    }
+    v4u af[WMB], bf[2][WNB];     // weight fragments double-buffered, activation fragments refilled in place
+#pragma unroll
+    for (int i = 0; i < WMB; ++i) af[i] = *reinterpret_cast<const v4u*>(base_a + arow + i * 4096 + coff[0]);
+#pragma unroll
+    for (int j = 0; j < WNB; ++j) bf[0][j] = *reinterpret_cast<const v4u*>(base_b + brow + j * 4096 + coff[0]);
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
-      v4u af[WMB], bf[WNB];
+      const int cb = kk & 1, nb = cb ^ 1;
+      v4u dq[PPS];
 #pragma unroll
-      for (int i = 0; i < WMB; ++i) af[i] = *reinterpret_cast<const v4u*>(base + arow + i * 4096 + coff[kk]);
+      for (int t = 0; t < SUB; ++t) {
+        // a share of this slice's MFMAs
 #pragma unroll
-      for (int j = 0; j < WNB; ++j) bf[j] = *reinterpret_cast<const v4u*>(base + brow + j * 4096 + coff[kk]);
+        for (int q = t * (NM / SUB); q < (t + 1) * (NM / SUB); ++q) {
+          const int i = q / WNB, j = q % WNB;
+          acc[i][j] = T::mfma32(bf[cb][j], af[i], acc[i][j]);   // rows = n, columns = m
+        }
+        // a share of the fragment reads of the next slice
+        if (kk < 3) {
 #pragma unroll
-      for (int i = 0; i < WMB; ++i)
+          for (int i = 0; i < WMB; ++i) {
+            // activation fragment i has just had its last use in this slice: refill it in place
+            const int last_q = i * WNB + WNB - 1;
+            if (last_q >= t * (NM / SUB) && last_q < (t + 1) * (NM / SUB))
+              af[i] = *reinterpret_cast<const v4u*>(base_a + arow + i * 4096 + coff[kk + 1]);
+          }
 #pragma unroll
-        for (int j = 0; j < WNB; ++j) acc[i][j] = T::mfma32(bf[j], af[i], acc[i][j]);   // rows = n, columns = m
+          for (int j = 0; j < WNB; ++j)
+            if (j % SUB == t) bf[nb][j] = *reinterpret_cast<const v4u*>(base_b + brow + j * 4096 + coff[kk + 1]);
+        }
+        // a share of the dequantisation
+        if constexpr (stage_on) {
+#pragma unroll
+          for (int pc = 0; pc < 2 * W_LD; ++pc) {
+            if (pc * 4 / (2 * W_LD) != kk) continue;
+            const int slot = pc % PPS;
+            const int i = pc >> 1, which = pc & 1;
+            const uint32_t wsel = half ? (which ? wcur[i].w : wcur[i].z) : (which ? wcur[i].y : wcur[i].x);
+            if constexpr (SUB == 4) {
+              dq[slot][t] = dequant_part<BF16>(wsel, scur[i], zcur[i], t);
+            } else {
+              dq[slot] = dequant_scaled<BF16>(wsel, scur[i], zcur[i]);
+            }
+            if (t == SUB - 1) {
+              const int row = (i * NW + wave) * 16 + r;
+              const int c0 = (row & 1) * 8 + o + which * 4, sw = (row >> 1) & 15;
+              *reinterpret_cast<v4u*>(Bn + (row >> 1) * 256 + ((c0 ^ sw) * 16)) = dq[slot];
+            }
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   };
 
-  // ---- prologue: stage step 0 (group 0, half 0) ----
+  // Vector-memory operations retire in issue order.  At the end of step s the activation tile of step s+1 (requested
+  // during step s-1) must have landed, while the requests made during step s -- the tile of step s+2 and, on even
+  // steps, the next group's weight words -- may stay in flight: wait until at most that many are outstanding.
+  using TT = std::true_type;
+  using FF = std::false_type;
+
+  // ---- prologue: activation tiles of steps 0 and 1, weights of step 0 (group 0, half 0) ----
   issue_a(0, 0);
-  load_w(0, 0);
-  store_w(0, 0, 0);
+  issue_a(1, 1);
+  load_w(0);
+  advance_w();
+  store_w0();
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
-  for (int g = 0; g < p.G; ++g) {
-    const int set = g & 1;
-    // even step 2g (buffer 0): stage step 2g+1 = (g, half 1) into buffer 1; request group g+1
-    issue_a(2 * g + 1, 1);
-    if (g + 1 < p.G) load_w(g + 1, set ^ 1);
-    store_w(1, 1, set);
-    compute(0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    // odd step 2g+1 (buffer 1): stage step 2g+2 = (g+1, half 0) into buffer 0
-    if (g + 1 < p.G) {
-      issue_a(2 * g + 2, 0);
-      store_w(0, 0, set ^ 1);
-    }
-    compute(1);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+  int a_cur = 0;                      // activation stage of the current step (step mod 3)
+  auto nxt = [](int x) { return x == 2 ? 0 : x + 1; };
+  // LDS writes of this wavefront done, requests older than the newest `n` landed, then the workgroup barrier.  (A
+  // plain __syncthreads() carries a fence that drains every outstanding load.)
+  auto sync_step = [&](auto n_c) {
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(decltype(n_c)::value) : "memory");
+  };
+  for (int g = 0; g + 1 < p.G; ++g) {
+    // even step 2g: dequantise (g, half 1) for step 2g+1; request the tile of step 2g+2 and the words of group g+1
+    load_w(g + 1);
+    fused_step(a_cur, 0, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 2, 1);
+    sync_step(std::integral_constant<int, A_LD + KW>{});
+    a_cur = nxt(a_cur);
+    // odd step 2g+1: dequantise (g+1, half 0) for step 2g+2; request the tile of step 2g+3
+    advance_w();
+    fused_step(a_cur, 1, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 3, 0);
+    sync_step(std::integral_constant<int, A_LD>{});
+    a_cur = nxt(a_cur);
   }
+  // last group: its second half is still dequantised, nothing is requested any more
+  fused_step(a_cur, 0, TT{}, FF{}, 0, 0, 1);
+  sync_step(std::integral_constant<int, 0>{});
+  a_cur = nxt(a_cur);
+  fused_step(a_cur, 1, FF{}, FF{}, 0, 0, 0);
 
   // ---- epilogue: four consecutive accumulator registers = four consecutive n of one row ----
 #pragma unroll
@@ -415,7 +528,7 @@ static int launch_prefill(const PrefillParams& p, hipStream_t s) {
 
 template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP>
 static int launch_prefill2(const PrefillParams& p, hipStream_t s) {
-  const size_t lds = (size_t)2 * (BM + BN) * 128;
+  const size_t lds = (size_t)(3 * BM + 2 * BN) * 128;
   auto kern = w4a16_prefill2_kernel<BF16, BM, BN, WAVES_M, WAVES_N, HAS_ZP>;
   static bool attr_done = false;
   if (!attr_done) {
