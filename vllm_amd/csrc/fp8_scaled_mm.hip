@@ -16,6 +16,8 @@
 // k0 + 32*q .. k0 + 32*q + 31 of its row.
 #include "vaq_common.h"
 
+#include <type_traits>
+
 namespace vaq {
 
 struct Fp8MMParams {
@@ -296,6 +298,157 @@ __global__ __launch_bounds__(256) void fp8_mm_tile2_kernel(const Fp8MMParams p) 
   tile_epilogue<BF16_OUT, WMB, WNB>(p, acc, m0, n0, wm, wn, lane);
 }
 
+// ----------------------------------------------------------------------------- tile kernel, multi-stage direct-to-LDS
+// The kernel the M > 32 path normally uses.  Differences from fp8_mm_tile2_kernel:
+//  * one MFMA k-slice (64 bytes of K) per stage, NST stages in a ring: the requests for step s+NST-1 go out at the
+//    start of step s, so a tile has NST-2 full steps to arrive before anybody waits for it (with two stages of 128
+//    bytes the wait at the end of every step saw most of the L2 latency);
+//  * vector-memory operations retire in issue order, so "the tile of step s+1 has landed" is `vmcnt <= requests issued
+//    after it`, a compile-time constant; the workgroup barrier is the bare instruction (a __syncthreads() carries a fence
+//    that drains every outstanding load);
+//  * LDS rows are 64 bytes; four rows form one 256-byte line of 16 chunks (chunk index (row & 3) * 4 + c) and the chunk
+//    index is XOR-ed with (row >> 2) & 3.  The LDS has 64 banks (256 bytes per cycle): 16 lanes reading 16 consecutive
+//    rows at the same k chunk touch 16 different 16-byte bank groups;
+//  * WAVES_M x WAVES_N wavefronts; tiles are handed out in bands of 8 tile rows inside each XCD's contiguous range so
+//    that the tiles resident on one XCD share activation rows and weight columns in its L2.
+// Requires K % 64 == 0 (a partial last step would read the neighbouring row instead of zeros) and M*lda, N*ldb < 2^32.
+template <bool BF16_OUT, int BM, int BN, int WAVES_M, int WAVES_N, int NST>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(const Fp8MMParams p) {
+  constexpr int NW = WAVES_M * WAVES_N;
+  constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;
+  constexpr int WMB = TM / 32, WNB = TN / 32;
+  constexpr int A_ST = BM * 64, B_ST = BN * 64, STAGE = A_ST + B_ST;
+  constexpr int A_LD = BM / (16 * NW), B_LD = BN / (16 * NW);     // DMA instructions per wavefront and step (16 rows each)
+  constexpr int LPW = A_LD + B_LD;
+  static_assert(A_LD >= 1 && B_LD >= 1, "tile too small for this many wavefronts");
+  static_assert((NST - 2) * LPW <= 63, "wait counter range");
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds8[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  const int total = tiles_m * tiles_n;
+  int t = blockIdx.x;
+  if (total % 8 == 0) t = (t & 7) * (total / 8) + (t >> 3);          // one contiguous range of tile ids per XCD
+  constexpr int GM = 8;                                              // band height in tiles
+  const int band = t / (GM * tiles_n);
+  const int first_m = band * GM;
+  const int gsz = min(tiles_m - first_m, GM);
+  const int tin = t - band * GM * tiles_n;
+  const int tm = first_m + tin % gsz, tn = tin / gsz;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.a), 0, (int)((uint32_t)p.M * (uint32_t)p.lda), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.b), 0, (int)((uint32_t)p.N * (uint32_t)p.ldb), 0x00020000);
+  // DMA instruction: 16 rows x 64 bytes = four 256-byte lines; lane l lands in slot l: line j = r0/4 + (l >> 4), swizzled
+  // chunk l & 15 -> c16 = (l & 15) ^ (j & 3), row = 4j + (c16 >> 2), chunk = c16 & 3.  r0 is a multiple of 16, so j & 3 = l >> 4.
+  const int c16 = (lane & 15) ^ (lane >> 4);
+  const int lrow = 4 * (lane >> 4) + (c16 >> 2);
+  const uint32_t voff_a = (uint32_t)lrow * (uint32_t)p.lda + (uint32_t)(c16 & 3) * 16u;
+  const uint32_t voff_b = (uint32_t)lrow * (uint32_t)p.ldb + (uint32_t)(c16 & 3) * 16u;
+
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  auto issue_loads = [&](int step, int stage) {
+    uint8_t* Ab = lds8 + (size_t)stage * STAGE;
+    uint8_t* Bb = Ab + A_ST;
+#pragma unroll
+    for (int i = 0; i < A_LD; ++i) {
+      const int r0 = (wave * A_LD + i) * 16;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(Ab + r0 * 64), 16, (int)voff_a,
+                                               (int)((uint32_t)(m0 + r0) * (uint32_t)p.lda + (uint32_t)step * 64u), 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < B_LD; ++i) {
+      const int r0 = (wave * B_LD + i) * 16;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(Bb + r0 * 64), 16, (int)voff_b,
+                                               (int)((uint32_t)(n0 + r0) * (uint32_t)p.ldb + (uint32_t)step * 64u), 0, 0);
+    }
+  };
+
+  v16f acc[WMB][WNB];
+#pragma unroll
+  for (int i = 0; i < WMB; ++i)
+#pragma unroll
+    for (int j = 0; j < WNB; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // operand reads: row = lane & 31 of a 32-row block (blocks start at multiples of 32 rows), the lane's 32 bytes are
+  // chunks 2*kh and 2*kh+1 (kh = lane >> 5)
+  const int kh = lane >> 5;
+  uint32_t coff[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+    coff[h] = (uint32_t)(((lane & 31) >> 2) * 256 + ((((lane & 3) * 4 + kh * 2 + h) ^ ((lane >> 2) & 3)) * 16));
+  const uint32_t arow = (uint32_t)(wm * TM * 64);
+  const uint32_t brow = (uint32_t)(A_ST + wn * TN * 64);
+
+  // (Reading the fragments of step s+1 during the MFMAs of step s -- one more stage of slack, double-buffered weight
+  // fragments -- was measured 5% slower than reading them at the start of their own step, and is not done.)
+  auto compute = [&](int stage) {
+    const uint8_t* base = lds8 + (size_t)stage * STAGE;
+    v8i af[WMB], bf[WNB];
+#pragma unroll
+    for (int j = 0; j < WNB; ++j) {
+      const v4i lo = *reinterpret_cast<const v4i*>(base + brow + j * 2048 + coff[0]);
+      const v4i hi = *reinterpret_cast<const v4i*>(base + brow + j * 2048 + coff[1]);
+      bf[j] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
+#pragma unroll
+    for (int i = 0; i < WMB; ++i) {
+      const v4i lo = *reinterpret_cast<const v4i*>(base + arow + i * 2048 + coff[0]);
+      const v4i hi = *reinterpret_cast<const v4i*>(base + arow + i * 2048 + coff[1]);
+      af[i] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
+#pragma unroll
+    for (int i = 0; i < WMB; ++i)
+#pragma unroll
+      for (int j = 0; j < WNB; ++j) acc[i][j] = mfma_fp8_32(bf[j], af[i], acc[i][j]);   // rows = n, columns = m
+  };
+  // end of a step: LDS reads of this wavefront done, requests older than the newest `n` landed, then the bare barrier
+  auto sync_step = [&](auto n_c) {
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(decltype(n_c)::value) : "memory");
+  };
+  using WAIT_STEADY = std::integral_constant<int, (NST - 2) * LPW>;
+  using WAIT_NONE = std::integral_constant<int, 0>;
+
+  // Invariant at the start of step s: the tile of step s complete in LDS, the tiles of steps s+1 .. s+NST-2 requested,
+  // stage (s-1) % NST free.  The requests of step s+NST-1 go out first thing in step s.
+  const int steps = p.K / 64;
+  if (steps >= NST) {
+#pragma unroll
+    for (int s0 = 0; s0 < NST - 1; ++s0) issue_loads(s0, s0);
+    sync_step(WAIT_STEADY{});           // tile 0 landed
+    int cur = 0, dst = NST - 1;
+    int step = 0;
+    for (; step + NST - 1 < steps; ++step) {
+      issue_loads(step + NST - 1, dst);
+      compute(cur);
+      sync_step(WAIT_STEADY{});
+      cur = cur + 1 == NST ? 0 : cur + 1;
+      dst = dst + 1 == NST ? 0 : dst + 1;
+    }
+    for (; step < steps; ++step) {      // nothing left to request: drain
+      compute(cur);
+      sync_step(WAIT_NONE{});
+      cur = cur + 1 == NST ? 0 : cur + 1;
+    }
+  } else {
+    // short K: no ring, one tile at a time
+    for (int step = 0; step < steps; ++step) {
+      issue_loads(step, 0);
+      sync_step(WAIT_NONE{});
+      compute(0);
+      sync_step(WAIT_NONE{});
+    }
+  }
+
+  tile_epilogue<BF16_OUT, WMB, WNB>(p, acc, m0, n0, wm, wn, lane);
+}
+
 // ----------------------------------------------------------------------------- stream kernel (M <= 32)
 // blockDim = (64, WK).  Wavefront w owns K steps [w*KS, (w+1)*KS) of 128 bytes; activations of that slab live in
 // registers for the whole kernel; the workgroup walks a contiguous range of 16-row weight tiles.
@@ -438,13 +591,50 @@ static int launch_tile2(const Fp8MMParams& p, hipStream_t s) {
   return VAQ_OK;
 }
 
+template <bool BF16_OUT, int BM, int BN, int WAVES_M, int WAVES_N, int NST>
+static int launch_tile3(const Fp8MMParams& p, hipStream_t s) {
+  const size_t lds = (size_t)NST * (BM + BN) * 64;
+  auto kern = fp8_mm_tile3_kernel<BF16_OUT, BM, BN, WAVES_M, WAVES_N, NST>;
+  static bool attr_done = false;
+  if (!attr_done) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
+        hipSuccess) {
+      set_error("fp8_scaled_mm: cannot reserve %zu bytes of LDS", lds);
+      (void)hipGetLastError();
+      return VAQ_ERR_LAUNCH;
+    }
+    attr_done = true;
+  }
+  const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(WAVES_M * WAVES_N * 64), lds, s, p);
+  return VAQ_OK;
+}
+
+static int g_fp8_tile3_cfg = 0;    // 0: automatic, -1: off (two-stage kernel), >0: a fixed tile shape (benchmarking)
 static int g_fp8_tile_impl = 0;   // 0: direct-to-LDS kernel when its preconditions hold, 1: always the register-staged kernel
 
 template <bool BF16_OUT>
 static int dispatch_tile(const Fp8MMParams& p, hipStream_t s) {
-  const bool direct_ok = g_fp8_tile_impl == 0 && p.K % F8_BK == 0 && (uint64_t)p.M * (uint64_t)p.lda < (1ull << 32) &&
+  const bool direct_ok = g_fp8_tile_impl == 0 && p.K % 64 == 0 && (uint64_t)p.M * (uint64_t)p.lda < (1ull << 32) &&
                          (uint64_t)p.N * (uint64_t)p.ldb < (1ull << 32);
-  if (direct_ok) {
+  if (direct_ok && g_fp8_tile_impl == 0 && g_fp8_tile3_cfg >= 0) {
+    const int cus3 = num_cus_current_device();
+    auto tiles3 = [&](int bm, int bn) { return (int64_t)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
+    int cfg = g_fp8_tile3_cfg;
+    if (cfg == 0)
+      cfg = tiles3(256, 256) >= cus3 ? 1 : (tiles3(128, 256) * 8 >= cus3 * 7 ? 7 : (tiles3(128, 128) * 2 >= cus3 ? 3 : 4));
+    switch (cfg) {
+      case 1: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 5>(p, s);
+      case 2: return launch_tile3<BF16_OUT, 256, 256, 2, 2, 5>(p, s);
+      case 3: return launch_tile3<BF16_OUT, 128, 128, 2, 2, 5>(p, s);
+      case 4: return launch_tile3<BF16_OUT, 64, 128, 2, 2, 5>(p, s);
+      case 5: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 4>(p, s);
+      case 6: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 3>(p, s);
+      case 7: return launch_tile3<BF16_OUT, 128, 256, 2, 4, 5>(p, s);
+      default: break;
+    }
+  }
+  if (direct_ok && p.K % F8_BK == 0) {
     const int cus2 = num_cus_current_device();
     auto tiles2 = [&](int bm, int bn) { return (int64_t)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
     if (tiles2(256, 256) >= cus2) return launch_tile2<BF16_OUT, 4, 4>(p, s);
@@ -541,6 +731,7 @@ extern "C" int vaq_fp8_scaled_mm(const uint8_t* a, int64_t lda, const uint8_t* b
 // Benchmark / tuning aid, not part of the drop-in surface.  path: 0 auto, 1 stream, 2 tile; gx: stream-kernel grid.
 extern "C" void vaq_debug_set_fp8_config(int path, int gx) {
   vaq::g_force_fp8_path = path % 10;
-  vaq::g_fp8_tile_impl = path / 10;       // tens digit: 1 = force the register-staged tile kernel
+  vaq::g_fp8_tile_impl = (path / 10) % 10;     // tens digit: 1 = force the register-staged tile kernel
+  vaq::g_fp8_tile3_cfg = path / 100 == 9 ? -1 : path / 100;   // hundreds digit: multi-stage tile shape (9 = off)
   vaq::g_force_fp8_gx = gx;
 }

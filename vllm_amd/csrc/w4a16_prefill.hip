@@ -263,9 +263,14 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
 
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   const int total = tiles_m * tiles_n;
-  int bid = blockIdx.x;
-  if (total % 8 == 0) bid = (bid & 7) * (total / 8) + (bid >> 3);   // one contiguous band of tiles per XCD
-  const int tm = bid % tiles_m, tn = bid / tiles_m;
+  int t = blockIdx.x;
+  if (total % 8 == 0) t = (t & 7) * (total / 8) + (t >> 3);          // one contiguous range of tile ids per XCD
+  constexpr int GM = 8;                                              // tiles are handed out in bands of 8 tile rows, so
+  const int band = t / (GM * tiles_n);                               // that the tiles resident on one XCD share
+  const int first_m = band * GM;                                     // activation rows and weight columns in its L2
+  const int gsz = min(tiles_m - first_m, GM);
+  const int tin = t - band * GM * tiles_n;
+  const int tm = first_m + tin % gsz, tn = tin / gsz;
   const int m0 = tm * BM, n0 = tn * BN, nt0 = n0 / 16;
 
   // ---- activation tile: direct-to-LDS loads ----
