@@ -53,6 +53,26 @@ def test_repack_bit_exact_both_layouts(device, k, n, act_order):
     assert np.array_equal(nl.native_unpack(native.cpu().numpy(), k, n), q_sorted)
 
 
+# ------------------------------------------------------------------------------------------------ permute_cols
+
+@pytest.mark.parametrize("m,k", [(1, 128), (3, 1024), (7, 4096), (130, 14336), (5, 70000)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_permute_cols_bit_exact(device, m, k, dtype):
+    """out[:, j] = a[:, perm[j]] (reference: permute_cols.cu, used by the act_order path); rows may be a strided view.
+    K = 70000 exceeds what the LDS-staged kernel holds and takes the direct-gather kernel."""
+    import vllm_amd._custom_ops as ops
+    g = torch.Generator().manual_seed(m * 131 + k)
+    big = torch.randn(m, k + 24, generator=g).to(dtype)
+    perm = torch.randperm(k, generator=g).to(torch.int32)
+    big_dev = big.to(device)
+    for lo, contiguous in ((0, True), (8, False), (3, False)):
+        a_cpu = big[:, lo:lo + k]
+        a_dev = big_dev[:, lo:lo + k].contiguous() if contiguous else big_dev[:, lo:lo + k]
+        out = ops.permute_cols(a_dev, perm.to(device))
+        assert out.shape == (m, k) and out.dtype == dtype and out.is_contiguous()
+        assert torch.equal(out.cpu().view(torch.int16), a_cpu[:, perm.long()].contiguous().view(torch.int16))
+
+
 # ------------------------------------------------------------------------------------------------ GEMM, small shapes
 
 SMALL = [(128, 64), (512, 256), (1024, 192), (2048, 576), (14336 // 4, 128)]
