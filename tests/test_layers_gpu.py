@@ -1,0 +1,243 @@
+"""GPU tests of the plugin surface: quantization configs -> linear methods -> ``create_weights`` /
+``process_weights_after_loading`` / ``apply`` on a device layer, checked against the CPU oracle; HIP-graph replays of the
+same layers; dispatcher checks of the custom ops (schema + fake tensors) with device arguments.
+
+The flow mirrors how the reference drives a quantized layer (linear.py:243-300, gptq_marlin.py:329-466, fp8.py:330-684):
+a checkpoint's tensors are copied into the parameters that ``create_weights`` registered, then
+``process_weights_after_loading`` rewrites them in place, then ``forward`` calls ``quant_method.apply``."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8 as of
+from oracle import w4a16 as o
+from tests.helpers import check_gemm_close, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _acts(m, k, dtype=torch.bfloat16, seed=0):
+    return torch.randn(m, k, generator=torch.Generator().manual_seed(seed)).to(dtype)
+
+
+def _gptq_layer(device, k, n_sizes, desc_act, dtype, seed, bias=False):
+    """A MergedColumnParallelLinear with a synthetic GPTQ checkpoint loaded; returns (layer, oracle case, bias)."""
+    from vllm_amd.layers.linear import MergedColumnParallelLinear
+    from vllm_amd.layers.quantization import get_quantization_config
+    n = sum(n_sizes)
+    cfg = get_quantization_config("gptq_marlin").from_config(dict(bits=4, group_size=128, desc_act=desc_act, sym=True))
+    layer = MergedColumnParallelLinear(k, n_sizes, quant_config=cfg, params_dtype=dtype, bias=bias, return_bias=False)
+    case = o.make_w4a16_case(k, n, 128, asym=False, act_order=desc_act, dtype=dtype, seed=seed)
+    layer = layer.to(device)
+    layer.qweight.data.copy_(to_dev(case["qweight"], device))
+    layer.scales.data.copy_(to_dev(case["scales"], device, dtype))
+    g_idx = case["g_idx"] if case["g_idx"] is not None else np.arange(k, dtype=np.int32) // 128
+    layer.g_idx.data.copy_(to_dev(g_idx, device))
+    # a symmetric GPTQ checkpoint stores zero point 8 (as 7 in the v1 format); the method ignores qzeros
+    layer.qzeros.data.fill_(0x77777777)
+    b = None
+    if bias:
+        b = (torch.randn(n, generator=torch.Generator().manual_seed(seed + 1)) * 0.5).to(dtype)
+        layer.bias.data.copy_(b.to(device))
+    layer.process_weights_after_loading()
+    return layer, case, b
+
+
+@pytest.mark.parametrize("desc_act", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_gptq_linear_method_end_to_end(device, desc_act, dtype):
+    k, n_sizes = 1024, [256, 128, 128]
+    layer, case, bias = _gptq_layer(device, k, n_sizes, desc_act, dtype, seed=3, bias=True)
+    from vllm_amd.layers.quantization.gptq_marlin import GPTQMarlinLinearMethod
+    assert isinstance(layer.quant_method, GPTQMarlinLinearMethod)
+    # the loader's parameters were rewritten in place (marlin.py:85-140): same names, repacked contents
+    assert layer.qweight.shape == (k // 16, 2 * sum(n_sizes)) and layer.qweight.dtype == torch.int32
+    w_ref = o.case_w_ref(case)
+    for m in (1, 16, 33, 200):
+        a = _acts(m, k, dtype, seed=m)
+        out = layer(a.to(device))
+        assert out.shape == (m, sum(n_sizes)) and out.dtype == dtype
+        check_gemm_close(out, o.gemm_ref(a, w_ref, bias), f"gptq method desc_act={desc_act} {dtype} m={m}")
+    # leading batch dimensions are flattened and restored (marlin_utils.py:449-450,:481)
+    a3 = _acts(6, k, dtype, seed=9).reshape(2, 3, k)
+    out3 = layer(a3.to(device))
+    assert out3.shape == (2, 3, sum(n_sizes))
+    check_gemm_close(out3.reshape(6, -1), o.gemm_ref(a3.reshape(6, k), w_ref, bias), "gptq method 3-d input")
+
+
+def _fp8_close(out, ref64, what):
+    """Holds the result to 2 ulp of the output type + 2e-3 of the mean magnitude against an fp64 accumulation of the
+    same quantised operands (bitwise parity of this GEMM is not pinned by any reference test)."""
+    out64 = out.detach().cpu().double()
+    assert torch.isfinite(out64).all(), what
+    ulp = 2.0 ** -7 if out.dtype == torch.bfloat16 else 2.0 ** -10
+    tol = 2 * ulp * ref64.abs() + 2e-3 * ref64.abs().mean()
+    bad = (out64 - ref64).abs() > tol
+    assert not bool(bad.any()), f"{what}: {int(bad.sum())} elements out of tolerance, worst {(out64 - ref64).abs().max():.3e}"
+
+
+def test_fp8_linear_method_from_16bit_checkpoint(device):
+    """Fp8Config on a bf16 checkpoint: weight quantised per tensor at load (fp8.py:497-500), activations per token."""
+    from vllm_amd.layers.linear import LinearBase
+    from vllm_amd.layers.quantization import get_quantization_config
+    k, n = 512, 384
+    # a config dict with quant_method "fp8" announces an FP8 checkpoint (fp8.py:191-205); on-the-fly quantisation of a
+    # 16-bit checkpoint is the config built without it
+    cfg = get_quantization_config("fp8")(is_checkpoint_fp8_serialized=False, activation_scheme="dynamic")
+    layer = LinearBase(k, n, quant_config=cfg, params_dtype=torch.bfloat16, bias=True, return_bias=False).to(device)
+    w = (torch.randn(n, k, generator=torch.Generator().manual_seed(1)) * 0.02).to(torch.bfloat16)
+    bias = (torch.randn(n, generator=torch.Generator().manual_seed(2)) * 0.01).to(torch.bfloat16)
+    layer.weight.data.copy_(w.to(device))
+    layer.bias.data.copy_(bias.to(device))
+    layer.process_weights_after_loading()
+    wq_ref, ws_ref = of.ref_dynamic_per_tensor_quant(w)
+    assert layer.weight.dtype == torch.float8_e4m3fn and layer.weight.shape == (k, n)
+    assert torch.equal(layer.weight.t().contiguous().cpu().view(torch.uint8), wq_ref.view(torch.uint8)), "weight codes"
+    assert torch.equal(layer.weight_scale.cpu().reshape(()), ws_ref.reshape(())), "weight scale"
+    for m in (1, 16, 100):
+        a = _acts(m, k, seed=m)
+        out = layer(a.to(device))
+        aq, sa = of.ref_dynamic_per_token_quant(a)
+        ref = of.scaled_mm_ref(aq, wq_ref.t(), sa, ws_ref, torch.float64, bias)
+        _fp8_close(out, ref, f"fp8 method m={m}")
+
+
+def test_fp8_linear_method_serialized_static_fused_shards(device):
+    """FP8 checkpoint of a fused module: one weight scale and one input scale per logical shard; the method requantises
+    to the largest weight scale and takes the largest input scale (fp8.py:517-570, w8a8_utils.py:105-156)."""
+    from vllm_amd.layers.linear import MergedColumnParallelLinear
+    from vllm_amd.layers.quantization import get_quantization_config
+    k, sizes = 256, [128, 192]
+    n = sum(sizes)
+    cfg = get_quantization_config("fp8").from_config(dict(quant_method="fp8", activation_scheme="static"))
+    assert cfg.is_checkpoint_fp8_serialized
+    layer = MergedColumnParallelLinear(k, sizes, quant_config=cfg, params_dtype=torch.bfloat16, return_bias=False).to(device)
+    g = torch.Generator().manual_seed(5)
+    shards, scales = [], torch.tensor([0.011, 0.017], dtype=torch.float32)
+    for i, width in enumerate(sizes):
+        wf = torch.randn(width, k, generator=g) * (0.6 + 0.5 * i)
+        shards.append(of.ref_static_quant(wf, scales[i]))
+    wq = torch.cat(shards, dim=0)
+    in_scales = torch.tensor([0.02, 0.015], dtype=torch.float32)
+    layer.weight.data.copy_(wq.to(device))
+    layer.weight_scale.data.copy_(scales.to(device))
+    layer.input_scale.data.copy_(in_scales.to(device))
+    layer.process_weights_after_loading()
+    # oracle of the load-time transformation
+    max_s = scales.max()
+    deq = torch.cat([shards[i].to(torch.float32) * scales[i] for i in range(2)], dim=0)
+    wq_ref = of.ref_static_quant(deq, max_s)
+    assert torch.equal(layer.weight.t().contiguous().cpu().view(torch.uint8), wq_ref.view(torch.uint8))
+    assert float(layer.weight_scale) == float(max_s) and float(layer.input_scale) == float(in_scales.max())
+    for m in (3, 64):
+        a = _acts(m, k, seed=m)
+        out = layer(a.to(device))
+        aq = of.ref_static_quant(a, in_scales.max())
+        ref = of.scaled_mm_ref(aq, wq_ref.t(), in_scales.max(), max_s, torch.float64, None)
+        _fp8_close(out, ref, f"fp8 static fused m={m}")
+
+
+def test_ptpc_fp8_linear_method(device):
+    """Per-token x per-channel (ptpc_fp8.py:82-137): bit-exact load-time weight quantisation, GEMM within tolerance."""
+    from vllm_amd.layers.linear import LinearBase
+    from vllm_amd.layers.quantization import get_quantization_config
+    k, n = 1024, 320
+    cfg = get_quantization_config("ptpc_fp8").from_config({})
+    layer = LinearBase(k, n, quant_config=cfg, params_dtype=torch.bfloat16, return_bias=False).to(device)
+    w = (torch.randn(n, k, generator=torch.Generator().manual_seed(7)) * 0.02).to(torch.bfloat16)
+    layer.weight.data.copy_(w.to(device))
+    layer.process_weights_after_loading()
+    wq_ref, ws_ref = of.ref_dynamic_per_token_quant(w)
+    assert torch.equal(layer.weight.t().contiguous().cpu().view(torch.uint8), wq_ref.view(torch.uint8))
+    assert torch.equal(layer.weight_scale.cpu(), ws_ref)
+    for m in (1, 40, 300):
+        a = _acts(m, k, seed=m)
+        out = layer(a.to(device))
+        aq, sa = of.ref_dynamic_per_token_quant(a)
+        _fp8_close(out, of.scaled_mm_ref(aq, wq_ref.t(), sa, ws_ref, torch.float64, None), f"ptpc m={m}")
+
+
+# ------------------------------------------------------------------------------------------------ HIP graphs
+
+@pytest.mark.parametrize("m", [4, 16, 96])
+def test_layers_replay_in_a_hip_graph(device, m):
+    """Capture a GPTQ layer (act_order: exercises the permute and split paths) and a PTPC FP8 layer in one HIP graph,
+    replay it several times with eager work and synchronisations in between, and compare every replay with the eager
+    result: the entry points must neither allocate behind the allocator's back nor record memset nodes."""
+    from vllm_amd.layers.linear import LinearBase
+    from vllm_amd.layers.quantization import get_quantization_config
+    k = 3584            # 28 groups: the decode kernels split K for M > 4
+    gptq, case, _ = _gptq_layer(device, k, [256], True, torch.bfloat16, seed=11)
+    cfg = get_quantization_config("ptpc_fp8").from_config({})
+    fp8 = LinearBase(256, 128, quant_config=cfg, params_dtype=torch.bfloat16, return_bias=False).to(device)
+    fp8.weight.data.copy_((torch.randn(128, 256, generator=torch.Generator().manual_seed(1)) * 0.05).to(torch.bfloat16).to(device))
+    fp8.process_weights_after_loading()
+
+    static_in = torch.zeros(m, k, dtype=torch.bfloat16, device=device)
+
+    def run():
+        return fp8(gptq(static_in))
+
+    inputs = [_acts(m, k, seed=s).to(device) for s in range(4)]
+    eager = []
+    for x in inputs:
+        static_in.copy_(x)
+        eager.append(run().clone())
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        static_in.copy_(inputs[0])
+        run()                      # warm-up on the capture stream
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            static_out = run()
+    torch.cuda.synchronize()
+    for rep in range(2):
+        for x, ref in zip(inputs, eager):
+            static_in.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_out, ref), f"replay differs from eager (m={m}, repetition {rep})"
+            # eager work between replays, as a serving loop would do
+            assert torch.equal(run(), ref)
+    assert bool((gptq.quant_method.kernel.workspace == 0).all()), "workspace counters not restored to zero"
+
+
+# ------------------------------------------------------------------------------------------------ dispatcher checks
+
+def test_custom_ops_pass_opcheck_on_device(device):
+    """Schema and fake-tensor checks of the registered ops with real device arguments (the reference runs the same
+    checks on its ops: tests/kernels/quantization/test_marlin_gemm.py:180-184,:334-352; test_fp8_quant.py:20-45)."""
+    import vllm_amd._custom_ops as ops  # noqa: F401  (registers the ops)
+    from vllm_amd.layers.quantization.utils import marlin_utils as mu
+    from vllm_amd.scalar_type import scalar_types
+    utils = ("test_schema", "test_faketensor")
+    k, n, m = 256, 128, 8
+    case = o.make_w4a16_case(k, n, 128, seed=0)
+    qweight = to_dev(case["qweight"], device)
+    empty = torch.empty(0, dtype=torch.int32, device=device)
+    torch.library.opcheck(torch.ops.vllm_amd.gptq_marlin_repack, (qweight, empty, k, n, 4, 1), test_utils=utils)
+    w = ops.gptq_marlin_repack(qweight, empty, k, n, 4)
+    scales = to_dev(case["scales"], device, torch.bfloat16)
+    a = _acts(m, k).to(device)
+    ws = mu.marlin_make_workspace_new(device)
+    torch.library.opcheck(torch.ops.vllm_amd.gptq_marlin_gemm,
+                          (a, None, w, None, scales, None, empty, empty, empty, ws, scalar_types.uint4b8.id, m, n, k,
+                           True, False, True, False), test_utils=utils)
+    perm = torch.randperm(k, generator=torch.Generator().manual_seed(0)).to(torch.int32).to(device)
+    torch.library.opcheck(torch.ops.vllm_amd.permute_cols, (a, perm), test_utils=utils)
+    # ops with FP8 tensors: the schema checker compares mutated arguments with arithmetic torch lacks for float8, so
+    # only the fake-tensor check applies
+    utils = ("test_faketensor",)
+    out = torch.empty(m, k, dtype=torch.float8_e4m3fn, device=device)
+    sc = torch.empty(m, 1, dtype=torch.float32, device=device)
+    torch.library.opcheck(torch.ops.vllm_amd.dynamic_per_token_scaled_fp8_quant, (out, a, sc, None), test_utils=utils)
+    one = torch.ones(1, dtype=torch.float32, device=device)
+    torch.library.opcheck(torch.ops.vllm_amd.static_scaled_fp8_quant, (out, a, one), test_utils=utils)
+    torch.library.opcheck(torch.ops.vllm_amd.dynamic_scaled_fp8_quant, (out, a, torch.zeros(1, dtype=torch.float32, device=device)),
+                          test_utils=utils)
+    bq = torch.randn(n, k, device=device).to(torch.float8_e4m3fn).t()
+    c = torch.empty(m, n, dtype=torch.bfloat16, device=device)
+    sb = torch.ones(n, 1, dtype=torch.float32, device=device)
+    torch.library.opcheck(torch.ops.vllm_amd.cutlass_scaled_mm, (c, out, bq, sc.fill_(1.0), sb, None), test_utils=utils)
