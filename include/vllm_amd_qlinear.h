@@ -61,6 +61,16 @@ int vaq_w4a16_repack(const int32_t* qweight, const int32_t* perm, int32_t* out, 
                      int num_bits, int layout, void* stream);
 
 /*
+ * AWQ int4 repack.  Replaces `awq_marlin_repack(Tensor b_q_weight, SymInt size_k, SymInt size_n, int num_bits)
+ * -> Tensor` (csrc/torch_bindings.cpp:325-327; device code csrc/quantization/gptq_marlin/awq_marlin_repack.cu:7-268).
+ *   qweight  int32 [size_k, size_n/8] contiguous (AutoAWQ: 8 nibbles along N per word, column 8c+{0,2,4,6,1,3,5,7}[p]
+ *            in nibble position p)
+ *   out      int32 [size_k/16, 2*size_n], same two layouts and the same size rules as vaq_w4a16_repack
+ */
+int vaq_w4a16_repack_awq(const int32_t* qweight, int32_t* out, int64_t size_k, int64_t size_n, int num_bits, int layout,
+                         void* stream);
+
+/*
  * Zero-point repack for the NATIVE layout: GPTQ/compressed-tensors `qzeros` values, packed 8 per int32 along N
  * in natural order, are what vaq_w4a16_gemm reads, so no device work is needed and no entry point exists for
  * it; the reference's marlin_zero_points (marlin_utils.py:326-346) is reproduced on the host side only.

@@ -198,6 +198,33 @@ def test_repack_and_scaled_mm_argument_checks():
         ops.scaled_fp8_quant(torch.zeros(2, 16, dtype=torch.bfloat16), use_per_token_if_dynamic=True)
 
 
+def test_awq_repack_argument_checks_and_helpers():
+    """Host checks of awq_marlin_repack (awq_marlin_repack.cu:208-232) and the AWQ zero-point conversion against the
+    oracle, both layouts (marlin_utils.py:349-370)."""
+    import vllm_amd._custom_ops as ops
+    from oracle import w4a16 as o
+    from vllm_amd.layers.quantization.utils import marlin_utils as mu
+    qw = torch.zeros(128, 8, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="not divisible by tile_k_size"):
+        ops._check_awq_repack_args(qw, 100, 64, 4)
+    with pytest.raises(RuntimeError, match="not divisible by tile_n_size"):
+        ops._check_awq_repack_args(qw, 128, 72, 4)
+    with pytest.raises(RuntimeError, match="num_bits must be 4 or 8"):
+        ops._check_awq_repack_args(qw, 128, 64, 3)
+    with pytest.raises(RuntimeError, match="Shape mismatch"):
+        ops._check_awq_repack_args(qw, 128, 128, 4)
+    with pytest.raises(RuntimeError, match="not on GPU"):
+        ops._check_awq_repack_args(qw, 128, 64, 4)
+    rng = np.random.default_rng(3)
+    groups, n = 6, 192
+    zp = rng.integers(0, 16, size=(groups, n), dtype=np.int32)
+    packed = torch.from_numpy(o.awq_pack(zp, 4))
+    got_marlin = mu.awq_to_marlin_zero_points(packed, groups, n, 4, layout="marlin")
+    assert np.array_equal(got_marlin.numpy(), o.awq_to_marlin_zero_points(o.awq_pack(zp, 4), groups, n, 4))
+    got_native = mu.awq_to_marlin_zero_points(packed, groups, n, 4)
+    assert np.array_equal(got_native.numpy(), o.pack_cols(zp, 4))
+
+
 def test_fake_tensor_shapes():
     """The fake (meta) implementations give the reference's output shapes (_custom_ops.py:524-545,
     gptq_marlin_repack.cu:324-334)."""

@@ -65,6 +65,41 @@ def test_gptq_linear_method_end_to_end(device, desc_act, dtype):
     check_gemm_close(out3.reshape(6, -1), o.gemm_ref(a3.reshape(6, k), w_ref, bias), "gptq method 3-d input")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_awq_linear_method_end_to_end(device, dtype):
+    """AutoAWQ checkpoint (weights and zero points packed along N with the AWQ interleave) through AWQMarlinConfig ->
+    AWQMarlinLinearMethod (awq_marlin.py:264-413) against the oracle's dequantise + fp64 GEMM."""
+    from vllm_amd.layers.linear import MergedColumnParallelLinear, UnquantizedLinearMethod
+    from vllm_amd.layers.quantization import get_quantization_config
+    from vllm_amd.layers.quantization.awq_marlin import AWQMarlinConfig, AWQMarlinLinearMethod
+    hf = dict(quant_method="awq", bits=4, group_size=128, zero_point=True, modules_to_not_convert=["lm_head"])
+    assert AWQMarlinConfig.override_quantization_method(hf, None) == "awq_marlin"
+    assert AWQMarlinConfig.override_quantization_method(hf, "awq") is None
+    assert not AWQMarlinConfig.is_awq_marlin_compatible(dict(hf, bits=8))
+    cfg = get_quantization_config("awq_marlin").from_config(hf)
+    k, sizes = 1024, [256, 192]
+    n = sum(sizes)
+    layer = MergedColumnParallelLinear(k, sizes, quant_config=cfg, params_dtype=dtype, bias=True, return_bias=False,
+                                       prefix="model.layers.0.mlp.gate_up_proj").to(device)
+    assert isinstance(layer.quant_method, AWQMarlinLinearMethod)
+    skipped = MergedColumnParallelLinear(k, sizes, quant_config=cfg, params_dtype=dtype, prefix="lm_head")
+    assert isinstance(skipped.quant_method, UnquantizedLinearMethod)
+    case = o.make_w4a16_case(k, n, 128, asym=True, act_order=False, dtype=dtype, seed=21)
+    layer.qweight.data.copy_(to_dev(o.awq_pack(case["q"], 4), device))
+    layer.qzeros.data.copy_(to_dev(o.awq_pack(case["zp_vals"], 4), device))
+    layer.scales.data.copy_(to_dev(case["scales"], device, dtype))
+    bias = (torch.randn(n, generator=torch.Generator().manual_seed(4)) * 0.5).to(dtype)
+    layer.bias.data.copy_(bias.to(device))
+    layer.process_weights_after_loading()
+    assert layer.qweight.shape == (k // 16, 2 * n) and layer.qzeros.shape == (k // 128, n // 8)
+    w_ref = o.case_w_ref(case)
+    for m in (1, 8, 17, 150):
+        a = _acts(m, k, dtype, seed=m)
+        out = layer(a.to(device))
+        assert out.shape == (m, n) and out.dtype == dtype
+        check_gemm_close(out, o.gemm_ref(a, w_ref, bias), f"awq method {dtype} m={m}")
+
+
 def _fp8_close(out, ref64, what):
     """Holds the result to 2 ulp of the output type + 2e-3 of the mean magnitude against an fp64 accumulation of the
     same quantised operands (bitwise parity of this GEMM is not pinned by any reference test)."""
@@ -218,6 +253,8 @@ def test_custom_ops_pass_opcheck_on_device(device):
     qweight = to_dev(case["qweight"], device)
     empty = torch.empty(0, dtype=torch.int32, device=device)
     torch.library.opcheck(torch.ops.vllm_amd.gptq_marlin_repack, (qweight, empty, k, n, 4, 1), test_utils=utils)
+    torch.library.opcheck(torch.ops.vllm_amd.awq_marlin_repack, (to_dev(o.awq_pack(case["q"], 4), device), k, n, 4, 0),
+                          test_utils=utils)
     w = ops.gptq_marlin_repack(qweight, empty, k, n, 4)
     scales = to_dev(case["scales"], device, torch.bfloat16)
     a = _acts(m, k).to(device)

@@ -53,6 +53,25 @@ def test_repack_bit_exact_both_layouts(device, k, n, act_order):
     assert np.array_equal(nl.native_unpack(native.cpu().numpy(), k, n), q_sorted)
 
 
+@pytest.mark.parametrize("k,n", [(128, 64), (128, 256), (1024, 256), (128 * 13, 64 * 37), (4096, 4096)])
+def test_awq_repack_bit_exact_both_layouts(device, k, n):
+    """Twin of the reference's test_awq_marlin_repack (test_marlin_gemm.py:168-209): AWQ-packed codes -> Marlin order
+    must equal the host construction `marlin_weights`; the native order must equal its specification."""
+    import vllm_amd._custom_ops as ops
+    rng = np.random.default_rng(k * 7 + n)
+    q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    qw = to_dev(o.awq_pack(q, 4), device)
+    assert qw.shape == (k, n // 8)
+    marlin = ops.awq_marlin_repack(qw, k, n, 4, layout="marlin")
+    native = ops.awq_marlin_repack(qw, k, n, 4)
+    assert marlin.shape == native.shape == (k // 16, 2 * n) and marlin.dtype == torch.int32
+    assert np.array_equal(marlin.cpu().numpy(), o.marlin_weights(q)), "marlin order differs from the oracle"
+    assert np.array_equal(native.cpu().numpy(), nl.native_pack(q)), "native order differs from its spec"
+    # the same codes through the GPTQ packing give the same bytes
+    assert torch.equal(native, ops.gptq_marlin_repack(to_dev(o.gptq_pack(q, 4), device),
+                                                      torch.empty(0, dtype=torch.int32, device=device), k, n, 4))
+
+
 # ------------------------------------------------------------------------------------------------ permute_cols
 
 @pytest.mark.parametrize("m,k", [(1, 128), (3, 1024), (7, 4096), (130, 14336), (5, 70000)])

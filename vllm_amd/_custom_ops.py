@@ -96,6 +96,43 @@ def _repack_fake(b_q_weight, perm, size_k, size_n, num_bits, layout=1):
                        dtype=b_q_weight.dtype, device=b_q_weight.device)
 
 
+def _check_awq_repack_args(b_q_weight: torch.Tensor, size_k: int, size_n: int, num_bits: int) -> None:
+    """Host checks of awq_marlin_repack.cu:208-232 in the same order."""
+    _check(size_k % GPTQ_MARLIN_TILE == 0, f"size_k = {size_k} is not divisible by tile_k_size = {GPTQ_MARLIN_TILE}")
+    _check(size_n % GPTQ_MARLIN_MIN_THREAD_N == 0,
+           f"size_n = {size_n} is not divisible by tile_n_size = {GPTQ_MARLIN_MIN_THREAD_N}")
+    _check(num_bits in (4, 8), f"num_bits must be 4 or 8. Got = {num_bits}")
+    pack_factor = 32 // num_bits
+    _check(b_q_weight.dim() == 2 and b_q_weight.size(0) == size_k,
+           f"b_q_weight.size(0) = {b_q_weight.size(0) if b_q_weight.dim() else None} is not size_k = {size_k}")
+    _check(size_n // pack_factor == b_q_weight.size(1),
+           f"Shape mismatch: b_q_weight.size(1) = {b_q_weight.size(1)}, size_n = {size_n}, pack_factor = {pack_factor}")
+    _check(_is_gpu(b_q_weight), "b_q_weight is not on GPU")
+    _check(b_q_weight.is_contiguous(), "b_q_weight is not contiguous")
+    _check(b_q_weight.dtype == torch.int32, "b_q_weight type is not kInt")
+    if num_bits != 4:
+        raise NotImplementedError("awq_marlin_repack: only num_bits = 4 is built for gfx950")
+
+
+def _awq_repack_impl(b_q_weight: torch.Tensor, size_k: int, size_n: int, num_bits: int,
+                     layout: int = _lib.VAQ_LAYOUT_NATIVE) -> torch.Tensor:
+    _check_awq_repack_args(b_q_weight, size_k, size_n, num_bits)
+    lib = _lib.load()
+    pack_factor = 32 // num_bits
+    with torch.cuda.device(b_q_weight.device):
+        out = torch.empty((size_k // GPTQ_MARLIN_TILE, size_n * GPTQ_MARLIN_TILE // pack_factor),
+                          dtype=torch.int32, device=b_q_weight.device)
+        _lib.check(lib.vaq_w4a16_repack_awq(_ptr(b_q_weight), _ptr(out), size_k, size_n, num_bits, layout,
+                                            _stream(b_q_weight.device)))
+    return out
+
+
+def _awq_repack_fake(b_q_weight, size_k, size_n, num_bits, layout=1):
+    pack_factor = 32 // num_bits
+    return torch.empty((size_k // GPTQ_MARLIN_TILE, size_n * GPTQ_MARLIN_TILE // pack_factor),
+                       dtype=b_q_weight.dtype, device=b_q_weight.device)
+
+
 # ============================================================================ W4A16 GEMM
 
 def _opt(t: torch.Tensor | None) -> torch.Tensor | None:
@@ -378,6 +415,9 @@ def _register(name: str, schema: str, impl, fake=None) -> None:
 _register("gptq_marlin_repack",
           "(Tensor b_q_weight, Tensor perm, SymInt size_k, SymInt size_n, int num_bits, int layout=1) -> Tensor",
           _repack_impl, _repack_fake)
+_register("awq_marlin_repack",
+          "(Tensor b_q_weight, SymInt size_k, SymInt size_n, int num_bits, int layout=1) -> Tensor",
+          _awq_repack_impl, _awq_repack_fake)
 _register("gptq_marlin_gemm",
           "(Tensor a, Tensor? c_or_none, Tensor b_q_weight, Tensor? b_bias_or_none, Tensor b_scales, "
           "Tensor? global_scale, Tensor? b_zeros_or_none, Tensor? g_idx_or_none, Tensor? perm_or_none, "
@@ -407,6 +447,13 @@ def gptq_marlin_repack(b_q_weight: torch.Tensor, perm: torch.Tensor, size_k: int
     reproduces the reference's Marlin order bit-for-bit.  Callers treat the result as opaque either way.
     """
     return _ops.gptq_marlin_repack(b_q_weight, perm, size_k, size_n, num_bits, _LAYOUTS[layout])
+
+
+def awq_marlin_repack(b_q_weight: torch.Tensor, size_k: int, size_n: int, num_bits: int, *,
+                      layout: str = "native") -> torch.Tensor:
+    """AutoAWQ int32[K, N/8] -> repacked int32[K/16, 2N] (reference: _custom_ops.py:1145-1148).  Same two layouts as
+    ``gptq_marlin_repack``: ``"marlin"`` is bit-exact with the reference, ``"native"`` is what the GEMM reads."""
+    return _ops.awq_marlin_repack(b_q_weight, size_k, size_n, num_bits, _LAYOUTS[layout])
 
 
 def gptq_marlin_gemm(a: torch.Tensor, c: torch.Tensor | None, b_q_weight: torch.Tensor, b_bias: torch.Tensor | None,

@@ -26,6 +26,7 @@ _SIGNATURES = {
     "vaq_abi_version": (c_int, []),
     "vaq_num_cus": (c_int, [c_int]),
     "vaq_w4a16_repack": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_int, c_void_p]),
+    "vaq_w4a16_repack_awq": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_int, c_void_p]),
     "vaq_w4a16_gemm_workspace": (c_int, [c_int64, c_int64, c_int64, c_int, c_int, POINTER(c_size_t), POINTER(c_size_t),
                                          POINTER(c_size_t)]),
     "vaq_w4a16_gemm": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,

@@ -1,7 +1,9 @@
-// GPTQ int4 weight repack for gfx950.
+// GPTQ / AWQ int4 weight repack for gfx950.
 //
 // Input : GPTQ checkpoint tensor int32 [K/8, N]; word (r, n) holds codes of rows 8r..8r+7 of column n, row 8r+e in
-//         bits [4e, 4e+4).
+//         bits [4e, 4e+4);
+//         or AWQ (AutoAWQ) checkpoint tensor int32 [K, N/8]; word (k, c) holds the codes of row k, columns 8c..8c+7,
+//         column 8c + {0,2,4,6,1,3,5,7}[p] in nibble position p.
 // Output: int32 [K/16, 2N] (same byte count) in one of two orders.
 //
 //  NATIVE (what the GEMM kernels stream)
@@ -32,13 +34,21 @@ __device__ inline uint32_t fetch_code(const uint32_t* __restrict__ qw, const int
   return (word >> ((src & 7) * 4)) & 0xFu;
 }
 
+// AWQ source: nibble position of column n inside its word is {0,4,1,5,2,6,3,7}[n % 8] (the inverse of the AutoAWQ
+// interleave {0,2,4,6,1,3,5,7}); reference: awq_marlin_repack.cu:95-103.
+__device__ inline uint32_t fetch_code_awq(const uint32_t* __restrict__ qw, int64_t k, int64_t n, int64_t size_n) {
+  const uint32_t word = qw[k * (size_n >> 3) + (n >> 3)];
+  const int pos = (int)(((n & 1) << 2) | ((n & 7) >> 1));
+  return (word >> (pos * 4)) & 0xFu;
+}
+
 __device__ inline uint32_t interleave_pack(const uint32_t v[8]) {
   // nibble position p <- element {0,2,4,6,1,3,5,7}[p]
   return v[0] | (v[2] << 4) | (v[4] << 8) | (v[6] << 12) | (v[1] << 16) | (v[3] << 20) | (v[5] << 24) | (v[7] << 28);
 }
 
 // One thread per output word; native layout.
-template <bool HAS_PERM>
+template <bool HAS_PERM, bool AWQ>
 __global__ __launch_bounds__(256) void repack_native_kernel(const uint32_t* __restrict__ qw,
                                                              const int32_t* __restrict__ perm,
                                                              uint32_t* __restrict__ out, int64_t size_k,
@@ -55,7 +65,12 @@ __global__ __launch_bounds__(256) void repack_native_kernel(const uint32_t* __re
     const int64_t k0 = kt * 128 + j * 32 + o * 8;
     const int64_t n = nt * 16 + r;
     uint32_t res;
-    if constexpr (HAS_PERM) {
+    if constexpr (AWQ) {
+      uint32_t v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = fetch_code_awq(qw, k0 + e, n, size_n);
+      res = interleave_pack(v);
+    } else if constexpr (HAS_PERM) {
       uint32_t v[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] = fetch_code(qw, perm, k0 + e, n, size_n);
@@ -73,6 +88,7 @@ __global__ __launch_bounds__(256) void repack_native_kernel(const uint32_t* __re
 }
 
 // One thread per output word; reference (Marlin) order.
+template <bool AWQ>
 __global__ __launch_bounds__(256) void repack_marlin_kernel(const uint32_t* __restrict__ qw,
                                                              const int32_t* __restrict__ perm,
                                                              uint32_t* __restrict__ out, int64_t size_k,
@@ -91,8 +107,13 @@ __global__ __launch_bounds__(256) void repack_marlin_kernel(const uint32_t* __re
     uint32_t v[8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      v[i] = fetch_code(qw, perm, kbase + off[i], n, size_n);
-      v[4 + i] = fetch_code(qw, perm, kbase + off[i], n + 8, size_n);
+      if constexpr (AWQ) {
+        v[i] = fetch_code_awq(qw, kbase + off[i], n, size_n);
+        v[4 + i] = fetch_code_awq(qw, kbase + off[i], n + 8, size_n);
+      } else {
+        v[i] = fetch_code(qw, perm, kbase + off[i], n, size_n);
+        v[4 + i] = fetch_code(qw, perm, kbase + off[i], n + 8, size_n);
+      }
     }
     out[idx] = interleave_pack(v);
   }
@@ -100,8 +121,8 @@ __global__ __launch_bounds__(256) void repack_marlin_kernel(const uint32_t* __re
 
 }  // namespace vaq
 
-extern "C" int vaq_w4a16_repack(const int32_t* qweight, const int32_t* perm, int32_t* out, int64_t size_k,
-                                int64_t size_n, int num_bits, int layout, void* stream) {
+static int repack_common(const int32_t* qweight, const int32_t* perm, int32_t* out, int64_t size_k, int64_t size_n,
+                         int num_bits, int layout, bool awq, void* stream) {
   using namespace vaq;
   VAQ_CHECK_SUPPORTED(num_bits == 4, "w4a16_repack: num_bits must be 4 (8-bit weights are not built). Got = %d",
                       num_bits);
@@ -121,16 +142,30 @@ extern "C" int vaq_w4a16_repack(const int32_t* qweight, const int32_t* perm, int
   hipStream_t s = (hipStream_t)stream;
   const uint32_t* qw = (const uint32_t*)qweight;
   uint32_t* o = (uint32_t*)out;
+  const dim3 grid((unsigned)blocks), block(threads);
   if (layout == VAQ_LAYOUT_NATIVE) {
-    if (perm)
-      hipLaunchKernelGGL(repack_native_kernel<true>, dim3((unsigned)blocks), dim3(threads), 0, s, qw, perm, o, size_k,
-                         size_n);
+    if (awq)
+      hipLaunchKernelGGL((repack_native_kernel<false, true>), grid, block, 0, s, qw, perm, o, size_k, size_n);
+    else if (perm)
+      hipLaunchKernelGGL((repack_native_kernel<true, false>), grid, block, 0, s, qw, perm, o, size_k, size_n);
     else
-      hipLaunchKernelGGL(repack_native_kernel<false>, dim3((unsigned)blocks), dim3(threads), 0, s, qw, perm, o, size_k,
-                         size_n);
+      hipLaunchKernelGGL((repack_native_kernel<false, false>), grid, block, 0, s, qw, perm, o, size_k, size_n);
   } else {
-    hipLaunchKernelGGL(repack_marlin_kernel, dim3((unsigned)blocks), dim3(threads), 0, s, qw, perm, o, size_k, size_n);
+    if (awq)
+      hipLaunchKernelGGL(repack_marlin_kernel<true>, grid, block, 0, s, qw, perm, o, size_k, size_n);
+    else
+      hipLaunchKernelGGL(repack_marlin_kernel<false>, grid, block, 0, s, qw, perm, o, size_k, size_n);
   }
   VAQ_CHECK_LAUNCH("w4a16_repack");
   return VAQ_OK;
+}
+
+extern "C" int vaq_w4a16_repack(const int32_t* qweight, const int32_t* perm, int32_t* out, int64_t size_k,
+                                int64_t size_n, int num_bits, int layout, void* stream) {
+  return repack_common(qweight, perm, out, size_k, size_n, num_bits, layout, false, stream);
+}
+
+extern "C" int vaq_w4a16_repack_awq(const int32_t* qweight, int32_t* out, int64_t size_k, int64_t size_n, int num_bits,
+                                    int layout, void* stream) {
+  return repack_common(qweight, nullptr, out, size_k, size_n, num_bits, layout, true, stream);
 }

@@ -5,7 +5,7 @@ from __future__ import annotations
 
 from .base_config import QuantizationConfig
 
-QUANTIZATION_METHODS: list[str] = ["gptq_marlin", "fp8", "ptpc_fp8"]
+QUANTIZATION_METHODS: list[str] = ["gptq_marlin", "awq_marlin", "fp8", "ptpc_fp8"]
 _CUSTOMIZED_METHOD_TO_QUANT_CONFIG: dict[str, type[QuantizationConfig]] = {}
 
 
@@ -28,11 +28,13 @@ def register_quantization_config(quantization: str):
 def get_quantization_config(quantization: str) -> type[QuantizationConfig]:
     if quantization not in QUANTIZATION_METHODS:
         raise ValueError(f"Invalid quantization method: {quantization}")
+    from .awq_marlin import AWQMarlinConfig
     from .fp8 import Fp8Config, PTPCFp8Config
     from .gptq_marlin import GPTQMarlinConfig
 
     method_to_config: dict[str, type[QuantizationConfig]] = {
         "gptq_marlin": GPTQMarlinConfig,
+        "awq_marlin": AWQMarlinConfig,
         "fp8": Fp8Config,
         "ptpc_fp8": PTPCFp8Config,
     }

@@ -192,3 +192,29 @@ def apply_gptq_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_s
                                   is_k_full=is_k_full, use_atomic_add=use_atomic_add, use_fp32_reduce=use_fp32_reduce,
                                   is_zp_float=False)
     return output.reshape(out_shape)
+
+
+def apply_awq_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
+                            weight_zp: torch.Tensor, g_idx: torch.Tensor, g_idx_sort_indices: torch.Tensor,
+                            workspace: torch.Tensor, quant_type: ScalarType, output_size_per_partition: int,
+                            input_size_per_partition: int, bias: torch.Tensor | None = None,
+                            use_fp32_reduce: bool = USE_FP32_REDUCE_DEFAULT) -> torch.Tensor:
+    """marlin_utils.py:485-530."""
+    reshaped_x = input.reshape(-1, input.shape[-1])
+    out_shape = input.shape[:-1] + (output_size_per_partition,)
+    use_atomic_add = should_use_atomic_add_reduce(m=reshaped_x.size(0), n=output_size_per_partition,
+                                                  k=reshaped_x.size(1), device=input.device, dtype=input.dtype)
+    output = ops.gptq_marlin_gemm(reshaped_x, None, weight, bias, weight_scale, None, weight_zp, g_idx,
+                                  g_idx_sort_indices, workspace, quant_type, size_m=reshaped_x.shape[0],
+                                  size_n=output_size_per_partition, size_k=input_size_per_partition,
+                                  use_atomic_add=use_atomic_add, use_fp32_reduce=use_fp32_reduce, is_zp_float=False)
+    return output.reshape(out_shape)
+
+
+def check_marlin_supports_layer(layer: torch.nn.Module, group_size: int) -> bool:
+    """marlin_utils.py:161-178: shape test of a linear layer before a method is attached to it."""
+    output_size_per_partition = getattr(layer, "output_size_per_partition", None) or layer.output_size
+    input_size_per_partition = getattr(layer, "input_size_per_partition", None) or layer.input_size
+    return check_marlin_supports_shape(output_size_per_partition=output_size_per_partition,
+                                       input_size_per_partition=input_size_per_partition,
+                                       input_size=layer.input_size, group_size=group_size)[0]
