@@ -184,20 +184,101 @@ def per_shape_decode(dev, sets, acts):
 
 
 def prefill_section(dev):
+    """BASELINE config 3: asymmetric uint4 + act_order, both readings of its act_order wording.  `rows`: g_idx from a
+    random permutation of the K rows (the reference's generator): activations are reordered on every call.  `groups`:
+    g_idx permutes whole groups: the linear method folds it into the scale / zero-point rows at load time, so the GEMM
+    runs without a permutation (same kernel as no act_order)."""
     rows = []
     gen = torch.Generator(device=dev).manual_seed(2)
     for (k, n) in LLAMA_SHAPES:
-        layer = W4Layer(k, n, dev, gen, asym=True, act_order=True)
-        for m in (512, 2048, 4096):
-            a = torch.randn(m, k, device=dev, generator=gen).to(torch.bfloat16)
-            inner = 4 if m <= 512 else 1
-            t = time_graph(lambda: [layer(a) for _ in range(inner)], iters=5, warmup=2, inner=inner)
-            fl = 2.0 * m * n * k
-            rows.append(dict(kind="w4a16_prefill_asym_actorder", K=k, N=n, M=m, us=t * 1e6, TFLOPs=fl / t / 1e12,
-                             mfma_frac=fl / t / 1e12 / BF16_PEAK_TFLOPS, GBps=w4a16_bytes(m, k, n, True) / t / 1e9))
-            log(f"[prefill     ] K={k:5d} N={n:5d} M={m:4d}: {t * 1e6:8.1f} us  {fl / t / 1e12:7.1f} TFLOP/s ({100 * fl / t / 1e12 / BF16_PEAK_TFLOPS:4.1f}% of 2.5 PF)")
-        del layer
+        for variant in ("rows", "groups"):
+            layer = W4Layer(k, n, dev, gen, asym=True, act_order=(variant == "rows"))
+            for m in (512, 2048, 4096):
+                a = torch.randn(m, k, device=dev, generator=gen).to(torch.bfloat16)
+                inner = 4 if m <= 512 else 1
+                t = time_graph(lambda: [layer(a) for _ in range(inner)], iters=5, warmup=2, inner=inner)
+                fl = 2.0 * m * n * k
+                rows.append(dict(kind=f"w4a16_prefill_asym_actorder_{variant}", K=k, N=n, M=m, us=t * 1e6, TFLOPs=fl / t / 1e12,
+                                 mfma_frac=fl / t / 1e12 / BF16_PEAK_TFLOPS, GBps=w4a16_bytes(m, k, n, True) / t / 1e9))
+                log(f"[prefill {variant:6s}] K={k:5d} N={n:5d} M={m:4d}: {t * 1e6:8.1f} us  {fl / t / 1e12:7.1f} TFLOP/s ({100 * fl / t / 1e12 / BF16_PEAK_TFLOPS:4.1f}% of 2.5 PF)")
+            del layer
     return rows
+
+
+def vendor_ceiling_section(dev):
+    """Practical ceilings on the same box and shapes: the vendor GEMM library through torch (bf16 `matmul`, row-wise
+    scaled FP8 `_scaled_mm`) at M = 4096.  Context for the MFMA fractions above, not part of the product path."""
+    rows = []
+    gen = torch.Generator(device=dev).manual_seed(4)
+    m = 4096
+    for (k, n) in LLAMA_SHAPES:
+        a = torch.randn(m, k, device=dev, generator=gen).to(torch.bfloat16)
+        w = (torch.randn(n, k, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+        fl = 2.0 * m * n * k
+        t = time_graph(lambda: [torch.matmul(a, w.t()) for _ in range(2)], iters=5, warmup=2, inner=2)
+        rows.append(dict(kind="vendor_bf16_matmul", K=k, N=n, M=m, us=t * 1e6, TFLOPs=fl / t / 1e12))
+        log(f"[vendor bf16 ] K={k:5d} N={n:5d} M={m:4d}: {t * 1e6:8.1f} us  {fl / t / 1e12:7.1f} TFLOP/s")
+        try:
+            aq = a.to(torch.float8_e4m3fn)
+            wq = w.to(torch.float8_e4m3fn)
+            sa = torch.ones(m, 1, device=dev, dtype=torch.float32)
+            sb = torch.ones(1, n, device=dev, dtype=torch.float32)
+            t = time_graph(lambda: [torch._scaled_mm(aq, wq.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16) for _ in range(2)],
+                           iters=5, warmup=2, inner=2)
+            rows.append(dict(kind="vendor_fp8_scaled_mm_rowwise", K=k, N=n, M=m, us=t * 1e6, TFLOPs=fl / t / 1e12))
+            log(f"[vendor fp8  ] K={k:5d} N={n:5d} M={m:4d}: {t * 1e6:8.1f} us  {fl / t / 1e12:7.1f} TFLOP/s")
+        except Exception as e:   # not every torch build exposes row-wise FP8 scaling
+            log(f"[vendor fp8  ] unavailable: {str(e)[:80]}")
+        del a, w
+    return rows
+
+
+def decode_step_section(dev):
+    """BASELINE config 5: one decode step of a random-init Llama-3-8B-architecture model, batch 32, context 1024.  All
+    32 x 4 linear layers run on the W4A16 GEMM (M = 32, distinct weights per layer: 3.6 GB); norms, rotary-free
+    attention over a bf16 KV cache, SiLU-mul, embedding and the bf16 lm_head are plain torch ops standing in for the
+    rest of the model.  Reports the step time, the share of it spent in the quantized GEMMs and tokens/s."""
+    import torch.nn.functional as F
+    gen = torch.Generator(device=dev).manual_seed(5)
+    B, CTX, H, NQ, NKV, HD, FF, V, L = 32, 1024, 4096, 32, 8, 128, 14336, 128256, 32
+    layers = []
+    for _ in range(L):
+        layers.append(dict(qkv=W4Layer(H, (NQ + 2 * NKV) * HD, dev, gen), o=W4Layer(H, H, dev, gen),
+                           gate_up=W4Layer(H, 2 * FF, dev, gen), down=W4Layer(FF, H, dev, gen),
+                           kc=torch.randn(B, NKV, CTX, HD, device=dev, generator=gen).to(torch.bfloat16),
+                           vc=torch.randn(B, NKV, CTX, HD, device=dev, generator=gen).to(torch.bfloat16),
+                           n1=torch.ones(H, device=dev, dtype=torch.bfloat16), n2=torch.ones(H, device=dev, dtype=torch.bfloat16)))
+    emb = (torch.randn(V, H, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+    lm_head = (torch.randn(V, H, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+    ids = torch.randint(0, V, (B,), device=dev, generator=gen)
+
+    def step(linear_only=False):
+        x = emb[ids]
+        for ly in layers:
+            h = x if linear_only else F.rms_norm(x, (H,), ly["n1"], 1e-5)
+            qkv = ly["qkv"](h)
+            if linear_only:
+                att = qkv[:, :H]
+            else:
+                q = qkv[:, :NQ * HD].view(B, NQ, 1, HD)
+                att = F.scaled_dot_product_attention(q, ly["kc"], ly["vc"], enable_gqa=True).reshape(B, H)
+            x = x + ly["o"](att.contiguous()) if not linear_only else ly["o"](att.contiguous())
+            h = x if linear_only else F.rms_norm(x, (H,), ly["n2"], 1e-5)
+            gu = ly["gate_up"](h)
+            act = gu[:, :FF].contiguous() if linear_only else F.silu(gu[:, :FF]) * gu[:, FF:]
+            x = ly["down"](act) if linear_only else x + ly["down"](act)
+        return x if linear_only else torch.matmul(x, lm_head.t())
+
+    t_full = time_graph(lambda: step(False), iters=5, warmup=2)
+    t_lin = time_graph(lambda: step(True), iters=5, warmup=2)
+    gemm_bytes = L * sum(w4a16_bytes(B, k, n) for (k, n) in LLAMA_SHAPES)
+    row = dict(kind="llama3_8b_decode_step", batch=B, context=CTX, layers=L, step_us=t_full * 1e6, linear_us=t_lin * 1e6,
+               linear_share=t_lin / t_full, tokens_per_s=B / t_full, tokens_per_s_linear_only=B / t_lin,
+               linear_GBps=gemm_bytes / t_lin / 1e9, linear_hbm_frac=gemm_bytes / t_lin / 1e9 / HBM_PEAK_GBS)
+    log(f"[decode step ] batch {B} ctx {CTX}: {t_full * 1e6:.0f} us/step = {B / t_full:.0f} tok/s; the 128 W4A16 GEMMs (M=32) take "
+        f"{t_lin * 1e6:.0f} us = {100 * t_lin / t_full:.0f}% of the step, {gemm_bytes / t_lin / 1e9:.0f} GB/s "
+        f"({100 * gemm_bytes / t_lin / 1e9 / HBM_PEAK_GBS:.1f}% of 8 TB/s)")
+    return [row]
 
 
 def fp8_section(dev):
@@ -320,7 +401,8 @@ def main():
     del sets
     torch.cuda.empty_cache()
     if not args.no_extra:
-        for name, fn in (("prefill", prefill_section), ("fp8", fp8_section)):
+        for name, fn in (("prefill", prefill_section), ("fp8", fp8_section), ("vendor_ceiling", vendor_ceiling_section),
+                         ("decode_step", decode_step_section)):
             try:
                 extra[name] = fn(dev)
             except Exception as e:

@@ -65,6 +65,37 @@ def test_gptq_linear_method_end_to_end(device, desc_act, dtype):
     check_gemm_close(out3.reshape(6, -1), o.gemm_ref(a3.reshape(6, k), w_ref, bias), "gptq method 3-d input")
 
 
+def test_gptq_group_level_act_order_is_folded_at_load(device):
+    """g_idx that permutes whole groups (BASELINE config 3's wording): the method gathers the scale rows at load time and
+    runs without any activation reorder; results equal the oracle's act_order semantics."""
+    from vllm_amd.layers.linear import LinearBase
+    from vllm_amd.layers.quantization import get_quantization_config
+    k, n = 2048, 256
+    cfg = get_quantization_config("gptq_marlin").from_config(dict(bits=4, group_size=128, desc_act=True, sym=True))
+    case = o.make_w4a16_case(k, n, 128, act_order=True, group_level_perm=True, seed=31)
+    layer = LinearBase(k, n, quant_config=cfg, params_dtype=torch.bfloat16, return_bias=False).to(device)
+    layer.qweight.data.copy_(to_dev(case["qweight"], device))
+    layer.scales.data.copy_(to_dev(case["scales"], device, torch.bfloat16))
+    layer.g_idx.data.copy_(to_dev(case["g_idx"], device))
+    layer.process_weights_after_loading()
+    assert layer.quant_method.kernel.act_order_folded
+    assert layer.g_idx.numel() == 0 and layer.g_idx_sort_indices.numel() == 0
+    w_ref = o.case_w_ref(case)
+    for m in (2, 16, 100):
+        a = _acts(m, k, seed=m)
+        check_gemm_close(layer(a.to(device)), o.gemm_ref(a, w_ref), f"folded act_order m={m}")
+    # a row-level permutation is not folded
+    case2 = o.make_w4a16_case(k, n, 128, act_order=True, seed=32)
+    layer2 = LinearBase(k, n, quant_config=cfg, params_dtype=torch.bfloat16, return_bias=False).to(device)
+    layer2.qweight.data.copy_(to_dev(case2["qweight"], device))
+    layer2.scales.data.copy_(to_dev(case2["scales"], device, torch.bfloat16))
+    layer2.g_idx.data.copy_(to_dev(case2["g_idx"], device))
+    layer2.process_weights_after_loading()
+    assert not layer2.quant_method.kernel.act_order_folded and layer2.g_idx_sort_indices.numel() == k
+    a = _acts(9, k, seed=1)
+    check_gemm_close(layer2(a.to(device)), o.gemm_ref(a, o.case_w_ref(case2)), "row-level act_order")
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_awq_linear_method_end_to_end(device, dtype):
     """AutoAWQ checkpoint (weights and zero points packed along N with the AWQ interleave) through AWQMarlinConfig ->

@@ -10,21 +10,23 @@ int w4a16_decode2_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* co
 int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
                          const int32_t* perm, const void* bias, void* c, float* c_tmp, int32_t* counters,
                          int64_t counter_ints, int M, int N, int K, int dtype, hipStream_t s);
+int w4a16_prefill_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* counter_ints);
 int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
-                         const void* bias, void* c, int M, int N, int K, int dtype, hipStream_t s);
+                         const void* bias, void* c, float* c_tmp, int32_t* counters, int64_t counter_ints, int M, int N,
+                         int K, int dtype, hipStream_t s);
 
 constexpr int64_t DECODE_MAX_M = 32;
 static int g_decode_impl = -1;  // -1: automatic, 0: LDS-staged activations (w4a16_decode2.hip), 1: register-resident (w4a16_decode.hip)
 
 // Measured on MI355X (Llama-3-8B shapes): staging the activations once per workgroup in LDS (one independent task
-// per wavefront, no barrier in the K loop) wins everywhere except for M > 2 on wide layers (many n-tiles per compute
+// per wavefront, no barrier in the K loop) wins everywhere except for 2 < M <= 16 on wide layers (many n-tiles per compute
 // unit), where the register-resident kernel, whose wavefronts walk over n-tiles with their slice of the activations
 // held in registers, is slightly ahead.
 static int decode_impl_for(int64_t size_m, int64_t size_n, int64_t lda) {
   // the LDS-staged kernel addresses A through a 32-bit buffer offset
   if (size_m * lda * 2 >= (1ll << 31)) return 1;
   if (g_decode_impl >= 0) return g_decode_impl;
-  return (size_n <= 8192 || size_m <= 2) ? 0 : 1;
+  return (size_n <= 8192 || size_m <= 2 || size_m > 16) ? 0 : 1;
 }
 
 static int check_shape(int64_t size_m, int64_t size_n, int64_t size_k) {
@@ -63,7 +65,7 @@ extern "C" int vaq_w4a16_gemm_workspace(int64_t size_m, int64_t size_n, int64_t 
     return VAQ_OK;
   }
   if (has_perm) *a_tmp_bytes = (size_t)size_m * (size_t)size_k * 2;
-  return VAQ_OK;
+  return w4a16_prefill_workspace((int)size_m, (int)size_n, (int)size_k, c_tmp_bytes, counter_ints);
 }
 
 extern "C" int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
@@ -116,7 +118,8 @@ extern "C" int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, cons
     a_eff = a_tmp;
     lda_eff = size_k;
   }
-  return w4a16_prefill_launch(a_eff, lda_eff, b, scales, zeros, bias, c, (int)size_m, (int)size_n, (int)size_k, dtype, s);
+  return w4a16_prefill_launch(a_eff, lda_eff, b, scales, zeros, bias, c, c_tmp, counters, counter_ints, (int)size_m,
+                              (int)size_n, (int)size_k, dtype, s);
 }
 
 // Benchmark / tuning aid, not part of the drop-in surface: choose the decode implementation (-1 = automatic, 0 = LDS-staged

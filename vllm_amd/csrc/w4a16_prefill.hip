@@ -28,7 +28,9 @@ struct PrefillParams {
   const uint32_t* zeros;
   const uint16_t* bias;
   uint16_t* c;
-  int M, N, K, G, NT;
+  float* c_tmp;        // fp32 partial tiles when K is split over workgroups (SK > 1)
+  int32_t* counters;   // arrival counters, zero on entry, left zero
+  int M, N, K, G, NT, SK;
 };
 
 constexpr int PF_BK = 64;
@@ -444,10 +446,14 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
   using TT = std::true_type;
   using FF = std::false_type;
 
-  // ---- prologue: activation tiles of steps 0 and 1, weights of step 0 (group 0, half 0) ----
-  issue_a(0, 0);
-  issue_a(1, 1);
-  load_w(0);
+  // K may be split over blockIdx.y: this workgroup covers the groups [g_lo, g_hi)
+  const int split = blockIdx.y;
+  const int g_lo = (int)(((int64_t)p.G * split) / p.SK), g_hi = (int)(((int64_t)p.G * (split + 1)) / p.SK);
+
+  // ---- prologue: activation tiles of the first two steps, weights of the first step (group g_lo, half 0) ----
+  issue_a(2 * g_lo, 0);
+  issue_a(2 * g_lo + 1, 1);
+  load_w(g_lo);
   advance_w();
   store_w0();
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -460,7 +466,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
   auto sync_step = [&](auto n_c) {
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(decltype(n_c)::value) : "memory");
   };
-  for (int g = 0; g + 1 < p.G; ++g) {
+  for (int g = g_lo; g + 1 < g_hi; ++g) {
     // even step 2g: dequantise (g, half 1) for step 2g+1; request the tile of step 2g+2 and the words of group g+1
     load_w(g + 1);
     fused_step(a_cur, 0, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 2, 1);
@@ -477,6 +483,49 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
   sync_step(std::integral_constant<int, 0>{});
   a_cur = nxt(a_cur);
   fused_step(a_cur, 1, FF{}, FF{}, 0, 0, 0);
+
+  // ---- split K: hand the partial tile over; the last of the SK workgroups to arrive sums them in split order ----
+  if (p.SK > 1) {
+    // 16-byte buffer stores / loads with the sc1 cache-policy bit (device scope: written through to, and read from,
+    // memory that all XCDs share -- each XCD has its own L2).  One unit of NV4 KiB per (tile, wavefront).
+    constexpr int NV4 = WMB * WNB * 4;                     // 16-byte pieces per lane
+    constexpr int SC1 = 16;
+    const uint32_t unit = (uint32_t)((t * NW + wave) * NV4) * 1024u;           // bytes
+    const uint32_t split_stride = (uint32_t)total * (uint32_t)(NW * NV4) * 1024u;
+    const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(p.c_tmp, 0, (int)(split_stride * (uint32_t)p.SK), 0x00020000);
+#pragma unroll
+    for (int i = 0; i < WMB; ++i)
+#pragma unroll
+      for (int j = 0; j < WNB; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), rt, lane * 16,
+                                                 (int)(split * split_stride + unit + ((i * WNB + j) * 4 + q) * 1024), SC1);
+        }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // partial tile acknowledged before the counter moves
+    int32_t* ctr = p.counters + (int64_t)t * NW + wave;
+    int old = 0;
+    if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    old = __shfl(old, 0);
+    if (old != p.SK - 1) return;
+#pragma unroll
+    for (int i = 0; i < WMB; ++i)
+#pragma unroll
+      for (int j = 0; j < WNB; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          v4f sum = {0.f, 0.f, 0.f, 0.f};
+          for (int s2 = 0; s2 < p.SK; ++s2) {             // fixed order: deterministic
+            const v4u r = __builtin_amdgcn_raw_buffer_load_b128(
+                rt, lane * 16, (int)(s2 * split_stride + unit + ((i * WNB + j) * 4 + q) * 1024), SC1);
+            sum += __builtin_bit_cast(v4f, r);
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = sum[e];
+        }
+    if (lane == 0) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
 
   // ---- epilogue: four consecutive accumulator registers = four consecutive n of one row ----
 #pragma unroll
@@ -546,7 +595,7 @@ static int launch_prefill2(const PrefillParams& p, hipStream_t s) {
     attr_done = true;
   }
   const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
-  hipLaunchKernelGGL(kern, dim3(tiles), dim3(WAVES_M * WAVES_N * 64), lds, s, p);
+  hipLaunchKernelGGL(kern, dim3(tiles, p.SK), dim3(WAVES_M * WAVES_N * 64), lds, s, p);
   return VAQ_OK;
 }
 
@@ -568,28 +617,73 @@ static int dispatch_tile(const PrefillParams& p, int tile, hipStream_t s) {
   return VAQ_ERR_UNSUPPORTED;
 }
 
-static int g_force_tile = -1;
+static int g_force_tile = -1, g_force_split = 0;
 
-static int pick_tile(int M, int N, int64_t lda) {
+static int pick_tile(int M, int N, bool direct_ok) {
   if (g_force_tile >= 0) return g_force_tile;
-  const bool direct_ok = (uint64_t)M * (uint64_t)lda * 2 < (1ull << 32);
-  if (direct_ok) {
-    const int cus2 = num_cus_current_device();
-    auto tiles2 = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    // measured: the 256x256 / 8-wavefront tile wins as soon as it fills ~60 % of the compute units
-    if (tiles2(256, 256) * 10 >= cus2 * 6) return 10;
-    if (tiles2(128, 128) * 2 >= cus2) return 12;
-    return 14;
-  }
   const int cus = num_cus_current_device();
   auto tiles = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+  if (direct_ok) {
+    // measured: the 256x256 / 8-wavefront tile wins as soon as it fills ~60 % of the compute units
+    if (tiles(256, 256) * 10 >= cus * 6) return 10;
+    if (tiles(128, 128) >= cus) return 12;
+    return 14;                                               // with K split over workgroups when it leaves units idle
+  }
   if (tiles(256, 256) >= cus) return 0;
   if (tiles(128, 128) >= cus) return 1;
   return 2;
 }
 
+struct PrefillPlan {
+  int tile, sk, bm, bn, nw;
+  int64_t tiles;
+};
+
+// Tile shape and K split for a problem.  K is split (direct-to-LDS tiles only) when the output tiles alone leave
+// compute units idle: as many splits as bring the workgroup count to about two per compute unit, at most 8, every
+// split at least 8 groups (16 K steps) long, 32 groups when the tiles already fill the device -- measured on the Llama
+// shapes for M = 48 .. 512.
+static PrefillPlan plan_prefill(int M, int N, int K, bool direct_ok) {
+  PrefillPlan pl;
+  pl.tile = pick_tile(M, N, direct_ok);
+  switch (pl.tile) {
+    case 10: pl.bm = 256; pl.bn = 256; pl.nw = 8; break;
+    case 11: pl.bm = 256; pl.bn = 256; pl.nw = 4; break;
+    case 12: pl.bm = 128; pl.bn = 128; pl.nw = 4; break;
+    case 13: pl.bm = 128; pl.bn = 256; pl.nw = 8; break;
+    case 14: pl.bm = 64; pl.bn = 128; pl.nw = 4; break;
+    default: pl.bm = 0; pl.bn = 0; pl.nw = 0; break;
+  }
+  pl.sk = 1;
+  pl.tiles = 0;
+  if (pl.bm == 0) return pl;
+  pl.tiles = (int64_t)((M + pl.bm - 1) / pl.bm) * ((N + pl.bn - 1) / pl.bn);
+  const int cus = num_cus_current_device();
+  const int G = K / 128;
+  int sk = 1;
+  if (pl.tiles < 2 * (int64_t)cus) {
+    sk = (int)((2 * (int64_t)cus) / pl.tiles);
+    if (sk > 8) sk = 8;
+    const int min_groups = pl.tiles < cus ? 8 : 32;     // a device already full of tiles only splits a very long K
+    if (sk > G / min_groups) sk = G / min_groups;
+    if (sk < 1) sk = 1;
+  }
+  if (g_force_split > 0) sk = g_force_split <= G ? g_force_split : G;
+  while (sk > 1 && (uint64_t)sk * (uint64_t)pl.tiles * pl.bm * pl.bn * 4 >= (1ull << 32)) --sk;   // 32-bit buffer offsets
+  pl.sk = sk;
+  return pl;
+}
+
+int w4a16_prefill_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* counter_ints) {
+  const PrefillPlan pl = plan_prefill(M, N, K, true);
+  *c_tmp_bytes = pl.sk > 1 ? (size_t)pl.sk * (size_t)pl.tiles * pl.bm * pl.bn * sizeof(float) : 0;
+  *counter_ints = pl.sk > 1 ? (size_t)pl.tiles * pl.nw : 0;
+  return VAQ_OK;
+}
+
 int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
-                         const void* bias, void* c, int M, int N, int K, int dtype, hipStream_t s) {
+                         const void* bias, void* c, float* c_tmp, int32_t* counters, int64_t counter_ints, int M, int N,
+                         int K, int dtype, hipStream_t s) {
   PrefillParams p;
   p.a = (const uint16_t*)a;
   p.lda = lda;
@@ -598,14 +692,20 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
   p.zeros = (const uint32_t*)zeros;
   p.bias = (const uint16_t*)bias;
   p.c = (uint16_t*)c;
+  p.c_tmp = c_tmp;
+  p.counters = counters;
   p.M = M; p.N = N; p.K = K;
   p.G = K / 128;
   p.NT = N / 16;
-  const int tile = pick_tile(M, N, lda);
+  const bool direct_ok = (uint64_t)M * (uint64_t)lda * 2 < (1ull << 32);
+  PrefillPlan pl = plan_prefill(M, N, K, direct_ok);
+  // without scratch from the caller (or with too small a counter array) the unsplit kernel still gives the result
+  if (pl.sk > 1 && (c_tmp == nullptr || counters == nullptr || counter_ints < pl.tiles * pl.nw)) pl.sk = 1;
+  p.SK = pl.sk;
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
-  if (bf16) rc = zp ? dispatch_tile<true, true>(p, tile, s) : dispatch_tile<true, false>(p, tile, s);
-  else rc = zp ? dispatch_tile<false, true>(p, tile, s) : dispatch_tile<false, false>(p, tile, s);
+  if (bf16) rc = zp ? dispatch_tile<true, true>(p, pl.tile, s) : dispatch_tile<true, false>(p, pl.tile, s);
+  else rc = zp ? dispatch_tile<false, true>(p, pl.tile, s) : dispatch_tile<false, false>(p, pl.tile, s);
   if (rc != VAQ_OK) return rc;
   VAQ_CHECK_LAUNCH("w4a16_gemm(prefill)");
   return VAQ_OK;
@@ -615,4 +715,8 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
 
 // Benchmark / tuning aid, not part of the drop-in surface: force the prefill tile (-1 = automatic,
 // 0 = 256x256, 1 = 128x128, 2 = 64x128).  Process-global and not thread-safe.
-extern "C" void vaq_debug_set_prefill_tile(int tile) { vaq::g_force_tile = tile; }
+extern "C" void vaq_debug_set_prefill_tile(int tile) {
+  // tile < 0: automatic; otherwise tile id + 100 * (forced K split, 0 = automatic)
+  vaq::g_force_tile = tile < 0 ? -1 : tile % 100;
+  vaq::g_force_split = tile < 0 ? 0 : tile / 100;
+}

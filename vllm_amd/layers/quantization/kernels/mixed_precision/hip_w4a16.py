@@ -50,7 +50,27 @@ class HipW4A16LinearKernel(MPLinearKernel):
         if self.w_zp_name is None:
             self.w_zp_name = "w_zp"
 
-        if c.has_g_idx:
+        # act_order whose g_idx moves whole groups (every run of `group_size` consecutive rows carries one group id, each
+        # id once) needs no row permutation at all: the rows are already grouped, only group j's scales / zero points
+        # sit in row g_idx[j * group_size].  Gather those rows once here and run the layer as if it had no act_order:
+        # same weights, no activation reorder on any call.
+        group_ids = None
+        if c.has_g_idx and c.group_size > 0 and size_k % c.group_size == 0:
+            g_idx_full = getattr(layer, self.w_gidx_name).data
+            blocks = g_idx_full.reshape(size_k // c.group_size, c.group_size)
+            first = blocks[:, 0]
+            if bool((blocks == first[:, None]).all()) and first.numel() == getattr(layer, self.w_s_name).shape[0] and \
+                    bool((torch.bincount(first.long(), minlength=first.numel()) == 1).all()):
+                group_ids = first.long()
+        self.act_order_folded = group_ids is not None
+
+        if group_ids is not None:
+            getattr(layer, self.w_s_name).data = getattr(layer, self.w_s_name).data[group_ids].contiguous()
+            if c.zero_points:
+                getattr(layer, self.w_zp_name).data = getattr(layer, self.w_zp_name).data[group_ids].contiguous()
+            setattr(layer, self.w_gidx_name, marlin_make_empty_g_idx(device))
+            layer.g_idx_sort_indices = marlin_make_empty_g_idx(device)
+        elif c.has_g_idx:
             g_idx, g_idx_sort_indices = marlin_sort_g_idx(getattr(layer, self.w_gidx_name))
             self._transform_param(layer, self.w_gidx_name, lambda _: g_idx)
             layer.g_idx_sort_indices = g_idx_sort_indices
