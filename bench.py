@@ -335,7 +335,10 @@ def counter_pass(dev):
 def cpu_baseline(budget_s: float = 15.0):
     """The reference's CPU-runnable path, restated by the oracle: unpack int4 -> (q - 8).to(bf16) * s -> torch.matmul,
     dequantisation included in every call (the reference path dequantises per call).  Bounded sample of the headline
-    workload: whole steps (the 12 GEMMs) are repeated until about `budget_s` seconds of CPU work have been timed."""
+    workload: whole steps (the 12 GEMMs) are repeated until about `budget_s` seconds of CPU work have been timed.
+    Two smaller side figures ride along in the sample text: the same GEMMs with weights dequantised beforehand (matmul
+    only), and the FP8 path (per-token quant + fp32 scaled matmul, the reference's `baseline_scaled_mm`) on one layer."""
+    from oracle import fp8 as of
     from oracle import w4a16 as o
     threads = torch.get_num_threads()
     rng = np.random.default_rng(0)
@@ -357,9 +360,34 @@ def cpu_baseline(budget_s: float = 15.0):
                 assert out.shape == (m, n)
         steps_done += 1
     log(f"[cpu baseline] {steps_done} step(s) of 12 GEMMs in {total_t:.1f} s on {threads} threads: {total_b / total_t / 1e9:.3f} GB/s")
+    # matmul only (weights dequantised once, outside the timed region): one step
+    pre_t, pre_b = 0.0, 0
+    for (k, n, qweight, scales) in layers:
+        w = o.dequantize(o.unpack_rows(qweight, 4), scales, 8, GROUP)
+        for m in DECODE_MS:
+            a = torch.randn(m, k).to(torch.bfloat16)
+            t0 = time.perf_counter()
+            o.gemm_ref_like_reference(a, w)
+            pre_t += time.perf_counter() - t0
+            pre_b += w4a16_bytes(m, k, n)
+        del w
+    log(f"[cpu baseline] matmul only, weights dequantised beforehand: {pre_b / pre_t / 1e9:.3f} GB/s (one step, {pre_t:.2f} s)")
+    # FP8 path on the 4096 x 4096 layer, M = 16
+    k, n, m = 4096, 4096, 16
+    wq, ws = of.make_fp8_weight(n, k)
+    a = torch.randn(m, k).to(torch.bfloat16)
+    t0 = time.perf_counter()
+    reps = 3
+    for _ in range(reps):
+        aq, sa = of.ref_dynamic_per_token_quant(a)
+        of.scaled_mm_ref(aq, wq.t(), sa, ws, torch.bfloat16, None, order="baseline")
+    f8_t = (time.perf_counter() - t0) / reps
+    log(f"[cpu baseline] FP8 quant + scaled matmul, M={m} K={k} N={n}: {f8_t * 1e3:.1f} ms = {fp8_mm_bytes(m, k, n, False) / f8_t / 1e9:.3f} GB/s")
     return dict(value=round(total_b / total_t / 1e9, 4), unit="GB/s", cores=threads, kind="port",
                 sample=f"{steps_done} full step(s) of the headline workload (12 GEMMs each) through the oracle: unpack + "
-                       f"dequantise (bf16) + torch.matmul per call, {total_t:.1f} s of CPU time")
+                       f"dequantise (bf16) + torch.matmul per call, {total_t:.1f} s of CPU time; side figures: matmul only "
+                       f"with pre-dequantised weights {pre_b / pre_t / 1e9:.3f} GB/s (one step); FP8 per-token quant + "
+                       f"scaled matmul at M={m}, {k}x{n}: {fp8_mm_bytes(m, k, n, False) / f8_t / 1e9:.3f} GB/s")
 
 
 # --------------------------------------------------------------------------------------------- main

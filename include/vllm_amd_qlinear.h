@@ -146,6 +146,21 @@ int vaq_fp8_scaled_mm(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t l
                       const float* sb, int64_t sb_count, const void* bias, void* out, int64_t ldc, int out_dtype,
                       int64_t size_m, int64_t size_n, int64_t size_k, void* stream);
 
+/*
+ * The same GEMM with caller-provided scratch, which lets the tile kernel split K over workgroups when M and N alone
+ * leave compute units idle (a few hundred tokens on the narrow layers).  Sizes come from the query; both may be 0.
+ *   c_tmp     fp32 partial tiles, 16-byte aligned, contents irrelevant on entry
+ *   counters  int32 arrival counters that must be ZERO on entry and are left zero (calls sharing them must not overlap)
+ * With NULL / too small scratch the call behaves exactly like vaq_fp8_scaled_mm.  (The reference's cutlass_scaled_mm has
+ * no workspace argument: CUTLASS allocates its own, scaled_mm_entry.cu.)
+ */
+int vaq_fp8_scaled_mm_workspace(int64_t size_m, int64_t size_n, int64_t size_k, size_t* c_tmp_bytes,
+                                size_t* counter_ints);
+int vaq_fp8_scaled_mm_ws(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t ldb, const float* sa, int64_t sa_count,
+                         const float* sb, int64_t sb_count, const void* bias, void* out, int64_t ldc, int out_dtype,
+                         int64_t size_m, int64_t size_n, int64_t size_k, float* c_tmp, int64_t c_tmp_bytes,
+                         int32_t* counters, int64_t counter_ints, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

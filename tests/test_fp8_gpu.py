@@ -198,6 +198,23 @@ def test_scaled_mm_exact_small_integers(device):
         assert torch.equal(out.cpu().float(), a @ w.t()), (m, n, k)
 
 
+def test_scaled_mm_split_k_exact_and_deterministic(device):
+    """Few output tiles and a long K: the tile kernel splits K over workgroups (fp32 partial tiles through the op's
+    scratch, arrival counters left zero).  Small-integer operands make every partial sum exact, so the split result
+    must equal the integer GEMM; two runs must agree bit for bit."""
+    import vllm_amd._custom_ops as ops
+    g = torch.Generator().manual_seed(1)
+    for m, n, k in ((200, 256, 14336), (96, 128, 8192 + 64), (257, 384, 16384)):
+        a = torch.randint(-2, 3, (m, k), generator=g).float()
+        w = torch.randint(-1, 2, (n, k), generator=g).float()
+        args = (a.to(torch.float8_e4m3fn).to(device), w.to(torch.float8_e4m3fn).to(device).t(),
+                torch.ones(m, 1, device=device), torch.ones(n, 1, device=device), torch.float16)
+        out = ops.cutlass_scaled_mm(*args)
+        assert torch.equal(out.cpu().float(), a @ w.t()), (m, n, k)
+        assert torch.equal(out, ops.cutlass_scaled_mm(*args))
+        assert bool((ops._fp8_counters(torch.device(device)) == 0).all()), "arrival counters not restored to zero"
+
+
 @pytest.mark.parametrize("k,n", LLAMA_SHAPES)
 def test_config4_llama_shapes(device, k, n):
     """BASELINE config 4: M in {1, 16, 256, 4096}, per-token x per-channel (+bias); activations quantised on the GPU

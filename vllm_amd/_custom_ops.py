@@ -394,10 +394,39 @@ def _scaled_mm_impl(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor, a_scale
     if a.size(0) == 0:
         return
     lib = _lib.load()
-    with torch.cuda.device(a.device):
-        _lib.check(lib.vaq_fp8_scaled_mm(_ptr(a), a.stride(0), _ptr(b), b.stride(1), _ptr(a_scales), a_scales.numel(),
-                                         _ptr(b_scales), b_scales.numel(), _ptr(bias), _ptr(out), out.stride(0),
-                                         _dtype_tag(out.dtype), a.size(0), b.size(1), a.size(1), _stream(a.device)))
+    dev = a.device
+    with torch.cuda.device(dev):
+        # scratch for the K split of mid-sized M: partial tiles from the caching allocator (capture-safe), arrival
+        # counters from one zeroed per-device array that the kernel leaves zero
+        n_ctmp, n_cnt = ctypes.c_size_t(), ctypes.c_size_t()
+        _lib.check(lib.vaq_fp8_scaled_mm_workspace(a.size(0), b.size(1), a.size(1), ctypes.byref(n_ctmp),
+                                                   ctypes.byref(n_cnt)))
+        c_tmp = counters = None
+        if n_ctmp.value:
+            counters = _fp8_counters(dev)
+            if counters.numel() >= n_cnt.value:
+                c_tmp = torch.empty((n_ctmp.value // 4,), dtype=torch.float32, device=dev)
+            else:
+                counters = None
+        _lib.check(lib.vaq_fp8_scaled_mm_ws(_ptr(a), a.stride(0), _ptr(b), b.stride(1), _ptr(a_scales), a_scales.numel(),
+                                            _ptr(b_scales), b_scales.numel(), _ptr(bias), _ptr(out), out.stride(0),
+                                            _dtype_tag(out.dtype), a.size(0), b.size(1), a.size(1), _ptr(c_tmp),
+                                            n_ctmp.value if c_tmp is not None else 0, _ptr(counters),
+                                            counters.numel() if counters is not None else 0, _stream(dev)))
+
+
+_FP8_COUNTERS: dict[int, torch.Tensor] = {}
+
+
+def _fp8_counters(dev: torch.device) -> torch.Tensor:
+    """One zeroed int32 array per device for the FP8 GEMM's K split (the reference's CUTLASS path owns its workspace
+    too).  Created on first use; calls that use it must not overlap on different streams."""
+    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    t = _FP8_COUNTERS.get(idx)
+    if t is None:
+        t = torch.zeros(16384, dtype=torch.int32, device=dev)
+        _FP8_COUNTERS[idx] = t
+    return t
 
 
 # ============================================================================ registration

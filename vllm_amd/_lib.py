@@ -40,6 +40,11 @@ _SIGNATURES = {
                                       c_void_p]),
     "vaq_fp8_scaled_mm": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
                                   c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p]),
+    "vaq_fp8_scaled_mm_workspace": (c_int, [c_int64, c_int64, c_int64, ctypes.POINTER(ctypes.c_size_t),
+                                            ctypes.POINTER(ctypes.c_size_t)]),
+    "vaq_fp8_scaled_mm_ws": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
+                                     c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p,
+                                     c_int64, c_void_p]),
 }
 # tuning aids exported by the library but not part of the drop-in header
 _DEBUG_SIGNATURES = {

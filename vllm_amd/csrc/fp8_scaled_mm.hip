@@ -33,6 +33,9 @@ struct Fp8MMParams {
   uint16_t* out;
   int64_t ldc;
   int M, N, K;
+  float* c_tmp = nullptr;        // fp32 partial tiles when K is split over workgroups (SK > 1)
+  int32_t* counters = nullptr;   // arrival counters, zero on entry, left zero
+  int SK = 1;
 };
 
 __device__ inline v16f mfma_fp8_32(v8i a, v8i b, v16f c) {
@@ -417,15 +420,19 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
 
   // Invariant at the start of step s: the tile of step s complete in LDS, the tiles of steps s+1 .. s+NST-2 requested,
   // stage (s-1) % NST free.  The requests of step s+NST-1 go out first thing in step s.
-  const int steps = p.K / 64;
+  // K may be split over blockIdx.y: this workgroup covers the 64-byte steps [s_lo, s_hi)
+  const int all_steps = p.K / 64;
+  const int split = blockIdx.y;
+  const int s_lo = (int)(((int64_t)all_steps * split) / p.SK), s_hi = (int)(((int64_t)all_steps * (split + 1)) / p.SK);
+  const int steps = s_hi - s_lo;
   if (steps >= NST) {
 #pragma unroll
-    for (int s0 = 0; s0 < NST - 1; ++s0) issue_loads(s0, s0);
+    for (int s0 = 0; s0 < NST - 1; ++s0) issue_loads(s_lo + s0, s0);
     sync_step(WAIT_STEADY{});           // tile 0 landed
     int cur = 0, dst = NST - 1;
     int step = 0;
     for (; step + NST - 1 < steps; ++step) {
-      issue_loads(step + NST - 1, dst);
+      issue_loads(s_lo + step + NST - 1, dst);
       compute(cur);
       sync_step(WAIT_STEADY{});
       cur = cur + 1 == NST ? 0 : cur + 1;
@@ -439,11 +446,54 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
   } else {
     // short K: no ring, one tile at a time
     for (int step = 0; step < steps; ++step) {
-      issue_loads(step, 0);
+      issue_loads(s_lo + step, 0);
       sync_step(WAIT_NONE{});
       compute(0);
       sync_step(WAIT_NONE{});
     }
+  }
+
+  // ---- split K: hand the partial tile over; the last of the SK workgroups to arrive sums them in split order.
+  // 16-byte buffer stores / loads with the sc1 cache-policy bit (device scope: each XCD has its own L2), one unit of
+  // NV4 KiB per (tile, wavefront), one arrival counter per unit. ----
+  if (p.SK > 1) {
+    constexpr int NV4 = WMB * WNB * 4;
+    constexpr int SC1 = 16;
+    const uint32_t unit = (uint32_t)((t * NW + wave) * NV4) * 1024u;
+    const uint32_t split_stride = (uint32_t)total * (uint32_t)(NW * NV4) * 1024u;
+    const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(p.c_tmp, 0, (int)(split_stride * (uint32_t)p.SK), 0x00020000);
+#pragma unroll
+    for (int i = 0; i < WMB; ++i)
+#pragma unroll
+      for (int j = 0; j < WNB; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), rt, lane * 16,
+                                                 (int)(split * split_stride + unit + ((i * WNB + j) * 4 + q) * 1024), SC1);
+        }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // partial tile acknowledged before the counter moves
+    int32_t* ctr = p.counters + (int64_t)t * NW + wave;
+    int old = 0;
+    if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    old = __shfl(old, 0);
+    if (old != p.SK - 1) return;
+#pragma unroll
+    for (int i = 0; i < WMB; ++i)
+#pragma unroll
+      for (int j = 0; j < WNB; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          v4f sum = {0.f, 0.f, 0.f, 0.f};
+          for (int s2 = 0; s2 < p.SK; ++s2) {             // fixed order: deterministic
+            const v4u r = __builtin_amdgcn_raw_buffer_load_b128(
+                rt, lane * 16, (int)(s2 * split_stride + unit + ((i * WNB + j) * 4 + q) * 1024), SC1);
+            sum += __builtin_bit_cast(v4f, r);
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = sum[e];
+        }
+    if (lane == 0) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
   tile_epilogue<BF16_OUT, WMB, WNB>(p, acc, m0, n0, wm, wn, lane);
@@ -606,24 +656,66 @@ static int launch_tile3(const Fp8MMParams& p, hipStream_t s) {
     attr_done = true;
   }
   const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
-  hipLaunchKernelGGL(kern, dim3(tiles), dim3(WAVES_M * WAVES_N * 64), lds, s, p);
+  hipLaunchKernelGGL(kern, dim3(tiles, p.SK), dim3(WAVES_M * WAVES_N * 64), lds, s, p);
   return VAQ_OK;
 }
 
 static int g_fp8_tile3_cfg = 0;    // 0: automatic, -1: off (two-stage kernel), >0: a fixed tile shape (benchmarking)
 static int g_fp8_tile_impl = 0;   // 0: direct-to-LDS kernel when its preconditions hold, 1: always the register-staged kernel
 
+static int g_fp8_force_split = 0;
+
+struct Fp8TilePlan {
+  int cfg, sk, bm, bn, nw;
+  int64_t tiles;
+};
+
+// Tile shape and K split of the multi-stage kernel.  K is split when the output tiles alone leave compute units idle:
+// about two workgroups per compute unit, at most 8 splits, each at least 64 steps (4096 bytes of K) long -- measured at
+// M = 256: the FP8 steps are short, so the hand-over only pays on a long K (1.35x on K = 14336, a loss on K = 4096).
+static Fp8TilePlan plan_tile3(int M, int N, int K) {
+  const int cus = num_cus_current_device();
+  auto tiles = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+  Fp8TilePlan pl;
+  pl.cfg = g_fp8_tile3_cfg;
+  if (pl.cfg <= 0)
+    pl.cfg = tiles(256, 256) >= cus ? 1 : (tiles(128, 256) * 8 >= cus * 7 ? 7 : (tiles(128, 128) >= cus ? 3 : 4));
+  switch (pl.cfg) {
+    case 3: pl.bm = 128; pl.bn = 128; pl.nw = 4; break;
+    case 4: pl.bm = 64; pl.bn = 128; pl.nw = 4; break;
+    case 7: pl.bm = 128; pl.bn = 256; pl.nw = 8; break;
+    case 2: pl.bm = 256; pl.bn = 256; pl.nw = 4; break;
+    default: pl.bm = 256; pl.bn = 256; pl.nw = 8; break;
+  }
+  pl.tiles = tiles(pl.bm, pl.bn);
+  int sk = 1;
+  const int steps = K / 64;
+  if (pl.tiles < cus) {
+    sk = (int)((2 * (int64_t)cus) / pl.tiles);
+    if (sk > 8) sk = 8;
+    if (sk > steps / 64) sk = steps / 64;
+    if (sk < 1) sk = 1;
+    while (sk & (sk - 1)) --sk;       // a power of two (3 splits measured slower than 2)
+  }
+  if (g_fp8_force_split > 0) sk = g_fp8_force_split <= steps ? g_fp8_force_split : steps;
+  while (sk > 1 && (uint64_t)sk * (uint64_t)pl.tiles * pl.bm * pl.bn * 4 >= (1ull << 32)) --sk;   // 32-bit buffer offsets
+  pl.sk = sk;
+  return pl;
+}
+
 template <bool BF16_OUT>
-static int dispatch_tile(const Fp8MMParams& p, hipStream_t s) {
+static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t counter_ints, hipStream_t s) {
+  Fp8MMParams p = p_in;
   const bool direct_ok = g_fp8_tile_impl == 0 && p.K % 64 == 0 && (uint64_t)p.M * (uint64_t)p.lda < (1ull << 32) &&
                          (uint64_t)p.N * (uint64_t)p.ldb < (1ull << 32);
   if (direct_ok && g_fp8_tile_impl == 0 && g_fp8_tile3_cfg >= 0) {
-    const int cus3 = num_cus_current_device();
-    auto tiles3 = [&](int bm, int bn) { return (int64_t)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
-    int cfg = g_fp8_tile3_cfg;
-    if (cfg == 0)
-      cfg = tiles3(256, 256) >= cus3 ? 1 : (tiles3(128, 256) * 8 >= cus3 * 7 ? 7 : (tiles3(128, 128) * 2 >= cus3 ? 3 : 4));
-    switch (cfg) {
+    Fp8TilePlan pl = plan_tile3(p.M, p.N, p.K);
+    // without (enough) scratch from the caller the unsplit kernel still gives the result
+    if (pl.sk > 1 && (p.c_tmp == nullptr || p.counters == nullptr || counter_ints < pl.tiles * pl.nw ||
+                      c_tmp_bytes < (int64_t)pl.sk * pl.tiles * pl.bm * pl.bn * 4))
+      pl.sk = 1;
+    p.SK = pl.sk;
+    switch (pl.cfg) {
       case 1: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 5>(p, s);
       case 2: return launch_tile3<BF16_OUT, 256, 256, 2, 2, 5>(p, s);
       case 3: return launch_tile3<BF16_OUT, 128, 128, 2, 2, 5>(p, s);
@@ -634,6 +726,7 @@ static int dispatch_tile(const Fp8MMParams& p, hipStream_t s) {
       default: break;
     }
   }
+  p.SK = 1;
   if (direct_ok && p.K % F8_BK == 0) {
     const int cus2 = num_cus_current_device();
     auto tiles2 = [&](int bm, int bn) { return (int64_t)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
@@ -681,10 +774,37 @@ static bool dispatch_stream(const Fp8MMParams& p, hipStream_t s) {
 
 }  // namespace vaq
 
+extern "C" int vaq_fp8_scaled_mm_workspace(int64_t size_m, int64_t size_n, int64_t size_k, size_t* c_tmp_bytes,
+                                           size_t* counter_ints) {
+  using namespace vaq;
+  VAQ_CHECK_ARG(c_tmp_bytes && counter_ints, "fp8_scaled_mm_workspace: null output pointer");
+  VAQ_CHECK_ARG(size_m >= 0 && size_n > 0 && size_k > 0 && size_m < (1ll << 31) && size_n < (1ll << 31) &&
+                    size_k < (1ll << 31), "fp8_scaled_mm_workspace: bad shape M=%lld N=%lld K=%lld", (long long)size_m,
+                (long long)size_n, (long long)size_k);
+  *c_tmp_bytes = 0;
+  *counter_ints = 0;
+  if (size_m <= 32 || size_k % 64 != 0 || g_fp8_tile_impl != 0 || g_fp8_tile3_cfg < 0) return VAQ_OK;
+  const Fp8TilePlan pl = plan_tile3((int)size_m, (int)size_n, (int)size_k);
+  if (pl.sk > 1) {
+    *c_tmp_bytes = (size_t)pl.sk * (size_t)pl.tiles * pl.bm * pl.bn * sizeof(float);
+    *counter_ints = (size_t)pl.tiles * pl.nw;
+  }
+  return VAQ_OK;
+}
+
 extern "C" int vaq_fp8_scaled_mm(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t ldb, const float* sa,
                                  int64_t sa_count, const float* sb, int64_t sb_count, const void* bias, void* out,
                                  int64_t ldc, int out_dtype, int64_t size_m, int64_t size_n, int64_t size_k,
                                  void* stream) {
+  return vaq_fp8_scaled_mm_ws(a, lda, b, ldb, sa, sa_count, sb, sb_count, bias, out, ldc, out_dtype, size_m, size_n,
+                              size_k, nullptr, 0, nullptr, 0, stream);
+}
+
+extern "C" int vaq_fp8_scaled_mm_ws(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t ldb, const float* sa,
+                                    int64_t sa_count, const float* sb, int64_t sb_count, const void* bias, void* out,
+                                    int64_t ldc, int out_dtype, int64_t size_m, int64_t size_n, int64_t size_k,
+                                    float* c_tmp, int64_t c_tmp_bytes, int32_t* counters, int64_t counter_ints,
+                                    void* stream) {
   using namespace vaq;
   VAQ_CHECK_ARG(size_m >= 0 && size_n > 0 && size_k > 0, "fp8_scaled_mm: bad shape M=%lld N=%lld K=%lld",
                 (long long)size_m, (long long)size_n, (long long)size_k);
@@ -715,13 +835,16 @@ extern "C" int vaq_fp8_scaled_mm(const uint8_t* a, int64_t lda, const uint8_t* b
   p.bias = (const uint16_t*)bias;
   p.out = (uint16_t*)out; p.ldc = ldc;
   p.M = (int)size_m; p.N = (int)size_n; p.K = (int)size_k;
+  p.c_tmp = c_tmp;
+  p.counters = counters;
+  VAQ_CHECK_ARG(c_tmp == nullptr || ((uintptr_t)c_tmp % 16) == 0, "fp8_scaled_mm: c_tmp must be 16-byte aligned");
   hipStream_t s = (hipStream_t)stream;
   const bool bf16 = out_dtype == VAQ_BF16;
   bool done = false;
   const bool want_stream = g_force_fp8_path == 1 || (g_force_fp8_path == 0 && size_m <= 32);
   if (want_stream && size_m <= 32) done = bf16 ? dispatch_stream<true>(p, s) : dispatch_stream<false>(p, s);
   if (!done) {
-    int rc = bf16 ? dispatch_tile<true>(p, s) : dispatch_tile<false>(p, s);
+    int rc = bf16 ? dispatch_tile<true>(p, c_tmp_bytes, counter_ints, s) : dispatch_tile<false>(p, c_tmp_bytes, counter_ints, s);
     if (rc != VAQ_OK) return rc;
   }
   VAQ_CHECK_LAUNCH("fp8_scaled_mm");
@@ -732,6 +855,7 @@ extern "C" int vaq_fp8_scaled_mm(const uint8_t* a, int64_t lda, const uint8_t* b
 extern "C" void vaq_debug_set_fp8_config(int path, int gx) {
   vaq::g_force_fp8_path = path % 10;
   vaq::g_fp8_tile_impl = (path / 10) % 10;     // tens digit: 1 = force the register-staged tile kernel
-  vaq::g_fp8_tile3_cfg = path / 100 == 9 ? -1 : path / 100;   // hundreds digit: multi-stage tile shape (9 = off)
+  vaq::g_fp8_tile3_cfg = (path / 100) % 10 == 9 ? -1 : (path / 100) % 10;   // hundreds digit: multi-stage tile shape (9 = off)
+  vaq::g_fp8_force_split = path / 1000;                     // thousands: forced K split (0 = automatic)
   vaq::g_force_fp8_gx = gx;
 }
