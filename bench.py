@@ -205,6 +205,29 @@ def prefill_section(dev):
     return rows
 
 
+def fused_norm_quant_section(dev):
+    """RMSNorm + per-token FP8 quant in one pass (the step in front of the FP8 GEMM) against its HBM roofline, and the
+    unfused pair (torch rms_norm, then scaled_fp8_quant) beside it."""
+    import torch.nn.functional as F
+    import vllm_amd._custom_ops as ops
+    rows = []
+    gen = torch.Generator(device=dev).manual_seed(6)
+    for k in (4096, 14336):
+        w = (1.0 + 0.1 * torch.randn(k, device=dev, generator=gen)).to(torch.bfloat16)
+        for m in (16, 256, 4096):
+            x = torch.randn(m, k, device=dev, generator=gen).to(torch.bfloat16)
+            t = time_graph(lambda: [ops.rms_norm_dynamic_per_token_quant(x, w, 1e-5, torch.float8_e4m3fn) for _ in range(20)],
+                           iters=5, warmup=2, inner=20)
+            tu = time_graph(lambda: [ops.scaled_fp8_quant(F.rms_norm(x, (k,), w, 1e-5), use_per_token_if_dynamic=True) for _ in range(20)],
+                            iters=5, warmup=2, inner=20)
+            b = 3 * m * k + 4 * m + 2 * k
+            rows.append(dict(kind="rms_norm_dynamic_per_token_fp8_quant", hidden=k, M=m, us=t * 1e6, GBps=b / t / 1e9,
+                             hbm_frac=b / t / 1e9 / HBM_PEAK_GBS, unfused_us=tu * 1e6, cold=False))
+            log(f"[norm+quant  ] hidden={k:5d} M={m:4d}: {t * 1e6:6.1f} us {b / t / 1e9:6.0f} GB/s ({100 * b / t / 1e9 / HBM_PEAK_GBS:4.1f}% of 8 TB/s) | "
+                f"unfused rms_norm + quant {tu * 1e6:6.1f} us")
+    return rows
+
+
 def vendor_ceiling_section(dev):
     """Practical ceilings on the same box and shapes: the vendor GEMM library through torch (bf16 `matmul`, row-wise
     scaled FP8 `_scaled_mm`) at M = 4096.  Context for the MFMA fractions above, not part of the product path."""
@@ -429,7 +452,8 @@ def main():
     del sets
     torch.cuda.empty_cache()
     if not args.no_extra:
-        for name, fn in (("prefill", prefill_section), ("fp8", fp8_section), ("vendor_ceiling", vendor_ceiling_section),
+        for name, fn in (("prefill", prefill_section), ("fp8", fp8_section), ("fused_norm_quant", fused_norm_quant_section),
+                         ("vendor_ceiling", vendor_ceiling_section),
                          ("decode_step", decode_step_section)):
             try:
                 extra[name] = fn(dev)

@@ -147,6 +147,20 @@ int vaq_fp8_scaled_mm(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t l
                       int64_t size_m, int64_t size_n, int64_t size_k, void* stream);
 
 /*
+ * RMSNorm (+ residual add) fused with dynamic per-token FP8 quantisation.  Replaces
+ * `rms_norm_dynamic_per_token_quant(Tensor! result, Tensor input, Tensor weight, Tensor! scale, float epsilon,
+ * Tensor? scale_ub, Tensor!? residual)` (csrc/torch_bindings.cpp:216-221; device code
+ * csrc/quantization/fused_kernels/fused_layernorm_dynamic_per_token_quant.cu, layernorm_utils.cuh:17-130) for FP8 output.
+ *   out       e4m3fn [tokens, hidden] contiguous;  scales fp32 [tokens]
+ *   input     [tokens, hidden] F16/BF16, row stride in_stride elements;  weight [hidden] same dtype
+ *   scale_ub  optional fp32 scalar (device);  residual optional [tokens, hidden] contiguous, updated in place with
+ *             input + residual
+ */
+int vaq_rms_norm_dynamic_per_token_fp8_quant(uint8_t* out, float* scales, const void* input, int64_t in_stride,
+                                             const void* weight, const float* scale_ub, float epsilon, void* residual,
+                                             int dtype, int64_t tokens, int64_t hidden, void* stream);
+
+/*
  * The same GEMM with caller-provided scratch, which lets the tile kernel split K over workgroups when M and N alone
  * leave compute units idle (a few hundred tokens on the narrow layers).  Sizes come from the query; both may be 0.
  *   c_tmp     fp32 partial tiles, 16-byte aligned, contents irrelevant on entry

@@ -135,6 +135,36 @@ def scaled_mm_ref(a_q: torch.Tensor, b_q: torch.Tensor, scale_a: torch.Tensor, s
     raise ValueError(order)
 
 
+def ref_rms_norm_dynamic_per_token_quant(x: torch.Tensor, weight: torch.Tensor, eps: float,
+                                         scale_ub: torch.Tensor | None = None, residual: torch.Tensor | None = None):
+    """Fused RMSNorm + per-token FP8 quant, operation order of
+    csrc/quantization/fused_kernels/layernorm_utils.cuh:17-130 (the reference's own test oracle is the unfused
+    composition, tests/kernels/core/test_fused_quant_layernorm.py:40-75):
+
+        xf = float(x) (+ float(residual));  new_residual = T(xf)
+        rms = rsqrt(sum(xf*xf)/hidden + eps)             # the sum here is accumulated in fp64, then rounded
+        y = float(T(T(xf * rms) * weight));  s = max(min(max|y|, ub)/448, 1/(448*512));  q = cast(clamp(y / s))
+
+    Returns (q e4m3fn, scales [tokens,1] fp32, new_residual or None).  The order of the fp32 additions inside the sum
+    is the one degree of freedom a device kernel has; everything else is bit-determined."""
+    dt = x.dtype
+    xf = x.to(torch.float32)
+    new_res = None
+    if residual is not None:
+        xf = xf + residual.to(torch.float32)
+        new_res = xf.to(dt)
+    hidden = x.shape[-1]
+    ss = (xf.double() * xf.double()).sum(dim=-1, keepdim=True).to(torch.float32)
+    rms = torch.rsqrt(ss / torch.tensor(float(hidden), dtype=torch.float32) + torch.tensor(eps, dtype=torch.float32))
+    y = ((xf * rms).to(dt) * weight.to(dt)).to(torch.float32)
+    amax = y.abs().amax(dim=-1, keepdim=True)
+    if scale_ub is not None:
+        amax = torch.minimum(amax, scale_ub.to(torch.float32).reshape(()))
+    s = torch.maximum(amax / FP8_MAX, torch.tensor(1.0 / (FP8_MAX * 512.0), dtype=torch.float32))
+    q = (y / s).clamp(-FP8_MAX, FP8_MAX).to(torch.float8_e4m3fn)
+    return q, s, new_res
+
+
 def make_fp8_weight(n: int, k: int, seed: int = 0, dtype: torch.dtype = torch.bfloat16):
     """BASELINE config 4 weight: ``randn([N,K])*0.02`` quantised per output channel (amax/448 fp32 scales).
     Returns (w_q [N,K] e4m3fn row-major, w_scale [N,1] fp32).  Per-channel quantisation of a weight is the same

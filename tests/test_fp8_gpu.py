@@ -198,6 +198,43 @@ def test_scaled_mm_exact_small_integers(device):
         assert torch.equal(out.cpu().float(), a @ w.t()), (m, n, k)
 
 
+@pytest.mark.parametrize("tokens,hidden", [(1, 17), (11, 1024), (1, 2), (4096, 64), (7, 5120), (83, 4096), (3, 17000)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("add_residual", [False, True])
+@pytest.mark.parametrize("use_ub", [False, True])
+def test_fused_rms_norm_per_token_quant(device, tokens, hidden, dtype, add_residual, use_ub):
+    """Twin of the reference's test_rms_norm (tests/kernels/core/test_fused_quant_layernorm.py:109-200, same size grid
+    and input scaling) for FP8 output.  Scales must agree to one fp32 ulp of the row statistics, the residual sum
+    exactly; codes may differ from the oracle only where the last bit of `rms` (the one order-dependent quantity) moves a
+    value across a rounding boundary: at most one code step, in at most 0.1 % of the elements."""
+    import vllm_amd._custom_ops as ops
+    g = torch.Generator().manual_seed(tokens * 31 + hidden)
+    scale = 1.0 / hidden
+    x = (torch.randn(tokens, hidden, generator=g) * scale).to(dtype)
+    res = (torch.randn(tokens, hidden, generator=g) * scale).to(dtype) if add_residual else None
+    w = (1.0 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
+    ub = None
+    if use_ub:
+        xf = x.float() + (res.float() if res is not None else 0.0)
+        normed = (xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + 1e-5)).to(dtype) * w
+        ub = normed.float().mean().abs().reshape(1) + 0.05
+    q_ref, s_ref, res_ref = f.ref_rms_norm_dynamic_per_token_quant(x, w, 1e-5, ub, res)
+    res_dev = res.to(device).clone() if res is not None else None
+    q, s = ops.rms_norm_dynamic_per_token_quant(x.to(device), w.to(device), 1e-5, torch.float8_e4m3fn,
+                                                ub.to(device) if ub is not None else None, res_dev)
+    assert q.shape == x.shape and q.dtype == torch.float8_e4m3fn and s.shape == (tokens, 1)
+    assert torch.allclose(s.cpu(), s_ref, rtol=3e-7, atol=0)
+    if add_residual:
+        assert torch.equal(res_dev.cpu(), res_ref)
+    a, b = _codes(q).astype(np.int32), _codes(q_ref).astype(np.int32)
+    diff = a != b
+    assert diff.mean() <= 1e-3, f"{diff.mean():.2e} of the codes differ"
+    if diff.any():
+        # neighbouring codes of the same sign differ by 1; across zero the pair is (0x00, 0x80) or a +-1 subnormal
+        step = np.abs((a & 0x7f) - (b & 0x7f))[diff]
+        assert step.max() <= 1, step.max()
+
+
 def test_scaled_mm_split_k_exact_and_deterministic(device):
     """Few output tiles and a long K: the tile kernel splits K over workgroups (fp32 partial tiles through the op's
     scratch, arrival counters left zero).  Small-integer operands make every partial sum exact, so the split result

@@ -125,3 +125,26 @@ def test_golden_vectors():
     # the codes of the fixture also satisfy the independent encoder
     ratio = (x.float().numpy() / gd["scales"]).astype(np.float32)
     assert np.array_equal(gd["codes"], f.e4m3fn_encode_rne_sat(np.clip(ratio, -448, 448)))
+
+
+def test_fused_rms_norm_quant_oracle_equals_unfused_composition():
+    """The fused oracle must equal RMSNorm (the reference layer's forward_native: fp32 statistics, cast to the
+    activation type, multiply by the weight; layernorm.py) followed by the unfused per-token quantiser, bit for bit
+    whenever the fp64 and fp32 row sums round alike (they do for these sizes), with and without residual / scale_ub."""
+    g = torch.Generator().manual_seed(0)
+    for dtype in (torch.bfloat16, torch.float16):
+        for hidden in (64, 1000, 4096):
+            x = (torch.randn(7, hidden, generator=g) / hidden ** 0.5).to(dtype)
+            res = (torch.randn(7, hidden, generator=g) / hidden ** 0.5).to(dtype)
+            w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
+            for residual in (None, res):
+                for ub in (None, torch.tensor(0.5)):
+                    q, s, new_res = f.ref_rms_norm_dynamic_per_token_quant(x, w, 1e-5, ub, residual)
+                    xf = x.float() + (residual.float() if residual is not None else 0.0)
+                    normed = (xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + 1e-5)).to(dtype) * w
+                    q2, s2 = f.ref_dynamic_per_token_quant(normed, ub)
+                    assert torch.allclose(s, s2, rtol=2e-7, atol=0)
+                    same = (q.view(torch.uint8) == q2.view(torch.uint8)).float().mean().item()
+                    assert same > 0.999, same
+                    if residual is not None:
+                        assert torch.equal(new_res, xf.to(dtype))

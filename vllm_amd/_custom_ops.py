@@ -429,6 +429,40 @@ def _fp8_counters(dev: torch.device) -> torch.Tensor:
     return t
 
 
+# ============================================================================ fused RMSNorm + per-token FP8 quant
+
+def _rms_norm_quant_impl(result: torch.Tensor, input: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor,
+                         epsilon: float, scale_ub: torch.Tensor | None, residual: torch.Tensor | None) -> None:
+    """Host checks of fused_layernorm_dynamic_per_token_quant.cu:141-170."""
+    _check(_is_gpu(input) and _is_gpu(result) and _is_gpu(weight) and _is_gpu(scale), "tensors must be on GPU")
+    if result.dtype != FP8_DTYPE:
+        raise NotImplementedError(f"rms_norm_dynamic_per_token_quant: only {FP8_DTYPE} output is built for gfx950 "
+                                  f"(got {result.dtype})")
+    _check(input.dtype in (torch.float16, torch.bfloat16), "input must be float16 or bfloat16")
+    _check(weight.dtype == input.dtype, "weight.dtype must equal input.dtype")
+    _check(scale.dtype == torch.float32, "scale must be float32")
+    _check(result.is_contiguous() and input.stride(-1) == 1, "out must be contiguous and input row-contiguous")
+    hidden = input.size(-1)
+    tokens = input.numel() // hidden if hidden else 0
+    _check(weight.numel() == hidden and weight.is_contiguous(), "weight must be a contiguous [hidden] tensor")
+    _check(scale.numel() == tokens and scale.is_contiguous(), "scale must hold one value per token")
+    if scale_ub is not None:
+        _check(scale_ub.dtype == torch.float32 and scale_ub.numel() == 1 and _is_gpu(scale_ub),
+               "scale_ub must be a float32 scalar on GPU")
+    if residual is not None:
+        _check(residual.dtype == input.dtype and residual.is_contiguous() and residual.shape == input.shape,
+               "residual must match input and be contiguous")
+    inp2 = input.reshape(-1, hidden) if input.dim() != 2 else input
+    _check(inp2.data_ptr() == input.data_ptr(), "input must be viewable as [tokens, hidden]")
+    if tokens == 0:
+        return
+    lib = _lib.load()
+    with torch.cuda.device(input.device):
+        _lib.check(lib.vaq_rms_norm_dynamic_per_token_fp8_quant(
+            _ptr(result), _ptr(scale), _ptr(input), inp2.stride(0), _ptr(weight), _ptr(scale_ub), float(epsilon),
+            _ptr(residual), _dtype_tag(input.dtype), tokens, hidden, _stream(input.device)))
+
+
 # ============================================================================ registration
 
 _NS = "vllm_amd"
@@ -461,6 +495,10 @@ _register("dynamic_scaled_fp8_quant", "(Tensor! result, Tensor input, Tensor! sc
           lambda result, input, scale: None)
 _register("dynamic_per_token_scaled_fp8_quant", "(Tensor! result, Tensor input, Tensor! scale, Tensor? scale_ub) -> ()",
           _per_token_quant_impl, lambda result, input, scale, scale_ub: None)
+_register("rms_norm_dynamic_per_token_quant",
+          "(Tensor! result, Tensor input, Tensor weight, Tensor! scale, float epsilon, Tensor? scale_ub, "
+          "Tensor!? residual) -> ()",
+          _rms_norm_quant_impl, lambda result, input, weight, scale, epsilon, scale_ub, residual: None)
 _register("cutlass_scaled_mm", "(Tensor! out, Tensor a, Tensor b, Tensor a_scales, Tensor b_scales, Tensor? bias) -> ()",
           _scaled_mm_impl, lambda out, a, b, a_scales, b_scales, bias: None)
 
@@ -499,6 +537,17 @@ def gptq_marlin_gemm(a: torch.Tensor, c: torch.Tensor | None, b_q_weight: torch.
 
 def permute_cols(a: torch.Tensor, perm: torch.Tensor) -> torch.Tensor:
     return _ops.permute_cols(a, perm)
+
+
+def rms_norm_dynamic_per_token_quant(input: torch.Tensor, weight: torch.Tensor, epsilon: float, quant_dtype: torch.dtype,
+                                     scale_ub: torch.Tensor | None = None,
+                                     residual: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """RMSNorm (+ in-place residual add) and dynamic per-token quantisation in one pass (reference:
+    _custom_ops.py:394-410).  Returns (quantised [.., hidden], scales [tokens, 1])."""
+    output = torch.empty_like(input, dtype=quant_dtype)
+    scales = torch.empty((input.numel() // input.shape[-1], 1), device=input.device, dtype=torch.float32)
+    _ops.rms_norm_dynamic_per_token_quant(output, input, weight, scales, epsilon, scale_ub, residual)
+    return output, scales
 
 
 def scaled_fp8_quant(input: torch.Tensor, scale: torch.Tensor | None = None, num_token_padding: int | None = None,

@@ -1,0 +1,217 @@
+// RMSNorm (+ residual add) fused with dynamic per-token FP8 (OCP e4m3fn) quantisation for gfx950: the step in front of a
+// per-token-scaled FP8 GEMM, done in one pass over the activations instead of a norm pass plus a quant pass.
+//
+// Arithmetic, in the order of the reference kernel (csrc/quantization/fused_kernels/layernorm_utils.cuh:17-130):
+//   x   = float(input) (+ float(residual); the sum, rounded to the activation type, is written back to `residual`)
+//   rms = rsqrtf(sum(x*x) / hidden + eps)                                   (fp32)
+//   y   = float( T(x * rms) * weight )        -- the product with the weight is rounded to the activation type T
+//   s   = max(min(max|y|, ub) / 448, 1/(448*512))
+//   q   = cvt(clamp(y / s, +-448))            -- a true division, like the unfused per-token quantiser
+// Only the order of the fp32 additions inside sum(x*x) is this kernel's own (per-thread partial sums over a strided
+// set of 8-element vectors, a butterfly over the 64 lanes, then the wavefronts in order); everything else is fixed by
+// the list above, so results agree with the reference up to that last-bit freedom of `rms`.
+//
+// HBM-bound: one workgroup per token; the row (and the residual sum) stays in registers between the three passes when
+// it has at most 256 x 8 x 8 = 16384 elements and is 16-byte aligned; other rows re-read global memory.
+#include "vaq_common.h"
+
+namespace vaq {
+
+namespace {
+
+constexpr float NQ_FP8_MAX = 448.0f;
+constexpr int NQ_T = 256;
+constexpr int NQ_V = 8;
+
+template <bool BF16>
+__device__ inline float nq_to_float(uint16_t v) { return F16Traits<BF16>::to_float(v); }
+
+// round a float to the 16-bit activation type and come back
+template <bool BF16>
+__device__ inline float nq_round16(float x) { return F16Traits<BF16>::to_float(F16Traits<BF16>::from_float(x)); }
+
+__device__ inline float nq_block_sum(float v, float* smem) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0) smem[wave] = v;
+  __syncthreads();
+  float r = smem[0];
+#pragma unroll
+  for (int i = 1; i < NQ_T / 64; ++i) r += smem[i];
+  __syncthreads();
+  return r;
+}
+
+__device__ inline float nq_block_max(float v, float* smem) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0) smem[wave] = v;
+  __syncthreads();
+  float r = smem[0];
+#pragma unroll
+  for (int i = 1; i < NQ_T / 64; ++i) r = fmaxf(r, smem[i]);
+  __syncthreads();
+  return r;
+}
+
+__device__ inline void nq_unpack8(v4u r, float* f, bool bf16) {
+  const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = bf16 ? nq_to_float<true>((uint16_t)(w[i] & 0xffffu)) : nq_to_float<false>((uint16_t)(w[i] & 0xffffu));
+    f[2 * i + 1] = bf16 ? nq_to_float<true>((uint16_t)(w[i] >> 16)) : nq_to_float<false>((uint16_t)(w[i] >> 16));
+  }
+}
+
+template <bool BF16, bool HAS_RES>
+__global__ __launch_bounds__(NQ_T) void rms_norm_per_token_fp8_kernel(uint8_t* __restrict__ out, float* __restrict__ scales,
+                                                                      const uint16_t* __restrict__ input,
+                                                                      const uint16_t* __restrict__ weight,
+                                                                      const float* __restrict__ scale_ub, float eps,
+                                                                      uint16_t* __restrict__ residual, int hidden,
+                                                                      int64_t in_stride) {
+  using T = F16Traits<BF16>;
+  __shared__ float smem[NQ_T / 64];
+  const int64_t tok = blockIdx.x;
+  const uint16_t* row = input + tok * in_stride;
+  uint16_t* res = HAS_RES ? residual + tok * (int64_t)hidden : nullptr;
+  uint8_t* orow = out + tok * (int64_t)hidden;
+  const int chunks = hidden / 8;
+  const bool cached = (hidden % 8 == 0) && chunks <= NQ_T * NQ_V && (in_stride % 8 == 0) &&
+                      ((reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(weight) |
+                        reinterpret_cast<uintptr_t>(out) | (HAS_RES ? reinterpret_cast<uintptr_t>(residual) : 0)) % 16 == 0);
+  const float min_scale = 1.0f / (NQ_FP8_MAX * 512.0f);
+
+  if (cached) {
+    float x[NQ_V][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int v = 0; v < NQ_V; ++v) {
+      const int c = threadIdx.x + v * NQ_T;
+      if (c < chunks) {
+        nq_unpack8(*reinterpret_cast<const v4u*>(row + c * 8), x[v], BF16);
+        if constexpr (HAS_RES) {
+          float r[8];
+          nq_unpack8(*reinterpret_cast<const v4u*>(res + c * 8), r, BF16);
+          v4u back;
+          uint32_t* bw = reinterpret_cast<uint32_t*>(&back);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) x[v][e] += r[e];
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            bw[e] = (uint32_t)T::from_float(x[v][2 * e]) | ((uint32_t)T::from_float(x[v][2 * e + 1]) << 16);
+          *reinterpret_cast<v4u*>(res + c * 8) = back;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += x[v][e] * x[v][e];
+      }
+    }
+    ss = nq_block_sum(ss, smem);
+    const float rms = rsqrtf(ss / (float)hidden + eps);
+    float amax = 0.f;
+#pragma unroll
+    for (int v = 0; v < NQ_V; ++v) {
+      const int c = threadIdx.x + v * NQ_T;
+      if (c < chunks) {
+        float w[8];
+        nq_unpack8(*reinterpret_cast<const v4u*>(weight + c * 8), w, BF16);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          x[v][e] = nq_round16<BF16>(nq_round16<BF16>(x[v][e] * rms) * w[e]);
+          amax = fmaxf(amax, fabsf(x[v][e]));
+        }
+      }
+    }
+    amax = nq_block_max(amax, smem);
+    if (scale_ub) amax = fminf(amax, *scale_ub);
+    const float s = fmaxf(amax / NQ_FP8_MAX, min_scale);
+    if (threadIdx.x == 0) scales[tok] = s;
+#pragma unroll
+    for (int v = 0; v < NQ_V; ++v) {
+      const int c = threadIdx.x + v * NQ_T;
+      if (c < chunks) {
+        v2u o;
+        uint32_t* ow = reinterpret_cast<uint32_t*>(&o);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          float q[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) q[e] = fmaxf(-NQ_FP8_MAX, fminf(x[v][4 * h + e] / s, NQ_FP8_MAX));
+          uint32_t lo = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false) & 0xffffu;
+          uint32_t hi = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], 0, false) & 0xffffu;
+          ow[h] = lo | (hi << 16);
+        }
+        *reinterpret_cast<v2u*>(orow + c * 8) = o;
+      }
+    }
+    return;
+  }
+
+  // general path: three passes over global memory, one element per thread and step
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += NQ_T) {
+    float x = nq_to_float<BF16>(row[i]);
+    if constexpr (HAS_RES) {
+      x += nq_to_float<BF16>(res[i]);
+    }
+    ss += x * x;
+  }
+  ss = nq_block_sum(ss, smem);
+  const float rms = rsqrtf(ss / (float)hidden + eps);
+  float amax = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += NQ_T) {
+    float x = nq_to_float<BF16>(row[i]);
+    if constexpr (HAS_RES) x += nq_to_float<BF16>(res[i]);
+    const float y = nq_round16<BF16>(nq_round16<BF16>(x * rms) * nq_to_float<BF16>(weight[i]));
+    amax = fmaxf(amax, fabsf(y));
+  }
+  amax = nq_block_max(amax, smem);
+  if (scale_ub) amax = fminf(amax, *scale_ub);
+  const float s = fmaxf(amax / NQ_FP8_MAX, min_scale);
+  if (threadIdx.x == 0) scales[tok] = s;
+  for (int i = threadIdx.x; i < hidden; i += NQ_T) {
+    float x = nq_to_float<BF16>(row[i]);
+    if constexpr (HAS_RES) {
+      x += nq_to_float<BF16>(res[i]);
+      res[i] = T::from_float(x);
+    }
+    const float y = nq_round16<BF16>(nq_round16<BF16>(x * rms) * nq_to_float<BF16>(weight[i]));
+    const float q = fmaxf(-NQ_FP8_MAX, fminf(y / s, NQ_FP8_MAX));
+    orow[i] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(q, q, 0, false) & 0xff);
+  }
+}
+
+}  // namespace
+
+}  // namespace vaq
+
+extern "C" int vaq_rms_norm_dynamic_per_token_fp8_quant(uint8_t* out, float* scales, const void* input, int64_t in_stride,
+                                                        const void* weight, const float* scale_ub, float epsilon,
+                                                        void* residual, int dtype, int64_t tokens, int64_t hidden,
+                                                        void* stream) {
+  using namespace vaq;
+  VAQ_CHECK_ARG(tokens >= 0 && hidden > 0 && hidden < (1ll << 31) && tokens < (1ll << 31),
+                "rms_norm_dynamic_per_token_quant: bad shape [%lld, %lld]", (long long)tokens, (long long)hidden);
+  VAQ_CHECK_ARG(dtype == VAQ_F16 || dtype == VAQ_BF16, "rms_norm_dynamic_per_token_quant: dtype tag %d", dtype);
+  VAQ_CHECK_ARG(in_stride >= hidden, "rms_norm_dynamic_per_token_quant: input row stride %lld < hidden %lld",
+                (long long)in_stride, (long long)hidden);
+  if (tokens == 0) return VAQ_OK;
+  VAQ_CHECK_ARG(out && scales && input && weight, "rms_norm_dynamic_per_token_quant: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)tokens), block(NQ_T);
+  const uint16_t* in = (const uint16_t*)input;
+  const uint16_t* w = (const uint16_t*)weight;
+  uint16_t* res = (uint16_t*)residual;
+  const bool bf16 = dtype == VAQ_BF16;
+  if (bf16) {
+    if (res) hipLaunchKernelGGL((rms_norm_per_token_fp8_kernel<true, true>), grid, block, 0, s, out, scales, in, w, scale_ub, epsilon, res, (int)hidden, in_stride);
+    else hipLaunchKernelGGL((rms_norm_per_token_fp8_kernel<true, false>), grid, block, 0, s, out, scales, in, w, scale_ub, epsilon, res, (int)hidden, in_stride);
+  } else {
+    if (res) hipLaunchKernelGGL((rms_norm_per_token_fp8_kernel<false, true>), grid, block, 0, s, out, scales, in, w, scale_ub, epsilon, res, (int)hidden, in_stride);
+    else hipLaunchKernelGGL((rms_norm_per_token_fp8_kernel<false, false>), grid, block, 0, s, out, scales, in, w, scale_ub, epsilon, res, (int)hidden, in_stride);
+  }
+  VAQ_CHECK_LAUNCH("rms_norm_dynamic_per_token_quant");
+  return VAQ_OK;
+}
