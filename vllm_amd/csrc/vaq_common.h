@@ -60,11 +60,8 @@ struct F16Traits<true> {
   static constexpr uint32_t EX = 0x43004300u;
   static constexpr float CODE_BIAS = 128.0f;
   __device__ static inline float to_float(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
-  __device__ static inline uint16_t from_float(float f) {   // round-to-nearest-even, NaN preserved
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+  __device__ static inline uint16_t from_float(float f) {   // v_cvt_pk_bf16_f32: round-to-nearest-even, NaN stays NaN
+    return __builtin_bit_cast(uint16_t, (__bf16)f);
   }
   __device__ static inline v4f mfma16(v4u a, v4u b, v4f c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
