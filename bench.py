@@ -225,6 +225,30 @@ def fused_norm_quant_section(dev):
                              hbm_frac=b / t / 1e9 / HBM_PEAK_GBS, unfused_us=tu * 1e6, cold=False))
             log(f"[norm+quant  ] hidden={k:5d} M={m:4d}: {t * 1e6:6.1f} us {b / t / 1e9:6.0f} GB/s ({100 * b / t / 1e9 / HBM_PEAK_GBS:4.1f}% of 8 TB/s) | "
                 f"unfused rms_norm + quant {tu * 1e6:6.1f} us")
+    # static-scale variants at the prefill size: norm (+ residual) + quant, and silu(gate) * up + quant (d = 14336)
+    one = torch.ones(1, device=dev, dtype=torch.float32)
+    m, k = 4096, 4096
+    w = (1.0 + 0.1 * torch.randn(k, device=dev, generator=gen)).to(torch.bfloat16)
+    x = torch.randn(m, k, device=dev, generator=gen).to(torch.bfloat16)
+    res = torch.randn(m, k, device=dev, generator=gen).to(torch.bfloat16)
+    out = torch.empty(m, k, device=dev, dtype=torch.float8_e4m3fn)
+    for kind, fn, b in (
+            ("rms_norm_static_fp8_quant", lambda: ops.rms_norm_static_fp8_quant(out, x, w, one, 1e-6), 3 * m * k + 2 * k),
+            ("fused_add_rms_norm_static_fp8_quant",
+             lambda: ops.fused_add_rms_norm_static_fp8_quant(out, x, res, w, one, 1e-6), 7 * m * k + 2 * k)):
+        t = time_graph(lambda: [fn() for _ in range(20)], iters=5, warmup=2, inner=20)
+        rows.append(dict(kind=kind, hidden=k, M=m, us=t * 1e6, GBps=b / t / 1e9, hbm_frac=b / t / 1e9 / HBM_PEAK_GBS, cold=False))
+        log(f"[norm+quant  ] {kind} hidden={k} M={m}: {t * 1e6:6.1f} us {b / t / 1e9:6.0f} GB/s ({100 * b / t / 1e9 / HBM_PEAK_GBS:4.1f}% of 8 TB/s)")
+    d = 14336
+    gu = torch.randn(m, 2 * d, device=dev, generator=gen).to(torch.bfloat16)
+    out2 = torch.empty(m, d, device=dev, dtype=torch.float8_e4m3fn)
+    t = time_graph(lambda: [ops.silu_and_mul_quant(out2, gu, one) for _ in range(10)], iters=5, warmup=2, inner=10)
+    tu = time_graph(lambda: [ops.scaled_fp8_quant(F.silu(gu[:, :d]) * gu[:, d:], one) for _ in range(10)], iters=5, warmup=2, inner=10)
+    b = 5 * m * d
+    rows.append(dict(kind="silu_and_mul_quant", d=d, M=m, us=t * 1e6, GBps=b / t / 1e9, hbm_frac=b / t / 1e9 / HBM_PEAK_GBS,
+                     unfused_us=tu * 1e6, cold=False))
+    log(f"[silu+quant  ] d={d} M={m}: {t * 1e6:6.1f} us {b / t / 1e9:6.0f} GB/s ({100 * b / t / 1e9 / HBM_PEAK_GBS:4.1f}% of 8 TB/s) | "
+        f"unfused silu*mul + quant {tu * 1e6:6.1f} us")
     return rows
 
 

@@ -161,6 +161,28 @@ int vaq_rms_norm_dynamic_per_token_fp8_quant(uint8_t* out, float* scales, const 
                                              int dtype, int64_t tokens, int64_t hidden, void* stream);
 
 /*
+ * RMSNorm (+ residual add) fused with static per-tensor FP8 quantisation.  With residual == NULL replaces
+ * `rms_norm_static_fp8_quant(Tensor! result, Tensor input, Tensor weight, Tensor scale, float epsilon)`
+ * (csrc/torch_bindings.cpp:200-205, device code csrc/layernorm_quant_kernels.cu:21-66); with a residual replaces
+ * `fused_add_rms_norm_static_fp8_quant(Tensor! result, Tensor input, Tensor! residual, Tensor weight, Tensor scale,
+ * float epsilon)` (csrc/torch_bindings.cpp:208-213, csrc/layernorm_quant_kernels.cu:72-178): residual is updated in
+ * place with input + residual, input is left untouched.
+ *   out  e4m3fn [tokens, hidden] contiguous;  input row stride in_stride elements;  scale fp32 scalar (device)
+ */
+int vaq_rms_norm_static_fp8_quant(uint8_t* out, const void* input, int64_t in_stride, const void* weight,
+                                  const float* scale, float epsilon, void* residual, int dtype, int64_t tokens,
+                                  int64_t hidden, void* stream);
+
+/*
+ * out[t, i] = fp8(silu(input[t, i]) * input[t, d + i] / scale).  Replaces
+ * `silu_and_mul_quant(Tensor! result, Tensor input, Tensor scale)` (csrc/torch_bindings.cpp:121-123, device code
+ * csrc/quantization/activation_kernels.cu:35-119, 560-568).
+ *   out  e4m3fn [tokens, d] contiguous;  input [tokens, 2*d] F16/BF16 contiguous;  scale fp32 scalar (device)
+ */
+int vaq_silu_and_mul_fp8_quant(uint8_t* out, const void* input, const float* scale, int dtype, int64_t tokens, int64_t d,
+                               void* stream);
+
+/*
  * The same GEMM with caller-provided scratch, which lets the tile kernel split K over workgroups when M and N alone
  * leave compute units idle (a few hundred tokens on the narrow layers).  Sizes come from the query; both may be 0.
  *   c_tmp     fp32 partial tiles, 16-byte aligned, contents irrelevant on entry

@@ -165,6 +165,47 @@ def ref_rms_norm_dynamic_per_token_quant(x: torch.Tensor, weight: torch.Tensor, 
     return q, s, new_res
 
 
+def ref_rms_norm_static_fp8_quant(x: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, eps: float,
+                                  residual: torch.Tensor | None = None):
+    """Fused RMSNorm (+ residual) + static per-tensor FP8 quant, operation order of
+    csrc/layernorm_quant_kernels.cu:21-66 (no residual) and :138-178 (residual):
+
+        z = x  or  T(float(x) + float(residual))  (written back to residual);  xf = float(z)
+        rms = rsqrt(sum(xf*xf)/hidden + eps)            # sum accumulated in fp64 here, then rounded
+        y = float(T(T(xf * rms) * weight));  q = cast(clamp(y * (1/scale), +-448))
+
+    Returns (q e4m3fn, new_residual or None)."""
+    dt = x.dtype
+    new_res = None
+    z = x
+    if residual is not None:
+        z = (x.to(torch.float32) + residual.to(torch.float32)).to(dt)
+        new_res = z
+    xf = z.to(torch.float32)
+    hidden = x.shape[-1]
+    ss = (xf.double() * xf.double()).sum(dim=-1, keepdim=True).to(torch.float32)
+    rms = torch.rsqrt(ss / torch.tensor(float(hidden), dtype=torch.float32) + torch.tensor(eps, dtype=torch.float32))
+    y = ((xf * rms).to(dt) * weight.to(dt)).to(torch.float32)
+    inv = torch.tensor(1.0, dtype=torch.float32) / scale.to(torch.float32).reshape(())
+    q = (y * inv).clamp(-FP8_MAX, FP8_MAX).to(torch.float8_e4m3fn)
+    return q, new_res
+
+
+def ref_silu_and_mul_quant(x: torch.Tensor, scale: torch.Tensor):
+    """silu(x[..., :d]) * x[..., d:] quantised with a static scale, operation order of
+    csrc/quantization/activation_kernels.cu:35-119: silu in fp32 (x / (1 + exp(-x))) rounded to the activation type,
+    the product rounded to the activation type, then q = cast(clamp(float(product) * (1/scale), +-448)).  exp here
+    is torch's fp32 exp, which may differ from a device's expf in the last bit."""
+    dt = x.dtype
+    d = x.shape[-1] // 2
+    a = x[..., :d].to(torch.float32)
+    b = x[..., d:]
+    s = (a / (1.0 + torch.exp(-a))).to(dt)
+    v = (s * b).to(torch.float32)
+    inv = torch.tensor(1.0, dtype=torch.float32) / scale.to(torch.float32).reshape(())
+    return (v * inv).clamp(-FP8_MAX, FP8_MAX).to(torch.float8_e4m3fn)
+
+
 def make_fp8_weight(n: int, k: int, seed: int = 0, dtype: torch.dtype = torch.bfloat16):
     """BASELINE config 4 weight: ``randn([N,K])*0.02`` quantised per output channel (amax/448 fp32 scales).
     Returns (w_q [N,K] e4m3fn row-major, w_scale [N,1] fp32).  Per-channel quantisation of a weight is the same

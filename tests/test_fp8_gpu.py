@@ -235,6 +235,69 @@ def test_fused_rms_norm_per_token_quant(device, tokens, hidden, dtype, add_resid
         assert step.max() <= 1, step.max()
 
 
+def _assert_codes_close(q, q_ref, frac):
+    a, b = _codes(q).astype(np.int32), _codes(q_ref).astype(np.int32)
+    diff = a != b
+    assert diff.mean() <= frac, f"{diff.mean():.2e} of the codes differ"
+    if diff.any():
+        assert np.abs((a & 0x7f) - (b & 0x7f))[diff].max() <= 1
+
+
+@pytest.mark.parametrize("tokens,hidden", [(7, 8), (83, 768), (83, 769), (83, 5120), (4096, 64), (3, 8199), (2, 17000)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("add_residual", [False, True])
+@pytest.mark.parametrize("quant_scale", [1.0, 0.01, 10.0])
+@pytest.mark.parametrize("strided_input", [False, True])
+def test_fused_rms_norm_static_quant(device, tokens, hidden, dtype, add_residual, quant_scale, strided_input):
+    """Twin of the reference's test_fused_rms_norm_quant (tests/kernels/core/test_layernorm.py:63-153: same size grid
+    corners, input scaling 1/(2*hidden), quant scales and the strided-input case).  Residual sum exact; codes equal to the
+    oracle's except where the last bit of `rms` moves a value over a rounding boundary (<= 0.1 %, one code step).
+    The input must be left untouched by the residual variant."""
+    import vllm_amd._custom_ops as ops
+    g = torch.Generator().manual_seed(tokens * 31 + hidden)
+    last = 2 * hidden if strided_input else hidden
+    x_base = (torch.randn(tokens, last, generator=g) / (2 * hidden)).to(dtype)
+    x = x_base[..., :hidden]
+    res = (torch.randn(tokens, hidden, generator=g) / (2 * hidden)).to(dtype) if add_residual else None
+    w = (1.0 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
+    scale = torch.tensor([quant_scale], dtype=torch.float32)
+    q_ref, res_ref = f.ref_rms_norm_static_fp8_quant(x, w, scale, 1e-6, res)
+    xb_dev = x_base.to(device)
+    x_dev = xb_dev[..., :hidden]
+    assert x_dev.is_contiguous() != strided_input or tokens == 1
+    out = torch.empty(tokens, hidden, dtype=torch.float8_e4m3fn, device=device)
+    if add_residual:
+        res_dev = res.to(device)
+        ops.fused_add_rms_norm_static_fp8_quant(out, x_dev, res_dev, w.to(device), scale.to(device), 1e-6)
+        assert torch.equal(res_dev.cpu(), res_ref)
+    else:
+        ops.rms_norm_static_fp8_quant(out, x_dev, w.to(device), scale.to(device), 1e-6)
+    assert torch.equal(xb_dev.cpu(), x_base)
+    _assert_codes_close(out, q_ref, 1e-3)
+
+
+@pytest.mark.parametrize("tokens", [1, 17, 86, 1234, 3045])
+@pytest.mark.parametrize("hidden", [16, 48, 128, 1562, 4096, 28672])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_silu_and_mul_quant(device, tokens, hidden, dtype):
+    """Twin of the reference's test_silu_and_mul (tests/kernels/test_fused_quant_activation.py:33-68, same size grid
+    plus Llama-3-8B's 2*14336).  Codes equal to the oracle's except where the device's expf and the CPU's exp differ in
+    the last bit and that moves a value over a rounding boundary (<= 0.2 %, one code step)."""
+    import vllm_amd._custom_ops as ops
+    g = torch.Generator().manual_seed(tokens + hidden)
+    scale = torch.randn(1, generator=g).abs() + 0.05
+    x = torch.randn(tokens, hidden, generator=g).to(dtype)
+    out = torch.empty(tokens, hidden // 2, dtype=torch.float8_e4m3fn, device=device)
+    ops.silu_and_mul_quant(out, x.to(device), scale.to(device))
+    _assert_codes_close(out, f.ref_silu_and_mul_quant(x, scale), 2e-3)
+    # 3-d input, as the layer passes it
+    if tokens == 86:
+        x3 = x.reshape(2, 43, hidden)
+        out3 = torch.empty(2, 43, hidden // 2, dtype=torch.float8_e4m3fn, device=device)
+        ops.silu_and_mul_quant(out3, x3.to(device), scale.to(device))
+        assert torch.equal(out3.reshape(tokens, -1).view(torch.uint8), out.view(torch.uint8))
+
+
 def test_scaled_mm_split_k_exact_and_deterministic(device):
     """Few output tiles and a long K: the tile kernel splits K over workgroups (fp32 partial tiles through the op's
     scratch, arrival counters left zero).  Small-integer operands make every partial sum exact, so the split result

@@ -57,6 +57,11 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
         _lib.check(rc)
     rc = lib.vaq_fp8_quant_per_token(None, _lib.VAQ_BF16, 8, None, 16, None, None, 4, 16, None)
     assert rc == _lib.VAQ_ERR_INVALID_ARG and b"row strides" in lib.vaq_last_error()
+    rc = lib.vaq_rms_norm_static_fp8_quant(None, None, 8, None, None, 1e-6, None, _lib.VAQ_BF16, 4, 16, None)
+    assert rc == _lib.VAQ_ERR_INVALID_ARG and b"row stride" in lib.vaq_last_error()
+    rc = lib.vaq_silu_and_mul_fp8_quant(None, None, None, _lib.VAQ_F32, 4, 16, None)
+    assert rc == _lib.VAQ_ERR_INVALID_ARG and b"dtype" in lib.vaq_last_error()
+    assert lib.vaq_silu_and_mul_fp8_quant(None, None, None, _lib.VAQ_BF16, 0, 16, None) == _lib.VAQ_OK
     # M == 0 is a no-op that touches nothing
     assert lib.vaq_w4a16_gemm(None, 4096, None, None, None, None, None, None, None, None, None, 0, 0, 4096, 4096, 128,
                               _lib.VAQ_BF16, _lib.VAQ_WTYPE_U4B8, 0, None) == _lib.VAQ_OK

@@ -309,3 +309,11 @@ def test_custom_ops_pass_opcheck_on_device(device):
     c = torch.empty(m, n, dtype=torch.bfloat16, device=device)
     sb = torch.ones(n, 1, dtype=torch.float32, device=device)
     torch.library.opcheck(torch.ops.vllm_amd.cutlass_scaled_mm, (c, out, bq, sc.fill_(1.0), sb, None), test_utils=utils)
+    w = torch.ones(k, dtype=torch.bfloat16, device=device)
+    torch.library.opcheck(torch.ops.vllm_amd.rms_norm_static_fp8_quant, (out, a, w, one, 1e-6), test_utils=utils)
+    torch.library.opcheck(torch.ops.vllm_amd.fused_add_rms_norm_static_fp8_quant, (out, a, a.clone(), w, one, 1e-6),
+                          test_utils=utils)
+    torch.library.opcheck(torch.ops.vllm_amd.rms_norm_dynamic_per_token_quant, (out, a, w, sc, 1e-6, None, a.clone()),
+                          test_utils=utils)
+    half = torch.empty(m, k // 2, dtype=torch.float8_e4m3fn, device=device)
+    torch.library.opcheck(torch.ops.vllm_amd.silu_and_mul_quant, (half, a, one), test_utils=utils)

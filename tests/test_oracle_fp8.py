@@ -148,3 +148,38 @@ def test_fused_rms_norm_quant_oracle_equals_unfused_composition():
                     assert same > 0.999, same
                     if residual is not None:
                         assert torch.equal(new_res, xf.to(dtype))
+
+
+def test_static_fused_norm_and_silu_oracles_equal_unfused_compositions():
+    """The static-scale fused oracles against independent compositions, as the reference's own tests check the kernels
+    (tests/kernels/core/test_layernorm.py:81-153, tests/kernels/test_fused_quant_activation.py:19-68): RMSNorm written
+    with mean() and rsqrt, then the static quantiser oracle; torch.nn.functional.silu (the SiluAndMul layer's
+    forward_native) times the gate, then the static quantiser oracle.  Bit-equal except where a last-bit difference of
+    rsqrt/exp moves a value over a rounding boundary (< 0.2 % of the codes, one code step)."""
+    g = torch.Generator().manual_seed(3)
+    for dtype in (torch.bfloat16, torch.float16):
+        for hidden in (64, 1000, 4096):
+            x = (torch.randn(7, hidden, generator=g) / (2 * hidden)).to(dtype)
+            res = (torch.randn(7, hidden, generator=g) / (2 * hidden)).to(dtype)
+            w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
+            for qs in (1.0, 0.01):
+                scale = torch.tensor([qs])
+                for residual in (None, res):
+                    q, new_res = f.ref_rms_norm_static_fp8_quant(x, w, scale, 1e-6, residual)
+                    z = x if residual is None else (x + residual)
+                    zf = z.float()
+                    normed = (zf * torch.rsqrt(zf.pow(2).mean(-1, keepdim=True) + 1e-6)).to(dtype) * w
+                    q2 = f.ref_static_quant(normed, scale)
+                    a, b = q.view(torch.uint8).int(), q2.view(torch.uint8).int()
+                    assert (a != b).float().mean().item() < 2e-3
+                    assert ((a & 0x7f) - (b & 0x7f)).abs().max().item() <= 1
+                    if residual is not None:
+                        assert torch.equal(new_res, z)
+            y = torch.randn(5, 2 * hidden, generator=g).to(dtype)
+            scale = torch.tensor([0.05])
+            q = f.ref_silu_and_mul_quant(y, scale)
+            q2 = f.ref_static_quant(torch.nn.functional.silu(y[..., :hidden]) * y[..., hidden:], scale)
+            a, b = q.view(torch.uint8).int(), q2.view(torch.uint8).int()
+            assert (a != b).float().mean().item() < 2e-3
+            assert ((a & 0x7f) - (b & 0x7f)).abs().max().item() <= 1
+

@@ -463,6 +463,61 @@ def _rms_norm_quant_impl(result: torch.Tensor, input: torch.Tensor, weight: torc
             _ptr(residual), _dtype_tag(input.dtype), tokens, hidden, _stream(input.device)))
 
 
+def _rms_norm_static_common(who, result, input, residual, weight, scale, epsilon) -> None:
+    """Host checks of layernorm_quant_kernels.cu:181-188 / 225-236."""
+    _check(_is_gpu(input) and _is_gpu(result) and _is_gpu(weight) and _is_gpu(scale), "tensors must be on GPU")
+    if result.dtype != FP8_DTYPE:
+        raise NotImplementedError(f"{who}: only {FP8_DTYPE} output is built for gfx950 (got {result.dtype})")
+    _check(input.dtype in (torch.float16, torch.bfloat16), f"{who}: input must be float16 or bfloat16")
+    _check(weight.dtype == input.dtype, "weight.dtype must equal input.dtype")
+    _check(scale.dtype == torch.float32 and scale.numel() == 1, "scale must be a float32 scalar")
+    _check(result.is_contiguous(), "out must be contiguous")
+    _check(input.stride(-1) == 1, "input rows must be contiguous")
+    hidden = input.size(-1)
+    tokens = input.numel() // hidden if hidden else 0
+    _check(result.numel() == input.numel(), "out must have the shape of input")
+    _check(weight.numel() == hidden and weight.is_contiguous(), "weight must be a contiguous [hidden] tensor")
+    if residual is not None:
+        _check(residual.is_contiguous(), "residual must be contiguous")
+        _check(residual.dtype == input.dtype and residual.shape == input.shape, "residual must match input")
+    inp2 = input.reshape(-1, hidden) if input.dim() != 2 else input
+    _check(inp2.data_ptr() == input.data_ptr(), "input must be viewable as [tokens, hidden]")
+    if tokens == 0:
+        return
+    lib = _lib.load()
+    with torch.cuda.device(input.device):
+        _lib.check(lib.vaq_rms_norm_static_fp8_quant(
+            _ptr(result), _ptr(input), inp2.stride(0), _ptr(weight), _ptr(scale), float(epsilon), _ptr(residual),
+            _dtype_tag(input.dtype), tokens, hidden, _stream(input.device)))
+
+
+def _rms_norm_static_impl(result, input, weight, scale, epsilon) -> None:
+    _rms_norm_static_common("rms_norm_static_fp8_quant", result, input, None, weight, scale, epsilon)
+
+
+def _fused_add_rms_norm_static_impl(result, input, residual, weight, scale, epsilon) -> None:
+    _rms_norm_static_common("fused_add_rms_norm_static_fp8_quant", result, input, residual, weight, scale, epsilon)
+
+
+def _silu_and_mul_quant_impl(result: torch.Tensor, input: torch.Tensor, scale: torch.Tensor) -> None:
+    """Host checks of activation_kernels.cu:560-568."""
+    _check(_is_gpu(input) and _is_gpu(result) and _is_gpu(scale), "tensors must be on GPU")
+    _check(result.dtype == FP8_DTYPE, f"silu_and_mul_quant: out must be {FP8_DTYPE}")
+    _check(input.dtype in (torch.float16, torch.bfloat16), "silu_and_mul_quant: input must be float16 or bfloat16")
+    _check(input.size(-1) % 2 == 0, "silu_and_mul_quant: the last dimension of input must be even")
+    _check(scale.dtype == torch.float32 and scale.numel() == 1, "scale must be a float32 scalar")
+    d = input.size(-1) // 2
+    tokens = input.numel() // input.size(-1) if d else 0
+    _check(input.is_contiguous() and result.is_contiguous(), "input and out must be contiguous")
+    _check(result.numel() == tokens * d, "out must be [..., d] for input [..., 2*d]")
+    if tokens == 0:
+        return
+    lib = _lib.load()
+    with torch.cuda.device(input.device):
+        _lib.check(lib.vaq_silu_and_mul_fp8_quant(_ptr(result), _ptr(input), _ptr(scale), _dtype_tag(input.dtype), tokens,
+                                                  d, _stream(input.device)))
+
+
 # ============================================================================ registration
 
 _NS = "vllm_amd"
@@ -499,6 +554,13 @@ _register("rms_norm_dynamic_per_token_quant",
           "(Tensor! result, Tensor input, Tensor weight, Tensor! scale, float epsilon, Tensor? scale_ub, "
           "Tensor!? residual) -> ()",
           _rms_norm_quant_impl, lambda result, input, weight, scale, epsilon, scale_ub, residual: None)
+_register("rms_norm_static_fp8_quant", "(Tensor! result, Tensor input, Tensor weight, Tensor scale, float epsilon) -> ()",
+          _rms_norm_static_impl, lambda result, input, weight, scale, epsilon: None)
+_register("fused_add_rms_norm_static_fp8_quant",
+          "(Tensor! result, Tensor input, Tensor! residual, Tensor weight, Tensor scale, float epsilon) -> ()",
+          _fused_add_rms_norm_static_impl, lambda result, input, residual, weight, scale, epsilon: None)
+_register("silu_and_mul_quant", "(Tensor! result, Tensor input, Tensor scale) -> ()",
+          _silu_and_mul_quant_impl, lambda result, input, scale: None)
 _register("cutlass_scaled_mm", "(Tensor! out, Tensor a, Tensor b, Tensor a_scales, Tensor b_scales, Tensor? bias) -> ()",
           _scaled_mm_impl, lambda out, a, b, a_scales, b_scales, bias: None)
 
@@ -548,6 +610,24 @@ def rms_norm_dynamic_per_token_quant(input: torch.Tensor, weight: torch.Tensor, 
     scales = torch.empty((input.numel() // input.shape[-1], 1), device=input.device, dtype=torch.float32)
     _ops.rms_norm_dynamic_per_token_quant(output, input, weight, scales, epsilon, scale_ub, residual)
     return output, scales
+
+
+def rms_norm_static_fp8_quant(out: torch.Tensor, input: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor,
+                              epsilon: float) -> None:
+    """``out = fp8(rms_norm(input) * weight / scale)``; the reference exposes it only as ``torch.ops._C`` op
+    (csrc/torch_bindings.cpp:200-205)."""
+    _ops.rms_norm_static_fp8_quant(out, input, weight, scale, epsilon)
+
+
+def fused_add_rms_norm_static_fp8_quant(out: torch.Tensor, input: torch.Tensor, residual: torch.Tensor,
+                                        weight: torch.Tensor, scale: torch.Tensor, epsilon: float) -> None:
+    """``residual += input; out = fp8(rms_norm(residual) * weight / scale)`` (csrc/torch_bindings.cpp:208-213)."""
+    _ops.fused_add_rms_norm_static_fp8_quant(out, input, residual, weight, scale, epsilon)
+
+
+def silu_and_mul_quant(out: torch.Tensor, input: torch.Tensor, scale: torch.Tensor) -> None:
+    """``out = fp8(silu(input[..., :d]) * input[..., d:] / scale)`` (csrc/torch_bindings.cpp:121-123)."""
+    _ops.silu_and_mul_quant(out, input, scale)
 
 
 def scaled_fp8_quant(input: torch.Tensor, scale: torch.Tensor | None = None, num_token_padding: int | None = None,

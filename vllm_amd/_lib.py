@@ -42,6 +42,9 @@ _SIGNATURES = {
                                   c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p]),
     "vaq_rms_norm_dynamic_per_token_fp8_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p,
                                                          ctypes.c_float, c_void_p, c_int, c_int64, c_int64, c_void_p]),
+    "vaq_rms_norm_static_fp8_quant": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, ctypes.c_float, c_void_p,
+                                              c_int, c_int64, c_int64, c_void_p]),
+    "vaq_silu_and_mul_fp8_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p]),
     "vaq_fp8_scaled_mm_workspace": (c_int, [c_int64, c_int64, c_int64, ctypes.POINTER(ctypes.c_size_t),
                                             ctypes.POINTER(ctypes.c_size_t)]),
     "vaq_fp8_scaled_mm_ws": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p,

@@ -11,6 +11,11 @@
 // set of 8-element vectors, a butterfly over the 64 lanes, then the wavefronts in order); everything else is fixed by
 // the list above, so results agree with the reference up to that last-bit freedom of `rms`.
 //
+// The static-scale variant (reference: csrc/layernorm_quant_kernels.cu:21-178, ops rms_norm_static_fp8_quant and
+// fused_add_rms_norm_static_fp8_quant) differs in two places: with a residual the sum is rounded to the activation type
+// first and the statistics are taken from the rounded value, and the quantisation multiplies by 1/scale of the given
+// per-tensor scale:  q = cvt(clamp(y * (1/scale), +-448)).
+//
 // HBM-bound: one workgroup per token; the row (and the residual sum) stays in registers between the three passes when
 // it has at most 256 x 8 x 8 = 16384 elements and is 16-byte aligned; other rows re-read global memory.
 #include "vaq_common.h"
@@ -183,6 +188,151 @@ __global__ __launch_bounds__(NQ_T) void rms_norm_per_token_fp8_kernel(uint8_t* _
   }
 }
 
+template <bool BF16, bool HAS_RES>
+__global__ __launch_bounds__(NQ_T) void rms_norm_static_fp8_kernel(uint8_t* __restrict__ out,
+                                                                   const uint16_t* __restrict__ input,
+                                                                   const uint16_t* __restrict__ weight,
+                                                                   const float* __restrict__ scale, float eps,
+                                                                   uint16_t* __restrict__ residual, int hidden,
+                                                                   int64_t in_stride) {
+  using T = F16Traits<BF16>;
+  __shared__ float smem[NQ_T / 64];
+  const int64_t tok = blockIdx.x;
+  const uint16_t* row = input + tok * in_stride;
+  uint16_t* res = HAS_RES ? residual + tok * (int64_t)hidden : nullptr;
+  uint8_t* orow = out + tok * (int64_t)hidden;
+  const int chunks = hidden / 8;
+  const bool cached = (hidden % 8 == 0) && chunks <= NQ_T * NQ_V && (in_stride % 8 == 0) &&
+                      ((reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(weight) |
+                        reinterpret_cast<uintptr_t>(out) | (HAS_RES ? reinterpret_cast<uintptr_t>(residual) : 0)) % 16 == 0);
+  const float inv = 1.0f / *scale;
+
+  if (cached) {
+    float x[NQ_V][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int v = 0; v < NQ_V; ++v) {
+      const int c = threadIdx.x + v * NQ_T;
+      if (c < chunks) {
+        nq_unpack8(*reinterpret_cast<const v4u*>(row + c * 8), x[v], BF16);
+        if constexpr (HAS_RES) {
+          float r[8];
+          nq_unpack8(*reinterpret_cast<const v4u*>(res + c * 8), r, BF16);
+          v4u back;
+          uint32_t* bw = reinterpret_cast<uint32_t*>(&back);
+          uint16_t z[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            z[e] = T::from_float(x[v][e] + r[e]);
+            x[v][e] = T::to_float(z[e]);
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) bw[e] = (uint32_t)z[2 * e] | ((uint32_t)z[2 * e + 1] << 16);
+          *reinterpret_cast<v4u*>(res + c * 8) = back;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += x[v][e] * x[v][e];
+      }
+    }
+    ss = nq_block_sum(ss, smem);
+    const float rms = rsqrtf(ss / (float)hidden + eps);
+#pragma unroll
+    for (int v = 0; v < NQ_V; ++v) {
+      const int c = threadIdx.x + v * NQ_T;
+      if (c < chunks) {
+        float w[8];
+        nq_unpack8(*reinterpret_cast<const v4u*>(weight + c * 8), w, BF16);
+        v2u o;
+        uint32_t* ow = reinterpret_cast<uint32_t*>(&o);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          float q[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float y = nq_round16<BF16>(nq_round16<BF16>(x[v][4 * h + e] * rms) * w[4 * h + e]);
+            q[e] = fmaxf(-NQ_FP8_MAX, fminf(y * inv, NQ_FP8_MAX));
+          }
+          uint32_t lo = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false) & 0xffffu;
+          uint32_t hi = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], 0, false) & 0xffffu;
+          ow[h] = lo | (hi << 16);
+        }
+        *reinterpret_cast<v2u*>(orow + c * 8) = o;
+      }
+    }
+    return;
+  }
+
+  // general path: two passes over global memory, one element per thread and step
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += NQ_T) {
+    float x = nq_to_float<BF16>(row[i]);
+    if constexpr (HAS_RES) {
+      const uint16_t z = T::from_float(x + nq_to_float<BF16>(res[i]));
+      res[i] = z;
+      x = T::to_float(z);
+    }
+    ss += x * x;
+  }
+  ss = nq_block_sum(ss, smem);  // its barrier also orders this workgroup's own writes to `res` before the re-reads
+  const float rms = rsqrtf(ss / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += NQ_T) {
+    const float x = nq_to_float<BF16>(HAS_RES ? res[i] : row[i]);
+    const float y = nq_round16<BF16>(nq_round16<BF16>(x * rms) * nq_to_float<BF16>(weight[i]));
+    const float q = fmaxf(-NQ_FP8_MAX, fminf(y * inv, NQ_FP8_MAX));
+    orow[i] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(q, q, 0, false) & 0xff);
+  }
+}
+
+// silu(x) * y of the two halves of each row, quantised with a given per-tensor scale.
+// reference: csrc/quantization/activation_kernels.cu:35-119 -- silu is rounded to the activation type, so is the product.
+template <bool BF16>
+__device__ inline float silu_mul16(float x, float y) {
+  const float s = nq_round16<BF16>(x / (1.0f + expf(-x)));
+  return nq_round16<BF16>(s * y);
+}
+
+template <bool BF16, bool VEC>
+__global__ __launch_bounds__(NQ_T) void silu_and_mul_fp8_kernel(uint8_t* __restrict__ out,
+                                                                const uint16_t* __restrict__ input,
+                                                                const float* __restrict__ scale, int64_t tokens, int d) {
+  const float inv = 1.0f / *scale;
+  if constexpr (VEC) {
+    const int chunks = d / 8;
+    const int64_t total = tokens * chunks;
+    for (int64_t idx = (int64_t)blockIdx.x * NQ_T + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * NQ_T) {
+      const int64_t tok = idx / chunks;
+      const int c = (int)(idx - tok * chunks);
+      const uint16_t* xr = input + tok * 2 * (int64_t)d + c * 8;
+      float x[8], y[8];
+      nq_unpack8(*reinterpret_cast<const v4u*>(xr), x, BF16);
+      nq_unpack8(*reinterpret_cast<const v4u*>(xr + d), y, BF16);
+      v2u o;
+      uint32_t* ow = reinterpret_cast<uint32_t*>(&o);
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        float q[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          q[e] = fmaxf(-NQ_FP8_MAX, fminf(silu_mul16<BF16>(x[4 * h + e], y[4 * h + e]) * inv, NQ_FP8_MAX));
+        uint32_t lo = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false) & 0xffffu;
+        uint32_t hi = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], 0, false) & 0xffffu;
+        ow[h] = lo | (hi << 16);
+      }
+      *reinterpret_cast<v2u*>(out + tok * (int64_t)d + c * 8) = o;
+    }
+  } else {
+    const int64_t total = tokens * d;
+    for (int64_t idx = (int64_t)blockIdx.x * NQ_T + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * NQ_T) {
+      const int64_t tok = idx / d;
+      const int i = (int)(idx - tok * d);
+      const uint16_t* xr = input + tok * 2 * (int64_t)d;
+      const float v = silu_mul16<BF16>(nq_to_float<BF16>(xr[i]), nq_to_float<BF16>(xr[d + i]));
+      const float q = fmaxf(-NQ_FP8_MAX, fminf(v * inv, NQ_FP8_MAX));
+      out[idx] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(q, q, 0, false) & 0xff);
+    }
+  }
+}
+
 }  // namespace
 
 }  // namespace vaq
@@ -213,5 +363,59 @@ extern "C" int vaq_rms_norm_dynamic_per_token_fp8_quant(uint8_t* out, float* sca
     else hipLaunchKernelGGL((rms_norm_per_token_fp8_kernel<false, false>), grid, block, 0, s, out, scales, in, w, scale_ub, epsilon, res, (int)hidden, in_stride);
   }
   VAQ_CHECK_LAUNCH("rms_norm_dynamic_per_token_quant");
+  return VAQ_OK;
+}
+
+extern "C" int vaq_rms_norm_static_fp8_quant(uint8_t* out, const void* input, int64_t in_stride, const void* weight,
+                                             const float* scale, float epsilon, void* residual, int dtype,
+                                             int64_t tokens, int64_t hidden, void* stream) {
+  using namespace vaq;
+  VAQ_CHECK_ARG(tokens >= 0 && hidden > 0 && hidden < (1ll << 31) && tokens < (1ll << 31),
+                "rms_norm_static_fp8_quant: bad shape [%lld, %lld]", (long long)tokens, (long long)hidden);
+  VAQ_CHECK_ARG(dtype == VAQ_F16 || dtype == VAQ_BF16, "rms_norm_static_fp8_quant: dtype tag %d", dtype);
+  VAQ_CHECK_ARG(in_stride >= hidden, "rms_norm_static_fp8_quant: input row stride %lld < hidden %lld",
+                (long long)in_stride, (long long)hidden);
+  if (tokens == 0) return VAQ_OK;
+  VAQ_CHECK_ARG(out && input && weight && scale, "rms_norm_static_fp8_quant: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)tokens), block(NQ_T);
+  const uint16_t* in = (const uint16_t*)input;
+  const uint16_t* w = (const uint16_t*)weight;
+  uint16_t* res = (uint16_t*)residual;
+  if (dtype == VAQ_BF16) {
+    if (res) hipLaunchKernelGGL((rms_norm_static_fp8_kernel<true, true>), grid, block, 0, s, out, in, w, scale, epsilon, res, (int)hidden, in_stride);
+    else hipLaunchKernelGGL((rms_norm_static_fp8_kernel<true, false>), grid, block, 0, s, out, in, w, scale, epsilon, res, (int)hidden, in_stride);
+  } else {
+    if (res) hipLaunchKernelGGL((rms_norm_static_fp8_kernel<false, true>), grid, block, 0, s, out, in, w, scale, epsilon, res, (int)hidden, in_stride);
+    else hipLaunchKernelGGL((rms_norm_static_fp8_kernel<false, false>), grid, block, 0, s, out, in, w, scale, epsilon, res, (int)hidden, in_stride);
+  }
+  VAQ_CHECK_LAUNCH("rms_norm_static_fp8_quant");
+  return VAQ_OK;
+}
+
+extern "C" int vaq_silu_and_mul_fp8_quant(uint8_t* out, const void* input, const float* scale, int dtype, int64_t tokens,
+                                          int64_t d, void* stream) {
+  using namespace vaq;
+  VAQ_CHECK_ARG(tokens >= 0 && d >= 0 && d < (1ll << 30) && tokens < (1ll << 31),
+                "silu_and_mul_quant: bad shape [%lld, 2*%lld]", (long long)tokens, (long long)d);
+  VAQ_CHECK_ARG(dtype == VAQ_F16 || dtype == VAQ_BF16, "silu_and_mul_quant: dtype tag %d", dtype);
+  if (tokens == 0 || d == 0) return VAQ_OK;
+  VAQ_CHECK_ARG(out && input && scale, "silu_and_mul_quant: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  const bool vec = d % 8 == 0 && ((uintptr_t)input % 16) == 0 && ((uintptr_t)out % 8) == 0;
+  const int64_t work = vec ? tokens * (d / 8) : tokens * d;
+  int64_t blocks = (work + NQ_T - 1) / NQ_T;
+  const int64_t cap = (int64_t)num_cus_current_device() * 32;
+  if (blocks > cap) blocks = cap;
+  const dim3 grid((unsigned)blocks), block(NQ_T);
+  const uint16_t* in = (const uint16_t*)input;
+  if (dtype == VAQ_BF16) {
+    if (vec) hipLaunchKernelGGL((silu_and_mul_fp8_kernel<true, true>), grid, block, 0, s, out, in, scale, tokens, (int)d);
+    else hipLaunchKernelGGL((silu_and_mul_fp8_kernel<true, false>), grid, block, 0, s, out, in, scale, tokens, (int)d);
+  } else {
+    if (vec) hipLaunchKernelGGL((silu_and_mul_fp8_kernel<false, true>), grid, block, 0, s, out, in, scale, tokens, (int)d);
+    else hipLaunchKernelGGL((silu_and_mul_fp8_kernel<false, false>), grid, block, 0, s, out, in, scale, tokens, (int)d);
+  }
+  VAQ_CHECK_LAUNCH("silu_and_mul_quant");
   return VAQ_OK;
 }
