@@ -91,12 +91,13 @@ int vaq_w4a16_gemm_workspace(int64_t size_m, int64_t size_n, int64_t size_k, int
  * Replaces `gptq_marlin_gemm(...)` (csrc/torch_bindings.cpp:309-315; csrc/quantization/gptq_marlin/gptq_marlin.cu:674-959).
  *   a        [M, K] 16-bit, row stride lda elements (lda % 8 == 0, base 16-byte aligned), unit column stride
  *   b        NATIVE-layout weights from vaq_w4a16_repack
- *   scales   [K/group_size, N] in the activation dtype, contiguous
- *   zeros    int32 [K/group_size, N/8] natural nibble order (wtype U4) or NULL (wtype U4B8)
+ *   scales   [K/group_size, N] ([1, N] for group_size -1) in the activation dtype, contiguous
+ *   zeros    int32 [K/group_size, N/8] ([1, N/8] for -1) natural nibble order (wtype U4) or NULL (wtype U4B8)
  *   perm     int32 [K] act_order sort indices or NULL  (is_k_full semantics: group of sorted row r is r / group_size)
  *   bias     [N] activation dtype or NULL
  *   c        [M, N] activation dtype, contiguous
- *   group_size  128 (the only size built; others return VAQ_ERR_UNSUPPORTED)
+ *   group_size  128, 64, 32, or -1 / K for channelwise scales (the reference's MARLIN_SUPPORTED_GROUP_SIZES,
+ *               marlin_utils.py:24); anything else returns VAQ_ERR_UNSUPPORTED
  * M == 0 is a no-op.  Kernel choice (decode: M <= 32, MFMA GEMV with in-register dequant; prefill: LDS-staged MFMA)
  * is internal; `force_path` = 0 auto, 1 decode, 2 prefill (tests / benchmarks).
  */

@@ -223,6 +223,8 @@ def dequantize(q: np.ndarray, scales: torch.Tensor, zp: np.ndarray | int, group_
     both the torch CPU multiply and the device ``__hmul2`` (marlin_template.h:162-171) produce.
     """
     k, n = q.shape
+    if group_size == -1:
+        group_size = k          # channelwise: one group spans K (marlin_utils.py:66, quant_utils.py:395-396)
     grp = (np.arange(k) // group_size) if g_idx is None else np.asarray(g_idx).astype(np.int64)
     grp_t = torch.from_numpy(np.asarray(grp, dtype=np.int64))
     if isinstance(zp, (int, np.integer)):
@@ -269,9 +271,12 @@ def make_w4a16_case(k: int, n: int, group_size: int = 128, *, asym: bool = False
     ``qweight`` int32[K/8,N] = gptq_pack(q), ``scales`` [G,N] ``dtype`` (made in fp16 then cast, as a checkpoint
     loader would), ``zp_vals`` int32[G,N] / ``qzeros`` int32[G,N/8] (asym only, else None),
     ``g_idx`` int32[K] (act_order only: group of row r, = (arange(K)//g)[rand_perm], quant_utils.py:357-366),
-    ``group_size``.  ``group_level_perm`` permutes whole groups instead of single rows.
+    ``group_size`` (-1: channelwise, one group).  ``group_level_perm`` permutes whole groups instead of single rows.
     """
     rng = np.random.default_rng(seed)
+    orig_group_size = group_size
+    if group_size == -1:
+        group_size = k
     g = k // group_size
     q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
     tg = torch.Generator().manual_seed(seed)
@@ -286,7 +291,7 @@ def make_w4a16_case(k: int, n: int, group_size: int = 128, *, asym: bool = False
             rand_perm = rng.permutation(k)
         g_idx = (np.arange(k) // group_size).astype(np.int32)[rand_perm]
     return dict(q=q, qweight=gptq_pack(q, 4), scales=scales, zp_vals=zp_vals,
-                qzeros=pack_cols(zp_vals, 4) if asym else None, g_idx=g_idx, group_size=group_size)
+                qzeros=pack_cols(zp_vals, 4) if asym else None, g_idx=g_idx, group_size=orig_group_size)
 
 
 def case_w_ref(case: dict) -> torch.Tensor:

@@ -38,7 +38,7 @@ class W4A16Layer:
         self.w = ops.gptq_marlin_repack(qweight, self.sort_idx, k, n, 4)
         self.scales = mu.marlin_permute_scales(to_dev(case["scales"], device, dtype), k, n, self.g)
         if case["zp_vals"] is not None:
-            self.zp = mu.marlin_zero_points(to_dev(case["zp_vals"], device), k // self.g, n, 4)
+            self.zp = mu.marlin_zero_points(to_dev(case["zp_vals"], device), case["zp_vals"].shape[0], n, 4)
             self.wtype = scalar_types.uint4
         else:
             self.zp = empty

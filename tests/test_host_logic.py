@@ -48,7 +48,7 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     rc = lib.vaq_w4a16_gemm(None, 4096, None, None, None, None, None, None, None, None, None, 0, 16, 4096 + 32, 4096,
                             128, _lib.VAQ_BF16, _lib.VAQ_WTYPE_U4B8, 0, None)
     assert rc == _lib.VAQ_ERR_INVALID_ARG and b"min_thread_n" in lib.vaq_last_error()
-    rc = lib.vaq_w4a16_gemm(None, 4096, None, None, None, None, None, None, None, None, None, 0, 16, 4096, 4096, 64,
+    rc = lib.vaq_w4a16_gemm(None, 4096, None, None, None, None, None, None, None, None, None, 0, 16, 4096, 4096, 256,
                             _lib.VAQ_BF16, _lib.VAQ_WTYPE_U4B8, 0, None)
     assert rc == _lib.VAQ_ERR_UNSUPPORTED and b"group_size" in lib.vaq_last_error()
     rc = lib.vaq_fp8_scaled_mm(None, 100, None, 128, None, 1, None, 1, None, None, 128, _lib.VAQ_BF16, 4, 128, 128, None)
@@ -138,7 +138,8 @@ def test_shape_and_type_support_checks():
     for bad in ((4096 + 32, 4096, 4096, 128), (4096, 4096 + 64, 4096 + 64, 128)):
         with pytest.raises(ValueError):
             mu.verify_marlin_supports_shape(*bad)
-    assert mu.check_marlin_supported(st.uint4b8, 128) and not mu.check_marlin_supported(st.uint4b8, 64)
+    assert mu.check_marlin_supported(st.uint4b8, 128) and not mu.check_marlin_supported(st.uint4b8, 256)
+    assert all(mu.check_marlin_supported(st.uint4b8, g) for g in (-1, 32, 64))
     assert mu.check_marlin_supported(st.uint4, 128, has_zp=True) and not mu.check_marlin_supported(st.uint4, 128)
     with pytest.raises(ValueError):
         mu.verify_marlin_supported(st.uint8b128, 128)
@@ -268,7 +269,9 @@ def test_plugin_surface_contract():
     assert GPTQMarlinConfig.override_quantization_method(dict(quant_method="gptq", bits=4, group_size=128, sym=True, desc_act=False), None) == "gptq_marlin"
     mp = MPLinearLayerConfig((4096, 4096), (4096, 4096), st.uint4, torch.bfloat16, 128, True, False)
     assert choose_mp_linear_kernel(mp) is HipW4A16LinearKernel
-    bad = MPLinearLayerConfig((4096, 4096), (4096, 4096), st.uint4b8, torch.bfloat16, 32, False, False)
+    assert choose_mp_linear_kernel(MPLinearLayerConfig((4096, 4096), (4096, 4096), st.uint4b8, torch.bfloat16, 32, False,
+                                                       False)) is HipW4A16LinearKernel
+    bad = MPLinearLayerConfig((4096, 4096), (4096, 4096), st.uint4b8, torch.bfloat16, 256, False, False)
     with pytest.raises(ValueError, match="Group size"):
         choose_mp_linear_kernel(bad)
     os.environ["VLLM_DISABLED_KERNELS"] = "HipW4A16LinearKernel"

@@ -131,6 +131,47 @@ def test_awq_linear_method_end_to_end(device, dtype):
         check_gemm_close(out, o.gemm_ref(a, w_ref, bias), f"awq method {dtype} m={m}")
 
 
+@pytest.mark.parametrize("group_size", [-1, 32, 64])
+def test_gptq_and_awq_methods_other_group_sizes(device, group_size):
+    """The linear methods at the reference's other supported group sizes (marlin_utils.py:24): a GPTQ layer (channelwise
+    when group_size = -1; otherwise with act_order, once row-level and once moving whole groups, which is folded at load
+    also for 32- and 64-row groups) and an AWQ layer."""
+    from vllm_amd.layers.linear import LinearBase
+    from vllm_amd.layers.quantization import get_quantization_config
+    k, n = 1024, 256
+    desc_act = group_size != -1
+    cfg = get_quantization_config("gptq_marlin").from_config(dict(bits=4, group_size=group_size, desc_act=desc_act, sym=True))
+    for group_level in ((False, True) if desc_act else (False,)):
+        case = o.make_w4a16_case(k, n, group_size, act_order=desc_act, group_level_perm=group_level, seed=50 + group_size)
+        layer = LinearBase(k, n, quant_config=cfg, params_dtype=torch.bfloat16, return_bias=False).to(device)
+        assert layer.scales.shape == case["scales"].shape
+        layer.qweight.data.copy_(to_dev(case["qweight"], device))
+        layer.scales.data.copy_(to_dev(case["scales"], device, torch.bfloat16))
+        gs = k if group_size == -1 else group_size
+        g_idx = case["g_idx"] if case["g_idx"] is not None else np.arange(k, dtype=np.int32) // gs
+        layer.g_idx.data.copy_(to_dev(g_idx, device))
+        layer.process_weights_after_loading()
+        assert layer.quant_method.kernel.act_order_folded == group_level
+        w_ref = o.case_w_ref(case)
+        for m in (1, 16, 32, 150):
+            a = _acts(m, k, seed=m)
+            check_gemm_close(layer(a.to(device)), o.gemm_ref(a, w_ref), f"gptq g={group_size} folded={group_level} m={m}")
+    if group_size == -1:
+        return      # AutoAWQ has no channelwise checkpoints
+    hf = dict(quant_method="awq", bits=4, group_size=group_size, zero_point=True)
+    cfg = get_quantization_config("awq_marlin").from_config(hf)
+    case = o.make_w4a16_case(k, n, group_size, asym=True, seed=60 + group_size)
+    layer = LinearBase(k, n, quant_config=cfg, params_dtype=torch.bfloat16, return_bias=False).to(device)
+    layer.qweight.data.copy_(to_dev(o.awq_pack(case["q"], 4), device))
+    layer.qzeros.data.copy_(to_dev(o.awq_pack(case["zp_vals"], 4), device))
+    layer.scales.data.copy_(to_dev(case["scales"], device, torch.bfloat16))
+    layer.process_weights_after_loading()
+    w_ref = o.case_w_ref(case)
+    for m in (1, 16, 32, 150):
+        a = _acts(m, k, seed=m)
+        check_gemm_close(layer(a.to(device)), o.gemm_ref(a, w_ref), f"awq g={group_size} m={m}")
+
+
 def _fp8_close(out, ref64, what):
     """Holds the result to 2 ulp of the output type + 2e-3 of the mean magnitude against an fp64 accumulation of the
     same quantised operands (bitwise parity of this GEMM is not pinned by any reference test)."""

@@ -140,6 +140,55 @@ def test_prefill_gemm_split_k(device, k, n, m, asym):
     assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
 
 
+@pytest.mark.parametrize("group_size", [-1, 32, 64])
+@pytest.mark.parametrize("k,n", [(128, 64), (1024, 192), (2048, 576), (14336 // 4, 128)])
+@pytest.mark.parametrize("m", [1, 4, 16, 17, 32, 33, 200, 257])
+@pytest.mark.parametrize("asym,act_order", [(False, False), (True, False), (True, True)])
+def test_gemm_other_group_sizes(device, group_size, k, n, m, asym, act_order):
+    """Channelwise scales (group_size -1) and groups of 32 / 64 rows -- the other entries of the reference's
+    MARLIN_SUPPORTED_GROUP_SIZES (marlin_utils.py:24; its GEMM test sweeps them, test_marlin_gemm.py:228-361) -- on both
+    the decode and the prefill kernels, with zero points and with act_order."""
+    if act_order and (group_size == -1 or k == 128):
+        pytest.skip("act_order needs more than one group (gptq_marlin.cu:805)")
+    case = o.make_w4a16_case(k, n, group_size, asym=asym, act_order=act_order, seed=k + n + m + group_size)
+    layer = W4A16Layer(case, device)
+    a = _acts(m, k, device, seed=m)
+    out = layer(a)
+    check_gemm_close(out, o.gemm_ref(a.cpu(), o.case_w_ref(case)), f"g={group_size} k={k} n={n} m={m}")
+    assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
+
+
+@pytest.mark.parametrize("group_size", [-1, 32, 64])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m", [1, 48])
+def test_one_hot_activation_other_group_sizes_exact(device, decode_kernel, group_size, dtype, m):
+    """One-hot rows of A select single dequantised weight rows: every row must come back as rn16((q - z) * s) of ITS
+    group, bit for bit -- a wrong scale or zero-point row for any sub-block of a 128-row tile shows here."""
+    k, n = 512, 128
+    case = o.make_w4a16_case(k, n, group_size, asym=True, dtype=dtype, seed=13 + group_size)
+    layer = W4A16Layer(case, device, dtype)
+    w = o.case_w_ref(case)
+    for base in (0, 7):
+        rows = [(37 * i + 32 * (i % 4) + base) % k for i in range(m)]
+        a = torch.zeros(m, k, dtype=dtype)
+        for i, r in enumerate(rows):
+            a[i, r] = 1
+        assert torch.equal(layer(a.to(device)).cpu(), w[rows])
+
+
+def test_gemm_other_group_sizes_llama_shape(device):
+    """Llama-3-8B's down_proj (K = 14336: K split over workgroups on the decode path) at group sizes 32 / 64 / -1."""
+    k, n = 14336, 4096
+    for group_size in (32, 64, -1):
+        case = o.make_w4a16_case(k, n, group_size, asym=group_size == 32, seed=group_size + 40)
+        layer = W4A16Layer(case, device)
+        w_ref = o.case_w_ref(case)
+        for m in (1, 16, 32, 160):
+            a = _acts(m, k, device, seed=m)
+            check_gemm_close(layer(a), o.gemm_ref(a.cpu(), w_ref), f"g={group_size} m={m}")
+        assert bool((layer.workspace == 0).all())
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("m", [1, 3, 16, 96])
 def test_gemm_fp16_and_bias(device, decode_kernel, dtype, m):

@@ -238,10 +238,12 @@ def _check_gemm_args(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, 
     if has_act_order and not is_k_full:
         raise NotImplementedError("gptq_marlin_gemm: is_k_full = False (act_order x row-parallel shard) is not built; "
                                   "one-GPU layers always have is_k_full = True")
-    if group_size == -1 and size_k == 128:
-        group_size = 128          # one group spanning K = 128 rows is the same thing as group_size 128
-    if group_size != 128:
-        raise NotImplementedError(f"gptq_marlin_gemm: group_size = {group_size} is not built for gfx950 (only 128)")
+    if group_size not in (-1, 32, 64, 128):
+        if group_size == size_k:
+            group_size = -1       # one group spanning all of K is channelwise
+        else:
+            raise NotImplementedError(f"gptq_marlin_gemm: group_size = {group_size} is not built for gfx950 "
+                                      "(only -1, 32, 64, 128)")
     _check(size_k % GPTQ_MARLIN_MIN_THREAD_K == 0,
            f"size_k = {size_k}, is not divisible by min_thread_k = {GPTQ_MARLIN_MIN_THREAD_K}")
     wtype = _lib.VAQ_WTYPE_U4 if has_zp else _lib.VAQ_WTYPE_U4B8

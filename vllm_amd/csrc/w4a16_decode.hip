@@ -37,6 +37,7 @@ struct DecodeParams {
   v4f* c_tmp;
   int32_t* counters;
   int M, N, K, G, NT, SK, WK;
+  int GR, s_stride, z_stride;   // rows of scales / zeros and the element strides between them (1 row, strides 0: channelwise)
   uint32_t k_mask, k_ex;   // 0x000f000f and the exponent pattern, passed as run-time values (see and_or)
 };
 
@@ -98,8 +99,8 @@ __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodePar
   // Weights, scales and zero points are read through buffer descriptors: the per-tile part of the address is a
   // scalar offset, the per-lane part a constant, so a load costs no vector ALU work.
   const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b, (uint64_t)p.K * p.N / 2);
-  const __amdgpu_buffer_rsrc_t rs = make_rsrc(p.scales, (uint64_t)p.G * p.N * 2);
-  const __amdgpu_buffer_rsrc_t rz = make_rsrc(HAS_ZP ? (const void*)p.zeros : (const void*)p.scales, (uint64_t)p.G * (p.N / 8) * 4);
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(p.scales, (uint64_t)p.GR * p.N * 2);
+  const __amdgpu_buffer_rsrc_t rz = make_rsrc(HAS_ZP ? (const void*)p.zeros : (const void*)p.scales, (uint64_t)p.GR * (p.N / 8) * 4);
   const int vo_b = lane * 16, vo_s = o * 8, vo_z = (o >> 1) * 4;
 
   v4u wq[D][TG];
@@ -112,8 +113,8 @@ __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodePar
   for (int t = 0; t < TG; ++t) {
     const uint32_t g = (uint32_t)min(g0 + t, p.G - 1);
     ob[t] = g * 1024u;
-    os_[t] = g * (uint32_t)p.N * 2u;
-    oz[t] = g * (uint32_t)(p.N >> 3) * 4u;
+    os_[t] = g * (uint32_t)p.s_stride * 2u;
+    oz[t] = g * (uint32_t)p.z_stride * 4u;
   }
   auto issue_load = [&](int u, int nt, int t) {
     wq[u][t] = __builtin_amdgcn_raw_buffer_load_b128(rb, vo_b, (int)(ob[t] + (uint32_t)nt * (uint32_t)p.G * 1024u), 2);
@@ -404,7 +405,7 @@ int w4a16_decode_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* cou
 
 int w4a16_decode_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
                         const int32_t* perm, const void* bias, void* c, float* c_tmp, int32_t* counters,
-                        int64_t counter_ints, int M, int N, int K, int dtype, hipStream_t s) {
+                        int64_t counter_ints, int M, int N, int K, bool channelwise, int dtype, hipStream_t s) {
   DecodeParams p;
   p.a = (const uint16_t*)a;
   p.lda = lda;
@@ -419,6 +420,9 @@ int w4a16_decode_launch(const void* a, int64_t lda, const int32_t* b, const void
   p.M = M; p.N = N; p.K = K;
   p.G = K / 128;
   p.NT = N / 16;
+  p.GR = channelwise ? 1 : p.G;
+  p.s_stride = channelwise ? 0 : N;
+  p.z_stride = channelwise ? 0 : N / 8;
   p.k_mask = 0x000f000fu;
   p.k_ex = dtype == VAQ_BF16 ? 0x43004300u : 0x64006400u;
   const DecodeConfig cfg = pick_decode_config(M, N, K);

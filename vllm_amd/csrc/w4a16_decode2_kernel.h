@@ -1,0 +1,378 @@
+// W4A16 decode-shaped GEMM (M <= 32), barrier-free variant: activations staged in LDS, one independent task per
+// wavefront.  C[M,N] = A[M,K] . dequant(B[K,N]) (+bias), same arithmetic as w4a16_decode.hip.
+//
+//  * A workgroup is WKS slices of K  x  WN n-tiles (16 columns each) = up to 16 wavefronts.  Wavefront (wks, wn)
+//    streams the GS consecutive 1 KiB weight tiles (= quantisation groups) of its slice for its n-tile through a
+//    register ring of min(GS, 2) slots; no wavefront ever waits for another one inside the K loop.
+//  * The activations of the workgroup's K slab (WKS*GS groups) are written once to LDS in MFMA-B-operand order
+//    ([k-octet][m] 16-byte slots, rows m >= M zero, XOR-swizzled so that both the row-contiguous fill and the
+//    operand reads are bank-conflict free) and read back with one ds_read_b128 per MFMA.  The activation loads are
+//    issued before the first weight loads, in branch-free code (see step 1).  Only MR rows per m-block are staged
+//    (MR = 1, 4 or 16, the smallest that holds M): MFMA columns are independent, so lanes of the columns m >= MR read
+//    the slot of row m mod MR and their results are never stored.  With few rows a whole K = 14336 slab fits LDS and
+//    K need not be split over workgroups.
+//  * Per tile: 4 x { dequantise one word to 8 biased 16-bit numbers (7 VALU ops), MFMA with the activations, MFMA of
+//    the constant operand -(BIAS + zero) with the same activations }, then acc += scale * P (fp32).  The second MFMA
+//    removes the bias and the zero point exactly as `P - (BIAS+z)*S` would, without keeping S anywhere.
+//  * Quantisation groups of 64 or 32 rows (SUBG = 2 or 4 groups per tile): the same, per sub-group of 2 or 1 MFMA pairs.
+//    Channelwise scales are one row read with a row stride of 0.
+//  * WKS > 1: one LDS reduction at the end (wavefronts wks == 0 sum their column's slices).  K slabs that do not fit
+//    LDS (SK > 1 workgroups per n-tile) hand partial tiles over through device-scope write-through stores and an
+//    arrival counter, summed in fixed order by the last arriver.
+#pragma once
+#include "vaq_common.h"
+
+#include <type_traits>
+
+namespace vaq {
+
+struct Decode2Params {
+  const uint16_t* a;
+  int64_t lda;
+  const v4u* b;
+  const uint16_t* scales;
+  const uint32_t* zeros;
+  const int32_t* perm;
+  const uint16_t* bias;
+  uint16_t* c;
+  float* c_tmp;
+  int32_t* counters;
+  int M, N, K, G, NT, SK, WKS, WN;
+  int GR;                  // rows of the scale / zero-point tensors (G * SUBG, or 1 for channelwise scales)
+  int s_stride, z_stride;  // elements between consecutive rows of scales (N) / zeros (N/8); 0 for channelwise
+  uint32_t k_mask, k_ex;   // 0x000f000f and the exponent pattern, passed as run-time values (see and_or)
+};
+
+static __device__ inline void d2_store_partial(float* dst, v4f v) {
+  __hip_atomic_store(dst + 0, v.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(dst + 1, v.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(dst + 2, v.z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(dst + 3, v.w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+static __device__ inline v4f d2_load_partial(const float* src) {
+  v4f v;
+  v.x = __hip_atomic_load(src + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  v.y = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  v.z = __hip_atomic_load(src + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  v.w = __hip_atomic_load(src + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return v;
+}
+
+// (x & mask) | ex.  mask and ex reach the kernel as run-time arguments: with literal constants the compiler emits two
+// instructions (a VOP3 op of this architecture cannot carry two literals); with register operands it selects the
+// single v_and_or_b32, and unlike inline assembly the instruction stays visible to the MFMA hazard recogniser.
+static __device__ inline uint32_t d2_and_or(uint32_t x, uint32_t mask, uint32_t ex) { return (x & mask) | ex; }
+
+static __device__ inline __amdgpu_buffer_rsrc_t d2_rsrc(const void* base, uint64_t bytes) {
+  const uint32_t n = bytes > 0xffffffffull ? 0xffffffffu : (uint32_t)bytes;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)n, 0x00020000);
+}
+
+constexpr int D2_WAVES = 16;
+
+template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG>
+__global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Decode2Params p) {
+  using T = F16Traits<BF16>;
+  static_assert(SUBG == 1 || SUBG == 2 || SUBG == 4, "quantisation groups per 128-row tile");
+  static_assert(MR == 16 || MB == 1, "compact row staging is for a single m-block");
+  // Ring slots.  Two tiles in flight per wavefront measured best: a wavefront does not get past its load instructions
+  // until the memory pipeline has accepted them, and with deeper rings (every wavefront of the device asking for
+  // 7-8 KiB at once) the first MFMA of each wavefront starts when most of the stream has already been served, so the
+  // arithmetic no longer overlaps it.
+  constexpr int R = GS < 2 ? GS : 2;
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+  const int lane = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(threadIdx.y);
+  const int o = lane >> 4, r16 = lane & 15;
+  const int WKS = p.WKS, WN = p.WN;
+  const int wks = w / WN, wn = w - wks * WN;
+  const int sk = blockIdx.y;
+  const int slab_groups = WKS * GS;
+  const int slab_g0 = sk * slab_groups;             // first group of this workgroup's K slab
+  const int nt_raw = blockIdx.x * WN + wn;
+  const bool nt_ok = nt_raw < p.NT;
+  const int nt = nt_ok ? nt_raw : p.NT - 1;
+  const int g_first = slab_g0 + wks * GS;           // this wavefront's first group
+
+  // ---- 1. activations of the K slab -> LDS, with the first R weight tiles requested in between ----
+  // Loads retire in issue order as far as the wait counter is concerned, so the activation loads go out FIRST: the
+  // wait before the LDS writes then leaves the weight tiles in flight instead of draining them.
+  // slot (16 bytes) of (m-block mb, row ml, k-octet ko):  mb*KO*MR + ko*MR + (ml ^ (ko & (MR-1)))
+  const __amdgpu_buffer_rsrc_t rb = d2_rsrc(p.b, (uint64_t)p.K * p.N / 2);
+  const __amdgpu_buffer_rsrc_t rs = d2_rsrc(p.scales, (uint64_t)p.GR * p.N * 2);
+  const __amdgpu_buffer_rsrc_t rz = d2_rsrc(HAS_ZP ? (const void*)p.zeros : (const void*)p.scales, (uint64_t)p.GR * (p.N / 8) * 4);
+  const int vo_b = lane * 16, vo_s = o * 8, vo_z = (r16 >> 3) * 4;
+  v4u wq[R];
+  v2u sc[R][SUBG];
+  uint32_t zq[R][SUBG];
+  auto issue_load = [&](int slot, int gi) {
+    const uint32_t g = (uint32_t)min(g_first + gi, p.G - 1);     // clamped: activations past K are zero
+    wq[slot] = __builtin_amdgcn_raw_buffer_load_b128(rb, vo_b, (int)(((uint32_t)nt * (uint32_t)p.G + g) * 1024u), 2);
+#pragma unroll
+    for (int sj = 0; sj < SUBG; ++sj) {
+      const uint32_t row = g * (uint32_t)SUBG + (uint32_t)sj;
+      sc[slot][sj] = __builtin_amdgcn_raw_buffer_load_b64(rs, vo_s, (int)((row * (uint32_t)p.s_stride + (uint32_t)nt * 16u) * 2u), 0);
+      if constexpr (HAS_ZP)
+        zq[slot][sj] = __builtin_amdgcn_raw_buffer_load_b32(rz, vo_z, (int)((row * (uint32_t)p.z_stride + (uint32_t)nt * 2u) * 4u), 0);
+      else
+        zq[slot][sj] = 0u;
+    }
+  };
+
+  const int KO = slab_groups * 16;                   // k-octets in the slab
+  // 16 bytes behind the activations for lanes without a chunk (the start of the reduction buffer, unused until the K
+  // loop is over, when there is one)
+  const uint32_t dummy_slot = (uint32_t)(KO * MR * MB);
+  {
+    // chunk c = m * KO + ko (16 bytes: row m, k-octet ko); thread tid handles c = tid, tid + NTHR, ...  The (m, ko)
+    // pair is advanced incrementally: one scalar division per kernel instead of one vector division per chunk.
+    const int tid = w * 64 + lane;
+    const int chunks = KO * MR * MB;
+    const int64_t k_slab0 = (int64_t)slab_g0 * 128;
+    const int NTHR = WKS * WN * 64;
+    const int step_m = NTHR / KO, step_ko = NTHR - step_m * KO;     // scalar
+    int m = tid / KO, ko = tid - m * KO;
+    if (p.perm == nullptr) {
+      // Straight-line code, no branch between the loads and the LDS writes (at a join the compiler's wait-count
+      // bookkeeping falls back to draining every load): the rows are read through a buffer descriptor that ends with
+      // the last valid element, chunks that do not exist get an out-of-range offset and come back as zeros, and
+      // their lanes write to a dummy slot.  FB chunks per thread cover a full-size slab in the first pass.
+      constexpr int FB = MR == 1 ? 2 : 8;
+      const __amdgpu_buffer_rsrc_t ra = d2_rsrc(p.a, ((uint64_t)(p.M - 1) * (uint64_t)p.lda + (uint64_t)p.K) * 2);
+      auto fill_pass = [&](auto first) {
+        v4u v[FB];
+        uint32_t slot[FB];
+#pragma unroll
+        for (int i = 0; i < FB; ++i) {
+          const int64_t k = k_slab0 + (int64_t)ko * 8;
+          const bool ok = m < MR * MB && m < p.M && k < p.K;
+          const uint32_t off = ok ? (uint32_t)(((int64_t)m * p.lda + k) * 2) : 0x80000000u;
+          v[i] = __builtin_amdgcn_raw_buffer_load_b128(ra, (int)off, 0, 0);
+          const int mb = m / MR, ml = m % MR;
+          slot[i] = m < MR * MB ? (uint32_t)(mb * KO * MR + ko * MR + (ml ^ (ko & (MR - 1)))) : dummy_slot;
+          m += step_m;
+          ko += step_ko;
+          if (ko >= KO) {
+            ko -= KO;
+            m += 1;
+          }
+        }
+        if constexpr (decltype(first)::value) {
+#pragma unroll
+          for (int s = 0; s < R; ++s) issue_load(s, s);
+        }
+#pragma unroll
+        for (int i = 0; i < FB; ++i) *reinterpret_cast<v4u*>(lds + (size_t)slot[i] * 16) = v[i];
+      };
+      fill_pass(std::true_type{});
+      for (int c0 = NTHR * FB; c0 < chunks; c0 += NTHR * FB) fill_pass(std::false_type{});
+    } else {
+      // act_order: the columns of A are gathered through `perm`; two dependent levels of loads, weights requested first
+#pragma unroll
+      for (int s = 0; s < R; ++s) issue_load(s, s);
+      for (int c0 = 0; c0 < chunks; c0 += NTHR * 4) {
+        v4u v[4];
+        int mm[4], kk[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          mm[i] = m;
+          kk[i] = ko;
+          const int64_t k = k_slab0 + (int64_t)ko * 8;
+          v[i] = v4u{0u, 0u, 0u, 0u};
+          if (m < MR * MB && m < p.M && k < p.K) {
+            const uint16_t* row = p.a + (int64_t)m * p.lda;
+            const v4i p0 = *reinterpret_cast<const v4i*>(p.perm + k);
+            const v4i p1 = *reinterpret_cast<const v4i*>(p.perm + k + 4);
+            v[i].x = (uint32_t)row[p0.x] | ((uint32_t)row[p0.y] << 16);
+            v[i].y = (uint32_t)row[p0.z] | ((uint32_t)row[p0.w] << 16);
+            v[i].z = (uint32_t)row[p1.x] | ((uint32_t)row[p1.y] << 16);
+            v[i].w = (uint32_t)row[p1.z] | ((uint32_t)row[p1.w] << 16);
+          }
+          m += step_m;
+          ko += step_ko;
+          if (ko >= KO) {
+            ko -= KO;
+            m += 1;
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (mm[i] < MR * MB) {
+            const int mb = mm[i] / MR, ml = mm[i] % MR;
+            const int slot = mb * KO * MR + kk[i] * MR + (ml ^ (kk[i] & (MR - 1)));
+            *reinterpret_cast<v4u*>(lds + (size_t)slot * 16) = v[i];
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- 3. the K loop of this wavefront: GS tiles, fully unrolled ----
+  // operand read of MFMA jj of local group gl: k-octet = gl*16 + jj*4 + o  ->  (ko & 15) = jj*4 + o
+  uint32_t abase[4];
+#pragma unroll
+  for (int jj = 0; jj < 4; ++jj) {
+    const int kol = jj * 4 + o;
+    abase[jj] = (uint32_t)(((wks * GS * 16 + kol) * MR + ((r16 ^ kol) & (MR - 1))) * 16);
+  }
+  uint32_t ex;     // kept in a vector register so that (x & MSK) | ex is a legal single VOP3 instruction (one scalar operand)
+  asm volatile("v_mov_b32 %0, %1" : "=v"(ex) : "s"(p.k_ex));
+  const uint32_t MSK = p.k_mask;
+  constexpr uint32_t NEG_BIAS_BITS = BF16 ? 0xC300u : 0xE400u;     // -(BIAS) as a 16-bit pattern; "| z" adds the zero point
+  v4f acc[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) acc[mb] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  // One tile: `slot` is a compile-time constant wherever this is expanded; `reissue` refills the slot R tiles ahead.
+  auto do_tile = [&](int gi, int slot, bool reissue) {
+    const uint32_t wj[4] = {wq[slot].x, wq[slot].y, wq[slot].z, wq[slot].w};
+    v2u sct[SUBG];
+    uint32_t zqt[SUBG];
+#pragma unroll
+    for (int sj = 0; sj < SUBG; ++sj) {
+      sct[sj] = sc[slot][sj];
+      zqt[sj] = zq[slot][sj];
+    }
+    if (reissue) issue_load(slot, gi + R);
+
+#pragma unroll
+    for (int sj = 0; sj < SUBG; ++sj) {
+      uint32_t zbits;
+      if constexpr (HAS_ZP) zbits = NEG_BIAS_BITS | ((zqt[sj] >> ((r16 & 7) * 4)) & 0xFu);
+      else zbits = NEG_BIAS_BITS | 8u;
+      const uint32_t z2 = zbits | (zbits << 16);
+      const v4u zop = {z2, z2, z2, z2};
+
+      v4f P[MB];
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) P[mb] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int jj = sj * (4 / SUBG); jj < (sj + 1) * (4 / SUBG); ++jj) {
+        v4u aop;
+        aop.x = d2_and_or(wj[jj], MSK, ex);
+        aop.y = d2_and_or(wj[jj] >> 4, MSK, ex);
+        aop.z = d2_and_or(wj[jj] >> 8, MSK, ex);
+        aop.w = d2_and_or(wj[jj] >> 12, MSK, ex);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+          const v4u bop = *reinterpret_cast<const v4u*>(lds + abase[jj] + (uint32_t)(mb * KO * MR * 16) + (uint32_t)(gi * 256 * MR));
+          P[mb] = T::mfma16(aop, bop, P[mb]);
+          P[mb] = T::mfma16(zop, bop, P[mb]);
+        }
+      }
+      float s[4];
+      if constexpr (BF16) {
+        s[0] = __uint_as_float(sct[sj].x << 16);
+        s[1] = __uint_as_float(sct[sj].x & 0xffff0000u);
+        s[2] = __uint_as_float(sct[sj].y << 16);
+        s[3] = __uint_as_float(sct[sj].y & 0xffff0000u);
+      } else {
+        s[0] = T::to_float((uint16_t)(sct[sj].x & 0xffffu));
+        s[1] = T::to_float((uint16_t)(sct[sj].x >> 16));
+        s[2] = T::to_float((uint16_t)(sct[sj].y & 0xffffu));
+        s[3] = T::to_float((uint16_t)(sct[sj].y >> 16));
+      }
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[mb][r] = fmaf(s[r], P[mb][r], acc[mb][r]);
+    }
+  };
+  if constexpr (GS <= 4) {
+#pragma unroll
+    for (int gi = 0; gi < GS; ++gi) do_tile(gi, gi % R, gi + R < GS);
+  } else {
+    // Long streams run as a rolled loop of R tiles per trip (short code: these kernels alternate with others and
+    // start with a cold instruction cache).  Every trip of the loop refills its slots unconditionally -- a branch
+    // around a load would make the compiler's wait counts drain the ring -- and the last tiles are peeled.
+    constexpr int MAIN = ((GS - R) / R) * R;      // tiles consumed inside the loop
+#pragma unroll 1
+    for (int g0 = 0; g0 < MAIN; g0 += R) {
+#pragma unroll
+      for (int u = 0; u < R; ++u) do_tile(g0 + u, u, true);
+    }
+#pragma unroll
+    for (int gi = MAIN; gi < GS; ++gi) do_tile(gi, gi % R, gi + R < GS);
+  }
+
+  // ---- 4. reduce the K slices of the workgroup ----
+  v4f* red = reinterpret_cast<v4f*>(lds + (size_t)KO * MR * MB * 16);     // [16 waves][MB][64]
+  if (WKS > 1) {
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) red[(w * MB + mb) * 64 + lane] = acc[mb];
+    __syncthreads();
+    if (wks != 0) return;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      v4f t = acc[mb];
+      for (int s2 = 1; s2 < WKS; ++s2) t += red[((s2 * WN + wn) * MB + mb) * 64 + lane];
+      acc[mb] = t;
+    }
+  }
+  if (!nt_ok) return;
+
+  // ---- 5. hand over across workgroups if K is split, then write the 16-bit outputs ----
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    v4f val = acc[mb];
+    bool write_out = true;
+    if (p.SK > 1) {
+      const int64_t slot = (((int64_t)nt * MB + mb) * 64 + lane) * 4;
+      const int64_t sk_stride = (int64_t)p.NT * MB * 64 * 4;
+      d2_store_partial(p.c_tmp + sk * sk_stride + slot, val);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // partial tile acknowledged before the counter moves
+      int old = 0;
+      if (lane == 0) old = __hip_atomic_fetch_add(&p.counters[nt * MB + mb], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      old = __shfl(old, 0);
+      write_out = (old == p.SK - 1);
+      if (write_out) {
+        val = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int s2 = 0; s2 < p.SK; ++s2) val += d2_load_partial(p.c_tmp + s2 * sk_stride + slot);   // fixed order
+        if (lane == 0) __hip_atomic_store(&p.counters[nt * MB + mb], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    const int m = mb * 16 + r16;
+    if (write_out && m < p.M) {
+      const int n = nt * 16 + o * 4;
+      if (p.bias) {
+        const v2u bb = *reinterpret_cast<const v2u*>(p.bias + n);
+        val[0] += T::to_float((uint16_t)(bb.x & 0xffffu));
+        val[1] += T::to_float((uint16_t)(bb.x >> 16));
+        val[2] += T::to_float((uint16_t)(bb.y & 0xffffu));
+        val[3] += T::to_float((uint16_t)(bb.y >> 16));
+      }
+      v2u outv;
+      outv.x = (uint32_t)T::from_float(val[0]) | ((uint32_t)T::from_float(val[1]) << 16);
+      outv.y = (uint32_t)T::from_float(val[2]) | ((uint32_t)T::from_float(val[3]) << 16);
+      *reinterpret_cast<v2u*>(p.c + (int64_t)m * p.N + n) = outv;
+    }
+  }
+}
+
+template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG>
+static int launch_decode2(const Decode2Params& p, hipStream_t s) {
+  const int WN = p.WN;
+  const size_t lds = (size_t)p.WKS * GS * 256 * MR * MB + (p.WKS > 1 ? (size_t)D2_WAVES * MB * 1024 : 16);
+  auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP, MR, SUBG>;
+  static size_t attr_lds = 0;
+  if (lds > attr_lds) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
+        hipSuccess) {
+      set_error("w4a16_gemm(decode): cannot reserve %zu bytes of LDS", lds);
+      (void)hipGetLastError();
+      return VAQ_ERR_LAUNCH;
+    }
+    attr_lds = lds;
+  }
+  const int gx = (p.NT + WN - 1) / WN;
+  hipLaunchKernelGGL(kern, dim3(gx, p.SK), dim3(64, p.WKS * WN), lds, s, p);
+  return VAQ_OK;
+}
+
+// Groups of 64 / 32 rows (sub = 2 / 4 per tile); defined in w4a16_decode2_sub.hip: 16 staged rows per m-block only,
+// groups per wavefront gs in {1, 2, 4, 8, 16}.
+int decode2_launch_sub(const Decode2Params& p, int sub, int gs, int MB, bool bf16, bool zp, hipStream_t s);
+
+}  // namespace vaq

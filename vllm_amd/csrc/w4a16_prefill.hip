@@ -1,616 +1,23 @@
-// W4A16 prefill-shaped GEMM (M > 32) for gfx950: C[M,N] = A[M,K] . dequant(B[K,N]) (+bias).
-//
-// MFMA-bound.  One workgroup (4 wavefronts, 2 x 2) computes a BM x BN output tile with v_mfma_f32_32x32x16;
-// each wavefront owns (BM/2) x (BN/2) of it as WMB x WNB accumulator blocks of 32 x 32 fp32.
-//
-//  * K is walked in steps of 64.  A[BM x 64] goes global -> registers -> LDS unchanged.  The weight tile is read
-//    in the NATIVE order (one 16-byte load per lane covers 128 k of one column, i.e. two K steps), dequantised
-//    *with* its group scale and zero point to the 16-bit activation type and written to LDS as [n][k] so that both
-//    MFMA operands are 16-byte, k-contiguous LDS reads.
-//  * Dequantisation is exact: code -> fp32 (v_cvt_f32_ubyte), w = fma(code, s, -(z*s)) is the exact real number
-//    (code - z) * s (<= 16 significant bits), then one round-to-nearest-even to bf16/fp16.  That is bit-for-bit the
-//    weight `(q - z).to(dtype) * s` of the reference's dequantise-then-matmul path.
-//  * LDS rows are padded to 72 elements (144 B): 16-byte accesses by 8 consecutive rows hit 8 disjoint bank groups.
-//  * LDS is double buffered: while the MFMAs of step i run from buffer i&1, step i+1 is staged into the other
-//    buffer; one barrier per step.  Global loads for step i+2 are issued right after the registers are drained.
-//  * act_order: the caller passes activations already gathered through `perm` (vaq_permute_cols).
-#include "vaq_common.h"
-
-#include <type_traits>
+// Host side of the prefill kernels (w4a16_prefill_kernel.h): tile and K-split choice, workspace sizes, launch of the
+// instances for quantisation groups of 128 rows and channelwise scales.
+#include "w4a16_prefill_kernel.h"
 
 namespace vaq {
 
-struct PrefillParams {
-  const uint16_t* a;
-  int64_t lda;
-  const v4u* b;
-  const uint16_t* scales;
-  const uint32_t* zeros;
-  const uint16_t* bias;
-  uint16_t* c;
-  float* c_tmp;        // fp32 partial tiles when K is split over workgroups (SK > 1)
-  int32_t* counters;   // arrival counters, zero on entry, left zero
-  int M, N, K, G, NT, SK;
-};
-
-constexpr int PF_BK = 64;
-constexpr int PF_PITCH = 72;   // LDS row pitch in 16-bit elements
-
-template <bool BF16>
-__device__ inline uint32_t pack2(float lo, float hi) {
-  if constexpr (BF16) {
-    typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
-    v2bf r = {(__bf16)lo, (__bf16)hi};   // v_cvt_pk_bf16_f32, round-to-nearest-even
-    return __builtin_bit_cast(uint32_t, r);
-  } else {
-    return (uint32_t)F16Traits<false>::from_float(lo) | ((uint32_t)F16Traits<false>::from_float(hi) << 16);
-  }
-}
-
-// One native weight word (8 codes of 8 consecutive k) -> 8 scaled 16-bit weights in k order.
-template <bool BF16>
-__device__ inline v4u dequant_scaled(uint32_t w, float s, float neg_zs) {
-  const uint32_t t = w & 0x0f0f0f0fu;          // nibble positions 0,2,4,6 -> elements 0,4,1,5
-  const uint32_t u = (w >> 4) & 0x0f0f0f0fu;   // nibble positions 1,3,5,7 -> elements 2,6,3,7
-  const float e0 = fmaf((float)(t & 0xffu), s, neg_zs);
-  const float e4 = fmaf((float)((t >> 8) & 0xffu), s, neg_zs);
-  const float e1 = fmaf((float)((t >> 16) & 0xffu), s, neg_zs);
-  const float e5 = fmaf((float)(t >> 24), s, neg_zs);
-  const float e2 = fmaf((float)(u & 0xffu), s, neg_zs);
-  const float e6 = fmaf((float)((u >> 8) & 0xffu), s, neg_zs);
-  const float e3 = fmaf((float)((u >> 16) & 0xffu), s, neg_zs);
-  const float e7 = fmaf((float)(u >> 24), s, neg_zs);
-  v4u r;
-  r.x = pack2<BF16>(e0, e1);
-  r.y = pack2<BF16>(e2, e3);
-  r.z = pack2<BF16>(e4, e5);
-  r.w = pack2<BF16>(e6, e7);
-  return r;
-}
-
-// Quarter t of dequant_scaled: register t of its result (elements 2t and 2t+1).
-template <bool BF16>
-__device__ inline uint32_t dequant_part(uint32_t w, float s, float neg_zs, int t) {
-  const uint32_t x = ((t & 1) ? (w >> 4) : w) & 0x0f0f0f0fu;
-  const int sh = (t >> 1) * 8;
-  const float lo = fmaf((float)((x >> sh) & 0xffu), s, neg_zs);
-  const float hi = fmaf((float)((x >> (sh + 16)) & 0xffu), s, neg_zs);
-  return pack2<BF16>(lo, hi);
-}
-
-template <bool BF16, int WMB, int WNB, bool HAS_ZP>
-__global__ __launch_bounds__(256) void w4a16_prefill_kernel(const PrefillParams p) {
-  using T = F16Traits<BF16>;
-  constexpr int BM = 64 * WMB, BN = 64 * WNB;
-  constexpr int A_CH = BM / 32;    // 16-byte chunks of A per thread per step
-  constexpr int W_LD = BN / 64;    // 16-byte weight loads per thread per group
-  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-  uint16_t* As = lds;                           // [2][BM][PITCH]
-  uint16_t* Bs = lds + 2 * BM * PF_PITCH;       // [2][BN][PITCH]
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-
-  // XCD-aware tile order: consecutive workgroup ids land on different XCDs (round-robin over 8), so give each XCD a
-  // contiguous band of tile ids; tiles in a band share A rows / W columns in that XCD's L2.
-  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
-  const int total = tiles_m * tiles_n;
-  int bid = blockIdx.x;
-  {
-    const int per = (total + 7) / 8;
-    const int xcd = bid & 7, idx = bid >> 3;
-    const int remapped = xcd * per + idx;
-    // only valid as a bijection when total % 8 == 0; otherwise keep the plain order
-    if (total % 8 == 0) bid = remapped;
-  }
-  // walk tiles column-band-major in groups of 8 m-tiles so that neighbours share weights
-  const int tm = bid % tiles_m, tn = bid / tiles_m;
-  const int m0 = tm * BM, n0 = tn * BN, nt0 = n0 / 16;
-
-  // ---- per-thread staging state ----
-  v4u areg[A_CH];
-  v4u wreg[W_LD];
-  float ws[W_LD], wnz[W_LD];     // scale and -(zero*scale) of the current group, per owned column
-
-  auto load_a = [&](int step) {
-#pragma unroll
-    for (int i = 0; i < A_CH; ++i) {
-      const int c = tid + 256 * i;
-      const int row = c >> 3, ch = c & 7;
-      const int m = m0 + row;
-      v4u v = {0u, 0u, 0u, 0u};
-      if (m < p.M) v = *reinterpret_cast<const v4u*>(p.a + (int64_t)m * p.lda + step * PF_BK + ch * 8);
-      areg[i] = v;
-    }
-  };
-  auto store_a = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < A_CH; ++i) {
-      const int c = tid + 256 * i;
-      const int row = c >> 3, ch = c & 7;
-      *reinterpret_cast<v4u*>(As + ((size_t)buf * BM + row) * PF_PITCH + ch * 8) = areg[i];
-    }
-  };
-  auto load_w = [&](int g) {
-#pragma unroll
-    for (int i = 0; i < W_LD; ++i) {
-      const int ntl = i * 4 + wave;
-      const int nt = nt0 + ntl;
-      v4u v = {0u, 0u, 0u, 0u};
-      float s = 0.f, z = 8.f;
-      if (nt < p.NT) {
-        v = p.b[((int64_t)nt * p.G + g) * 64 + lane];
-        const int n = nt * 16 + (lane & 15);
-        s = T::to_float(p.scales[(int64_t)g * p.N + n]);
-        if constexpr (HAS_ZP) {
-          const uint32_t zw = p.zeros[(int64_t)g * (p.N >> 3) + (n >> 3)];
-          z = (float)((zw >> ((n & 7) * 4)) & 0xFu);
-        }
-      }
-      wreg[i] = v;
-      ws[i] = s;
-      wnz[i] = -(z * s);   // exact: <= 4 + 11 significant bits
-    }
-  };
-  auto store_w = [&](int buf, int half) {
-    const int o = lane >> 4, r = lane & 15;
-#pragma unroll
-    for (int i = 0; i < W_LD; ++i) {
-      const int ntl = i * 4 + wave;
-      const uint32_t w0 = half ? wreg[i].z : wreg[i].x;
-      const uint32_t w1 = half ? wreg[i].w : wreg[i].y;
-      uint16_t* rowp = Bs + ((size_t)buf * BN + ntl * 16 + r) * PF_PITCH + o * 8;
-      *reinterpret_cast<v4u*>(rowp) = dequant_scaled<BF16>(w0, ws[i], wnz[i]);
-      *reinterpret_cast<v4u*>(rowp + 32) = dequant_scaled<BF16>(w1, ws[i], wnz[i]);
-    }
-  };
-
-  v16f acc[WMB][WNB];
-#pragma unroll
-  for (int i = 0; i < WMB; ++i)
-#pragma unroll
-    for (int j = 0; j < WNB; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-
-  const int steps = p.K / PF_BK;
-
-  // ---- prologue: stage step 0, issue loads for step 1 ----
-  load_a(0);
-  load_w(0);
-  store_a(0);
-  store_w(0, 0);
-  if (steps > 1) load_a(1);
-  __syncthreads();
-
-  for (int step = 0; step < steps; ++step) {
-    const int cur = step & 1;
-    // stage step+1 into the other buffer
-    if (step + 1 < steps) {
-      const int nstep = step + 1;
-      store_a(cur ^ 1);
-      store_w(cur ^ 1, nstep & 1);
-      if (nstep + 1 < steps) {
-        load_a(nstep + 1);
-        if (nstep & 1) load_w((nstep + 1) >> 1);   // both halves of the group consumed: fetch the next group
-      }
-    }
-    // MFMAs of this step
-    const uint16_t* Ab = As + ((size_t)cur * BM + wm * 32 * WMB + (lane & 31)) * PF_PITCH + (lane >> 5) * 8;
-    const uint16_t* Bb = Bs + ((size_t)cur * BN + wn * 32 * WNB + (lane & 31)) * PF_PITCH + (lane >> 5) * 8;
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      v4u af[WMB], bf[WNB];
-#pragma unroll
-      for (int i = 0; i < WMB; ++i) af[i] = *reinterpret_cast<const v4u*>(Ab + (size_t)i * 32 * PF_PITCH + kk * 16);
-#pragma unroll
-      for (int j = 0; j < WNB; ++j) bf[j] = *reinterpret_cast<const v4u*>(Bb + (size_t)j * 32 * PF_PITCH + kk * 16);
-#pragma unroll
-      for (int i = 0; i < WMB; ++i)
-#pragma unroll
-        for (int j = 0; j < WNB; ++j) acc[i][j] = T::mfma32(af[i], bf[j], acc[i][j]);
-    }
-    __syncthreads();
-  }
-
-  // ---- epilogue: lane holds column n = lane%32, rows 8*(e/4) + 4*(lane/32) + e%4 of each 32x32 block ----
-#pragma unroll
-  for (int j = 0; j < WNB; ++j) {
-    const int n = n0 + wn * 32 * WNB + j * 32 + (lane & 31);
-    if (n >= p.N) continue;
-    float bv = 0.f;
-    if (p.bias) bv = T::to_float(p.bias[n]);
-#pragma unroll
-    for (int i = 0; i < WMB; ++i) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int m = m0 + wm * 32 * WMB + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-        if (m < p.M) p.c[(int64_t)m * p.N + n] = T::from_float(acc[i][j][e] + bv);
-      }
-    }
-  }
-}
-
-// ----------------------------------------------------------------------------- direct-to-LDS variant
-// Same arithmetic, different plumbing:
-//  * the activation tile goes global -> LDS with `buffer_load_dwordx4 ... lds` (no registers, no VALU);
-//  * LDS tiles are unpadded: a pair of 128-byte rows is one 256-byte line of 16 chunks (16 B each, chunk index
-//    (row & 1) * 8 + c), and the chunk index is XOR-ed with (row >> 1) & 15.  The LDS of this architecture has 64 banks
-//    (256 bytes per cycle): 16 lanes that touch 16 consecutive rows at the same k chunk -- the operand reads and the
-//    dequantised-weight writes -- then hit 16 different 16-byte bank groups, and so do the 16 lanes of a DMA line;
-//  * WAVES_M x WAVES_N wavefronts per workgroup (8 = two per SIMD lets one wavefront dequantise while the other one
-//    issues MFMAs);
-//  * the MFMAs take the weight fragment as A operand, so four consecutive accumulator registers are four consecutive
-//    output columns of one row: packed 8-byte stores in the epilogue;
-//  * weight words of group g+1 are requested one K step before they are needed (two register sets, by group parity).
-template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP>
-__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(const PrefillParams p) {
-  using T = F16Traits<BF16>;
-  constexpr int NW = WAVES_M * WAVES_N;
-  constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;
-  constexpr int WMB = TM / 32, WNB = TN / 32;
-  constexpr int W_LD = BN / (16 * NW);            // 16-byte weight loads per thread per group
-  constexpr int A_LD = BM / (8 * NW);             // direct-to-LDS instructions per wavefront per step
-  constexpr int A_ST = BM * 128, W_ST = BN * 128; // bytes per activation / weight stage
-  constexpr int W_BASE = 3 * A_ST;                // three activation stages, then two weight stages
-  constexpr int KW = W_LD * (HAS_ZP ? 3 : 2);     // vector-memory instructions of one load_w
-  static_assert(W_LD >= 1 && A_LD >= 1, "tile too small for this many wavefronts");
-  extern __shared__ __attribute__((aligned(16))) uint8_t lds8[];
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-
-  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
-  const int total = tiles_m * tiles_n;
-  int t = blockIdx.x;
-  if (total % 8 == 0) t = (t & 7) * (total / 8) + (t >> 3);          // one contiguous range of tile ids per XCD
-  constexpr int GM = 8;                                              // tiles are handed out in bands of 8 tile rows, so
-  const int band = t / (GM * tiles_n);                               // that the tiles resident on one XCD share
-  const int first_m = band * GM;                                     // activation rows and weight columns in its L2
-  const int gsz = min(tiles_m - first_m, GM);
-  const int tin = t - band * GM * tiles_n;
-  const int tm = first_m + tin % gsz, tn = tin / gsz;
-  const int m0 = tm * BM, n0 = tn * BN, nt0 = n0 / 16;
-
-  // ---- activation tile: direct-to-LDS loads ----
-  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint16_t*>(p.a), 0, (int)((uint32_t)p.M * (uint32_t)p.lda * 2u), 0x00020000);
-  // DMA instruction i of this wavefront fills rows r0 .. r0+7 (r0 = (wave*A_LD + i) * 8): lane l lands in LDS slot
-  // r0*8 + l, i.e. row pair j = r0/2 + (l >> 4), swizzled chunk l & 15; it must therefore fetch the element that
-  // belongs there: c16 = (l & 15) ^ (j & 15), row = 2j + (c16 >> 3), chunk = c16 & 7.
-  uint32_t voff_a[A_LD];
-#pragma unroll
-  for (int i = 0; i < A_LD; ++i) {
-    const int j = (wave * A_LD + i) * 4 + (lane >> 4);
-    const int c16 = (lane & 15) ^ (j & 15);
-    const int lrow = 2 * (lane >> 4) + (c16 >> 3);
-    voff_a[i] = ((uint32_t)lrow * (uint32_t)p.lda) * 2u + (uint32_t)(c16 & 7) * 16u;
-  }
-  typedef __attribute__((address_space(3))) void* lds_ptr_t;
-  auto issue_a = [&](int step, int buf) {
-    uint8_t* Ab = lds8 + (size_t)buf * A_ST;
-#pragma unroll
-    for (int i = 0; i < A_LD; ++i) {
-      const int r0 = (wave * A_LD + i) * 8;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(Ab + r0 * 128), 16, (int)voff_a[i],
-                                               (int)(((uint32_t)(m0 + r0) * (uint32_t)p.lda + (uint32_t)step * 64u) * 2u), 0, 0);
-    }
-  };
-
-  // ---- weight words: the group being dequantised (cur) and the next one in flight (nxt).  Two named sets with a
-  // register copy per group, not one array indexed by the group's parity: a run-time index into a register array turns
-  // every access into a select chain, and the loads would have to be waited for as soon as they are issued. ----
-  v4u wcur[W_LD], wnxt[W_LD];
-  float scur[W_LD], zcur[W_LD], snxt[W_LD], znxt[W_LD];      // scale and -(zero * scale)
-  const int o = lane >> 4, r = lane & 15;
-  auto load_w = [&](int g) {
-#pragma unroll
-    for (int i = 0; i < W_LD; ++i) {
-      const int ntl = i * NW + wave;
-      const int nt = min(nt0 + ntl, p.NT - 1);          // clamped: columns past N are computed but never stored
-      wnxt[i] = p.b[((int64_t)nt * p.G + g) * 64 + lane];
-      const int n = nt * 16 + r;
-      const float sv = T::to_float(p.scales[(int64_t)g * p.N + n]);
-      float z = 8.f;
-      if constexpr (HAS_ZP) {
-        const uint32_t zw = p.zeros[(int64_t)g * (p.N >> 3) + (n >> 3)];
-        z = (float)((zw >> ((n & 7) * 4)) & 0xFu);
-      }
-      snxt[i] = sv;
-      znxt[i] = -(z * sv);   // exact: <= 4 + 11 significant bits
-    }
-  };
-  auto advance_w = [&]() {
-#pragma unroll
-    for (int i = 0; i < W_LD; ++i) {
-      wcur[i] = wnxt[i];
-      scur[i] = snxt[i];
-      zcur[i] = znxt[i];
-    }
-  };
-  // Prologue only: dequantise half 0 of the current group into weight stage 0.
-  auto store_w0 = [&]() {
-    uint8_t* Bb = lds8 + W_BASE;
-#pragma unroll
-    for (int pc = 0; pc < 2 * W_LD; ++pc) {
-      const int i = pc >> 1, which = pc & 1;
-      const int row = (i * NW + wave) * 16 + r;
-      const uint32_t wsel = which ? wcur[i].y : wcur[i].x;
-      const int c0 = (row & 1) * 8 + o + which * 4, sw = (row >> 1) & 15;
-      *reinterpret_cast<v4u*>(Bb + (row >> 1) * 256 + ((c0 ^ sw) * 16)) = dequant_scaled<BF16>(wsel, scur[i], zcur[i]);
-    }
-  };
-  auto issue_a_one = [&](int step, int buf, int i) {
-    uint8_t* Ab = lds8 + (size_t)buf * A_ST;
-    const int r0 = (wave * A_LD + i) * 8;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(Ab + r0 * 128), 16, (int)voff_a[i],
-                                             (int)(((uint32_t)(m0 + r0) * (uint32_t)p.lda + (uint32_t)step * 64u) * 2u), 0, 0);
-  };
-
-  v16f acc[WMB][WNB];
-#pragma unroll
-  for (int i = 0; i < WMB; ++i)
-#pragma unroll
-    for (int j = 0; j < WNB; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-
-  // operand reads: row = lane & 31 of a 32-row block (blocks start at multiples of 32 rows), chunk kk*2 + (lane >> 5)
-  const int kh = lane >> 5;
-  uint32_t coff[4];
-#pragma unroll
-  for (int kk = 0; kk < 4; ++kk)
-    coff[kk] = (uint32_t)(((lane & 31) >> 1) * 256 + ((((lane & 1) * 8 + kk * 2 + kh) ^ ((lane >> 1) & 15)) * 16));
-  const uint32_t arow = (uint32_t)(wm * TM * 128);
-  const uint32_t brow = (uint32_t)(wn * TN * 128);
-
-  // One K step (64 wide = 4 MFMA k-slices) on activation stage `a_cur` and weight stage `w_cur`, fused with the staging
-  // work for later steps: the DMA requests of the activation tile two steps ahead (into stage `a_dst`), and the
-  // dequantisation of the next step's weights into the other weight stage.  The fragments of slice kk+1 are read
-  // while the MFMAs of slice kk run; the staging work is cut into sub-steps that alternate with shares of the MFMAs
-  // (sched_barrier keeps the compiler from regrouping them).
-  auto fused_step = [&](int a_cur, int w_cur, auto stage_c, auto dma_c, int a_dst, int a_step, int half) {
-    constexpr bool stage_on = decltype(stage_c)::value;
-    constexpr bool dma_on = decltype(dma_c)::value;
-    constexpr int NM = WMB * WNB;                    // MFMAs per slice
-    constexpr int SUB = (NM % 4 == 0) ? 4 : 1;       // sub-steps per slice
-    constexpr int PPS = (2 * W_LD + 3) / 4;          // dequantisation pieces per slice (at most)
-    const uint8_t* base_a = lds8 + (size_t)a_cur * A_ST;
-    const uint8_t* base_b = lds8 + W_BASE + (size_t)w_cur * W_ST;
-    uint8_t* Bn = lds8 + W_BASE + (size_t)(w_cur ^ 1) * W_ST;
-    if constexpr (dma_on) {
-#pragma unroll
-      for (int i = 0; i < A_LD; ++i) issue_a_one(a_step, a_dst, i);
-    }
-    v4u af[WMB], bf[2][WNB];     // weight fragments double-buffered, activation fragments refilled in place
-#pragma unroll
-    for (int i = 0; i < WMB; ++i) af[i] = *reinterpret_cast<const v4u*>(base_a + arow + i * 4096 + coff[0]);
-#pragma unroll
-    for (int j = 0; j < WNB; ++j) bf[0][j] = *reinterpret_cast<const v4u*>(base_b + brow + j * 4096 + coff[0]);
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      const int cb = kk & 1, nb = cb ^ 1;
-      v4u dq[PPS];
-#pragma unroll
-      for (int t = 0; t < SUB; ++t) {
-        // a share of this slice's MFMAs
-#pragma unroll
-        for (int q = t * (NM / SUB); q < (t + 1) * (NM / SUB); ++q) {
-          const int i = q / WNB, j = q % WNB;
-          acc[i][j] = T::mfma32(bf[cb][j], af[i], acc[i][j]);   // rows = n, columns = m
-        }
-        // a share of the fragment reads of the next slice
-        if (kk < 3) {
-#pragma unroll
-          for (int i = 0; i < WMB; ++i) {
-            // activation fragment i has just had its last use in this slice: refill it in place
-            const int last_q = i * WNB + WNB - 1;
-            if (last_q >= t * (NM / SUB) && last_q < (t + 1) * (NM / SUB))
-              af[i] = *reinterpret_cast<const v4u*>(base_a + arow + i * 4096 + coff[kk + 1]);
-          }
-#pragma unroll
-          for (int j = 0; j < WNB; ++j)
-            if (j % SUB == t) bf[nb][j] = *reinterpret_cast<const v4u*>(base_b + brow + j * 4096 + coff[kk + 1]);
-        }
-        // a share of the dequantisation
-        if constexpr (stage_on) {
-#pragma unroll
-          for (int pc = 0; pc < 2 * W_LD; ++pc) {
-            if (pc * 4 / (2 * W_LD) != kk) continue;
-            const int slot = pc % PPS;
-            const int i = pc >> 1, which = pc & 1;
-            const uint32_t wsel = half ? (which ? wcur[i].w : wcur[i].z) : (which ? wcur[i].y : wcur[i].x);
-            if constexpr (SUB == 4) {
-              dq[slot][t] = dequant_part<BF16>(wsel, scur[i], zcur[i], t);
-            } else {
-              dq[slot] = dequant_scaled<BF16>(wsel, scur[i], zcur[i]);
-            }
-            if (t == SUB - 1) {
-              const int row = (i * NW + wave) * 16 + r;
-              const int c0 = (row & 1) * 8 + o + which * 4, sw = (row >> 1) & 15;
-              *reinterpret_cast<v4u*>(Bn + (row >> 1) * 256 + ((c0 ^ sw) * 16)) = dq[slot];
-            }
-          }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-  };
-
-  // Vector-memory operations retire in issue order.  At the end of step s the activation tile of step s+1 (requested
-  // during step s-1) must have landed, while the requests made during step s -- the tile of step s+2 and, on even
-  // steps, the next group's weight words -- may stay in flight: wait until at most that many are outstanding.
-  using TT = std::true_type;
-  using FF = std::false_type;
-
-  // K may be split over blockIdx.y: this workgroup covers the groups [g_lo, g_hi)
-  const int split = blockIdx.y;
-  const int g_lo = (int)(((int64_t)p.G * split) / p.SK), g_hi = (int)(((int64_t)p.G * (split + 1)) / p.SK);
-
-  // ---- prologue: activation tiles of the first two steps, weights of the first step (group g_lo, half 0) ----
-  issue_a(2 * g_lo, 0);
-  issue_a(2 * g_lo + 1, 1);
-  load_w(g_lo);
-  advance_w();
-  store_w0();
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-
-  int a_cur = 0;                      // activation stage of the current step (step mod 3)
-  auto nxt = [](int x) { return x == 2 ? 0 : x + 1; };
-  // LDS writes of this wavefront done, requests older than the newest `n` landed, then the workgroup barrier.  (A
-  // plain __syncthreads() carries a fence that drains every outstanding load.)
-  auto sync_step = [&](auto n_c) {
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(decltype(n_c)::value) : "memory");
-  };
-  for (int g = g_lo; g + 1 < g_hi; ++g) {
-    // even step 2g: dequantise (g, half 1) for step 2g+1; request the tile of step 2g+2 and the words of group g+1
-    load_w(g + 1);
-    fused_step(a_cur, 0, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 2, 1);
-    sync_step(std::integral_constant<int, A_LD + KW>{});
-    a_cur = nxt(a_cur);
-    // odd step 2g+1: dequantise (g+1, half 0) for step 2g+2; request the tile of step 2g+3
-    advance_w();
-    fused_step(a_cur, 1, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 3, 0);
-    sync_step(std::integral_constant<int, A_LD>{});
-    a_cur = nxt(a_cur);
-  }
-  // last group: its second half is still dequantised, nothing is requested any more
-  fused_step(a_cur, 0, TT{}, FF{}, 0, 0, 1);
-  sync_step(std::integral_constant<int, 0>{});
-  a_cur = nxt(a_cur);
-  fused_step(a_cur, 1, FF{}, FF{}, 0, 0, 0);
-
-  // ---- split K: hand the partial tile over; the last of the SK workgroups to arrive sums them in split order ----
-  if (p.SK > 1) {
-    // 16-byte buffer stores / loads with the sc1 cache-policy bit (device scope: written through to, and read from,
-    // memory that all XCDs share -- each XCD has its own L2).  One unit of NV4 KiB per (tile, wavefront).
-    constexpr int NV4 = WMB * WNB * 4;                     // 16-byte pieces per lane
-    constexpr int SC1 = 16;
-    const uint32_t unit = (uint32_t)((t * NW + wave) * NV4) * 1024u;           // bytes
-    const uint32_t split_stride = (uint32_t)total * (uint32_t)(NW * NV4) * 1024u;
-    const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(p.c_tmp, 0, (int)(split_stride * (uint32_t)p.SK), 0x00020000);
-#pragma unroll
-    for (int i = 0; i < WMB; ++i)
-#pragma unroll
-      for (int j = 0; j < WNB; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), rt, lane * 16,
-                                                 (int)(split * split_stride + unit + ((i * WNB + j) * 4 + q) * 1024), SC1);
-        }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // partial tile acknowledged before the counter moves
-    int32_t* ctr = p.counters + (int64_t)t * NW + wave;
-    int old = 0;
-    if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    old = __shfl(old, 0);
-    if (old != p.SK - 1) return;
-#pragma unroll
-    for (int i = 0; i < WMB; ++i)
-#pragma unroll
-      for (int j = 0; j < WNB; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          v4f sum = {0.f, 0.f, 0.f, 0.f};
-          for (int s2 = 0; s2 < p.SK; ++s2) {             // fixed order: deterministic
-            const v4u r = __builtin_amdgcn_raw_buffer_load_b128(
-                rt, lane * 16, (int)(s2 * split_stride + unit + ((i * WNB + j) * 4 + q) * 1024), SC1);
-            sum += __builtin_bit_cast(v4f, r);
-          }
-#pragma unroll
-          for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = sum[e];
-        }
-    if (lane == 0) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-
-  // ---- epilogue: four consecutive accumulator registers = four consecutive n of one row ----
-#pragma unroll
-  for (int i = 0; i < WMB; ++i) {
-    const int m = m0 + wm * TM + i * 32 + (lane & 31);
-    if (m >= p.M) continue;
-    uint16_t* orow = p.c + (int64_t)m * p.N;
-#pragma unroll
-    for (int j = 0; j < WNB; ++j) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = n0 + wn * TN + j * 32 + 8 * q + 4 * (lane >> 5);
-        if (n >= p.N) continue;
-        float ov[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) ov[e] = acc[i][j][4 * q + e];
-        if (p.bias) {
-          const v2u bb = *reinterpret_cast<const v2u*>(p.bias + n);
-          ov[0] += T::to_float((uint16_t)(bb.x & 0xffffu));
-          ov[1] += T::to_float((uint16_t)(bb.x >> 16));
-          ov[2] += T::to_float((uint16_t)(bb.y & 0xffffu));
-          ov[3] += T::to_float((uint16_t)(bb.y >> 16));
-        }
-        v2u pk;
-        pk.x = pack2<BF16>(ov[0], ov[1]);
-        pk.y = pack2<BF16>(ov[2], ov[3]);
-        *reinterpret_cast<v2u*>(orow + n) = pk;
-      }
-    }
-  }
-}
-
 // ----------------------------------------------------------------------------- host side
-
-template <bool BF16, int WMB, int WNB, bool HAS_ZP>
-static int launch_prefill(const PrefillParams& p, hipStream_t s) {
-  constexpr int BM = 64 * WMB, BN = 64 * WNB;
-  const size_t lds = (size_t)2 * (BM + BN) * PF_PITCH * sizeof(uint16_t);
-  auto kern = w4a16_prefill_kernel<BF16, WMB, WNB, HAS_ZP>;
-  static bool attr_done = false;   // idempotent attribute; a benign race sets it twice
-  if (!attr_done) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
-        hipSuccess) {
-      set_error("w4a16_gemm(prefill): cannot reserve %zu bytes of LDS", lds);
-      (void)hipGetLastError();
-      return VAQ_ERR_LAUNCH;
-    }
-    attr_done = true;
-  }
-  const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
-  hipLaunchKernelGGL(kern, dim3(tiles), dim3(256), lds, s, p);
-  return VAQ_OK;
-}
-
-template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP>
-static int launch_prefill2(const PrefillParams& p, hipStream_t s) {
-  const size_t lds = (size_t)(3 * BM + 2 * BN) * 128;
-  auto kern = w4a16_prefill2_kernel<BF16, BM, BN, WAVES_M, WAVES_N, HAS_ZP>;
-  static bool attr_done = false;
-  if (!attr_done) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
-        hipSuccess) {
-      set_error("w4a16_gemm(prefill): cannot reserve %zu bytes of LDS", lds);
-      (void)hipGetLastError();
-      return VAQ_ERR_LAUNCH;
-    }
-    attr_done = true;
-  }
-  const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
-  hipLaunchKernelGGL(kern, dim3(tiles, p.SK), dim3(WAVES_M * WAVES_N * 64), lds, s, p);
-  return VAQ_OK;
-}
 
 // tile ids: 0..2 = register-staged kernel (256x256, 128x128, 64x128); 10.. = direct-to-LDS kernel
 template <bool BF16, bool HAS_ZP>
 static int dispatch_tile(const PrefillParams& p, int tile, hipStream_t s) {
   switch (tile) {
-    case 10: return launch_prefill2<BF16, 256, 256, 2, 4, HAS_ZP>(p, s);   // 8 wavefronts, 128 x 64 each
-    case 11: return launch_prefill2<BF16, 256, 256, 2, 2, HAS_ZP>(p, s);   // 4 wavefronts, 128 x 128 each
-    case 12: return launch_prefill2<BF16, 128, 128, 2, 2, HAS_ZP>(p, s);   // 4 wavefronts, 64 x 64 each
-    case 13: return launch_prefill2<BF16, 128, 256, 2, 4, HAS_ZP>(p, s);   // 8 wavefronts, 64 x 64 each
-    case 14: return launch_prefill2<BF16, 64, 128, 2, 2, HAS_ZP>(p, s);    // 4 wavefronts, 32 x 64 each
-    case 0: return launch_prefill<BF16, 4, 4, HAS_ZP>(p, s);   // 256 x 256
-    case 1: return launch_prefill<BF16, 2, 2, HAS_ZP>(p, s);   // 128 x 128
-    case 2: return launch_prefill<BF16, 1, 2, HAS_ZP>(p, s);   //  64 x 128
+    case 10: return launch_prefill2<BF16, 256, 256, 2, 4, HAS_ZP, 1>(p, s);   // 8 wavefronts, 128 x 64 each
+    case 11: return launch_prefill2<BF16, 256, 256, 2, 2, HAS_ZP, 1>(p, s);   // 4 wavefronts, 128 x 128 each
+    case 12: return launch_prefill2<BF16, 128, 128, 2, 2, HAS_ZP, 1>(p, s);   // 4 wavefronts, 64 x 64 each
+    case 13: return launch_prefill2<BF16, 128, 256, 2, 4, HAS_ZP, 1>(p, s);   // 8 wavefronts, 64 x 64 each
+    case 14: return launch_prefill2<BF16, 64, 128, 2, 2, HAS_ZP, 1>(p, s);    // 4 wavefronts, 32 x 64 each
+    case 0: return launch_prefill<BF16, 4, 4, HAS_ZP, 1>(p, s);   // 256 x 256
+    case 1: return launch_prefill<BF16, 2, 2, HAS_ZP, 1>(p, s);   // 128 x 128
+    case 2: return launch_prefill<BF16, 1, 2, HAS_ZP, 1>(p, s);   //  64 x 128
     default: break;
   }
   set_error("w4a16_gemm(prefill): unknown tile id %d", tile);
@@ -683,7 +90,7 @@ int w4a16_prefill_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* co
 
 int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
                          const void* bias, void* c, float* c_tmp, int32_t* counters, int64_t counter_ints, int M, int N,
-                         int K, int dtype, hipStream_t s) {
+                         int K, int sub, bool channelwise, int dtype, hipStream_t s) {
   PrefillParams p;
   p.a = (const uint16_t*)a;
   p.lda = lda;
@@ -697,6 +104,8 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
   p.M = M; p.N = N; p.K = K;
   p.G = K / 128;
   p.NT = N / 16;
+  p.s_stride = channelwise ? 0 : N;
+  p.z_stride = channelwise ? 0 : N / 8;
   const bool direct_ok = (uint64_t)M * (uint64_t)lda * 2 < (1ull << 32);
   PrefillPlan pl = plan_prefill(M, N, K, direct_ok);
   // without scratch from the caller (or with too small a counter array) the unsplit kernel still gives the result
@@ -704,7 +113,8 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
   p.SK = pl.sk;
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
-  if (bf16) rc = zp ? dispatch_tile<true, true>(p, pl.tile, s) : dispatch_tile<true, false>(p, pl.tile, s);
+  if (sub > 1) rc = prefill_launch_sub(p, sub, pl.tile, bf16, zp, s);
+  else if (bf16) rc = zp ? dispatch_tile<true, true>(p, pl.tile, s) : dispatch_tile<true, false>(p, pl.tile, s);
   else rc = zp ? dispatch_tile<false, true>(p, pl.tile, s) : dispatch_tile<false, false>(p, pl.tile, s);
   if (rc != VAQ_OK) return rc;
   VAQ_CHECK_LAUNCH("w4a16_gemm(prefill)");
