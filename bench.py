@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-linear hot path on one MI355X.
 
-Headline workload (``config.workload``): BASELINE config 2 -- decode-shaped W4A16 GEMMs, the four Llama-3-8B
+Headline workload (``config.workload``): BASELINE.json config 2 -- decode-shaped W4A16 GEMMs, the four Llama-3-8B
 projection shapes (K,N) x M in {1,4,16}, group 128, symmetric int4, bf16 activations.  One *step* is one pass over
 those 12 GEMMs, launched through the public op surface (``vllm_amd._custom_ops.gptq_marlin_gemm`` -> C ABI) and
 replayed as a HIP graph, as a serving loop would run them.  Every GEMM of a step reads its own copy of the weights and
@@ -184,7 +184,7 @@ def per_shape_decode(dev, sets, acts):
 
 
 def prefill_section(dev):
-    """BASELINE config 3: asymmetric uint4 + act_order, both readings of its act_order wording.  `rows`: g_idx from a
+    """BASELINE.json config 3: asymmetric uint4 + act_order, both readings of its act_order wording.  `rows`: g_idx from a
     random permutation of the K rows (the reference's generator): activations are reordered on every call.  `groups`:
     g_idx permutes whole groups: the linear method folds it into the scale / zero-point rows at load time, so the GEMM
     runs without a permutation (same kernel as no act_order)."""
@@ -281,7 +281,7 @@ def vendor_ceiling_section(dev):
 
 
 def decode_step_section(dev):
-    """BASELINE config 5: one decode step of a random-init Llama-3-8B-architecture model, batch 32, context 1024.  All
+    """BASELINE.json config 5: one decode step of a random-init Llama-3-8B-architecture model, batch 32, context 1024.  All
     32 x 4 linear layers run on the W4A16 GEMM (M = 32, distinct weights per layer: 3.6 GB); norms, rotary-free
     attention over a bf16 KV cache, SiLU-mul, embedding and the bf16 lm_head are plain torch ops standing in for the
     rest of the model.  Reports the step time, the share of it spent in the quantized GEMMs and tokens/s."""
@@ -499,7 +499,7 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": "BASELINE configs[1]: decode W4A16 GEMMs, (K,N) in {(4096,6144),(4096,4096),(4096,28672),"
+        "config": {"workload": "BASELINE.json configs[1]: decode W4A16 GEMMs, (K,N) in {(4096,6144),(4096,4096),(4096,28672),"
                                "(14336,4096)} x M in {1,4,16}, group 128, symmetric int4, bf16 act, fp32 acc; one step = "
                                "12 GEMMs in a HIP graph, weights cold (650 MB cycling)",
                    "launches_per_step": launches},

@@ -40,6 +40,7 @@ extern "C" {
 /* Weight code types (what b_q_type.id selects in the reference, vllm/scalar_type.py:327-351). */
 #define VAQ_WTYPE_U4B8 0 /* symmetric: code - 8            */
 #define VAQ_WTYPE_U4 1   /* asymmetric: code - zeros[g][n] */
+#define VAQ_WTYPE_U8B128 2 /* 8-bit symmetric: code - 128 (weights from vaq_w4a16_repack with num_bits = 8) */
 
 /* Text of the last error on the calling thread ("" if none). */
 const char* vaq_last_error(void);
@@ -49,13 +50,13 @@ int vaq_abi_version(void);
 int vaq_num_cus(int device);
 
 /*
- * GPTQ int4 repack.  Replaces `gptq_marlin_repack(Tensor b_q_weight, Tensor perm, SymInt size_k,
+ * GPTQ int4 / int8 repack.  Replaces `gptq_marlin_repack(Tensor b_q_weight, Tensor perm, SymInt size_k,
  * SymInt size_n, int num_bits) -> Tensor` (csrc/torch_bindings.cpp:320-321; device code
  * csrc/quantization/gptq_marlin/gptq_marlin_repack.cu:7-322).
- *   qweight  int32 [size_k/8, size_n] contiguous (8 nibbles along K per word)
+ *   qweight  int32 [size_k/8, size_n] contiguous (8 nibbles along K per word); num_bits 8: [size_k/4, size_n], 4 bytes
  *   perm     int32 [size_k] act_order sort indices (output row r takes input row perm[r]) or NULL
- *   out      int32 [size_k/16, 2*size_n]
- * num_bits must be 4.  size_k % 16 == 0, size_n % 64 == 0 (NATIVE additionally size_k % 128 == 0).
+ *   out      int32 [size_k/16, 2*size_n]; num_bits 8: [size_k/16, 4*size_n]
+ * num_bits must be 4 or 8.  size_k % 16 == 0, size_n % 64 == 0 (NATIVE additionally size_k % 128 == 0).
  */
 int vaq_w4a16_repack(const int32_t* qweight, const int32_t* perm, int32_t* out, int64_t size_k, int64_t size_n,
                      int num_bits, int layout, void* stream);
@@ -90,14 +91,14 @@ int vaq_w4a16_gemm_workspace(int64_t size_m, int64_t size_n, int64_t size_k, int
  * W4A16 GEMM  C[M,N] = A[:, perm] . dequant(B) (+ bias), fp32 accumulation, one rounding to the 16-bit dtype.
  * Replaces `gptq_marlin_gemm(...)` (csrc/torch_bindings.cpp:309-315; csrc/quantization/gptq_marlin/gptq_marlin.cu:674-959).
  *   a        [M, K] 16-bit, row stride lda elements (lda % 8 == 0, base 16-byte aligned), unit column stride
- *   b        NATIVE-layout weights from vaq_w4a16_repack
+ *   b        NATIVE-layout weights from vaq_w4a16_repack (num_bits 8 for wtype U8B128)
  *   scales   [K/group_size, N] ([1, N] for group_size -1) in the activation dtype, contiguous
  *   zeros    int32 [K/group_size, N/8] ([1, N/8] for -1) natural nibble order (wtype U4) or NULL (wtype U4B8)
  *   perm     int32 [K] act_order sort indices or NULL  (is_k_full semantics: group of sorted row r is r / group_size)
  *   bias     [N] activation dtype or NULL
  *   c        [M, N] activation dtype, contiguous
  *   group_size  128, 64, 32, or -1 / K for channelwise scales (the reference's MARLIN_SUPPORTED_GROUP_SIZES,
- *               marlin_utils.py:24); anything else returns VAQ_ERR_UNSUPPORTED
+ *               marlin_utils.py:24); anything else returns VAQ_ERR_UNSUPPORTED, and so do 64 / 32 with U8B128
  * M == 0 is a no-op.  Kernel choice (decode: M <= 32, MFMA GEMV with in-register dequant; prefill: LDS-staged MFMA)
  * is internal; `force_path` = 0 auto, 1 decode, 2 prefill (tests / benchmarks).
  */

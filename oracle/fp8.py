@@ -207,7 +207,7 @@ def ref_silu_and_mul_quant(x: torch.Tensor, scale: torch.Tensor):
 
 
 def make_fp8_weight(n: int, k: int, seed: int = 0, dtype: torch.dtype = torch.bfloat16):
-    """BASELINE config 4 weight: ``randn([N,K])*0.02`` quantised per output channel (amax/448 fp32 scales).
+    """BASELINE.json config 4 weight: ``randn([N,K])*0.02`` quantised per output channel (amax/448 fp32 scales).
     Returns (w_q [N,K] e4m3fn row-major, w_scale [N,1] fp32).  Per-channel quantisation of a weight is the same
     per-row op as the activation quant (ptpc_fp8.py:107-123)."""
     g = torch.Generator().manual_seed(seed)

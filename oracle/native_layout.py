@@ -6,6 +6,9 @@ Tile (kt, nt) = rows 128*kt.., columns 16*nt.. is the 256-word block number nt*(
 L = 16*o + r, holds the codes of rows 128*kt + 32*j + 8*o + e (e = 0..7) of column 16*nt + r; code e sits in nibble
 position p with {0,2,4,6,1,3,5,7}[p] == e.  The inverse (`native_unpack`) is the documented map back to the logical
 [K, N] code matrix.
+
+8-bit codes are stored as two 4-bit planes: the 1 KiB block 2*(nt*(K/128)+kt) is the tile of the high nibbles
+(code >> 4) in the order above, the block after it the tile of the low nibbles (code & 15).
 """
 from __future__ import annotations
 
@@ -49,3 +52,20 @@ def native_unpack(packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
     q = np.zeros((size_k, size_n), dtype=np.int32)
     q[rows, n[:, None]] = codes.astype(np.int32)
     return q
+
+
+def native_pack8(q: np.ndarray) -> np.ndarray:
+    """Logical 8-bit codes int[K, N] -> int32 [K/16, 4N]: per tile the high-nibble plane, then the low-nibble plane."""
+    size_k, size_n = q.shape
+    q = np.asarray(q).astype(np.int32)
+    hi = native_pack(q >> 4).reshape(-1, 256)
+    lo = native_pack(q & 15).reshape(-1, 256)
+    return np.stack([hi, lo], axis=1).reshape(size_k // 16, 4 * size_n)
+
+
+def native_unpack8(packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    """Inverse of :func:`native_pack8`."""
+    planes = np.asarray(packed).reshape(-1, 2, 256)
+    hi = native_unpack(planes[:, 0].reshape(size_k // 16, 2 * size_n), size_k, size_n)
+    lo = native_unpack(planes[:, 1].reshape(size_k // 16, 2 * size_n), size_k, size_n)
+    return (hi << 4) | lo

@@ -12,6 +12,7 @@ import torch
 TILE = 16          # marlin tile edge, marlin_utils.py:19
 TILE_N = 64        # repack kernel n-tile, gptq_marlin_repack.cu:12-13 (tile_k_size=16, tile_n_size=64)
 INTERLEAVE4 = (0, 2, 4, 6, 1, 3, 5, 7)   # marlin_utils_test.py:82, gptq_marlin_repack.cu:180
+INTERLEAVE8 = (0, 2, 1, 3)               # 8-bit codes: marlin_utils_test.py:84, gptq_marlin_repack.cu:191
 
 
 def pack_factor(num_bits: int) -> int:
@@ -81,7 +82,7 @@ def awq_pack(q: np.ndarray, num_bits: int) -> np.ndarray:
 
 def get_weight_perm(num_bits: int = 4) -> np.ndarray:
     """Index list of marlin_utils_test.py:66-93 (1024 entries over one 16x64 tile pair)."""
-    assert num_bits == 4
+    assert num_bits in (4, 8)
     base = []
     for i in range(32):
         col = i // 4
@@ -90,8 +91,8 @@ def get_weight_perm(num_bits: int = 4) -> np.ndarray:
         for j in range(4):
             base.extend(p + 256 * j for p in one)
     perm = np.asarray(base, dtype=np.int64)
-    il = np.asarray(INTERLEAVE4)
-    return perm.reshape(-1, 8)[:, il].ravel()
+    il = np.asarray(INTERLEAVE4 if num_bits == 4 else INTERLEAVE8)
+    return perm.reshape(-1, il.size)[:, il].ravel()
 
 
 def marlin_permute_weights(q: np.ndarray, perm: np.ndarray) -> np.ndarray:
@@ -103,25 +104,31 @@ def marlin_permute_weights(q: np.ndarray, perm: np.ndarray) -> np.ndarray:
 
 
 def marlin_weights(q: np.ndarray, num_bits: int = 4) -> np.ndarray:
-    """marlin_utils_test.py:48-63: permute + pack 8 nibbles/int32 along the tiled axis -> int32 [K/16, 2N]."""
+    """marlin_utils_test.py:48-63: permute + pack 8 nibbles (4 bytes) per int32 along the tiled axis -> int32
+    [K/16, 2N] (4-bit) or [K/16, 4N] (8-bit)."""
     w = marlin_permute_weights(np.asarray(q), get_weight_perm(num_bits))
     return pack_cols(w, num_bits)
 
 
 # --------------------------------------------------------------------------- marlin weight layout, description 2
 
-def marlin_repack_thread_map(qweight: np.ndarray, perm: np.ndarray | None, size_k: int, size_n: int) -> np.ndarray:
+def marlin_repack_thread_map(qweight: np.ndarray, perm: np.ndarray | None, size_k: int, size_n: int,
+                             num_bits: int = 4) -> np.ndarray:
     """Thread->element restatement of the device repack kernel, gptq_marlin_repack.cu:112-203.
 
-    ``qweight`` is the GPTQ tensor int32[K/8, N]; ``perm`` int32[K] (act_order sort indices) or None/empty.
-    Output int32 [K/16, 2N].  Written as explicit loops over (k_tile, n_tile, warp, lane) vectorised over tiles.
+    ``qweight`` is the GPTQ tensor int32[K/pack_factor, N]; ``perm`` int32[K] (act_order sort indices) or None/empty.
+    Output int32 [K/16, 2N] (4-bit: one word per thread, :177-188) or [K/16, 4N] (8-bit: two words per thread, one per
+    column, :189-203).  Written as explicit loops over (warp, lane) vectorised over tiles.
     """
+    pf = pack_factor(num_bits)
     qw = np.asarray(qweight).view(np.uint32)
-    assert qw.shape == (size_k // 8, size_n)
+    assert qw.shape == (size_k // pf, size_n)
     k_tiles, n_tiles = size_k // 16, size_n // TILE_N
     has_perm = perm is not None and len(perm) > 0
-    out = np.zeros((k_tiles * n_tiles * 128,), dtype=np.uint32)
+    tile_words = 16 * TILE_N // pf
+    out = np.zeros((k_tiles * n_tiles * tile_words,), dtype=np.uint32)
     tc_offsets = (0, 1, 8, 9)
+    mask = np.uint32((1 << num_bits) - 1)
     kt = np.arange(k_tiles).reshape(-1, 1)
     nt = np.arange(n_tiles).reshape(1, -1)
     for warp in range(4):
@@ -134,21 +141,29 @@ def marlin_repack_thread_map(qweight: np.ndarray, perm: np.ndarray | None, size_
                     k_in_tile = tc_row + off
                     dst_k = kt * 16 + k_in_tile                      # row of the (sorted) logical matrix
                     src_k = np.asarray(perm)[dst_k] if has_perm else dst_k
-                    word = qw[src_k // 8, nt * TILE_N + cur_n + half]
-                    vals.append((word >> ((src_k % 8) * 4).astype(np.uint32)) & np.uint32(0xF))
-            res = np.zeros((k_tiles, n_tiles), dtype=np.uint32)
-            for i, src in enumerate(INTERLEAVE4):
-                res |= vals[src] << np.uint32(4 * i)
-            out_idx = (kt * n_tiles + nt) * 128 + th * 4 + warp
-            out[out_idx.ravel()] = res.ravel()
-    return out.view(np.int32).reshape(k_tiles, size_n * 16 // 8)
+                    word = qw[src_k // pf, nt * TILE_N + cur_n + half]
+                    vals.append((word >> ((src_k % pf) * num_bits).astype(np.uint32)) & mask)
+            if num_bits == 4:
+                res = np.zeros((k_tiles, n_tiles), dtype=np.uint32)
+                for i, src in enumerate(INTERLEAVE4):
+                    res |= vals[src] << np.uint32(4 * i)
+                out_idx = (kt * n_tiles + nt) * tile_words + th * 4 + warp
+                out[out_idx.ravel()] = res.ravel()
+            else:
+                for which in (0, 1):
+                    res = np.zeros((k_tiles, n_tiles), dtype=np.uint32)
+                    for i, src in enumerate(INTERLEAVE8):
+                        res |= vals[4 * which + src] << np.uint32(8 * i)
+                    out_idx = (kt * n_tiles + nt) * tile_words + th * 8 + warp * 2 + which
+                    out[out_idx.ravel()] = res.ravel()
+    return out.view(np.int32).reshape(k_tiles, size_n * 16 // pf)
 
 
-def marlin_unpack_to_logical(marlin_w: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
-    """Inverse of :func:`marlin_weights` (int32 [K/16, 2N] -> nibble matrix [K, N]); used for invariants."""
-    perm = get_weight_perm(4)
+def marlin_unpack_to_logical(marlin_w: np.ndarray, size_k: int, size_n: int, num_bits: int = 4) -> np.ndarray:
+    """Inverse of :func:`marlin_weights` (int32 [K/16, 2N or 4N] -> code matrix [K, N]); used for invariants."""
+    perm = get_weight_perm(num_bits)
     inv = np.argsort(perm)
-    flat = unpack_cols(marlin_w, 4)                      # [K/16, 16N]
+    flat = unpack_cols(marlin_w, num_bits)               # [K/16, 16N]
     t = flat.reshape(-1, perm.size)[:, inv].reshape(size_k // TILE, size_n // TILE, TILE, TILE)
     return t.transpose(0, 2, 1, 3).reshape(size_k, size_n)
 
@@ -216,8 +231,8 @@ def dequantize(q: np.ndarray, scales: torch.Tensor, zp: np.ndarray | int, group_
                g_idx: np.ndarray | None = None) -> torch.Tensor:
     """``w_ref = (w_q - zp).to(dtype) * w_s`` -- quant_utils.py:441, evaluated in the 16-bit activation dtype.
 
-    ``q`` int [K, N] codes 0..15 in *storage row order*; ``scales`` [G, N] bf16/fp16 CPU tensor;
-    ``zp`` either the uint4b8 bias (8) or an int [G, N] array; ``g_idx`` [K] group of each stored row
+    ``q`` int [K, N] codes (0..15, or 0..255 for 8-bit weights) in *storage row order*; ``scales`` [G, N] bf16/fp16 CPU tensor;
+    ``zp`` either the bias of the symmetric type (8 for uint4b8, 128 for uint8b128) or an int [G, N] array; ``g_idx`` [K] group of each stored row
     (act_order) or None for ``row // group_size``.
     The product ``(q - z) * s`` is an exact fp32 value rounded once to the 16-bit dtype, which is what
     both the torch CPU multiply and the device ``__hmul2`` (marlin_template.h:162-171) produce.
@@ -261,24 +276,27 @@ def rel_err_max(out: torch.Tensor, ref: torch.Tensor) -> float:
     return float((out.double() - ref.double()).abs().max() / ref.double().abs().max())
 
 
-# --------------------------------------------------------------------------- synthetic layers (BASELINE configs)
+# --------------------------------------------------------------------------- synthetic layers (BASELINE.json configs)
 
 def make_w4a16_case(k: int, n: int, group_size: int = 128, *, asym: bool = False, act_order: bool = False,
-                    group_level_perm: bool = False, dtype: torch.dtype = torch.bfloat16, seed: int = 0) -> dict:
-    """Synthetic GPTQ layer in checkpoint format, as the BASELINE configs specify it.
+                    group_level_perm: bool = False, dtype: torch.dtype = torch.bfloat16, seed: int = 0,
+                    num_bits: int = 4) -> dict:
+    """Synthetic GPTQ layer in checkpoint format, as the BASELINE.json configs specify it.
 
     Keys: ``q`` int32[K,N] codes 0..15 (row r multiplies activation column r, as in a GPTQ checkpoint),
     ``qweight`` int32[K/8,N] = gptq_pack(q), ``scales`` [G,N] ``dtype`` (made in fp16 then cast, as a checkpoint
     loader would), ``zp_vals`` int32[G,N] / ``qzeros`` int32[G,N/8] (asym only, else None),
     ``g_idx`` int32[K] (act_order only: group of row r, = (arange(K)//g)[rand_perm], quant_utils.py:357-366),
-    ``group_size`` (-1: channelwise, one group).  ``group_level_perm`` permutes whole groups instead of single rows.
+    ``group_size`` (-1: channelwise, one group), ``num_bits`` (4, or 8: codes 0..255 with the fixed zero point 128,
+    the ``uint8b128`` type).  ``group_level_perm`` permutes whole groups instead of single rows.
     """
     rng = np.random.default_rng(seed)
     orig_group_size = group_size
     if group_size == -1:
         group_size = k
     g = k // group_size
-    q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    assert num_bits == 4 or not asym, "8-bit codes are symmetric only (uint8b128)"
+    q = rng.integers(0, 1 << num_bits, size=(k, n), dtype=np.int32)
     tg = torch.Generator().manual_seed(seed)
     scales = (torch.randn(g, n, generator=tg).abs() * 0.01 + 1e-3).to(torch.float16).to(dtype)
     zp_vals = rng.integers(0, 16, size=(g, n), dtype=np.int32) if asym else None
@@ -290,11 +308,11 @@ def make_w4a16_case(k: int, n: int, group_size: int = 128, *, asym: bool = False
         else:
             rand_perm = rng.permutation(k)
         g_idx = (np.arange(k) // group_size).astype(np.int32)[rand_perm]
-    return dict(q=q, qweight=gptq_pack(q, 4), scales=scales, zp_vals=zp_vals,
-                qzeros=pack_cols(zp_vals, 4) if asym else None, g_idx=g_idx, group_size=orig_group_size)
+    return dict(q=q, qweight=gptq_pack(q, num_bits), scales=scales, zp_vals=zp_vals,
+                qzeros=pack_cols(zp_vals, 4) if asym else None, g_idx=g_idx, group_size=orig_group_size, num_bits=num_bits)
 
 
 def case_w_ref(case: dict) -> torch.Tensor:
     """Dequantised weight [K, N] such that ``C = A @ w_ref`` (rows in checkpoint order)."""
-    zp = 8 if case["zp_vals"] is None else case["zp_vals"]
+    zp = (1 << (case.get("num_bits", 4) - 1)) if case["zp_vals"] is None else case["zp_vals"]     # uint4b8: 8, uint8b128: 128
     return dequantize(case["q"], case["scales"], zp, case["group_size"], case["g_idx"])

@@ -35,14 +35,15 @@ class W4A16Layer:
             self.g_idx, self.sort_idx = mu.marlin_sort_g_idx(g_idx)
         else:
             self.g_idx, self.sort_idx = empty, empty
-        self.w = ops.gptq_marlin_repack(qweight, self.sort_idx, k, n, 4)
+        bits = case.get("num_bits", 4)
+        self.w = ops.gptq_marlin_repack(qweight, self.sort_idx, k, n, bits)
         self.scales = mu.marlin_permute_scales(to_dev(case["scales"], device, dtype), k, n, self.g)
         if case["zp_vals"] is not None:
             self.zp = mu.marlin_zero_points(to_dev(case["zp_vals"], device), case["zp_vals"].shape[0], n, 4)
             self.wtype = scalar_types.uint4
         else:
             self.zp = empty
-            self.wtype = scalar_types.uint4b8
+            self.wtype = scalar_types.uint4b8 if bits == 4 else scalar_types.uint8b128
         self.workspace = mu.marlin_make_workspace_new(device)
 
     def __call__(self, a: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:

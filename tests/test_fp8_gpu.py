@@ -317,7 +317,7 @@ def test_scaled_mm_split_k_exact_and_deterministic(device):
 
 @pytest.mark.parametrize("k,n", LLAMA_SHAPES)
 def test_config4_llama_shapes(device, k, n):
-    """BASELINE config 4: M in {1, 16, 256, 4096}, per-token x per-channel (+bias); activations quantised on the GPU
+    """BASELINE.json config 4: M in {1, 16, 256, 4096}, per-token x per-channel (+bias); activations quantised on the GPU
     (bit-exact with the oracle), M = 4096 checked on sampled rows."""
     import vllm_amd._custom_ops as ops
     w_q, sb = f.make_fp8_weight(n, k, seed=1)

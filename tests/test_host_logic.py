@@ -39,7 +39,9 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     lib = _lib.load()
     rc = lib.vaq_w4a16_repack(None, None, None, 100, 64, 4, _lib.VAQ_LAYOUT_NATIVE, None)
     assert rc == _lib.VAQ_ERR_INVALID_ARG and b"size_k = 100" in lib.vaq_last_error()
-    rc = lib.vaq_w4a16_repack(None, None, None, 128, 64, 8, _lib.VAQ_LAYOUT_NATIVE, None)
+    rc = lib.vaq_w4a16_repack(None, None, None, 128, 64, 2, _lib.VAQ_LAYOUT_NATIVE, None)
+    assert rc == _lib.VAQ_ERR_INVALID_ARG and b"num_bits" in lib.vaq_last_error()
+    rc = lib.vaq_w4a16_repack_awq(None, None, 128, 64, 8, _lib.VAQ_LAYOUT_NATIVE, None)
     assert rc == _lib.VAQ_ERR_UNSUPPORTED
     with pytest.raises(NotImplementedError):
         _lib.check(rc)
@@ -141,8 +143,11 @@ def test_shape_and_type_support_checks():
     assert mu.check_marlin_supported(st.uint4b8, 128) and not mu.check_marlin_supported(st.uint4b8, 256)
     assert all(mu.check_marlin_supported(st.uint4b8, g) for g in (-1, 32, 64))
     assert mu.check_marlin_supported(st.uint4, 128, has_zp=True) and not mu.check_marlin_supported(st.uint4, 128)
+    mu.verify_marlin_supported(st.uint8b128, 128)
     with pytest.raises(ValueError):
-        mu.verify_marlin_supported(st.uint8b128, 128)
+        mu.verify_marlin_supported(st.uint8b128, 64)
+    with pytest.raises(ValueError):
+        mu.verify_marlin_supported(st.uint8, 128, has_zp=True)
 
 
 # ------------------------------------------------------------------------------------------------ op argument validation
@@ -265,7 +270,9 @@ def test_plugin_surface_contract():
     shapes = {n: tuple(p.shape) for n, p in layer.named_parameters()}
     assert shapes == {"qweight": (512, 6144), "g_idx": (4096,), "scales": (32, 6144), "qzeros": (32, 768)}
     assert GPTQMarlinConfig.is_gptq_marlin_compatible(dict(quant_method="gptq", bits=4, group_size=128, sym=True, desc_act=False))
-    assert not GPTQMarlinConfig.is_gptq_marlin_compatible(dict(quant_method="gptq", bits=8, group_size=128, sym=True, desc_act=False))
+    assert GPTQMarlinConfig.is_gptq_marlin_compatible(dict(quant_method="gptq", bits=8, group_size=128, sym=True, desc_act=False))
+    assert not GPTQMarlinConfig.is_gptq_marlin_compatible(dict(quant_method="gptq", bits=8, group_size=32, sym=True, desc_act=False))
+    assert not GPTQMarlinConfig.is_gptq_marlin_compatible(dict(quant_method="gptq", bits=4, group_size=128, sym=False, desc_act=False))
     assert GPTQMarlinConfig.override_quantization_method(dict(quant_method="gptq", bits=4, group_size=128, sym=True, desc_act=False), None) == "gptq_marlin"
     mp = MPLinearLayerConfig((4096, 4096), (4096, 4096), st.uint4, torch.bfloat16, 128, True, False)
     assert choose_mp_linear_kernel(mp) is HipW4A16LinearKernel

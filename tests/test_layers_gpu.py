@@ -66,7 +66,7 @@ def test_gptq_linear_method_end_to_end(device, desc_act, dtype):
 
 
 def test_gptq_group_level_act_order_is_folded_at_load(device):
-    """g_idx that permutes whole groups (BASELINE config 3's wording): the method gathers the scale rows at load time and
+    """g_idx that permutes whole groups (BASELINE.json config 3's wording): the method gathers the scale rows at load time and
     runs without any activation reorder; results equal the oracle's act_order semantics."""
     from vllm_amd.layers.linear import LinearBase
     from vllm_amd.layers.quantization import get_quantization_config
@@ -170,6 +170,32 @@ def test_gptq_and_awq_methods_other_group_sizes(device, group_size):
     for m in (1, 16, 32, 150):
         a = _acts(m, k, seed=m)
         check_gemm_close(layer(a.to(device)), o.gemm_ref(a, w_ref), f"awq g={group_size} m={m}")
+
+
+@pytest.mark.parametrize("group_size,desc_act", [(128, False), (128, True), (-1, False)])
+def test_gptq_8bit_method_end_to_end(device, group_size, desc_act):
+    """A GPTQ 8-bit checkpoint (bits = 8, sym: the uint8b128 type, gptq_marlin.py:92-95) through GPTQMarlinConfig and
+    the linear method: qweight packs 4 codes per int32 along K."""
+    from vllm_amd.layers.linear import LinearBase
+    from vllm_amd.layers.quantization import get_quantization_config
+    from vllm_amd.scalar_type import scalar_types
+    k, n = 1024, 256
+    cfg = get_quantization_config("gptq_marlin").from_config(dict(bits=8, group_size=group_size, desc_act=desc_act, sym=True))
+    assert cfg.quant_type == scalar_types.uint8b128 and cfg.pack_factor == 4
+    case = o.make_w4a16_case(k, n, group_size, act_order=desc_act, seed=70 + group_size, num_bits=8)
+    layer = LinearBase(k, n, quant_config=cfg, params_dtype=torch.bfloat16, return_bias=False).to(device)
+    assert layer.qweight.shape == (k // 4, n)
+    layer.qweight.data.copy_(to_dev(case["qweight"], device))
+    layer.scales.data.copy_(to_dev(case["scales"], device, torch.bfloat16))
+    gs = k if group_size == -1 else group_size
+    g_idx = case["g_idx"] if case["g_idx"] is not None else np.arange(k, dtype=np.int32) // gs
+    layer.g_idx.data.copy_(to_dev(g_idx, device))
+    layer.process_weights_after_loading()
+    assert layer.qweight.shape == (k // 16, 4 * n)
+    w_ref = o.case_w_ref(case)
+    for m in (1, 16, 32, 150):
+        a = _acts(m, k, seed=m)
+        check_gemm_close(layer(a.to(device)), o.gemm_ref(a, w_ref), f"gptq 8-bit g={group_size} act_order={desc_act} m={m}")
 
 
 def _fp8_close(out, ref64, what):

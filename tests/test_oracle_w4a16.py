@@ -68,6 +68,26 @@ def test_two_descriptions_of_marlin_order_agree(k, n):
     assert np.array_equal(by_index_list, by_thread_map)
 
 
+@pytest.mark.parametrize("k,n", REF_GRID[:6] + [(128 * 13, 64 * 37)])
+def test_two_descriptions_of_marlin_order_agree_8bit(k, n):
+    """8-bit codes (uint8b128 weights): the host index list with interleave (0, 2, 1, 3) (marlin_utils_test.py:66-93) and
+    the device kernel's thread map (two words per thread, gptq_marlin_repack.cu:189-203) must describe the same order;
+    with act_order the thread map equals the order of the permuted rows; the order is a permutation of the codes."""
+    rng = np.random.default_rng(k * 5 + n)
+    q = rng.integers(0, 256, size=(k, n), dtype=np.int32)
+    qw = o.gptq_pack(q, 8)
+    assert qw.shape == (k // 4, n)
+    by_index_list = o.marlin_weights(q, 8)
+    assert by_index_list.shape == (k // 16, 4 * n)
+    assert np.array_equal(by_index_list, o.marlin_repack_thread_map(qw, None, k, n, 8))
+    perm = rng.permutation(k).astype(np.int32)
+    assert np.array_equal(o.marlin_repack_thread_map(qw, perm, k, n, 8), o.marlin_weights(q[perm], 8))
+    assert np.array_equal(o.marlin_unpack_to_logical(by_index_list, k, n, 8), q)
+    # first word of a tile: thread 0 / warp 0 -> rows {0, 8, 1, 9} of column 0
+    w0 = int(np.asarray(by_index_list).view(np.uint32)[0, 0])
+    assert [(w0 >> (8 * i)) & 0xff for i in range(4)] == [q[0, 0], q[8, 0], q[1, 0], q[9, 0]]
+
+
 @pytest.mark.parametrize("k,n", [(128, 64), (1024, 256), (128 * 13, 64 * 4)])
 def test_marlin_order_with_perm_equals_order_of_permuted_rows(k, n):
     rng = np.random.default_rng(3)
@@ -192,3 +212,16 @@ def test_golden_vectors():
     assert np.array_equal(o.marlin_repack_thread_map(g["qweight"], g["perm"], *q.shape), g["marlin_perm"])
     assert np.array_equal(nl.native_pack(q), g["native"])
     assert np.array_equal(o.marlin_zero_points(g["zp"], g["zp"].shape[0], q.shape[1], 4), g["marlin_zp"])
+
+
+def test_native_layout_8bit_is_two_nibble_planes():
+    k, n = 256, 64
+    rng = np.random.default_rng(8)
+    q = rng.integers(0, 256, size=(k, n), dtype=np.int32)
+    p8 = nl.native_pack8(q)
+    assert p8.shape == (k // 16, 4 * n)
+    assert np.array_equal(nl.native_unpack8(p8, k, n), q)
+    blocks = p8.reshape(-1, 256)
+    assert np.array_equal(blocks[0::2].reshape(k // 16, 2 * n), nl.native_pack(q >> 4))
+    assert np.array_equal(blocks[1::2].reshape(k // 16, 2 * n), nl.native_pack(q & 15))
+

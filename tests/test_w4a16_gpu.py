@@ -72,6 +72,29 @@ def test_awq_repack_bit_exact_both_layouts(device, k, n):
                                                       torch.empty(0, dtype=torch.int32, device=device), k, n, 4))
 
 
+@pytest.mark.parametrize("k,n", [(128, 64), (1024, 256), (128 * 13, 64 * 37), (4096, 4096)])
+@pytest.mark.parametrize("act_order", [False, True])
+def test_repack_8bit_bit_exact_both_layouts(device, k, n, act_order):
+    """num_bits = 8 of the reference's test_gptq_marlin_repack (test_marlin_gemm.py:98-156): the Marlin order must equal
+    the host construction, the native order (two nibble planes per tile) its specification."""
+    import vllm_amd._custom_ops as ops
+    rng = np.random.default_rng(k + n + 8)
+    q = rng.integers(0, 256, size=(k, n), dtype=np.int32)
+    qw = to_dev(o.gptq_pack(q, 8), device)
+    if act_order:
+        perm_np = rng.permutation(k).astype(np.int32)
+        perm = to_dev(perm_np, device)
+        q_sorted = q[perm_np]
+    else:
+        perm = torch.empty(0, dtype=torch.int32, device=device)
+        q_sorted = q
+    marlin = ops.gptq_marlin_repack(qw, perm, k, n, 8, layout="marlin")
+    native = ops.gptq_marlin_repack(qw, perm, k, n, 8)
+    assert marlin.shape == native.shape == (k // 16, 4 * n) and marlin.dtype == torch.int32
+    assert np.array_equal(marlin.cpu().numpy(), o.marlin_weights(q_sorted, 8)), "marlin order differs from the oracle"
+    assert np.array_equal(native.cpu().numpy(), nl.native_pack8(q_sorted)), "native order differs from its spec"
+
+
 # ------------------------------------------------------------------------------------------------ permute_cols
 
 @pytest.mark.parametrize("m,k", [(1, 128), (3, 1024), (7, 4096), (130, 14336), (5, 70000)])
@@ -189,6 +212,49 @@ def test_gemm_other_group_sizes_llama_shape(device):
         assert bool((layer.workspace == 0).all())
 
 
+@pytest.mark.parametrize("group_size", [128, -1])
+@pytest.mark.parametrize("k,n", [(128, 64), (1024, 192), (2048, 576), (14336 // 4, 128), (14336, 256)])
+@pytest.mark.parametrize("m", [1, 4, 16, 17, 32, 33, 200, 257])
+@pytest.mark.parametrize("act_order", [False, True])
+def test_gemm_8bit_weights(device, group_size, k, n, m, act_order):
+    """uint8b128 weights (GPTQ 8-bit symmetric; the reference's GEMM test includes the type, test_marlin_gemm.py:228-361)
+    on the decode and the prefill kernels."""
+    if act_order and (group_size == -1 or k == 128):
+        pytest.skip("act_order needs more than one group (gptq_marlin.cu:805)")
+    case = o.make_w4a16_case(k, n, group_size, act_order=act_order, seed=k + n + m, num_bits=8)
+    layer = W4A16Layer(case, device)
+    a = _acts(m, k, device, seed=m)
+    out = layer(a)
+    check_gemm_close(out, o.gemm_ref(a.cpu(), o.case_w_ref(case)), f"8-bit g={group_size} k={k} n={n} m={m}")
+    assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m", [1, 4, 16, 32, 48])
+def test_one_hot_activation_8bit_exact(device, dtype, m):
+    """One-hot rows of A with 8-bit weights: rn16((q - 128) * s) bit for bit, on every kernel variant by M."""
+    k, n = 512, 128
+    case = o.make_w4a16_case(k, n, 128, dtype=dtype, seed=21, num_bits=8)
+    layer = W4A16Layer(case, device, dtype)
+    w = o.case_w_ref(case)
+    rows = [(37 * i + 5) % k for i in range(m)]
+    a = torch.zeros(m, k, dtype=dtype)
+    for i, r in enumerate(rows):
+        a[i, r] = 1
+    assert torch.equal(layer(a.to(device)).cpu(), w[rows])
+
+
+def test_gemm_8bit_llama_shapes(device):
+    for k, n in LLAMA_SHAPES:
+        case = o.make_w4a16_case(k, n, 128, seed=k + n, num_bits=8)
+        layer = W4A16Layer(case, device)
+        w_ref = o.case_w_ref(case)
+        for m in (1, 16, 32, 300):
+            a = _acts(m, k, device, seed=m)
+            check_gemm_close(layer(a), o.gemm_ref(a.cpu(), w_ref), f"8-bit k={k} n={n} m={m}")
+        assert bool((layer.workspace == 0).all())
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("m", [1, 3, 16, 96])
 def test_gemm_fp16_and_bias(device, decode_kernel, dtype, m):
@@ -262,10 +328,10 @@ def test_m_zero_returns_empty(device):
     assert out.shape == (0, 64)
 
 
-# ------------------------------------------------------------------------------------------------ BASELINE sizes
+# ------------------------------------------------------------------------------------------------ BASELINE.json sizes
 
 def test_config1_reference_cpu_case(device):
-    """BASELINE config 1: M=16, K=N=4096, g=128, symmetric: bit-exact repack + output tolerance."""
+    """BASELINE.json config 1: M=16, K=N=4096, g=128, symmetric: bit-exact repack + output tolerance."""
     k = n = 4096
     case = o.make_w4a16_case(k, n, 128, seed=0)
     layer = W4A16Layer(case, device)

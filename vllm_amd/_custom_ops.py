@@ -73,8 +73,6 @@ def _check_repack_args(b_q_weight, perm, size_k, size_n, num_bits) -> None:
     _check(perm.is_contiguous(), "perm is not contiguous")
     _check(perm.dtype == torch.int32, "perm type is not at::kInt")
     _check(perm.numel() in (0, size_k), f"perm.numel() = {perm.numel()} must be 0 or size_k = {size_k}")
-    if num_bits != 4:
-        raise NotImplementedError("gptq_marlin_repack: only num_bits = 4 is built for gfx950")
 
 
 def _repack_impl(b_q_weight: torch.Tensor, perm: torch.Tensor, size_k: int, size_n: int, num_bits: int,
@@ -231,8 +229,9 @@ def _check_gemm_args(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, 
     _check(b_scales.dtype == a.dtype, f"b_scales dtype {b_scales.dtype} must equal the activation dtype {a.dtype}")
 
     # what this build implements out of everything the reference accepts
-    if b_q_type.size_bits != 4 or b_q_type not in (scalar_types.uint4, scalar_types.uint4b8):
-        raise NotImplementedError(f"gptq_marlin_gemm: weight type {b_q_type} is not built for gfx950 (uint4b8 / uint4)")
+    if b_q_type not in (scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8b128):
+        raise NotImplementedError(f"gptq_marlin_gemm: weight type {b_q_type} is not built for gfx950 "
+                                  "(uint4b8 / uint4 / uint8b128)")
     if is_zp_float:
         raise NotImplementedError("gptq_marlin_gemm: float zero points (is_zp_float) are not built for gfx950")
     if has_act_order and not is_k_full:
@@ -246,7 +245,13 @@ def _check_gemm_args(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, 
                                       "(only -1, 32, 64, 128)")
     _check(size_k % GPTQ_MARLIN_MIN_THREAD_K == 0,
            f"size_k = {size_k}, is not divisible by min_thread_k = {GPTQ_MARLIN_MIN_THREAD_K}")
-    wtype = _lib.VAQ_WTYPE_U4 if has_zp else _lib.VAQ_WTYPE_U4B8
+    if b_q_type == scalar_types.uint8b128:
+        if group_size not in (-1, 128):
+            raise NotImplementedError(f"gptq_marlin_gemm: uint8b128 weights with group_size = {group_size} are not built "
+                                      "for gfx950 (only -1, 128)")
+        wtype = _lib.VAQ_WTYPE_U8B128
+    else:
+        wtype = _lib.VAQ_WTYPE_U4 if has_zp else _lib.VAQ_WTYPE_U4B8
     return group_size, has_act_order, has_zp, wtype
 
 

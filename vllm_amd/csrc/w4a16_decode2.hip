@@ -12,20 +12,25 @@ struct Decode2Config {
 
 static int g2_force_gs = 0, g2_force_wks = 0, g2_force_wn = 0;
 
-static int round_gs(int x, int sub) {
+static int round_gs(int x, int sub, bool w8) {
   const int opts[] = {1, 2, 4, 7, 8, 14, 16};
-  for (int o : opts)
-    if (o >= x && (sub == 1 || (o & (o - 1)) == 0)) return o;     // sub-group instances exist for powers of two only
+  for (int o : opts) {
+    if (sub > 1 && (o & (o - 1)) != 0) continue;     // sub-group instances exist for powers of two only
+    if (w8 && (o & 1)) continue;                     // 8-bit codes: two tiles (nibble planes) per group
+    if (o >= x) return o;
+  }
   return 16;
 }
 
 // Groups per slab are limited by LDS (128 KiB of activations, 256 bytes per group and staged row): 512 / rows.
-static Decode2Config pick_decode2_config(int M, int N, int K, int sub) {
-  const int G = K / 128, NT = N / 16;
+// G, gslab, gs and slab_max below count weight tiles: one per 128 rows of K, two (nibble planes) for 8-bit codes.
+static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8) {
+  const int TPG = w8 ? 2 : 1;
+  const int G = K / 128 * TPG, NT = N / 16;
   const int MB = M <= 16 ? 1 : 2;
   Decode2Config c;
   c.mr = sub > 1 ? 16 : (M == 1 ? 1 : (M <= 4 ? 4 : 16));
-  const int slab_max = 512 / (c.mr * MB);
+  const int slab_max = 512 / (c.mr * MB) * TPG;
   c.sk = (G + slab_max - 1) / slab_max;
   const int gslab = (G + c.sk - 1) / c.sk;            // groups per slab
   const int cus = num_cus_current_device();
@@ -36,7 +41,7 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub) {
   while (wks * 2 <= want && wks < 16) wks *= 2;
   while (wks > 1 && wks > gslab) wks /= 2;
   if (g2_force_wks > 0) wks = g2_force_wks;
-  int gs = round_gs((gslab + wks - 1) / wks, sub);
+  int gs = round_gs((gslab + wks - 1) / wks, sub, w8);
   if (g2_force_gs > 0) gs = g2_force_gs;
   while (wks * gs > slab_max && wks > 1) wks /= 2;     // respect the LDS limit
   // the slab is now wks*gs groups; recompute the number of slabs
@@ -48,7 +53,7 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub) {
   // compute unit (i.e. spread over the device), then the smaller workgroup.
   int best_wn = 1;
   long best_rounds = -1, best_waves = -1;
-  const size_t lds_wg = (size_t)wks * gs * 256 * c.mr * MB + (wks > 1 ? (size_t)D2_WAVES * MB * 1024 : 16);
+  const size_t lds_wg = (size_t)wks * (gs / TPG) * 256 * c.mr * MB + (wks > 1 ? (size_t)D2_WAVES * MB * 1024 : 16);
   for (int wn = 1; wn <= D2_WAVES / wks; ++wn) {
     long slots = D2_WAVES / (wks * wn);
     const long lds_slots = (long)((size_t)(160 * 1024) / lds_wg);
@@ -120,8 +125,8 @@ static int dispatch_mr2(const Decode2Params& p, const Decode2Config& c, bool bf1
   }
 }
 
-int w4a16_decode2_workspace(int M, int N, int K, int sub, size_t* c_tmp_bytes, size_t* counter_ints) {
-  const Decode2Config c = pick_decode2_config(M, N, K, sub);
+int w4a16_decode2_workspace(int M, int N, int K, int sub, bool w8, size_t* c_tmp_bytes, size_t* counter_ints) {
+  const Decode2Config c = pick_decode2_config(M, N, K, sub, w8);
   const int MB = M <= 16 ? 1 : 2;
   const int NT = N / 16;
   *c_tmp_bytes = c.sk > 1 ? (size_t)c.sk * NT * MB * 64 * sizeof(v4f) : 0;
@@ -131,7 +136,7 @@ int w4a16_decode2_workspace(int M, int N, int K, int sub, size_t* c_tmp_bytes, s
 
 int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
                          const int32_t* perm, const void* bias, void* c, float* c_tmp, int32_t* counters,
-                         int64_t counter_ints, int M, int N, int K, int sub, bool channelwise, int dtype,
+                         int64_t counter_ints, int M, int N, int K, int sub, bool channelwise, bool w8, int dtype,
                          hipStream_t s) {
   Decode2Params p;
   p.a = (const uint16_t*)a;
@@ -145,14 +150,14 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
   p.c_tmp = c_tmp;
   p.counters = counters;
   p.M = M; p.N = N; p.K = K;
-  p.G = K / 128;
+  p.G = K / 128 * (w8 ? 2 : 1);
   p.NT = N / 16;
-  p.GR = channelwise ? 1 : p.G * sub;
+  p.GR = channelwise ? 1 : K / 128 * sub;
   p.s_stride = channelwise ? 0 : N;
   p.z_stride = channelwise ? 0 : N / 8;
   p.k_mask = 0x000f000fu;
   p.k_ex = dtype == VAQ_BF16 ? 0x43004300u : 0x64006400u;
-  const Decode2Config cfg = pick_decode2_config(M, N, K, sub);
+  const Decode2Config cfg = pick_decode2_config(M, N, K, sub, w8);
   p.SK = cfg.sk;
   p.WKS = cfg.wks;
   p.WN = cfg.wn;
@@ -165,7 +170,8 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
   }
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
-  if (sub > 1) rc = decode2_launch_sub(p, sub, cfg.gs, MB, bf16, zp, s);
+  if (w8) rc = decode2_launch_w8(p, cfg.gs, MB, cfg.mr, bf16, s);
+  else if (sub > 1) rc = decode2_launch_sub(p, sub, cfg.gs, MB, bf16, zp, s);
   else if (MB == 1) rc = dispatch_mr2<1>(p, cfg, bf16, zp, s);
   else rc = dispatch_types2<2, 16>(p, cfg.gs, bf16, zp, s);
   if (rc != VAQ_OK) return rc;

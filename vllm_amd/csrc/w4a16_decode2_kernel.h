@@ -16,6 +16,9 @@
 //    removes the bias and the zero point exactly as `P - (BIAS+z)*S` would, without keeping S anywhere.
 //  * Quantisation groups of 64 or 32 rows (SUBG = 2 or 4 groups per tile): the same, per sub-group of 2 or 1 MFMA pairs.
 //    Channelwise scales are one row read with a row stride of 0.
+//  * 8-bit codes (W8, symmetric, bias 128): the weights come as two 4-bit planes per tile (high nibbles, then low
+//    nibbles), code - 128 = 16 * (hi - 8) + lo.  Each plane is one tile of the stream, multiplied with the same
+//    activations; the high plane uses the constant operand -(BIAS + 8) and 16 * scale, the low plane -(BIAS + 0).
 //  * WKS > 1: one LDS reduction at the end (wavefronts wks == 0 sum their column's slices).  K slabs that do not fit
 //    LDS (SK > 1 workgroups per n-tile) hand partial tiles over through device-scope write-through stores and an
 //    arrival counter, summed in fixed order by the last arriver.
@@ -37,7 +40,7 @@ struct Decode2Params {
   uint16_t* c;
   float* c_tmp;
   int32_t* counters;
-  int M, N, K, G, NT, SK, WKS, WN;
+  int M, N, K, G, NT, SK, WKS, WN;   // G: weight tiles along K per 16-column strip (K/128, twice that for 8-bit codes)
   int GR;                  // rows of the scale / zero-point tensors (G * SUBG, or 1 for channelwise scales)
   int s_stride, z_stride;  // elements between consecutive rows of scales (N) / zeros (N/8); 0 for channelwise
   uint32_t k_mask, k_ex;   // 0x000f000f and the exponent pattern, passed as run-time values (see and_or)
@@ -70,10 +73,12 @@ static __device__ inline __amdgpu_buffer_rsrc_t d2_rsrc(const void* base, uint64
 
 constexpr int D2_WAVES = 16;
 
-template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG>
+template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, bool W8 = false>
 __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Decode2Params p) {
   using T = F16Traits<BF16>;
   static_assert(SUBG == 1 || SUBG == 2 || SUBG == 4, "quantisation groups per 128-row tile");
+  constexpr int TPG = W8 ? 2 : 1;                      // weight tiles per 128 rows of K
+  static_assert(!W8 || (SUBG == 1 && !HAS_ZP && GS % 2 == 0), "8-bit codes: two planes per group, symmetric, one group per tile");
   static_assert(MR == 16 || MB == 1, "compact row staging is for a single m-block");
   // Ring slots.  Two tiles in flight per wavefront measured best: a wavefront does not get past its load instructions
   // until the memory pipeline has accepted them, and with deeper rings (every wavefront of the device asking for
@@ -88,8 +93,8 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   const int WKS = p.WKS, WN = p.WN;
   const int wks = w / WN, wn = w - wks * WN;
   const int sk = blockIdx.y;
-  const int slab_groups = WKS * GS;
-  const int slab_g0 = sk * slab_groups;             // first group of this workgroup's K slab
+  const int slab_groups = WKS * GS;                 // tiles in this workgroup's K slab
+  const int slab_g0 = sk * slab_groups;             // first tile of the slab
   const int nt_raw = blockIdx.x * WN + wn;
   const bool nt_ok = nt_raw < p.NT;
   const int nt = nt_ok ? nt_raw : p.NT - 1;
@@ -99,7 +104,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   // Loads retire in issue order as far as the wait counter is concerned, so the activation loads go out FIRST: the
   // wait before the LDS writes then leaves the weight tiles in flight instead of draining them.
   // slot (16 bytes) of (m-block mb, row ml, k-octet ko):  mb*KO*MR + ko*MR + (ml ^ (ko & (MR-1)))
-  const __amdgpu_buffer_rsrc_t rb = d2_rsrc(p.b, (uint64_t)p.K * p.N / 2);
+  const __amdgpu_buffer_rsrc_t rb = d2_rsrc(p.b, (uint64_t)p.K * p.N / 2 * TPG);
   const __amdgpu_buffer_rsrc_t rs = d2_rsrc(p.scales, (uint64_t)p.GR * p.N * 2);
   const __amdgpu_buffer_rsrc_t rz = d2_rsrc(HAS_ZP ? (const void*)p.zeros : (const void*)p.scales, (uint64_t)p.GR * (p.N / 8) * 4);
   const int vo_b = lane * 16, vo_s = o * 8, vo_z = (r16 >> 3) * 4;
@@ -111,7 +116,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
     wq[slot] = __builtin_amdgcn_raw_buffer_load_b128(rb, vo_b, (int)(((uint32_t)nt * (uint32_t)p.G + g) * 1024u), 2);
 #pragma unroll
     for (int sj = 0; sj < SUBG; ++sj) {
-      const uint32_t row = g * (uint32_t)SUBG + (uint32_t)sj;
+      const uint32_t row = (g / (uint32_t)TPG) * (uint32_t)SUBG + (uint32_t)sj;
       sc[slot][sj] = __builtin_amdgcn_raw_buffer_load_b64(rs, vo_s, (int)((row * (uint32_t)p.s_stride + (uint32_t)nt * 16u) * 2u), 0);
       if constexpr (HAS_ZP)
         zq[slot][sj] = __builtin_amdgcn_raw_buffer_load_b32(rz, vo_z, (int)((row * (uint32_t)p.z_stride + (uint32_t)nt * 2u) * 4u), 0);
@@ -120,7 +125,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
     }
   };
 
-  const int KO = slab_groups * 16;                   // k-octets in the slab
+  const int KO = slab_groups / TPG * 16;             // k-octets in the slab
   // 16 bytes behind the activations for lanes without a chunk (the start of the reduction buffer, unused until the K
   // loop is over, when there is one)
   const uint32_t dummy_slot = (uint32_t)(KO * MR * MB);
@@ -129,7 +134,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
     // pair is advanced incrementally: one scalar division per kernel instead of one vector division per chunk.
     const int tid = w * 64 + lane;
     const int chunks = KO * MR * MB;
-    const int64_t k_slab0 = (int64_t)slab_g0 * 128;
+    const int64_t k_slab0 = (int64_t)(slab_g0 / TPG) * 128;
     const int NTHR = WKS * WN * 64;
     const int step_m = NTHR / KO, step_ko = NTHR - step_m * KO;     // scalar
     int m = tid / KO, ko = tid - m * KO;
@@ -215,7 +220,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
 #pragma unroll
   for (int jj = 0; jj < 4; ++jj) {
     const int kol = jj * 4 + o;
-    abase[jj] = (uint32_t)(((wks * GS * 16 + kol) * MR + ((r16 ^ kol) & (MR - 1))) * 16);
+    abase[jj] = (uint32_t)(((wks * (GS / TPG) * 16 + kol) * MR + ((r16 ^ kol) & (MR - 1))) * 16);
   }
   uint32_t ex;     // kept in a vector register so that (x & MSK) | ex is a legal single VOP3 instruction (one scalar operand)
   asm volatile("v_mov_b32 %0, %1" : "=v"(ex) : "s"(p.k_ex));
@@ -241,6 +246,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
     for (int sj = 0; sj < SUBG; ++sj) {
       uint32_t zbits;
       if constexpr (HAS_ZP) zbits = NEG_BIAS_BITS | ((zqt[sj] >> ((r16 & 7) * 4)) & 0xFu);
+      else if constexpr (W8) zbits = NEG_BIAS_BITS | ((slot & 1) ? 0u : 8u);     // slot parity == plane (ring of 2, GS even)
       else zbits = NEG_BIAS_BITS | 8u;
       const uint32_t z2 = zbits | (zbits << 16);
       const v4u zop = {z2, z2, z2, z2};
@@ -257,7 +263,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
         aop.w = d2_and_or(wj[jj] >> 12, MSK, ex);
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
-          const v4u bop = *reinterpret_cast<const v4u*>(lds + abase[jj] + (uint32_t)(mb * KO * MR * 16) + (uint32_t)(gi * 256 * MR));
+          const v4u bop = *reinterpret_cast<const v4u*>(lds + abase[jj] + (uint32_t)(mb * KO * MR * 16) + (uint32_t)((gi / TPG) * 256 * MR));
           P[mb] = T::mfma16(aop, bop, P[mb]);
           P[mb] = T::mfma16(zop, bop, P[mb]);
         }
@@ -273,6 +279,12 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
         s[1] = T::to_float((uint16_t)(sct[sj].x >> 16));
         s[2] = T::to_float((uint16_t)(sct[sj].y & 0xffffu));
         s[3] = T::to_float((uint16_t)(sct[sj].y >> 16));
+      }
+      if constexpr (W8) {
+        if ((slot & 1) == 0) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) s[r] *= 16.0f;        // high-nibble plane
+        }
       }
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
@@ -351,11 +363,11 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   }
 }
 
-template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG>
+template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, bool W8 = false>
 static int launch_decode2(const Decode2Params& p, hipStream_t s) {
   const int WN = p.WN;
-  const size_t lds = (size_t)p.WKS * GS * 256 * MR * MB + (p.WKS > 1 ? (size_t)D2_WAVES * MB * 1024 : 16);
-  auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP, MR, SUBG>;
+  const size_t lds = (size_t)p.WKS * (GS / (W8 ? 2 : 1)) * 256 * MR * MB + (p.WKS > 1 ? (size_t)D2_WAVES * MB * 1024 : 16);
+  auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP, MR, SUBG, W8>;
   static size_t attr_lds = 0;
   if (lds > attr_lds) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
@@ -374,5 +386,7 @@ static int launch_decode2(const Decode2Params& p, hipStream_t s) {
 // Groups of 64 / 32 rows (sub = 2 / 4 per tile); defined in w4a16_decode2_sub.hip: 16 staged rows per m-block only,
 // groups per wavefront gs in {1, 2, 4, 8, 16}.
 int decode2_launch_sub(const Decode2Params& p, int sub, int gs, int MB, bool bf16, bool zp, hipStream_t s);
+// 8-bit codes; defined in w4a16_decode2_w8.hip: gs in {2, 4, 8, 14, 16}, staged rows mr in {1, 4, 16} (16 when MB == 2).
+int decode2_launch_w8(const Decode2Params& p, int gs, int MB, int mr, bool bf16, hipStream_t s);
 
 }  // namespace vaq

@@ -7,14 +7,15 @@ int w4a16_decode_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* cou
 int w4a16_decode_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
                         const int32_t* perm, const void* bias, void* c, float* c_tmp, int32_t* counters,
                         int64_t counter_ints, int M, int N, int K, bool channelwise, int dtype, hipStream_t s);
-int w4a16_decode2_workspace(int M, int N, int K, int sub, size_t* c_tmp_bytes, size_t* counter_ints);
+int w4a16_decode2_workspace(int M, int N, int K, int sub, bool w8, size_t* c_tmp_bytes, size_t* counter_ints);
 int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
                          const int32_t* perm, const void* bias, void* c, float* c_tmp, int32_t* counters,
-                         int64_t counter_ints, int M, int N, int K, int sub, bool channelwise, int dtype, hipStream_t s);
+                         int64_t counter_ints, int M, int N, int K, int sub, bool channelwise, bool w8, int dtype,
+                         hipStream_t s);
 int w4a16_prefill_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* counter_ints);
 int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
                          const void* bias, void* c, float* c_tmp, int32_t* counters, int64_t counter_ints, int M, int N,
-                         int K, int sub, bool channelwise, int dtype, hipStream_t s);
+                         int K, int sub, bool channelwise, bool w8, int dtype, hipStream_t s);
 
 constexpr int64_t DECODE_MAX_M = 32;
 static int g_decode_impl = -1;  // -1: automatic, 0: LDS-staged activations (w4a16_decode2.hip), 1: register-resident (w4a16_decode.hip)
@@ -23,10 +24,10 @@ static int g_decode_impl = -1;  // -1: automatic, 0: LDS-staged activations (w4a
 // per wavefront, no barrier in the K loop) wins everywhere except for 2 < M <= 16 on wide layers (many n-tiles per compute
 // unit), where the register-resident kernel, whose wavefronts walk over n-tiles with their slice of the activations
 // held in registers, is slightly ahead.
-static int decode_impl_for(int64_t size_m, int64_t size_n, int64_t lda, int sub) {
+static int decode_impl_for(int64_t size_m, int64_t size_n, int64_t lda, int sub, bool w8) {
   // the LDS-staged kernel addresses A through a 32-bit buffer offset
   if (size_m * lda * 2 >= (1ll << 31)) return 1;
-  if (sub > 1) return 0;          // groups below 128 rows are built for the LDS-staged kernel only
+  if (sub > 1 || w8) return 0;    // groups below 128 rows and 8-bit codes are built for the LDS-staged kernel only
   if (g_decode_impl >= 0) return g_decode_impl;
   return (size_n <= 8192 || size_m <= 2 || size_m > 16) ? 0 : 1;
 }
@@ -39,7 +40,7 @@ static int check_shape(int64_t size_m, int64_t size_n, int64_t size_k) {
                 (long long)size_k);
   VAQ_CHECK_ARG(size_m < (1ll << 31) && size_n < (1ll << 31) && size_k < (1ll << 31) &&
                     size_k * size_n / 2 < (1ll << 32),
-                "w4a16_gemm: problem too large");
+                "w4a16_gemm: problem too large");   // (8-bit weights: K*N bytes, still below 2^33; offsets are checked per kernel)
   return VAQ_OK;
 }
 }  // namespace vaq
@@ -60,11 +61,15 @@ extern "C" int vaq_w4a16_gemm_workspace(int64_t size_m, int64_t size_n, int64_t 
     size_t t1 = 0, n1 = 0, t2 = 0, n2 = 0;
     rc = w4a16_decode_workspace((int)size_m, (int)size_n, (int)size_k, &t1, &n1);
     if (rc != VAQ_OK) return rc;
-    rc = w4a16_decode2_workspace((int)size_m, (int)size_n, (int)size_k, 1, &t2, &n2);
+    rc = w4a16_decode2_workspace((int)size_m, (int)size_n, (int)size_k, 1, false, &t2, &n2);
     if (rc != VAQ_OK) return rc;
     // a group size below 128 (unknown here) restricts the kernel's configurations: cover that choice as well
     size_t t3 = 0, n3 = 0;
-    rc = w4a16_decode2_workspace((int)size_m, (int)size_n, (int)size_k, 2, &t3, &n3);
+    rc = w4a16_decode2_workspace((int)size_m, (int)size_n, (int)size_k, 2, false, &t3, &n3);
+    if (rc != VAQ_OK) return rc;
+    if (t3 > t2) t2 = t3;
+    if (n3 > n2) n2 = n3;
+    rc = w4a16_decode2_workspace((int)size_m, (int)size_n, (int)size_k, 1, true, &t3, &n3);     // and 8-bit codes
     if (rc != VAQ_OK) return rc;
     if (t3 > t2) t2 = t3;
     if (n3 > n2) n2 = n3;
@@ -85,13 +90,18 @@ extern "C" int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, cons
   if (rc != VAQ_OK) return rc;
   VAQ_CHECK_ARG(dtype == VAQ_F16 || dtype == VAQ_BF16, "w4a16_gemm: only supports bfloat16 and float16 (dtype tag %d)",
                 dtype);
-  VAQ_CHECK_ARG(wtype == VAQ_WTYPE_U4B8 || wtype == VAQ_WTYPE_U4, "w4a16_gemm: unknown weight type tag %d", wtype);
+  VAQ_CHECK_ARG(wtype == VAQ_WTYPE_U4B8 || wtype == VAQ_WTYPE_U4 || wtype == VAQ_WTYPE_U8B128,
+                "w4a16_gemm: unknown weight type tag %d", wtype);
   VAQ_CHECK_ARG((wtype == VAQ_WTYPE_U4) == (zeros != nullptr),
-                "w4a16_gemm: b_q_type must be uint4 when has_zp = True and uint4b8 when has_zp = False");
+                "w4a16_gemm: b_q_type must be uint4 when has_zp = True and uint4b8 or uint8b128 when has_zp = False");
+  const bool w8 = wtype == VAQ_WTYPE_U8B128;
   const bool channelwise = group_size == -1 || (group_size == size_k && size_k != 128);
   VAQ_CHECK_SUPPORTED(channelwise || group_size == 128 || group_size == 64 || group_size == 32,
                       "w4a16_gemm: group_size = %d is not built (only -1, 32, 64, 128)", group_size);
   const int sub = channelwise ? 1 : 128 / group_size;
+  VAQ_CHECK_ARG(!w8 || size_k * size_n < (1ll << 32), "w4a16_gemm: problem too large for 8-bit weights");
+  VAQ_CHECK_SUPPORTED(!w8 || sub == 1, "w4a16_gemm: 8-bit weights with group_size = %d are not built (only -1, 128)",
+                      group_size);
   VAQ_CHECK_ARG(force_path >= 0 && force_path <= 2, "w4a16_gemm: force_path = %d", force_path);
   if (size_m == 0) return VAQ_OK;
   VAQ_CHECK_ARG(a && b && scales && c, "w4a16_gemm: null pointer");
@@ -112,11 +122,12 @@ extern "C" int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, cons
   } else if (force_path == 2) {
     decode = false;
   }
-  if (decode && decode_impl_for(size_m, size_n, lda, sub) == 0)
+  if (decode && decode_impl_for(size_m, size_n, lda, sub, w8) == 0)
     return w4a16_decode2_launch(a, lda, b, scales, zeros, perm, bias, c, c_tmp, counters, counter_ints, (int)size_m,
-                                (int)size_n, (int)size_k, sub, channelwise, dtype, s);
+                                (int)size_n, (int)size_k, sub, channelwise, w8, dtype, s);
   if (decode) {
-    VAQ_CHECK_SUPPORTED(sub == 1, "w4a16_gemm: group_size = %d with an A of 2 GiB or more is not built", group_size);
+    VAQ_CHECK_SUPPORTED(sub == 1 && !w8, "w4a16_gemm: group_size = %d / 8-bit weights with an A of 2 GiB or more are not built",
+                        group_size);
     return w4a16_decode_launch(a, lda, b, scales, zeros, perm, bias, c, c_tmp, counters, counter_ints, (int)size_m,
                                (int)size_n, (int)size_k, channelwise, dtype, s);
   }
@@ -132,7 +143,7 @@ extern "C" int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, cons
     lda_eff = size_k;
   }
   return w4a16_prefill_launch(a_eff, lda_eff, b, scales, zeros, bias, c, c_tmp, counters, counter_ints, (int)size_m,
-                              (int)size_n, (int)size_k, sub, channelwise, dtype, s);
+                              (int)size_n, (int)size_k, sub, channelwise, w8, dtype, s);
 }
 
 // Benchmark / tuning aid, not part of the drop-in surface: choose the decode implementation (-1 = automatic, 0 = LDS-staged

@@ -90,7 +90,7 @@ int w4a16_prefill_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* co
 
 int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
                          const void* bias, void* c, float* c_tmp, int32_t* counters, int64_t counter_ints, int M, int N,
-                         int K, int sub, bool channelwise, int dtype, hipStream_t s) {
+                         int K, int sub, bool channelwise, bool w8, int dtype, hipStream_t s) {
   PrefillParams p;
   p.a = (const uint16_t*)a;
   p.lda = lda;
@@ -107,13 +107,18 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
   p.s_stride = channelwise ? 0 : N;
   p.z_stride = channelwise ? 0 : N / 8;
   const bool direct_ok = (uint64_t)M * (uint64_t)lda * 2 < (1ull << 32);
+  if (w8 && !direct_ok) {
+    set_error("w4a16_gemm(prefill): 8-bit weights with an A of 4 GiB or more are not built");
+    return VAQ_ERR_UNSUPPORTED;
+  }
   PrefillPlan pl = plan_prefill(M, N, K, direct_ok);
   // without scratch from the caller (or with too small a counter array) the unsplit kernel still gives the result
   if (pl.sk > 1 && (c_tmp == nullptr || counters == nullptr || counter_ints < pl.tiles * pl.nw)) pl.sk = 1;
   p.SK = pl.sk;
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
-  if (sub > 1) rc = prefill_launch_sub(p, sub, pl.tile, bf16, zp, s);
+  if (w8) rc = prefill_launch_w8(p, pl.tile, bf16, s);
+  else if (sub > 1) rc = prefill_launch_sub(p, sub, pl.tile, bf16, zp, s);
   else if (bf16) rc = zp ? dispatch_tile<true, true>(p, pl.tile, s) : dispatch_tile<true, false>(p, pl.tile, s);
   else rc = zp ? dispatch_tile<false, true>(p, pl.tile, s) : dispatch_tile<false, false>(p, pl.tile, s);
   if (rc != VAQ_OK) return rc;

@@ -72,6 +72,36 @@ static __device__ inline v4u dequant_scaled(uint32_t w, float s, float neg_zs) {
   return r;
 }
 
+// 8-bit codes stored as two 4-bit planes: the words of the high and of the low nibbles of the same 8 codes.
+template <bool BF16>
+static __device__ inline v4u dequant_scaled8(uint32_t hi, uint32_t lo, float s, float neg_zs) {
+  const uint32_t t = ((hi & 0x0f0f0f0fu) << 4) | (lo & 0x0f0f0f0fu);          // bytes: elements 0,4,1,5
+  const uint32_t u = (hi & 0xf0f0f0f0u) | ((lo >> 4) & 0x0f0f0f0fu);           // bytes: elements 2,6,3,7
+  const float e0 = fmaf((float)(t & 0xffu), s, neg_zs);
+  const float e4 = fmaf((float)((t >> 8) & 0xffu), s, neg_zs);
+  const float e1 = fmaf((float)((t >> 16) & 0xffu), s, neg_zs);
+  const float e5 = fmaf((float)(t >> 24), s, neg_zs);
+  const float e2 = fmaf((float)(u & 0xffu), s, neg_zs);
+  const float e6 = fmaf((float)((u >> 8) & 0xffu), s, neg_zs);
+  const float e3 = fmaf((float)((u >> 16) & 0xffu), s, neg_zs);
+  const float e7 = fmaf((float)(u >> 24), s, neg_zs);
+  v4u r;
+  r.x = pack2<BF16>(e0, e1);
+  r.y = pack2<BF16>(e2, e3);
+  r.z = pack2<BF16>(e4, e5);
+  r.w = pack2<BF16>(e6, e7);
+  return r;
+}
+
+template <bool BF16>
+static __device__ inline uint32_t dequant_part8(uint32_t hi, uint32_t lo, float s, float neg_zs, int t) {
+  const uint32_t x = (t & 1) ? ((hi & 0xf0f0f0f0u) | ((lo >> 4) & 0x0f0f0f0fu)) : (((hi & 0x0f0f0f0fu) << 4) | (lo & 0x0f0f0f0fu));
+  const int sh = (t >> 1) * 8;
+  const float l = fmaf((float)((x >> sh) & 0xffu), s, neg_zs);
+  const float h = fmaf((float)((x >> (sh + 16)) & 0xffu), s, neg_zs);
+  return pack2<BF16>(l, h);
+}
+
 // Quarter t of dequant_scaled: register t of its result (elements 2t and 2t+1).
 template <bool BF16>
 static __device__ inline uint32_t dequant_part(uint32_t w, float s, float neg_zs, int t) {
@@ -261,9 +291,11 @@ __global__ __launch_bounds__(256) void w4a16_prefill_kernel(const PrefillParams 
 //  * the MFMAs take the weight fragment as A operand, so four consecutive accumulator registers are four consecutive
 //    output columns of one row: packed 8-byte stores in the epilogue;
 //  * weight words of group g+1 are requested one K step before they are needed (two register sets, by group parity).
-template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP, int SUBG>
+template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP, int SUBG, bool W8 = false>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(const PrefillParams p) {
   using T = F16Traits<BF16>;
+  static_assert(!W8 || (SUBG == 1 && !HAS_ZP), "8-bit codes: symmetric, one group per tile");
+  constexpr int TPG = W8 ? 2 : 1;                 // 1 KiB weight blocks per tile (8-bit: high-nibble plane, low-nibble plane)
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;
   constexpr int WMB = TM / 32, WNB = TN / 32;
@@ -271,7 +303,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
   constexpr int A_LD = BM / (8 * NW);             // direct-to-LDS instructions per wavefront per step
   constexpr int A_ST = BM * 128, W_ST = BN * 128; // bytes per activation / weight stage
   constexpr int W_BASE = 3 * A_ST;                // three activation stages, then two weight stages
-  constexpr int KW = W_LD * (1 + SUBG * (HAS_ZP ? 2 : 1));   // vector-memory instructions of one load_w
+  constexpr int KW = W_LD * (TPG + SUBG * (HAS_ZP ? 2 : 1));   // vector-memory instructions of one load_w
   static_assert(W_LD >= 1 && A_LD >= 1, "tile too small for this many wavefronts");
   extern __shared__ __attribute__((aligned(16))) uint8_t lds8[];
 
@@ -321,6 +353,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
   // register copy per group, not one array indexed by the group's parity: a run-time index into a register array turns
   // every access into a select chain, and the loads would have to be waited for as soon as they are issued. ----
   v4u wcur[W_LD], wnxt[W_LD];
+  v4u wcur_lo[W8 ? W_LD : 1], wnxt_lo[W8 ? W_LD : 1];      // 8-bit codes: the low-nibble plane (wcur / wnxt hold the high one)
   // scales, and for one group per tile -(zero * scale); with several groups per tile the zero points stay packed as one
   // byte per group (registers are short here) and the product is formed where it is used
   using ZT = std::conditional_t<SUBG == 1, float, uint32_t>;
@@ -332,14 +365,15 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
     for (int i = 0; i < W_LD; ++i) {
       const int ntl = i * NW + wave;
       const int nt = min(nt0 + ntl, p.NT - 1);          // clamped: columns past N are computed but never stored
-      wnxt[i] = p.b[((int64_t)nt * p.G + g) * 64 + lane];
+      wnxt[i] = p.b[(((int64_t)nt * p.G + g) * TPG) * 64 + lane];
+      if constexpr (W8) wnxt_lo[i] = p.b[(((int64_t)nt * p.G + g) * TPG + 1) * 64 + lane];
       const int n = nt * 16 + r;
       if constexpr (SUBG > 1) znxt[i] = 0u;
 #pragma unroll
       for (int sj = 0; sj < SUBG; ++sj) {
         const int64_t row = (int64_t)g * SUBG + sj;
         const float sv = T::to_float(p.scales[row * p.s_stride + n]);
-        uint32_t zc = 8u;
+        uint32_t zc = W8 ? 128u : 8u;
         if constexpr (HAS_ZP) {
           const uint32_t zw = p.zeros[row * p.z_stride + (n >> 3)];
           zc = (zw >> ((n & 7) * 4)) & 0xFu;
@@ -354,6 +388,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
 #pragma unroll
     for (int i = 0; i < W_LD; ++i) {
       wcur[i] = wnxt[i];
+      if constexpr (W8) wcur_lo[i] = wnxt_lo[i];
       zcur[i] = znxt[i];
 #pragma unroll
       for (int sj = 0; sj < SUBG; ++sj) scur[i][sj] = snxt[i][sj];
@@ -382,7 +417,10 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
       float sv, zv;
       sub_vals(i, which, sv, zv);
       const int c0 = (row & 1) * 8 + o + which * 4, sw = (row >> 1) & 15;
-      *reinterpret_cast<v4u*>(Bb + (row >> 1) * 256 + ((c0 ^ sw) * 16)) = dequant_scaled<BF16>(wsel, sv, zv);
+      v4u dv;
+      if constexpr (W8) dv = dequant_scaled8<BF16>(wsel, which ? wcur_lo[i].y : wcur_lo[i].x, sv, zv);
+      else dv = dequant_scaled<BF16>(wsel, sv, zv);
+      *reinterpret_cast<v4u*>(Bb + (row >> 1) * 256 + ((c0 ^ sw) * 16)) = dv;
     }
   };
   auto issue_a_one = [&](int step, int buf, int i) {
@@ -467,7 +505,11 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
             const uint32_t wsel = half ? (which ? wcur[i].w : wcur[i].z) : (which ? wcur[i].y : wcur[i].x);
             float sv, zv;
             sub_vals(i, half * 2 + which, sv, zv);
-            if constexpr (SUB == 4) {
+            if constexpr (W8) {
+              const uint32_t wlo = half ? (which ? wcur_lo[i].w : wcur_lo[i].z) : (which ? wcur_lo[i].y : wcur_lo[i].x);
+              if constexpr (SUB == 4) dq[slot][t] = dequant_part8<BF16>(wsel, wlo, sv, zv, t);
+              else dq[slot] = dequant_scaled8<BF16>(wsel, wlo, sv, zv);
+            } else if constexpr (SUB == 4) {
               dq[slot][t] = dequant_part<BF16>(wsel, sv, zv, t);
             } else {
               dq[slot] = dequant_scaled<BF16>(wsel, sv, zv);
@@ -622,10 +664,10 @@ static int launch_prefill(const PrefillParams& p, hipStream_t s) {
   return VAQ_OK;
 }
 
-template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP, int SUBG>
+template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP, int SUBG, bool W8 = false>
 static int launch_prefill2(const PrefillParams& p, hipStream_t s) {
   const size_t lds = (size_t)(3 * BM + 2 * BN) * 128;
-  auto kern = w4a16_prefill2_kernel<BF16, BM, BN, WAVES_M, WAVES_N, HAS_ZP, SUBG>;
+  auto kern = w4a16_prefill2_kernel<BF16, BM, BN, WAVES_M, WAVES_N, HAS_ZP, SUBG, W8>;
   static bool attr_done = false;
   if (!attr_done) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
@@ -644,5 +686,7 @@ static int launch_prefill2(const PrefillParams& p, hipStream_t s) {
 // Groups of 64 / 32 rows (sub = 2 / 4 per tile); defined in w4a16_prefill_sub.hip for the tile ids the automatic choice
 // uses (10, 12, 14 and 0, 1, 2).
 int prefill_launch_sub(const PrefillParams& p, int sub, int tile, bool bf16, bool zp, hipStream_t s);
+// 8-bit codes; defined in w4a16_prefill_w8.hip for the direct-to-LDS tile ids 10, 12, 14.
+int prefill_launch_w8(const PrefillParams& p, int tile, bool bf16, hipStream_t s);
 
 }  // namespace vaq

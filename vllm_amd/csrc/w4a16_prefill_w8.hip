@@ -1,0 +1,22 @@
+// Instances of the direct-to-LDS prefill kernel for 8-bit codes (uint8b128: two 4-bit planes per tile).
+#include "w4a16_prefill_kernel.h"
+
+namespace vaq {
+
+template <bool BF16>
+static int w8_dispatch_tile(const PrefillParams& p, int tile, hipStream_t s) {
+  switch (tile) {
+    case 10: return launch_prefill2<BF16, 256, 256, 2, 4, false, 1, true>(p, s);
+    case 12: return launch_prefill2<BF16, 128, 128, 2, 2, false, 1, true>(p, s);
+    case 14: return launch_prefill2<BF16, 64, 128, 2, 2, false, 1, true>(p, s);
+    default: break;
+  }
+  set_error("w4a16_gemm(prefill): tile id %d is not built for 8-bit weights", tile);
+  return VAQ_ERR_UNSUPPORTED;
+}
+
+int prefill_launch_w8(const PrefillParams& p, int tile, bool bf16, hipStream_t s) {
+  return bf16 ? w8_dispatch_tile<true>(p, tile, s) : w8_dispatch_tile<false>(p, tile, s);
+}
+
+}  // namespace vaq

@@ -22,6 +22,12 @@
 //    16*kt + 2*(th%4) + {0,1,8,9} for column 64*nt + 16*warp + th/4 (first four) and that column + 8 (last four),
 //    nibble order {0,2,4,6,1,3,5,7}.
 //
+// 8-bit codes (GPTQ int32 [K/4, N], row 4r+e in bits [8e, 8e+8)) go to int32 [K/16, 4N]:
+//  NATIVE  two 4-bit planes per tile: block 2*(nt*(K/128)+kt) holds the high nibbles (code >> 4) of the tile in the
+//          order above, the next block the low nibbles, so the 4-bit kernels' dequantisation applies to each plane.
+//  MARLIN  16 x 64 tiles of 256 words; words th*8 + warp*2 + {0, 1} hold, one byte each, rows 16*kt + 2*(th%4) +
+//          {0, 8, 1, 9} of column 64*nt + 16*warp + th/4 (word 0) and that column + 8 (word 1).
+//
 // With `perm` (act_order sort indices) output row k takes input row perm[k].
 #include "vaq_common.h"
 
@@ -40,6 +46,13 @@ __device__ inline uint32_t fetch_code_awq(const uint32_t* __restrict__ qw, int64
   const uint32_t word = qw[k * (size_n >> 3) + (n >> 3)];
   const int pos = (int)(((n & 1) << 2) | ((n & 7) >> 1));
   return (word >> (pos * 4)) & 0xFu;
+}
+
+__device__ inline uint32_t fetch_code8(const uint32_t* __restrict__ qw, const int32_t* __restrict__ perm, int64_t k,
+                                       int64_t n, int64_t size_n) {
+  int64_t src = perm ? (int64_t)perm[k] : k;
+  uint32_t word = qw[(src >> 2) * size_n + n];
+  return (word >> ((src & 3) * 8)) & 0xFFu;
 }
 
 __device__ inline uint32_t interleave_pack(const uint32_t v[8]) {
@@ -119,13 +132,64 @@ __global__ __launch_bounds__(256) void repack_marlin_kernel(const uint32_t* __re
   }
 }
 
+// 8-bit codes, native layout: one thread per output word of one nibble plane.
+__global__ __launch_bounds__(256) void repack_native8_kernel(const uint32_t* __restrict__ qw,
+                                                              const int32_t* __restrict__ perm,
+                                                              uint32_t* __restrict__ out, int64_t size_k,
+                                                              int64_t size_n) {
+  const int64_t total = size_k * size_n / 4;
+  const int64_t k_tiles = size_k / 128;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int j = idx & 3;
+    const int lane = (idx >> 2) & 63;
+    const int plane = (idx >> 8) & 1;
+    const int64_t tile = idx >> 9;
+    const int64_t nt = tile / k_tiles, kt = tile - nt * k_tiles;
+    const int o = lane >> 4, r = lane & 15;
+    const int64_t k0 = kt * 128 + j * 32 + o * 8;
+    const int64_t n = nt * 16 + r;
+    uint32_t v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t c = fetch_code8(qw, perm, k0 + e, n, size_n);
+      v[e] = plane ? (c & 0xFu) : (c >> 4);
+    }
+    out[idx] = interleave_pack(v);
+  }
+}
+
+// 8-bit codes, reference (Marlin) order: one thread per output word.
+__global__ __launch_bounds__(256) void repack_marlin8_kernel(const uint32_t* __restrict__ qw,
+                                                              const int32_t* __restrict__ perm,
+                                                              uint32_t* __restrict__ out, int64_t size_k,
+                                                              int64_t size_n) {
+  const int64_t total = size_k * size_n / 4;
+  const int64_t n_tiles = size_n / 64;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int which = idx & 1;
+    const int warp = (idx >> 1) & 3;
+    const int th = (idx >> 3) & 31;
+    const int64_t tile = idx >> 8;
+    const int64_t kt = tile / n_tiles, nt = tile - kt * n_tiles;
+    const int64_t n = nt * 64 + warp * 16 + (th >> 2) + which * 8;
+    const int64_t kbase = kt * 16 + (th & 3) * 2;
+    const int off[4] = {0, 8, 1, 9};     // byte i <- row offset {0, 1, 8, 9}[{0, 2, 1, 3}[i]]
+    uint32_t res = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) res |= fetch_code8(qw, perm, kbase + off[i], n, size_n) << (8 * i);
+    out[idx] = res;
+  }
+}
+
 }  // namespace vaq
 
 static int repack_common(const int32_t* qweight, const int32_t* perm, int32_t* out, int64_t size_k, int64_t size_n,
                          int num_bits, int layout, bool awq, void* stream) {
   using namespace vaq;
-  VAQ_CHECK_SUPPORTED(num_bits == 4, "w4a16_repack: num_bits must be 4 (8-bit weights are not built). Got = %d",
-                      num_bits);
+  VAQ_CHECK_ARG(num_bits == 4 || num_bits == 8, "w4a16_repack: num_bits must be 4 or 8. Got = %d", num_bits);
+  VAQ_CHECK_SUPPORTED(num_bits == 4 || !awq, "w4a16_repack: 8-bit AWQ weights are not built");
   VAQ_CHECK_ARG(size_k > 0 && size_k % 16 == 0, "w4a16_repack: size_k = %lld is not divisible by tile_k_size = 16",
                 (long long)size_k);
   VAQ_CHECK_ARG(size_n > 0 && size_n % 64 == 0, "w4a16_repack: size_n = %lld is not divisible by tile_n_size = 64",
@@ -134,7 +198,7 @@ static int repack_common(const int32_t* qweight, const int32_t* perm, int32_t* o
   VAQ_CHECK_ARG(layout != VAQ_LAYOUT_NATIVE || size_k % 128 == 0,
                 "w4a16_repack: native layout needs size_k %% 128 == 0, got size_k = %lld", (long long)size_k);
   VAQ_CHECK_ARG(qweight && out, "w4a16_repack: null pointer");
-  const int64_t total = size_k * size_n / 8;
+  const int64_t total = size_k * size_n / (32 / num_bits);
   const int threads = 256;
   int64_t blocks = (total + threads - 1) / threads;
   const int64_t cap = (int64_t)num_cus_current_device() * 16;
@@ -143,7 +207,10 @@ static int repack_common(const int32_t* qweight, const int32_t* perm, int32_t* o
   const uint32_t* qw = (const uint32_t*)qweight;
   uint32_t* o = (uint32_t*)out;
   const dim3 grid((unsigned)blocks), block(threads);
-  if (layout == VAQ_LAYOUT_NATIVE) {
+  if (num_bits == 8) {
+    if (layout == VAQ_LAYOUT_NATIVE) hipLaunchKernelGGL(repack_native8_kernel, grid, block, 0, s, qw, perm, o, size_k, size_n);
+    else hipLaunchKernelGGL(repack_marlin8_kernel, grid, block, 0, s, qw, perm, o, size_k, size_n);
+  } else if (layout == VAQ_LAYOUT_NATIVE) {
     if (awq)
       hipLaunchKernelGGL((repack_native_kernel<false, true>), grid, block, 0, s, qw, perm, o, size_k, size_n);
     else if (perm)

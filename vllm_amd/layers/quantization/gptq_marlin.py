@@ -20,8 +20,8 @@ logger = logging.getLogger(__name__)
 class GPTQMarlinConfig(QuantizationConfig):
     """Config class for GPTQ on the gfx950 W4A16 kernels."""
 
-    # (num_bits, is_sym) -> quant_type   (8-bit is not built)
-    TYPE_MAP = {(4, True): scalar_types.uint4b8}
+    # (num_bits, is_sym) -> quant_type   (gptq_marlin.py:92-95)
+    TYPE_MAP = {(4, True): scalar_types.uint4b8, (8, True): scalar_types.uint8b128}
 
     def __init__(self, weight_bits: int, group_size: int, desc_act: bool, is_sym: bool, lm_head_quantized: bool = False,
                  dynamic: dict[str, dict[str, int | bool]] | None = None, full_config: dict[str, Any] | None = None,

@@ -6,7 +6,8 @@ from __future__ import annotations
 import torch
 
 from vllm_amd import _custom_ops as ops
-from ...utils.marlin_utils import (HIP_W4A16_SUPPORTED_GROUP_SIZES, apply_gptq_marlin_linear,
+from ...utils.marlin_utils import (HIP_W4A16_SUPPORTED_GROUP_SIZES, HIP_W8A16_SUPPORTED_GROUP_SIZES,
+                                   apply_gptq_marlin_linear,
                                    check_marlin_supports_shape, marlin_is_k_full, marlin_make_empty_g_idx,
                                    marlin_make_workspace_new, marlin_permute_bias, marlin_permute_scales,
                                    marlin_sort_g_idx, marlin_zero_points, query_marlin_supported_quant_types)
@@ -25,7 +26,8 @@ class HipW4A16LinearKernel(MPLinearKernel):
         if c.weight_type not in quant_types:
             return False, (f"Quant type ({c.weight_type}) not supported by the gfx950 W4A16 kernel, supported types "
                            f"are: {quant_types}")
-        if c.group_size not in HIP_W4A16_SUPPORTED_GROUP_SIZES:
+        if c.group_size not in (HIP_W8A16_SUPPORTED_GROUP_SIZES if c.weight_type.size_bits == 8
+                                else HIP_W4A16_SUPPORTED_GROUP_SIZES):
             return False, (f"Group size ({c.group_size}) not supported by the gfx950 W4A16 kernel, supported group "
                            f"sizes are: {HIP_W4A16_SUPPORTED_GROUP_SIZES}")
         if c.act_type not in (torch.float16, torch.bfloat16):

@@ -23,6 +23,7 @@ GPTQ_MARLIN_MAX_PARALLEL = 16
 MARLIN_SUPPORTED_GROUP_SIZES = [-1, 32, 64, 128]
 # what the gfx950 kernels implement out of the above (marlin_utils.py:24)
 HIP_W4A16_SUPPORTED_GROUP_SIZES = [-1, 32, 64, 128]
+HIP_W8A16_SUPPORTED_GROUP_SIZES = [-1, 128]      # uint8b128 weights
 
 USE_FP32_REDUCE_DEFAULT = True
 
@@ -34,11 +35,11 @@ _INTERLEAVE4 = (0, 2, 4, 6, 1, 3, 5, 7)
 
 def query_marlin_supported_quant_types(has_zp: bool | None = None, include_fp_type: bool = True,
                                        device_capability: int | None = None) -> list[ScalarType]:
-    """marlin_utils.py:35-69, restricted to the 4-bit integer types built for gfx950."""
+    """marlin_utils.py:35-69, restricted to the integer types built for gfx950."""
     if has_zp is None:
         return (query_marlin_supported_quant_types(False, include_fp_type, device_capability) +
                 query_marlin_supported_quant_types(True, include_fp_type, device_capability))
-    return [scalar_types.uint4] if has_zp else [scalar_types.uint4b8]
+    return [scalar_types.uint4] if has_zp else [scalar_types.uint4b8, scalar_types.uint8b128]
 
 
 def _check_marlin_supported(quant_type: ScalarType, group_size: int | None, has_zp: bool,
@@ -50,6 +51,9 @@ def _check_marlin_supported(quant_type: ScalarType, group_size: int | None, has_
     if group_size is None or group_size not in HIP_W4A16_SUPPORTED_GROUP_SIZES:
         return (False, f"The gfx950 W4A16 kernels do not support group_size = {group_size}. Only group_sizes = "
                        f"{HIP_W4A16_SUPPORTED_GROUP_SIZES} are supported.")
+    if quant_type == scalar_types.uint8b128 and group_size not in HIP_W8A16_SUPPORTED_GROUP_SIZES:
+        return (False, f"The gfx950 kernels do not support group_size = {group_size} for {quant_type}. Only group_sizes = "
+                       f"{HIP_W8A16_SUPPORTED_GROUP_SIZES} are supported.")
     return True, None
 
 
