@@ -174,7 +174,7 @@ def test_gptq_and_awq_methods_other_group_sizes(device, group_size):
 
 @pytest.mark.parametrize("group_size,desc_act", [(128, False), (128, True), (-1, False)])
 def test_gptq_8bit_method_end_to_end(device, group_size, desc_act):
-    """A GPTQ 8-bit checkpoint (bits = 8, sym: the uint8b128 type, gptq_marlin.py:92-95) through GPTQMarlinConfig and
+    """A GPTQ 8-bit checkpoint (bits = 8, sym: the uint8b128 type, gptq_marlin.py:96-99) through GPTQMarlinConfig and
     the linear method: qweight packs 4 codes per int32 along K."""
     from vllm_amd.layers.linear import LinearBase
     from vllm_amd.layers.quantization import get_quantization_config

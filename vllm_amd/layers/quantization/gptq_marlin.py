@@ -20,7 +20,7 @@ logger = logging.getLogger(__name__)
 class GPTQMarlinConfig(QuantizationConfig):
     """Config class for GPTQ on the gfx950 W4A16 kernels."""
 
-    # (num_bits, is_sym) -> quant_type   (gptq_marlin.py:92-95)
+    # (num_bits, is_sym) -> quant_type   (gptq_marlin.py:96-99)
     TYPE_MAP = {(4, True): scalar_types.uint4b8, (8, True): scalar_types.uint8b128}
 
     def __init__(self, weight_bits: int, group_size: int, desc_act: bool, is_sym: bool, lm_head_quantized: bool = False,
