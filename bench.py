@@ -37,9 +37,10 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes moved per algorithmic byte over the 12 headline GEMMs, from two hardware-counter runs of
 # `bench.py --counter-pass` (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same counter reads for the 256 MiB
 # copy in that run (FETCH_SIZE reads 131083.5 for 262144 KiB -> x2.000, WRITE_SIZE reads 262144.0 -> x1.000):
-# fetch 361.87 MB + write 6.04 MB = 367.92 MB against 340.30 MB algorithmic.  The excess is about 10 % on the fetch
-# side of every small layer, the fp32 split-K partials of the K=14336, M=16 case, and activation re-reads at M=16.
-MEASURED_TRAFFIC_PER_ALGORITHMIC_BYTE = 367.92 / 340.30
+# fetch 361.79 MB + write 6.04 MB = 367.83 MB against 340.30 MB algorithmic.  The excess is about 10 % on the fetch
+# side of every small layer (a 128-byte line of a scale row spans four 16-column tiles whose workgroups sit on different
+# XCDs, each of which fetches the line), the fp32 split-K partials of the K=14336, M=16 case, and activation re-reads at M=16.
+MEASURED_TRAFFIC_PER_ALGORITHMIC_BYTE = 367.83 / 340.30
 BF16_PEAK_TFLOPS = 2500.0
 FP8_PEAK_TFLOPS = 5000.0
 GROUP = 128
@@ -249,6 +250,44 @@ def fused_norm_quant_section(dev):
                      unfused_us=tu * 1e6, cold=False))
     log(f"[silu+quant  ] d={d} M={m}: {t * 1e6:6.1f} us {b / t / 1e9:6.0f} GB/s ({100 * b / t / 1e9 / HBM_PEAK_GBS:4.1f}% of 8 TB/s) | "
         f"unfused silu*mul + quant {tu * 1e6:6.1f} us")
+    return rows
+
+
+def variants_section(dev):
+    """The other weight formats of the W4A16 GEMM -- groups of 64 / 32 rows, channelwise scales, 8-bit codes
+    (uint8b128) -- on gate_up_proj (4096 x 28672) at a decode size (cold weights, several copies cycling) and at
+    M = 4096.  Bytes count weights, scales and zero points of the format."""
+    from vllm_amd.scalar_type import scalar_types
+    rows = []
+    gen = torch.Generator(device=dev).manual_seed(7)
+    k, n = 4096, 28672
+    for name, gs, bits in (("g128", 128, 4), ("g64", 64, 4), ("g32", 32, 4), ("channelwise", -1, 4), ("8bit_g128", 128, 8)):
+        grp = 1 if gs == -1 else k // gs
+        copies = 6
+        layers = []
+        for _ in range(copies):
+            l = W4Layer(k, n, dev, gen)
+            if bits == 8:
+                l.w = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 16, 4 * n), dtype=torch.int32, device=dev, generator=gen)
+                l.wtype = scalar_types.uint8b128
+            l.s = (torch.randn(grp, n, device=dev, generator=gen).abs() * 0.01 + 1e-3).to(torch.bfloat16)
+            layers.append(l)
+        wbytes = k * n * bits // 8 + grp * n * 2
+        for m in (1, 16, 4096):
+            a = torch.randn(m, k, device=dev, generator=gen).to(torch.bfloat16)
+            use = layers if m <= 16 else layers[:2]
+
+            def fn():
+                for l in use:
+                    l(a)
+            t = time_graph(fn, iters=5, warmup=2, inner=len(use))
+            b = wbytes + 2 * m * (k + n)
+            fl = 2.0 * m * n * k
+            rows.append(dict(kind="w4a16_variant", variant=name, K=k, N=n, M=m, us=t * 1e6, GBps=b / t / 1e9,
+                             hbm_frac=b / t / 1e9 / HBM_PEAK_GBS, TFLOPs=fl / t / 1e12, cold=m <= 16))
+            log(f"[variant {name:11s}] K={k} N={n} M={m:4d}: {t * 1e6:8.1f} us  {b / t / 1e9:6.0f} GB/s ({100 * b / t / 1e9 / HBM_PEAK_GBS:4.1f}% of 8 TB/s)  "
+                f"{fl / t / 1e12:7.1f} TFLOP/s")
+        del layers
     return rows
 
 
@@ -477,6 +516,7 @@ def main():
     torch.cuda.empty_cache()
     if not args.no_extra:
         for name, fn in (("prefill", prefill_section), ("fp8", fp8_section), ("fused_norm_quant", fused_norm_quant_section),
+                         ("variants", variants_section),
                          ("vendor_ceiling", vendor_ceiling_section),
                          ("decode_step", decode_step_section)):
             try:

@@ -29,7 +29,7 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8) 
   const int G = K / 128 * TPG, NT = N / 16;
   const int MB = M <= 16 ? 1 : 2;
   Decode2Config c;
-  c.mr = sub > 1 ? 16 : (M == 1 ? 1 : (M <= 4 ? 4 : 16));
+  c.mr = M == 1 ? 1 : (M <= 4 ? 4 : 16);
   const int slab_max = 512 / (c.mr * MB) * TPG;
   c.sk = (G + slab_max - 1) / slab_max;
   const int gslab = (G + c.sk - 1) / c.sk;            // groups per slab
@@ -171,7 +171,8 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
   if (w8) rc = decode2_launch_w8(p, cfg.gs, MB, cfg.mr, bf16, s);
-  else if (sub > 1) rc = decode2_launch_sub(p, sub, cfg.gs, MB, bf16, zp, s);
+  else if (sub == 2) rc = decode2_launch_sub2(p, cfg.gs, MB, cfg.mr, bf16, zp, s);
+  else if (sub == 4) rc = decode2_launch_sub4(p, cfg.gs, MB, cfg.mr, bf16, zp, s);
   else if (MB == 1) rc = dispatch_mr2<1>(p, cfg, bf16, zp, s);
   else rc = dispatch_types2<2, 16>(p, cfg.gs, bf16, zp, s);
   if (rc != VAQ_OK) return rc;

@@ -383,9 +383,10 @@ static int launch_decode2(const Decode2Params& p, hipStream_t s) {
   return VAQ_OK;
 }
 
-// Groups of 64 / 32 rows (sub = 2 / 4 per tile); defined in w4a16_decode2_sub.hip: 16 staged rows per m-block only,
-// groups per wavefront gs in {1, 2, 4, 8, 16}.
-int decode2_launch_sub(const Decode2Params& p, int sub, int gs, int MB, bool bf16, bool zp, hipStream_t s);
+// Groups of 64 / 32 rows (2 / 4 per tile); defined in w4a16_decode2_sub2.hip / w4a16_decode2_sub4.hip: groups per
+// wavefront gs in {1, 2, 4, 8, 16}, staged rows mr in {1, 4, 16} (16 when MB == 2).
+int decode2_launch_sub2(const Decode2Params& p, int gs, int MB, int mr, bool bf16, bool zp, hipStream_t s);
+int decode2_launch_sub4(const Decode2Params& p, int gs, int MB, int mr, bool bf16, bool zp, hipStream_t s);
 // 8-bit codes; defined in w4a16_decode2_w8.hip: gs in {2, 4, 8, 14, 16}, staged rows mr in {1, 4, 16} (16 when MB == 2).
 int decode2_launch_w8(const Decode2Params& p, int gs, int MB, int mr, bool bf16, hipStream_t s);
 
