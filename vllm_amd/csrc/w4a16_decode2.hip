@@ -164,6 +164,8 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
   const int MB = M <= 16 ? 1 : 2;
   if (cfg.sk > 1) {
     VAQ_CHECK_ARG(c_tmp != nullptr && counters != nullptr, "w4a16_gemm: split-K needs c_tmp and counters");
+    VAQ_CHECK_ARG(((uintptr_t)c_tmp % 16) == 0, "w4a16_gemm: c_tmp must be 16-byte aligned");
+    VAQ_CHECK_ARG((uint64_t)cfg.sk * (uint64_t)p.NT * MB * 1024u < (1ull << 31), "w4a16_gemm: split-K scratch too large");
     VAQ_CHECK_ARG(counter_ints >= (int64_t)p.NT * MB,
                   "w4a16_gemm: workspace.numel = %lld is below min_workspace_size = %lld", (long long)counter_ints,
                   (long long)p.NT * MB);

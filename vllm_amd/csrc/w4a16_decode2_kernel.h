@@ -46,21 +46,6 @@ struct Decode2Params {
   uint32_t k_mask, k_ex;   // 0x000f000f and the exponent pattern, passed as run-time values (see and_or)
 };
 
-static __device__ inline void d2_store_partial(float* dst, v4f v) {
-  __hip_atomic_store(dst + 0, v.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(dst + 1, v.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(dst + 2, v.z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(dst + 3, v.w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-static __device__ inline v4f d2_load_partial(const float* src) {
-  v4f v;
-  v.x = __hip_atomic_load(src + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  v.y = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  v.z = __hip_atomic_load(src + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  v.w = __hip_atomic_load(src + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  return v;
-}
-
 // (x & mask) | ex.  mask and ex reach the kernel as run-time arguments: with literal constants the compiler emits two
 // instructions (a VOP3 op of this architecture cannot carry two literals); with register operands it selects the
 // single v_and_or_b32, and unlike inline assembly the instruction stays visible to the MFMA hazard recogniser.
@@ -326,25 +311,48 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   if (!nt_ok) return;
 
   // ---- 5. hand over across workgroups if K is split, then write the 16-bit outputs ----
+  // Partial tiles cross workgroups (and XCDs, whose L2 caches are not coherent with each other) through 16-byte buffer
+  // stores / loads with the sc1 cache-policy bit (device scope): one wait for the stores to be acknowledged, one arrival
+  // counter per n-tile; the last of the SK workgroups to arrive sums the partials in split order (deterministic).
+  if (p.SK > 1) {
+    constexpr int SC1 = 16;
+    const uint32_t sk_stride = (uint32_t)p.NT * (uint32_t)MB * 1024u;            // bytes per split
+    const __amdgpu_buffer_rsrc_t rt = d2_rsrc(p.c_tmp, (uint64_t)sk_stride * (uint64_t)p.SK);
+    const uint32_t unit = (uint32_t)nt * (uint32_t)MB * 1024u;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, acc[mb]), rt, lane * 16,
+                                             (int)((uint32_t)sk * sk_stride + unit + (uint32_t)mb * 1024u), SC1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // partial tiles acknowledged before the counter moves
+    int old = 0;
+    if (lane == 0) old = __hip_atomic_fetch_add(&p.counters[nt * MB], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    old = __shfl(old, 0);
+    if (old != p.SK - 1) return;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < p.SK; s0 += 4) {               // four splits in flight, added in split order
+      v4u part[4][MB];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t s2 = (uint32_t)min(s0 + i, p.SK - 1);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          part[i][mb] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s2 * sk_stride + unit + (uint32_t)mb * 1024u), SC1);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (s0 + i < p.SK) {
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) acc[mb] += __builtin_bit_cast(v4f, part[i][mb]);
+        }
+      }
+    }
+    if (lane == 0) __hip_atomic_store(&p.counters[nt * MB], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     v4f val = acc[mb];
-    bool write_out = true;
-    if (p.SK > 1) {
-      const int64_t slot = (((int64_t)nt * MB + mb) * 64 + lane) * 4;
-      const int64_t sk_stride = (int64_t)p.NT * MB * 64 * 4;
-      d2_store_partial(p.c_tmp + sk * sk_stride + slot, val);
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // partial tile acknowledged before the counter moves
-      int old = 0;
-      if (lane == 0) old = __hip_atomic_fetch_add(&p.counters[nt * MB + mb], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      old = __shfl(old, 0);
-      write_out = (old == p.SK - 1);
-      if (write_out) {
-        val = v4f{0.f, 0.f, 0.f, 0.f};
-        for (int s2 = 0; s2 < p.SK; ++s2) val += d2_load_partial(p.c_tmp + s2 * sk_stride + slot);   // fixed order
-        if (lane == 0) __hip_atomic_store(&p.counters[nt * MB + mb], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
+    const bool write_out = true;
     const int m = mb * 16 + r16;
     if (write_out && m < p.M) {
       const int n = nt * 16 + o * 4;
