@@ -298,6 +298,28 @@ def test_silu_and_mul_quant(device, tokens, hidden, dtype):
         assert torch.equal(out3.reshape(tokens, -1).view(torch.uint8), out.view(torch.uint8))
 
 
+@pytest.mark.parametrize("cfg", [1, 3, 4, 7, 13, 23, 14, 24, 17])
+def test_scaled_mm_every_tile_shape_exact(device, cfg):
+    """Every shape of the multi-stage tile kernel, forced through the tuning export (the automatic choice only reaches
+    some of them at any one problem size), including the ones that take two k-slices per step: small-integer operands
+    make the fp32 accumulation exact, so the result must equal the integer GEMM, also with K split over workgroups."""
+    import vllm_amd._custom_ops as ops
+    from vllm_amd import _lib
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(cfg)
+    try:
+        for m, n, k, split in ((300, 384, 1024, 0), (64, 256, 8192 + 128, 2), (513, 512, 640, 0)):
+            a = torch.randint(-2, 3, (m, k), generator=g).float()
+            w = torch.randint(-1, 2, (n, k), generator=g).float()
+            lib.vaq_debug_set_fp8_tile_cfg(cfg, split)
+            out = ops.cutlass_scaled_mm(a.to(torch.float8_e4m3fn).to(device), w.to(torch.float8_e4m3fn).to(device).t(),
+                                        torch.ones(m, 1, device=device), torch.ones(n, 1, device=device), torch.float16)
+            assert torch.equal(out.cpu().float(), a @ w.t()), (cfg, m, n, k)
+    finally:
+        lib.vaq_debug_set_fp8_tile_cfg(0, 0)
+    assert bool((ops._fp8_counters(torch.device(device)) == 0).all()), "arrival counters not restored to zero"
+
+
 def test_scaled_mm_split_k_exact_and_deterministic(device):
     """Few output tiles and a long K: the tile kernel splits K over workgroups (fp32 partial tiles through the op's
     scratch, arrival counters left zero).  Small-integer operands make every partial sum exact, so the split result

@@ -315,14 +315,16 @@ __global__ __launch_bounds__(256) void fp8_mm_tile2_kernel(const Fp8MMParams p) 
 //  * WAVES_M x WAVES_N wavefronts; tiles are handed out in bands of 8 tile rows inside each XCD's contiguous range so
 //    that the tiles resident on one XCD share activation rows and weight columns in its L2.
 // Requires K % 64 == 0 (a partial last step would read the neighbouring row instead of zeros) and M*lda, N*ldb < 2^32.
-template <bool BF16_OUT, int BM, int BN, int WAVES_M, int WAVES_N, int NST>
+template <bool BF16_OUT, int BM, int BN, int WAVES_M, int WAVES_N, int NST, int KS = 1>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(const Fp8MMParams p) {
+  // A step is KS k-slices of 64 bytes (KS = 2 for the small tiles, whose steps are otherwise shorter than the barrier
+  // and the LDS round trip that every step pays); a stage holds the KS slices of one step, each as [A tile | B tile].
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;
   constexpr int WMB = TM / 32, WNB = TN / 32;
-  constexpr int A_ST = BM * 64, B_ST = BN * 64, STAGE = A_ST + B_ST;
-  constexpr int A_LD = BM / (16 * NW), B_LD = BN / (16 * NW);     // DMA instructions per wavefront and step (16 rows each)
-  constexpr int LPW = A_LD + B_LD;
+  constexpr int A_ST = BM * 64, B_ST = BN * 64, SLICE = A_ST + B_ST, STAGE = KS * SLICE;
+  constexpr int A_LD = BM / (16 * NW), B_LD = BN / (16 * NW);     // DMA instructions per wavefront and slice (16 rows each)
+  constexpr int LPW = KS * (A_LD + B_LD);
   static_assert(A_LD >= 1 && B_LD >= 1, "tile too small for this many wavefronts");
   static_assert((NST - 2) * LPW <= 63, "wait counter range");
   extern __shared__ __attribute__((aligned(16))) uint8_t lds8[];
@@ -355,19 +357,23 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
 
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
   auto issue_loads = [&](int step, int stage) {
-    uint8_t* Ab = lds8 + (size_t)stage * STAGE;
-    uint8_t* Bb = Ab + A_ST;
 #pragma unroll
-    for (int i = 0; i < A_LD; ++i) {
-      const int r0 = (wave * A_LD + i) * 16;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(Ab + r0 * 64), 16, (int)voff_a,
-                                               (int)((uint32_t)(m0 + r0) * (uint32_t)p.lda + (uint32_t)step * 64u), 0, 0);
-    }
+    for (int ks = 0; ks < KS; ++ks) {
+      uint8_t* Ab = lds8 + (size_t)stage * STAGE + ks * SLICE;
+      uint8_t* Bb = Ab + A_ST;
+      const uint32_t koff = (uint32_t)(step * KS + ks) * 64u;
 #pragma unroll
-    for (int i = 0; i < B_LD; ++i) {
-      const int r0 = (wave * B_LD + i) * 16;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(Bb + r0 * 64), 16, (int)voff_b,
-                                               (int)((uint32_t)(n0 + r0) * (uint32_t)p.ldb + (uint32_t)step * 64u), 0, 0);
+      for (int i = 0; i < A_LD; ++i) {
+        const int r0 = (wave * A_LD + i) * 16;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(Ab + r0 * 64), 16, (int)voff_a,
+                                                 (int)((uint32_t)(m0 + r0) * (uint32_t)p.lda + koff), 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < B_LD; ++i) {
+        const int r0 = (wave * B_LD + i) * 16;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(Bb + r0 * 64), 16, (int)voff_b,
+                                                 (int)((uint32_t)(n0 + r0) * (uint32_t)p.ldb + koff), 0, 0);
+      }
     }
   };
 
@@ -392,7 +398,9 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
   // (Reading the fragments of step s+1 during the MFMAs of step s -- one more stage of slack, double-buffered weight
   // fragments -- was measured 5% slower than reading them at the start of their own step, and is not done.)
   auto compute = [&](int stage) {
-    const uint8_t* base = lds8 + (size_t)stage * STAGE;
+#pragma unroll
+   for (int ks = 0; ks < KS; ++ks) {
+    const uint8_t* base = lds8 + (size_t)stage * STAGE + ks * SLICE;
     v8i af[WMB], bf[WNB];
 #pragma unroll
     for (int j = 0; j < WNB; ++j) {
@@ -410,6 +418,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
     for (int i = 0; i < WMB; ++i)
 #pragma unroll
       for (int j = 0; j < WNB; ++j) acc[i][j] = mfma_fp8_32(bf[j], af[i], acc[i][j]);   // rows = n, columns = m
+   }
   };
   // end of a step: LDS reads of this wavefront done, requests older than the newest `n` landed, then the bare barrier
   auto sync_step = [&](auto n_c) {
@@ -420,8 +429,8 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
 
   // Invariant at the start of step s: the tile of step s complete in LDS, the tiles of steps s+1 .. s+NST-2 requested,
   // stage (s-1) % NST free.  The requests of step s+NST-1 go out first thing in step s.
-  // K may be split over blockIdx.y: this workgroup covers the 64-byte steps [s_lo, s_hi)
-  const int all_steps = p.K / 64;
+  // K may be split over blockIdx.y: this workgroup covers the steps [s_lo, s_hi)
+  const int all_steps = p.K / (64 * KS);
   const int split = blockIdx.y;
   const int s_lo = (int)(((int64_t)all_steps * split) / p.SK), s_hi = (int)(((int64_t)all_steps * (split + 1)) / p.SK);
   const int steps = s_hi - s_lo;
@@ -641,10 +650,10 @@ static int launch_tile2(const Fp8MMParams& p, hipStream_t s) {
   return VAQ_OK;
 }
 
-template <bool BF16_OUT, int BM, int BN, int WAVES_M, int WAVES_N, int NST>
+template <bool BF16_OUT, int BM, int BN, int WAVES_M, int WAVES_N, int NST, int KS = 1>
 static int launch_tile3(const Fp8MMParams& p, hipStream_t s) {
-  const size_t lds = (size_t)NST * (BM + BN) * 64;
-  auto kern = fp8_mm_tile3_kernel<BF16_OUT, BM, BN, WAVES_M, WAVES_N, NST>;
+  const size_t lds = (size_t)NST * KS * (BM + BN) * 64;
+  auto kern = fp8_mm_tile3_kernel<BF16_OUT, BM, BN, WAVES_M, WAVES_N, NST, KS>;
   static bool attr_done = false;
   if (!attr_done) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
@@ -680,10 +689,13 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   pl.cfg = g_fp8_tile3_cfg;
   if (pl.cfg <= 0)
     pl.cfg = tiles(256, 256) >= cus ? 1 : (tiles(128, 256) * 8 >= cus * 7 ? 7 : (tiles(128, 128) >= cus ? 3 : 4));
+  // the smallest tile with two k-slices per step: 5-8 % faster on a short K (half the barriers), no gain on a long one
+  if (g_fp8_tile3_cfg <= 0 && pl.cfg == 4 && K % 128 == 0 && K <= 8192) pl.cfg = 14;
+  if (pl.cfg >= 10 && K % 128 != 0) pl.cfg %= 10;      // two k-slices per step need K % 128 == 0
   switch (pl.cfg) {
-    case 3: pl.bm = 128; pl.bn = 128; pl.nw = 4; break;
-    case 4: pl.bm = 64; pl.bn = 128; pl.nw = 4; break;
-    case 7: pl.bm = 128; pl.bn = 256; pl.nw = 8; break;
+    case 3: case 13: case 23: pl.bm = 128; pl.bn = 128; pl.nw = 4; break;
+    case 4: case 14: case 24: pl.bm = 64; pl.bn = 128; pl.nw = 4; break;
+    case 7: case 17: pl.bm = 128; pl.bn = 256; pl.nw = 8; break;
     case 2: pl.bm = 256; pl.bn = 256; pl.nw = 4; break;
     default: pl.bm = 256; pl.bn = 256; pl.nw = 8; break;
   }
@@ -723,6 +735,12 @@ static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t c
       case 5: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 4>(p, s);
       case 6: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 3>(p, s);
       case 7: return launch_tile3<BF16_OUT, 128, 256, 2, 4, 5>(p, s);
+      // two k-slices per step (K % 128 == 0)
+      case 13: return launch_tile3<BF16_OUT, 128, 128, 2, 2, 4, 2>(p, s);
+      case 23: return launch_tile3<BF16_OUT, 128, 128, 2, 2, 2, 2>(p, s);
+      case 14: return launch_tile3<BF16_OUT, 64, 128, 2, 2, 5, 2>(p, s);
+      case 24: return launch_tile3<BF16_OUT, 64, 128, 2, 2, 3, 2>(p, s);
+      case 17: return launch_tile3<BF16_OUT, 128, 256, 2, 4, 3, 2>(p, s);
       default: break;
     }
   }
@@ -852,6 +870,10 @@ extern "C" int vaq_fp8_scaled_mm_ws(const uint8_t* a, int64_t lda, const uint8_t
 }
 
 // Benchmark / tuning aid, not part of the drop-in surface.  path: 0 auto, 1 stream, 2 tile; gx: stream-kernel grid.
+extern "C" void vaq_debug_set_fp8_tile_cfg(int cfg, int split) {     // cfg: 0 = automatic, -1 = off; split: 0 = automatic
+  vaq::g_fp8_tile3_cfg = cfg;
+  vaq::g_fp8_force_split = split;
+}
 extern "C" void vaq_debug_set_fp8_config(int path, int gx) {
   vaq::g_force_fp8_path = path % 10;
   vaq::g_fp8_tile_impl = (path / 10) % 10;     // tens digit: 1 = force the register-staged tile kernel
