@@ -135,6 +135,35 @@ def test_decode_gemm_small(device, decode_kernel, k, n, m, asym, act_order):
     assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
 
 
+@pytest.mark.parametrize("kernel", ["lds_staged", "register_resident"])
+@pytest.mark.parametrize("m", [1, 5, 16, 29])
+def test_decode_gemm_forced_split_k(device, kernel, m):
+    """K split over several workgroups on both decode kernels (forced through the tuning exports: the automatic choice
+    only splits a long K): partial tiles through `c_tmp`, arrival counters in `workspace`.  Against the oracle, twice for
+    determinism, counters left zero."""
+    from vllm_amd import _lib
+    lib = _lib.load()
+    k, n = 2048, 320
+    case = o.make_w4a16_case(k, n, 128, asym=True, seed=90 + m)
+    layer = W4A16Layer(case, device)
+    a = _acts(m, k, device, seed=m)
+    try:
+        if kernel == "lds_staged":
+            lib.vaq_debug_set_decode_impl(0)
+            lib.vaq_debug_set_decode2_config(2, 2 + 100 * 1)      # slabs of 4 groups: 4 splits
+        else:
+            lib.vaq_debug_set_decode_impl(1)
+            lib.vaq_debug_set_decode_config(1, 4, 0)              # 4 wavefronts of 1 group: 4 (M <= 16) splits
+        out = layer(a)
+        check_gemm_close(out, o.gemm_ref(a.cpu(), o.case_w_ref(case)), f"forced split-K {kernel} m={m}")
+        assert torch.equal(out, layer(a)), "split-K result is not deterministic run to run"
+        assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
+    finally:
+        lib.vaq_debug_set_decode_impl(-1)
+        lib.vaq_debug_set_decode2_config(0, 0)
+        lib.vaq_debug_set_decode_config(0, 0, 0)
+
+
 @pytest.mark.parametrize("k,n", SMALL)
 @pytest.mark.parametrize("m", [33, 64, 200, 257])
 @pytest.mark.parametrize("asym,act_order", [(False, False), (True, True)])

@@ -42,22 +42,9 @@ struct DecodeParams {
 };
 
 // Split-K partial tiles cross workgroups (and therefore XCDs, whose L2 caches are not coherent with each other)
-// through device-scope write-through stores and loads: no L2 write-back / invalidate is needed, only a wait for the
-// stores to be acknowledged before the arrival counter is bumped.
-__device__ inline void store_partial(float* dst, v4f v) {
-  __hip_atomic_store(dst + 0, v.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(dst + 1, v.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(dst + 2, v.z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(dst + 3, v.w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ inline v4f load_partial(const float* src) {
-  v4f v;
-  v.x = __hip_atomic_load(src + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  v.y = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  v.z = __hip_atomic_load(src + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  v.w = __hip_atomic_load(src + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  return v;
-}
+// through 16-byte buffer stores and loads with the sc1 cache-policy bit (device scope): no L2 write-back / invalidate is
+// needed, only a wait for the stores to be acknowledged before the arrival counter is bumped.
+constexpr int DEC_SC1 = 16;
 
 // (x & mask) | ex.  mask and ex reach the kernel as run-time arguments: with literal constants the compiler emits two
 // instructions (a VOP3 op of this architecture cannot carry two literals); with register operands it selects the
@@ -285,10 +272,11 @@ __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodePar
           v4f val = (p.WK > 1) ? tot : acc[mb];
           bool write_out = true;
           if (p.SK > 1) {
-            const int64_t slot = (((int64_t)nt * MB + mb) * 64 + lane) * 4;
-            const int64_t sk_stride = (int64_t)p.NT * MB * 64 * 4;
-            float* part = reinterpret_cast<float*>(p.c_tmp);
-            store_partial(part + sk * sk_stride + slot, val);
+            const uint32_t unit = (uint32_t)(nt * MB + mb) * 1024u;                  // bytes
+            const uint32_t sk_stride = (uint32_t)p.NT * (uint32_t)MB * 1024u;
+            const __amdgpu_buffer_rsrc_t rt = make_rsrc(p.c_tmp, (uint64_t)sk_stride * (uint64_t)p.SK);
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, val), rt, lane * 16,
+                                                   (int)((uint32_t)sk * sk_stride + unit), DEC_SC1);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // partial tile acknowledged before the counter moves
             int old = 0;
             if (lane == 0) old = __hip_atomic_fetch_add(&p.counters[nt * MB + mb], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -296,7 +284,16 @@ __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodePar
             write_out = (old == p.SK - 1);
             if (write_out) {
               val = v4f{0.f, 0.f, 0.f, 0.f};
-              for (int s2 = 0; s2 < p.SK; ++s2) val += load_partial(part + s2 * sk_stride + slot);   // fixed order
+              for (int s0 = 0; s0 < p.SK; s0 += 4) {             // four splits in flight, added in split order
+                v4u part[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                  part[i] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16,
+                                                                  (int)((uint32_t)min(s0 + i, p.SK - 1) * sk_stride + unit), DEC_SC1);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                  if (s0 + i < p.SK) val += __builtin_bit_cast(v4f, part[i]);
+              }
               if (lane == 0) __hip_atomic_store(&p.counters[nt * MB + mb], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
           }
@@ -342,10 +339,10 @@ static DecodeConfig pick_decode_config(int M, int N, int K) {
   if (MB == 2 && c.tg >= 4) c.tg = 2;
   const int kw = (G + c.tg - 1) / c.tg;          // wavefronts needed along K
   int wk_max = (c.tg >= 4 || (MB == 2 && c.tg == 2)) ? 8 : 16;
+  c.maxw = wk_max > 8 ? 16 : 8;                  // the instantiated launch bound; fewer wavefronts may run under it
   if (g_force_wk > 0 && g_force_wk < wk_max) wk_max = g_force_wk;
   c.sk = (kw + wk_max - 1) / wk_max;
   c.wk = (kw + c.sk - 1) / c.sk;
-  c.maxw = wk_max > 8 ? 16 : 8;
   const int cus = num_cus_current_device();
   int gx = g_force_gx > 0 ? g_force_gx : cus / c.sk;
   if (gx < 1) gx = 1;
@@ -431,6 +428,8 @@ int w4a16_decode_launch(const void* a, int64_t lda, const int32_t* b, const void
   const int MB = M <= 16 ? 1 : 2;
   if (cfg.sk > 1) {
     VAQ_CHECK_ARG(c_tmp != nullptr && counters != nullptr, "w4a16_gemm: split-K needs c_tmp and counters");
+    VAQ_CHECK_ARG(((uintptr_t)c_tmp % 16) == 0, "w4a16_gemm: c_tmp must be 16-byte aligned");
+    VAQ_CHECK_ARG((uint64_t)cfg.sk * (uint64_t)p.NT * 2048u < (1ull << 31), "w4a16_gemm: split-K scratch too large");
     VAQ_CHECK_ARG(counter_ints >= (int64_t)p.NT * MB,
                   "w4a16_gemm: workspace.numel = %lld is below min_workspace_size = %lld", (long long)counter_ints,
                   (long long)p.NT * MB);
