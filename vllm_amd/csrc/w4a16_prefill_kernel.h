@@ -684,9 +684,9 @@ static int launch_prefill2(const PrefillParams& p, hipStream_t s) {
 }
 
 // Groups of 64 / 32 rows (sub = 2 / 4 per tile); defined in w4a16_prefill_sub.hip for the tile ids the automatic choice
-// uses (10, 12, 14 and 0, 1, 2).
+// uses (10, 12, 14, 15 and 0, 1, 2).
 int prefill_launch_sub(const PrefillParams& p, int sub, int tile, bool bf16, bool zp, hipStream_t s);
-// 8-bit codes; defined in w4a16_prefill_w8.hip for the direct-to-LDS tile ids 10, 12, 14.
+// 8-bit codes; defined in w4a16_prefill_w8.hip for the direct-to-LDS tile ids 10, 12, 14, 15.
 int prefill_launch_w8(const PrefillParams& p, int tile, bool bf16, hipStream_t s);
 
 }  // namespace vaq

@@ -9,6 +9,7 @@ static int sub_dispatch_tile(const PrefillParams& p, int tile, hipStream_t s) {
     case 10: return launch_prefill2<BF16, 256, 256, 2, 4, HAS_ZP, SUBG>(p, s);
     case 12: return launch_prefill2<BF16, 128, 128, 2, 2, HAS_ZP, SUBG>(p, s);
     case 14: return launch_prefill2<BF16, 64, 128, 2, 2, HAS_ZP, SUBG>(p, s);
+    case 15: return launch_prefill2<BF16, 128, 64, 2, 2, HAS_ZP, SUBG>(p, s);
     case 0: return launch_prefill<BF16, 4, 4, HAS_ZP, SUBG>(p, s);
     case 1: return launch_prefill<BF16, 2, 2, HAS_ZP, SUBG>(p, s);
     case 2: return launch_prefill<BF16, 1, 2, HAS_ZP, SUBG>(p, s);

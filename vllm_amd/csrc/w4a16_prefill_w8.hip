@@ -9,6 +9,7 @@ static int w8_dispatch_tile(const PrefillParams& p, int tile, hipStream_t s) {
     case 10: return launch_prefill2<BF16, 256, 256, 2, 4, false, 1, true>(p, s);
     case 12: return launch_prefill2<BF16, 128, 128, 2, 2, false, 1, true>(p, s);
     case 14: return launch_prefill2<BF16, 64, 128, 2, 2, false, 1, true>(p, s);
+    case 15: return launch_prefill2<BF16, 128, 64, 2, 2, false, 1, true>(p, s);
     default: break;
   }
   set_error("w4a16_gemm(prefill): tile id %d is not built for 8-bit weights", tile);
