@@ -381,6 +381,21 @@ def test_config2_decode_llama_shapes(device, decode_kernel, k, n):
         assert torch.equal(out, layer(a)), "decode GEMM is not deterministic run to run"
 
 
+@pytest.mark.parametrize("k,n", LLAMA_SHAPES + [(1280, 192)])
+@pytest.mark.parametrize("m", [33, 40, 48, 64])
+def test_decode_three_and_four_m_blocks(device, k, n, m):
+    """32 < M <= 64 runs on the LDS-staged decode kernel with three / four m-blocks (K split over workgroups, the
+    reduction buffer on top of the activations); symmetric, and asymmetric with act_order."""
+    for asym, act_order in ((False, False), (True, True)):
+        case = o.make_w4a16_case(k, n, 128, asym=asym, act_order=act_order, seed=k + n + m)
+        layer = W4A16Layer(case, device)
+        a = _acts(m, k, device, seed=m)
+        out = layer(a)
+        check_gemm_close(out, o.gemm_ref(a.cpu(), o.case_w_ref(case)), f"k={k} n={n} m={m} asym={asym}")
+        assert torch.equal(out, layer(a)), "not deterministic run to run"
+        assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
+
+
 @pytest.mark.parametrize("k,n", LLAMA_SHAPES)
 @pytest.mark.parametrize("group_level", [False, True])
 def test_config3_prefill_llama_shapes_sampled(device, k, n, group_level):

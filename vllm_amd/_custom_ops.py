@@ -275,7 +275,7 @@ def _gemm_impl(a: torch.Tensor, c_or_none: torch.Tensor | None, b_q_weight: torc
         _lib.check(lib.vaq_w4a16_gemm_workspace(size_m, size_n, size_k, int(has_act_order), dev.index or 0,
                                                 ctypes.byref(n_ctmp), ctypes.byref(n_atmp), ctypes.byref(n_cnt)))
         # decode sizes need their counters; the tile kernel falls back to an unsplit K when the array is too small
-        _check(size_m > 32 or workspace.numel() >= n_cnt.value,
+        _check(size_m > 64 or workspace.numel() >= n_cnt.value,
                f"workspace.numel = {workspace.numel()} is below min_workspace_size = {n_cnt.value}")
         c_tmp = torch.empty((n_ctmp.value // 4,), dtype=torch.float32, device=dev) if n_ctmp.value else None
         a_tmp = torch.empty((n_atmp.value // 2,), dtype=a.dtype, device=dev) if n_atmp.value else None

@@ -27,7 +27,7 @@ static int round_gs(int x, int sub, bool w8) {
 static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8) {
   const int TPG = w8 ? 2 : 1;
   const int G = K / 128 * TPG, NT = N / 16;
-  const int MB = M <= 16 ? 1 : 2;
+  const int MB = (M + 15) / 16;
   Decode2Config c;
   c.mr = M == 1 ? 1 : (M <= 4 ? 4 : 16);
   const int slab_max = 512 / (c.mr * MB) * TPG;
@@ -44,6 +44,14 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8) 
   int gs = round_gs((gslab + wks - 1) / wks, sub, w8);
   if (g2_force_gs > 0) gs = g2_force_gs;
   while (wks * gs > slab_max && wks > 1) wks /= 2;     // respect the LDS limit
+  if (gs > slab_max) {                                 // rounding up went past it: largest instantiated size below
+    const int opts[] = {8, 7, 4, 2, 1};
+    for (int o : opts)
+      if (o <= slab_max && !(w8 && (o & 1)) && !(sub > 1 && (o & (o - 1)) != 0)) {
+        gs = o;
+        break;
+      }
+  }
   // the slab is now wks*gs groups; recompute the number of slabs
   c.sk = (G + wks * gs - 1) / (wks * gs);
   c.gs = gs;
@@ -53,7 +61,7 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8) 
   // compute unit (i.e. spread over the device), then the smaller workgroup.
   int best_wn = 1;
   long best_rounds = -1, best_waves = -1;
-  const size_t lds_wg = (size_t)wks * (gs / TPG) * 256 * c.mr * MB + (wks > 1 ? (size_t)D2_WAVES * MB * 1024 : 16);
+  const size_t lds_wg = decode2_lds_bytes(wks, gs / TPG, c.mr, MB);
   for (int wn = 1; wn <= D2_WAVES / wks; ++wn) {
     long slots = D2_WAVES / (wks * wn);
     const long lds_slots = (long)((size_t)(160 * 1024) / lds_wg);
@@ -127,7 +135,7 @@ static int dispatch_mr2(const Decode2Params& p, const Decode2Config& c, bool bf1
 
 int w4a16_decode2_workspace(int M, int N, int K, int sub, bool w8, size_t* c_tmp_bytes, size_t* counter_ints) {
   const Decode2Config c = pick_decode2_config(M, N, K, sub, w8);
-  const int MB = M <= 16 ? 1 : 2;
+  const int MB = (M + 15) / 16;
   const int NT = N / 16;
   *c_tmp_bytes = c.sk > 1 ? (size_t)c.sk * NT * MB * 64 * sizeof(v4f) : 0;
   *counter_ints = c.sk > 1 ? (size_t)NT * MB : 0;
@@ -161,7 +169,7 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
   p.SK = cfg.sk;
   p.WKS = cfg.wks;
   p.WN = cfg.wn;
-  const int MB = M <= 16 ? 1 : 2;
+  const int MB = (M + 15) / 16;
   if (cfg.sk > 1) {
     VAQ_CHECK_ARG(c_tmp != nullptr && counters != nullptr, "w4a16_gemm: split-K needs c_tmp and counters");
     VAQ_CHECK_ARG(((uintptr_t)c_tmp % 16) == 0, "w4a16_gemm: c_tmp must be 16-byte aligned");
@@ -175,6 +183,7 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
   if (w8) rc = decode2_launch_w8(p, cfg.gs, MB, cfg.mr, bf16, s);
   else if (sub == 2) rc = decode2_launch_sub2(p, cfg.gs, MB, cfg.mr, bf16, zp, s);
   else if (sub == 4) rc = decode2_launch_sub4(p, cfg.gs, MB, cfg.mr, bf16, zp, s);
+  else if (MB > 2) rc = decode2_launch_mb34(p, cfg.gs, MB, bf16, zp, s);
   else if (MB == 1) rc = dispatch_mr2<1>(p, cfg, bf16, zp, s);
   else rc = dispatch_types2<2, 16>(p, cfg.gs, bf16, zp, s);
   if (rc != VAQ_OK) return rc;

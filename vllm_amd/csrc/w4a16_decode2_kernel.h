@@ -295,8 +295,12 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   }
 
   // ---- 4. reduce the K slices of the workgroup ----
-  v4f* red = reinterpret_cast<v4f*>(lds + (size_t)KO * MR * MB * 16);     // [16 waves][MB][64]
+  // [16 waves][MB][64] partial tiles: behind the activations, or -- with three or four m-blocks, where both would not
+  // fit -- on top of them once every wavefront is through its K loop
+  constexpr bool RED_ALIAS = MB > 2;
+  v4f* red = reinterpret_cast<v4f*>(RED_ALIAS ? lds : lds + (size_t)KO * MR * MB * 16);
   if (WKS > 1) {
+    if constexpr (RED_ALIAS) __syncthreads();
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) red[(w * MB + mb) * 64 + lane] = acc[mb];
     __syncthreads();
@@ -371,10 +375,19 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   }
 }
 
+// LDS of a workgroup: activations of `groups` = WKS * (groups per wavefront) quantisation groups for MR x MB rows, 16
+// spare bytes, and the reduction buffer of the K slices (on top of the activations for MB > 2, see the kernel).
+static inline size_t decode2_lds_bytes(int wks, int groups_per_wave, int mr, int mb) {
+  const size_t act = (size_t)wks * groups_per_wave * 256 * mr * mb;
+  const size_t red = wks > 1 ? (size_t)D2_WAVES * mb * 1024 : 0;
+  if (mb > 2) return act + 16 > red ? act + 16 : red;
+  return act + (red ? red : 16);
+}
+
 template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, bool W8 = false>
 static int launch_decode2(const Decode2Params& p, hipStream_t s) {
   const int WN = p.WN;
-  const size_t lds = (size_t)p.WKS * (GS / (W8 ? 2 : 1)) * 256 * MR * MB + (p.WKS > 1 ? (size_t)D2_WAVES * MB * 1024 : 16);
+  const size_t lds = decode2_lds_bytes(p.WKS, GS / (W8 ? 2 : 1), MR, MB);
   auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP, MR, SUBG, W8>;
   static size_t attr_lds = 0;
   if (lds > attr_lds) {
@@ -395,6 +408,8 @@ static int launch_decode2(const Decode2Params& p, hipStream_t s) {
 // wavefront gs in {1, 2, 4, 8, 16}, staged rows mr in {1, 4, 16} (16 when MB == 2).
 int decode2_launch_sub2(const Decode2Params& p, int gs, int MB, int mr, bool bf16, bool zp, hipStream_t s);
 int decode2_launch_sub4(const Decode2Params& p, int gs, int MB, int mr, bool bf16, bool zp, hipStream_t s);
+// Three and four m-blocks (32 < M <= 64), groups of 128 rows / channelwise; defined in w4a16_decode2_mb34.hip.
+int decode2_launch_mb34(const Decode2Params& p, int gs, int MB, bool bf16, bool zp, hipStream_t s);
 // 8-bit codes; defined in w4a16_decode2_w8.hip: gs in {2, 4, 8, 14, 16}, staged rows mr in {1, 4, 16} (16 when MB == 2).
 int decode2_launch_w8(const Decode2Params& p, int gs, int MB, int mr, bool bf16, hipStream_t s);
 

@@ -17,7 +17,8 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
                          const void* bias, void* c, float* c_tmp, int32_t* counters, int64_t counter_ints, int M, int N,
                          int K, int sub, bool channelwise, bool w8, int dtype, hipStream_t s);
 
-constexpr int64_t DECODE_MAX_M = 32;
+constexpr int64_t DECODE_MAX_M = 64;          // up to four m-blocks of 16 rows on the LDS-staged kernel
+constexpr int64_t DECODE_MAX_M_2BLK = 32;     // the register-resident kernel, groups below 128 rows and 8-bit codes: two
 static int g_decode_impl = -1;  // -1: automatic, 0: LDS-staged activations (w4a16_decode2.hip), 1: register-resident (w4a16_decode.hip)
 
 // Measured on MI355X (Llama-3-8B shapes): staging the activations once per workgroup in LDS (one independent task
@@ -57,24 +58,35 @@ extern "C" int vaq_w4a16_gemm_workspace(int64_t size_m, int64_t size_n, int64_t 
   *counter_ints = 0;
   if (size_m == 0) return VAQ_OK;
   if (size_m <= DECODE_MAX_M) {
-    // enough for either decode kernel: which one runs also depends on the row stride of A, unknown here
-    size_t t1 = 0, n1 = 0, t2 = 0, n2 = 0;
-    rc = w4a16_decode_workspace((int)size_m, (int)size_n, (int)size_k, &t1, &n1);
-    if (rc != VAQ_OK) return rc;
+    // Enough for whichever kernel runs: that also depends on the row stride of A, the group size and the weight type,
+    // all unknown here.
+    size_t t = 0, n = 0, t2 = 0, n2 = 0;
+    auto take = [&]() {
+      if (t2 > t) t = t2;
+      if (n2 > n) n = n2;
+    };
     rc = w4a16_decode2_workspace((int)size_m, (int)size_n, (int)size_k, 1, false, &t2, &n2);
     if (rc != VAQ_OK) return rc;
-    // a group size below 128 (unknown here) restricts the kernel's configurations: cover that choice as well
-    size_t t3 = 0, n3 = 0;
-    rc = w4a16_decode2_workspace((int)size_m, (int)size_n, (int)size_k, 2, false, &t3, &n3);
-    if (rc != VAQ_OK) return rc;
-    if (t3 > t2) t2 = t3;
-    if (n3 > n2) n2 = n3;
-    rc = w4a16_decode2_workspace((int)size_m, (int)size_n, (int)size_k, 1, true, &t3, &n3);     // and 8-bit codes
-    if (rc != VAQ_OK) return rc;
-    if (t3 > t2) t2 = t3;
-    if (n3 > n2) n2 = n3;
-    *c_tmp_bytes = t1 > t2 ? t1 : t2;
-    *counter_ints = n1 > n2 ? n1 : n2;
+    take();
+    if (size_m <= DECODE_MAX_M_2BLK) {
+      rc = w4a16_decode_workspace((int)size_m, (int)size_n, (int)size_k, &t2, &n2);
+      if (rc != VAQ_OK) return rc;
+      take();
+      rc = w4a16_decode2_workspace((int)size_m, (int)size_n, (int)size_k, 2, false, &t2, &n2);   // groups below 128 rows
+      if (rc != VAQ_OK) return rc;
+      take();
+      rc = w4a16_decode2_workspace((int)size_m, (int)size_n, (int)size_k, 1, true, &t2, &n2);    // 8-bit codes
+      if (rc != VAQ_OK) return rc;
+      take();
+    } else {
+      // those cases take the prefill kernel above 32 rows
+      rc = w4a16_prefill_workspace((int)size_m, (int)size_n, (int)size_k, &t2, &n2);
+      if (rc != VAQ_OK) return rc;
+      take();
+      if (has_perm) *a_tmp_bytes = (size_t)size_m * (size_t)size_k * 2;
+    }
+    *c_tmp_bytes = t;
+    *counter_ints = n;
     return VAQ_OK;
   }
   if (has_perm) *a_tmp_bytes = (size_t)size_m * (size_t)size_k * 2;
@@ -114,10 +126,14 @@ extern "C" int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, cons
   VAQ_CHECK_ARG(!bias || ((uintptr_t)bias % 8) == 0, "w4a16_gemm: bias must be 8-byte aligned");
   hipStream_t s = (hipStream_t)stream;
 
-  bool decode = size_m <= DECODE_MAX_M;
+  // three and four m-blocks exist on the LDS-staged kernel for 4-bit codes in groups of 128 rows / channelwise
+  const bool two_blocks_only = sub > 1 || w8 || decode_impl_for(size_m, size_n, lda, sub, w8) != 0;
+  // (measured: four m-blocks beat the tile kernel by 1.5-2x on the narrow layers and lose 3 % on a 28672-wide one)
+  const int64_t dec_max = two_blocks_only ? DECODE_MAX_M_2BLK : (size_n > 8192 ? 48 : DECODE_MAX_M);
+  bool decode = size_m <= dec_max;
   if (force_path == 1) {
-    VAQ_CHECK_ARG(size_m <= DECODE_MAX_M, "w4a16_gemm: decode path forced with size_m = %lld > %lld", (long long)size_m,
-                  (long long)DECODE_MAX_M);
+    VAQ_CHECK_ARG(size_m <= dec_max, "w4a16_gemm: decode path forced with size_m = %lld > %lld", (long long)size_m,
+                  (long long)dec_max);
     decode = true;
   } else if (force_path == 2) {
     decode = false;
