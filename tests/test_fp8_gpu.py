@@ -87,6 +87,27 @@ def test_per_token_quant_strided_rows_and_padding(device):
     assert np.array_equal(_codes(q[:9]), _codes(q_ref)) and np.array_equal(s[:9].cpu().numpy(), s_ref.numpy())
 
 
+@pytest.mark.parametrize("hidden,tokens", [(8, 515), (1000, 601), (1024, 4096), (1032, 2051), (2048, 2050)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_per_token_quant_many_short_rows_bit_exact(device, hidden, tokens, dtype):
+    """Large batches of short rows take the kernel that keeps one row per wavefront (no barrier); ragged row lengths,
+    a row count that does not fill the last workgroup, strided rows, scale_ub.  Scales and codes bit-exact."""
+    import vllm_amd._custom_ops as ops
+    g = torch.Generator().manual_seed(hidden + tokens)
+    big = (torch.randn(tokens, hidden + 16, generator=g) * 3).to(dtype)
+    big[5] = 0
+    ub = torch.tensor([1.5], dtype=torch.float32)
+    big_dev = big.to(device)
+    for lo in (0, 8):
+        x = big[:, lo:lo + hidden]
+        for u in (None, ub):
+            q_ref, s_ref = f.ref_dynamic_per_token_quant(x, u)
+            q, s = ops.scaled_fp8_quant(big_dev[:, lo:lo + hidden], scale_ub=None if u is None else u.to(device),
+                                        use_per_token_if_dynamic=True)
+            assert np.array_equal(s.cpu().numpy(), s_ref.numpy())
+            assert np.array_equal(_codes(q), _codes(q_ref))
+
+
 @pytest.mark.parametrize("hidden", [17, 1024, 5137, 14336])
 @pytest.mark.parametrize("tokens", [1, 7, 300])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])

@@ -59,6 +59,7 @@ _DEBUG_SIGNATURES = {
     "vaq_debug_set_decode2_config": (None, [c_int, c_int]),
     "vaq_debug_set_fp8_config": (None, [c_int, c_int]),
     "vaq_debug_set_fp8_tile_cfg": (None, [c_int, c_int]),
+    "vaq_debug_set_quant_row_per_wave": (None, [c_int]),
 }
 
 _lib = None

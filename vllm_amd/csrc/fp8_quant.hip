@@ -18,6 +18,7 @@ namespace vaq {
 constexpr float FP8_MAX = 448.0f;
 constexpr int QT = 256;         // threads per workgroup
 constexpr int QV = 8;           // cached 8-element vectors per thread
+static int g_quant_row_per_wave = 1;    // tuning aid: 0 = always one workgroup per row
 
 template <typename T>
 __device__ inline float load_as_float(const T* p);
@@ -152,7 +153,80 @@ __global__ __launch_bounds__(QT) void fp8_quant_kernel(const T* __restrict__ in,
   }
 }
 
+// Dynamic per token, one row per WAVEFRONT: the row (at most 64 lanes x NV vectors x 8 elements) sits in the wavefront's
+// registers, the absmax is a butterfly over the lanes -- no LDS, no barrier, four rows per workgroup in flight
+// independently.  Same arithmetic as MODE 0 above (the maximum is order-independent, the division is the IEEE one).
+template <typename T, int NV>
+__global__ __launch_bounds__(QT) void fp8_quant_row_per_wave_kernel(const T* __restrict__ in, int64_t in_stride,
+                                                                     uint8_t* __restrict__ out, int64_t out_stride,
+                                                                     float* __restrict__ scales,
+                                                                     const float* __restrict__ scale_ub, int hidden,
+                                                                     int64_t rows) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * (QT / 64) + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T* x = in + row * in_stride;
+  uint8_t* y = out + row * out_stride;
+  const int nvec = hidden / 8;
+  Vec8<T> cache[NV];
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = lane + i * 64;
+    if (v < nvec) cache[i].load(x + (int64_t)v * 8);
+  }
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = lane + i * 64;
+    if (v < nvec) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(cache[i].f[e]));
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+  float s = scale_ub ? fminf(amax, *scale_ub) : amax;
+  s = fmaxf(s / FP8_MAX, 1.0f / (FP8_MAX * 512.0f));
+  if (lane == 0) scales[row] = s;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = lane + i * 64;
+    if (v < nvec) {
+      float q[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) q[e] = clamp448(cache[i].f[e] / s);
+      v2u o;
+      o.x = cvt2(q[0], q[1]) | (cvt2(q[2], q[3]) << 16);
+      o.y = cvt2(q[4], q[5]) | (cvt2(q[6], q[7]) << 16);
+      *reinterpret_cast<v2u*>(y + (int64_t)v * 8) = o;
+    }
+  }
+}
+
 __global__ void fill_zero_kernel(float* p) { *p = 0.f; }
+
+// The row-per-wavefront kernel takes 16-bit rows of at most 4096 elements whose addresses allow 16-byte loads and
+// 8-byte stores on every row (the caller only sends rows of up to 2048 elements).
+static bool row_per_wave_ok(const void* in, int in_dtype, int64_t in_stride, const uint8_t* out, int64_t out_stride,
+                            int64_t hidden) {
+  return (in_dtype == VAQ_BF16 || in_dtype == VAQ_F16) && hidden % 8 == 0 && hidden <= 64 * 8 * 8 &&
+         ((uintptr_t)in % 16) == 0 && in_stride % 8 == 0 && ((uintptr_t)out % 8) == 0 && out_stride % 8 == 0;
+}
+
+template <typename T>
+static void launch_row_per_wave(const void* in, int64_t in_stride, uint8_t* out, int64_t out_stride, float* scales,
+                                const float* ub, int64_t rows, int64_t hidden, hipStream_t s) {
+  const dim3 grid((unsigned)((rows + QT / 64 - 1) / (QT / 64))), block(QT);
+  if (hidden <= 64 * 8 * 2)
+    hipLaunchKernelGGL((fp8_quant_row_per_wave_kernel<T, 2>), grid, block, 0, s, (const T*)in, in_stride, out, out_stride,
+                       scales, ub, (int)hidden, rows);
+  else if (hidden <= 64 * 8 * 4)
+    hipLaunchKernelGGL((fp8_quant_row_per_wave_kernel<T, 4>), grid, block, 0, s, (const T*)in, in_stride, out, out_stride,
+                       scales, ub, (int)hidden, rows);
+  else
+    hipLaunchKernelGGL((fp8_quant_row_per_wave_kernel<T, 8>), grid, block, 0, s, (const T*)in, in_stride, out, out_stride,
+                       scales, ub, (int)hidden, rows);
+}
 
 template <int MODE>
 static int launch_quant(const void* in, int in_dtype, int64_t in_stride, uint8_t* out, int64_t out_stride,
@@ -196,9 +270,21 @@ extern "C" int vaq_fp8_quant_per_token(const void* in, int in_dtype, int64_t in_
   using namespace vaq;
   int rc = check_quant("fp8_quant_per_token", in, in_row_stride, out, out_row_stride, scales, rows, hidden);
   if (rc != VAQ_OK || rows == 0) return rc;
-  rc = launch_quant<0>(in, in_dtype, in_row_stride, out, out_row_stride, scales, scale_ub, rows, hidden,
-                       (hipStream_t)stream);
-  if (rc != VAQ_OK) return rc;
+  // Measured: a row per wavefront is 1.1-1.6x faster for short rows in large batches; with few rows a whole workgroup
+  // per row has the shorter latency, and from 4096 elements on the 64 registers of row data per lane cost more than the
+  // barriers saved.
+  const bool many_short_rows = hidden <= 1024 ? rows >= 512 : (hidden <= 2048 && rows >= 2048);
+  if (g_quant_row_per_wave && many_short_rows &&
+      row_per_wave_ok(in, in_dtype, in_row_stride, out, out_row_stride, hidden)) {
+    if (in_dtype == VAQ_BF16)
+      launch_row_per_wave<bf16_t>(in, in_row_stride, out, out_row_stride, scales, scale_ub, rows, hidden, (hipStream_t)stream);
+    else
+      launch_row_per_wave<f16_t>(in, in_row_stride, out, out_row_stride, scales, scale_ub, rows, hidden, (hipStream_t)stream);
+  } else {
+    rc = launch_quant<0>(in, in_dtype, in_row_stride, out, out_row_stride, scales, scale_ub, rows, hidden,
+                         (hipStream_t)stream);
+    if (rc != VAQ_OK) return rc;
+  }
   VAQ_CHECK_LAUNCH("fp8_quant_per_token");
   return VAQ_OK;
 }
@@ -232,3 +318,6 @@ extern "C" int vaq_fp8_quant_dynamic(const void* in, int in_dtype, int64_t in_ro
   VAQ_CHECK_LAUNCH("fp8_quant_dynamic");
   return VAQ_OK;
 }
+
+// Benchmark / tuning aid, not part of the drop-in surface: 0 = per-token quantisation always with one workgroup per row.
+extern "C" void vaq_debug_set_quant_row_per_wave(int on) { vaq::g_quant_row_per_wave = on; }

@@ -20,13 +20,18 @@
 // it has at most 256 x 8 x 8 = 16384 elements and is 16-byte aligned; other rows re-read global memory.
 #include "vaq_common.h"
 
+#include <type_traits>
+
 namespace vaq {
 
 namespace {
 
 constexpr float NQ_FP8_MAX = 448.0f;
 constexpr int NQ_T = 256;
-constexpr int NQ_V = 8;
+// Chunks of 8 elements per thread that the row-in-registers path holds (template parameter NV): 2, 4 or 8, the smallest
+// that covers the row -- the register arrays are sized by it, and with them the number of rows a compute unit works on
+// at a time.
+constexpr int NQ_V_MAX = 8;
 
 template <bool BF16>
 __device__ inline float nq_to_float(uint16_t v) { return F16Traits<BF16>::to_float(v); }
@@ -70,7 +75,7 @@ __device__ inline void nq_unpack8(v4u r, float* f, bool bf16) {
   }
 }
 
-template <bool BF16, bool HAS_RES>
+template <bool BF16, bool HAS_RES, int NV>
 __global__ __launch_bounds__(NQ_T) void rms_norm_per_token_fp8_kernel(uint8_t* __restrict__ out, float* __restrict__ scales,
                                                                       const uint16_t* __restrict__ input,
                                                                       const uint16_t* __restrict__ weight,
@@ -84,18 +89,20 @@ __global__ __launch_bounds__(NQ_T) void rms_norm_per_token_fp8_kernel(uint8_t* _
   uint16_t* res = HAS_RES ? residual + tok * (int64_t)hidden : nullptr;
   uint8_t* orow = out + tok * (int64_t)hidden;
   const int chunks = hidden / 8;
-  const bool cached = (hidden % 8 == 0) && chunks <= NQ_T * NQ_V && (in_stride % 8 == 0) &&
+  const bool cached = (hidden % 8 == 0) && chunks <= NQ_T * NV && (in_stride % 8 == 0) &&
                       ((reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(weight) |
                         reinterpret_cast<uintptr_t>(out) | (HAS_RES ? reinterpret_cast<uintptr_t>(residual) : 0)) % 16 == 0);
   const float min_scale = 1.0f / (NQ_FP8_MAX * 512.0f);
 
   if (cached) {
-    float x[NQ_V][8];
+    float x[NV][8];
+    v4u wv[NV];          // the weight chunks, requested together with the row: no dependent load after the reduction
     float ss = 0.f;
 #pragma unroll
-    for (int v = 0; v < NQ_V; ++v) {
+    for (int v = 0; v < NV; ++v) {
       const int c = threadIdx.x + v * NQ_T;
       if (c < chunks) {
+        wv[v] = *reinterpret_cast<const v4u*>(weight + c * 8);
         nq_unpack8(*reinterpret_cast<const v4u*>(row + c * 8), x[v], BF16);
         if constexpr (HAS_RES) {
           float r[8];
@@ -117,11 +124,11 @@ __global__ __launch_bounds__(NQ_T) void rms_norm_per_token_fp8_kernel(uint8_t* _
     const float rms = rsqrtf(ss / (float)hidden + eps);
     float amax = 0.f;
 #pragma unroll
-    for (int v = 0; v < NQ_V; ++v) {
+    for (int v = 0; v < NV; ++v) {
       const int c = threadIdx.x + v * NQ_T;
       if (c < chunks) {
         float w[8];
-        nq_unpack8(*reinterpret_cast<const v4u*>(weight + c * 8), w, BF16);
+        nq_unpack8(wv[v], w, BF16);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           x[v][e] = nq_round16<BF16>(nq_round16<BF16>(x[v][e] * rms) * w[e]);
@@ -134,7 +141,7 @@ __global__ __launch_bounds__(NQ_T) void rms_norm_per_token_fp8_kernel(uint8_t* _
     const float s = fmaxf(amax / NQ_FP8_MAX, min_scale);
     if (threadIdx.x == 0) scales[tok] = s;
 #pragma unroll
-    for (int v = 0; v < NQ_V; ++v) {
+    for (int v = 0; v < NV; ++v) {
       const int c = threadIdx.x + v * NQ_T;
       if (c < chunks) {
         v2u o;
@@ -188,7 +195,7 @@ __global__ __launch_bounds__(NQ_T) void rms_norm_per_token_fp8_kernel(uint8_t* _
   }
 }
 
-template <bool BF16, bool HAS_RES>
+template <bool BF16, bool HAS_RES, int NV>
 __global__ __launch_bounds__(NQ_T) void rms_norm_static_fp8_kernel(uint8_t* __restrict__ out,
                                                                    const uint16_t* __restrict__ input,
                                                                    const uint16_t* __restrict__ weight,
@@ -202,18 +209,20 @@ __global__ __launch_bounds__(NQ_T) void rms_norm_static_fp8_kernel(uint8_t* __re
   uint16_t* res = HAS_RES ? residual + tok * (int64_t)hidden : nullptr;
   uint8_t* orow = out + tok * (int64_t)hidden;
   const int chunks = hidden / 8;
-  const bool cached = (hidden % 8 == 0) && chunks <= NQ_T * NQ_V && (in_stride % 8 == 0) &&
+  const bool cached = (hidden % 8 == 0) && chunks <= NQ_T * NV && (in_stride % 8 == 0) &&
                       ((reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(weight) |
                         reinterpret_cast<uintptr_t>(out) | (HAS_RES ? reinterpret_cast<uintptr_t>(residual) : 0)) % 16 == 0);
   const float inv = 1.0f / *scale;
 
   if (cached) {
-    float x[NQ_V][8];
+    float x[NV][8];
+    v4u wv[NV];          // the weight chunks, requested together with the row
     float ss = 0.f;
 #pragma unroll
-    for (int v = 0; v < NQ_V; ++v) {
+    for (int v = 0; v < NV; ++v) {
       const int c = threadIdx.x + v * NQ_T;
       if (c < chunks) {
+        wv[v] = *reinterpret_cast<const v4u*>(weight + c * 8);
         nq_unpack8(*reinterpret_cast<const v4u*>(row + c * 8), x[v], BF16);
         if constexpr (HAS_RES) {
           float r[8];
@@ -237,11 +246,11 @@ __global__ __launch_bounds__(NQ_T) void rms_norm_static_fp8_kernel(uint8_t* __re
     ss = nq_block_sum(ss, smem);
     const float rms = rsqrtf(ss / (float)hidden + eps);
 #pragma unroll
-    for (int v = 0; v < NQ_V; ++v) {
+    for (int v = 0; v < NV; ++v) {
       const int c = threadIdx.x + v * NQ_T;
       if (c < chunks) {
         float w[8];
-        nq_unpack8(*reinterpret_cast<const v4u*>(weight + c * 8), w, BF16);
+        nq_unpack8(wv[v], w, BF16);
         v2u o;
         uint32_t* ow = reinterpret_cast<uint32_t*>(&o);
 #pragma unroll
@@ -337,6 +346,24 @@ __global__ __launch_bounds__(NQ_T) void silu_and_mul_fp8_kernel(uint8_t* __restr
 
 }  // namespace vaq
 
+namespace vaq {
+// run-time (dtype, residual, chunks per thread) -> compile-time template arguments
+template <typename F>
+static void nq_dispatch(bool bf16, bool has_res, int nv, F&& f) {
+  auto with_nv = [&](auto bf, auto rs) {
+    if (nv == 2) f(bf, rs, std::integral_constant<int, 2>{});
+    else if (nv == 4) f(bf, rs, std::integral_constant<int, 4>{});
+    else f(bf, rs, std::integral_constant<int, NQ_V_MAX>{});
+  };
+  auto with_res = [&](auto bf) {
+    if (has_res) with_nv(bf, std::true_type{});
+    else with_nv(bf, std::false_type{});
+  };
+  if (bf16) with_res(std::true_type{});
+  else with_res(std::false_type{});
+}
+}  // namespace vaq
+
 extern "C" int vaq_rms_norm_dynamic_per_token_fp8_quant(uint8_t* out, float* scales, const void* input, int64_t in_stride,
                                                         const void* weight, const float* scale_ub, float epsilon,
                                                         void* residual, int dtype, int64_t tokens, int64_t hidden,
@@ -355,13 +382,12 @@ extern "C" int vaq_rms_norm_dynamic_per_token_fp8_quant(uint8_t* out, float* sca
   const uint16_t* w = (const uint16_t*)weight;
   uint16_t* res = (uint16_t*)residual;
   const bool bf16 = dtype == VAQ_BF16;
-  if (bf16) {
-    if (res) hipLaunchKernelGGL((rms_norm_per_token_fp8_kernel<true, true>), grid, block, 0, s, out, scales, in, w, scale_ub, epsilon, res, (int)hidden, in_stride);
-    else hipLaunchKernelGGL((rms_norm_per_token_fp8_kernel<true, false>), grid, block, 0, s, out, scales, in, w, scale_ub, epsilon, res, (int)hidden, in_stride);
-  } else {
-    if (res) hipLaunchKernelGGL((rms_norm_per_token_fp8_kernel<false, true>), grid, block, 0, s, out, scales, in, w, scale_ub, epsilon, res, (int)hidden, in_stride);
-    else hipLaunchKernelGGL((rms_norm_per_token_fp8_kernel<false, false>), grid, block, 0, s, out, scales, in, w, scale_ub, epsilon, res, (int)hidden, in_stride);
-  }
+  const int nv = hidden <= NQ_T * 8 * 2 ? 2 : (hidden <= NQ_T * 8 * 4 ? 4 : NQ_V_MAX);
+  auto launch = [&](auto bf, auto rs, auto nvc) {
+    hipLaunchKernelGGL((rms_norm_per_token_fp8_kernel<decltype(bf)::value, decltype(rs)::value, decltype(nvc)::value>), grid, block,
+                       0, s, out, scales, in, w, scale_ub, epsilon, res, (int)hidden, in_stride);
+  };
+  nq_dispatch(bf16, res != nullptr, nv, launch);
   VAQ_CHECK_LAUNCH("rms_norm_dynamic_per_token_quant");
   return VAQ_OK;
 }
@@ -382,13 +408,12 @@ extern "C" int vaq_rms_norm_static_fp8_quant(uint8_t* out, const void* input, in
   const uint16_t* in = (const uint16_t*)input;
   const uint16_t* w = (const uint16_t*)weight;
   uint16_t* res = (uint16_t*)residual;
-  if (dtype == VAQ_BF16) {
-    if (res) hipLaunchKernelGGL((rms_norm_static_fp8_kernel<true, true>), grid, block, 0, s, out, in, w, scale, epsilon, res, (int)hidden, in_stride);
-    else hipLaunchKernelGGL((rms_norm_static_fp8_kernel<true, false>), grid, block, 0, s, out, in, w, scale, epsilon, res, (int)hidden, in_stride);
-  } else {
-    if (res) hipLaunchKernelGGL((rms_norm_static_fp8_kernel<false, true>), grid, block, 0, s, out, in, w, scale, epsilon, res, (int)hidden, in_stride);
-    else hipLaunchKernelGGL((rms_norm_static_fp8_kernel<false, false>), grid, block, 0, s, out, in, w, scale, epsilon, res, (int)hidden, in_stride);
-  }
+  const int nv = hidden <= NQ_T * 8 * 2 ? 2 : (hidden <= NQ_T * 8 * 4 ? 4 : NQ_V_MAX);
+  auto launch = [&](auto bf, auto rs, auto nvc) {
+    hipLaunchKernelGGL((rms_norm_static_fp8_kernel<decltype(bf)::value, decltype(rs)::value, decltype(nvc)::value>), grid, block, 0,
+                       s, out, in, w, scale, epsilon, res, (int)hidden, in_stride);
+  };
+  nq_dispatch(dtype == VAQ_BF16, res != nullptr, nv, launch);
   VAQ_CHECK_LAUNCH("rms_norm_static_fp8_quant");
   return VAQ_OK;
 }
