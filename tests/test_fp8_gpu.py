@@ -205,6 +205,27 @@ def test_scaled_mm_mixed_scales_fp16_and_padded_weight(device, m):
     _check_mm(out, ref, f"padded weight m={m}")
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_scaled_mm_random_shapes(device, seed):
+    """Seeded sweep over irregular problems: M from 1 to 700, N and K any multiple of 16 (K not a multiple of 64 or 128
+    takes the kernels' tail paths), every scale combination, bias or not, both output types."""
+    import vllm_amd._custom_ops as ops
+    rng = np.random.default_rng(2000 + seed)
+    for _ in range(6):
+        m = int(rng.choice([1, 2, 7, 16, 17, 32, 33, 63, 64, 65, 128, 200, 256, 257, 511, 700]))
+        n = 16 * int(rng.integers(1, 80))
+        k = 16 * int(rng.integers(1, 300))
+        per_token, per_channel, bias = bool(rng.integers(0, 2)), bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        out_dtype = torch.bfloat16 if rng.integers(0, 2) else torch.float16
+        a_q, sa, w_q, sb, b = _mm_case(m, k, n, seed=int(rng.integers(0, 1 << 30)), per_token=per_token,
+                                       per_channel=per_channel, bias=bias, out_dtype=out_dtype)
+        ref = f.scaled_mm_ref(a_q, w_q.t(), sa, sb, out_dtype, b)
+        out = ops.cutlass_scaled_mm(a_q.to(device), w_q.to(device).t(), sa.to(device), sb.to(device), out_dtype,
+                                    None if b is None else b.to(device))
+        _check_mm(out, ref, f"m={m} n={n} k={k} per_token={per_token} per_channel={per_channel} bias={bias} {out_dtype}")
+    assert bool((ops._fp8_counters(torch.device(device)) == 0).all())
+
+
 def test_scaled_mm_exact_small_integers(device):
     """With scales 1 and small-integer operands every partial sum is an exactly representable integer, so any
     dropped / duplicated k or transposed operand changes the result: the output must equal the integer GEMM."""

@@ -284,6 +284,31 @@ def test_gemm_8bit_llama_shapes(device):
         assert bool((layer.workspace == 0).all())
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_gemm_random_shapes_and_formats(device, seed):
+    """Seeded sweep over irregular problems: K any multiple of 128 (odd group counts, counts that no wavefront split
+    divides), N any multiple of 64, M from 1 to 300, every weight format and group size, act_order, bias, fp16 / bf16.
+    Each case against the oracle; the launch-shape choices of the kernels have many branches that only such sizes reach."""
+    rng = np.random.default_rng(1000 + seed)
+    for _ in range(6):
+        k = 128 * int(rng.integers(1, 40))
+        n = 64 * int(rng.integers(1, 20))
+        m = int(rng.choice([1, 2, 3, 5, 8, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 100, 129, 300]))
+        fmt = rng.choice(["u4b8", "u4", "u8b128"])
+        group_size = int(rng.choice([128, -1] if fmt == "u8b128" else [128, 64, 32, -1]))
+        act_order = bool(rng.integers(0, 2)) and group_size != -1 and k // group_size > 1
+        dtype = torch.bfloat16 if rng.integers(0, 2) else torch.float16
+        case = o.make_w4a16_case(k, n, group_size, asym=fmt == "u4", act_order=act_order, dtype=dtype,
+                                 seed=int(rng.integers(0, 1 << 30)), num_bits=8 if fmt == "u8b128" else 4)
+        layer = W4A16Layer(case, device, dtype)
+        a = _acts(m, k, device, dtype, seed=m + k)
+        bias = (torch.randn(n, generator=torch.Generator().manual_seed(n)) * 0.5).to(dtype) if rng.integers(0, 2) else None
+        what = f"k={k} n={n} m={m} {fmt} g={group_size} act_order={act_order} {dtype} bias={bias is not None}"
+        out = layer(a, None if bias is None else bias.to(device))
+        check_gemm_close(out, o.gemm_ref(a.cpu(), o.case_w_ref(case), bias), what)
+        assert bool((layer.workspace == 0).all()), what
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("m", [1, 3, 16, 96])
 def test_gemm_fp16_and_bias(device, decode_kernel, dtype, m):
