@@ -350,7 +350,8 @@ def test_scaled_mm_every_tile_shape_exact(device, cfg):
     lib = _lib.load()
     g = torch.Generator().manual_seed(cfg)
     try:
-        for m, n, k, split in ((300, 384, 1024, 0), (64, 256, 8192 + 128, 2), (513, 512, 640, 0)):
+        for m, n, k, split in ((300, 384, 1024, 0), (64, 256, 8192 + 128, 2), (513, 512, 640, 0), (257, 272, 384, 0),
+                               (100, 128, 448, 0), (520, 256, 64 * 13, 3)):
             a = torch.randint(-2, 3, (m, k), generator=g).float()
             w = torch.randint(-1, 2, (n, k), generator=g).float()
             lib.vaq_debug_set_fp8_tile_cfg(cfg, split)
