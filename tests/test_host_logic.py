@@ -309,3 +309,80 @@ def test_plugin_surface_contract():
     assert "my_method" in QUANTIZATION_METHODS and get_quantization_config("my_method") is MyConfig
     with pytest.raises(ValueError):
         get_quantization_config("no_such_method")
+
+
+# ------------------------------------------------------------------------------------------------ checkpoint loading
+
+def test_weight_loaders_place_checkpoint_tensors_in_fused_layers():
+    """The loader side of the plugin contract (parameter.py:129-408, linear.py:784-866,:948-1060): logical parts of
+    a fused layer arrive one checkpoint tensor at a time, each parameter knows its output / packed dimension, and a
+    tensor that is already fused on disk is cut into the parts.  Checked against plain concatenation."""
+    from vllm_amd.layers.linear import MergedColumnParallelLinear, QKVParallelLinear, RowParallelLinear
+    from vllm_amd.layers.quantization import get_quantization_config
+    from vllm_amd.parameter import (GroupQuantScaleParameter, PackedvLLMParameter, PerTensorScaleParameter,
+                                    RowvLLMParameter)
+    g = torch.Generator().manual_seed(0)
+    ri = lambda *shape: torch.randint(-2 ** 31, 2 ** 31 - 1, shape, dtype=torch.int32, generator=g)   # noqa: E731
+    k = 256
+
+    # GPTQ: qweight packed along K (output offsets unchanged), qzeros packed along N (output offsets / 8)
+    cfg = get_quantization_config("gptq_marlin").from_config(dict(bits=4, group_size=128, desc_act=False, sym=True))
+    sizes = [128, 192]
+    layer = MergedColumnParallelLinear(k, sizes, quant_config=cfg, params_dtype=torch.float16, bias=True)
+    assert isinstance(layer.qweight, PackedvLLMParameter) and layer.qweight.packed_dim == 0
+    assert isinstance(layer.qzeros, PackedvLLMParameter) and layer.qzeros.packed_dim == layer.qzeros.output_dim == 1
+    assert isinstance(layer.scales, GroupQuantScaleParameter) and isinstance(layer.g_idx, RowvLLMParameter)
+    parts = [dict(qweight=ri(k // 8, n), qzeros=ri(k // 128, n // 8), scales=torch.randn(k // 128, n, generator=g).half(),
+                  bias=torch.randn(n, generator=g).half()) for n in sizes]
+    g_idx = torch.arange(k, dtype=torch.int32) // 128
+    for name in ("qweight", "qzeros", "scales", "bias"):
+        for shard_id in (1, 0):                                         # any order
+            param = getattr(layer, name)
+            param.weight_loader(param, parts[shard_id][name], shard_id)
+        assert torch.equal(getattr(layer, name).data, torch.cat([p_[name] for p_ in parts], dim=-1)), name
+    layer.g_idx.weight_loader(layer.g_idx, g_idx)
+    assert torch.equal(layer.g_idx.data, g_idx)
+    # the same layer from tensors that are already fused on disk
+    layer2 = MergedColumnParallelLinear(k, sizes, quant_config=cfg, params_dtype=torch.float16)
+    for name in ("qweight", "qzeros", "scales"):
+        param = getattr(layer2, name)
+        param.weight_loader(param, getattr(layer, name).data.clone())
+        assert torch.equal(param.data, getattr(layer, name).data), name
+    with pytest.raises(ValueError):
+        layer.qweight.weight_loader(layer.qweight, ri(k // 8, 64), 0)   # wrong part size
+
+    # AWQ: weights AND zero points packed along N; q / k / v shard ids
+    cfg = get_quantization_config("awq_marlin").from_config(dict(quant_method="awq", bits=4, group_size=128, zero_point=True))
+    qkv = QKVParallelLinear(k, 64, 4, 2, quant_config=cfg, params_dtype=torch.float16)          # q 256, k 128, v 128
+    assert qkv.output_sizes == [256, 128, 128] and qkv.qweight.packed_dim == qkv.qweight.output_dim == 1
+    shards = {sid: dict(qweight=ri(k, n // 8), qzeros=ri(k // 128, n // 8),
+                        scales=torch.randn(k // 128, n, generator=g).half())
+              for sid, n in zip("qkv", qkv.output_sizes)}
+    for sid in "vqk":
+        for name in ("qweight", "qzeros", "scales"):
+            param = getattr(qkv, name)
+            param.weight_loader(param, shards[sid][name], sid)
+    for name in ("qweight", "qzeros", "scales"):
+        assert torch.equal(getattr(qkv, name).data, torch.cat([shards[sid][name] for sid in "qkv"], dim=-1)), name
+
+    # FP8 serialized: weight rows per part, one scale per part (a scalar on disk), static input scales
+    from vllm_amd.layers.quantization.fp8 import Fp8Config
+    fcfg = Fp8Config(is_checkpoint_fp8_serialized=True, activation_scheme="static")
+    f8 = QKVParallelLinear(k, 64, 4, 2, quant_config=fcfg, params_dtype=torch.bfloat16)
+    assert isinstance(f8.weight_scale, PerTensorScaleParameter) and f8.weight_scale.shape == (3,)
+    ws = {sid: torch.randint(0, 255, (n, k), dtype=torch.uint8, generator=g).view(torch.float8_e4m3fn)
+          for sid, n in zip("qkv", f8.output_sizes)}
+    for i, sid in enumerate("kvq"):
+        f8.weight.weight_loader(f8.weight, ws[sid], sid)
+        f8.weight_scale.weight_loader(f8.weight_scale, torch.tensor(0.5 + i), sid)
+        f8.input_scale.weight_loader(f8.input_scale, torch.tensor([0.25 * (i + 1)]), sid)
+    assert torch.equal(f8.weight.data.view(torch.uint8), torch.cat([ws[sid] for sid in "qkv"]).view(torch.uint8))
+    assert f8.weight_scale.data.tolist() == [2.5, 0.5, 1.5] and f8.input_scale.data.tolist() == [0.75, 0.25, 0.5]
+
+    # a plain (row-parallel) layer takes the whole tensor; a scalar checkpoint scale lands in a one-element parameter
+    row = RowParallelLinear(k, 64, quant_config=fcfg, params_dtype=torch.bfloat16)
+    w = torch.randint(0, 255, (64, k), dtype=torch.uint8, generator=g).view(torch.float8_e4m3fn)
+    row.weight.weight_loader(row.weight, w)
+    row.weight_scale.weight_loader(row.weight_scale, torch.tensor(0.125))
+    assert torch.equal(row.weight.data.view(torch.uint8), w.view(torch.uint8)) and row.weight_scale.data.tolist() == [0.125]
+

@@ -270,6 +270,62 @@ def test_fp8_linear_method_serialized_static_fused_shards(device):
         _fp8_close(out, ref, f"fp8 static fused m={m}")
 
 
+def test_layers_loaded_shard_by_shard_through_weight_loaders(device):
+    """Checkpoint tensors enter the layers the way a model loader delivers them -- `param.weight_loader(param, tensor,
+    shard_id)` per logical part, on a layer that already lives on the device (linear.py:820-866,:1009-1060) -- then
+    `process_weights_after_loading` and a forward pass against the oracle of the concatenated layer."""
+    from vllm_amd.layers.linear import MergedColumnParallelLinear, QKVParallelLinear
+    from vllm_amd.layers.quantization import get_quantization_config
+    k = 1024
+    # GPTQ gate_up_proj from separate gate / up tensors
+    sizes = [256, 192]
+    cfg = get_quantization_config("gptq_marlin").from_config(dict(bits=4, group_size=128, desc_act=False, sym=True))
+    layer = MergedColumnParallelLinear(k, sizes, quant_config=cfg, params_dtype=torch.bfloat16, return_bias=False).to(device)
+    cases = [o.make_w4a16_case(k, n, 128, seed=80 + i) for i, n in enumerate(sizes)]
+    for i, case in enumerate(cases):
+        layer.qweight.weight_loader(layer.qweight, to_dev(case["qweight"], device), i)
+        layer.scales.weight_loader(layer.scales, to_dev(case["scales"], device, torch.bfloat16), i)
+        layer.qzeros.weight_loader(layer.qzeros, torch.full((k // 128, sizes[i] // 8), 0x77777777, dtype=torch.int32), i)
+    layer.g_idx.weight_loader(layer.g_idx, torch.arange(k, dtype=torch.int32) // 128)
+    layer.process_weights_after_loading()
+    w_ref = torch.cat([o.case_w_ref(c) for c in cases], dim=1)
+    for m in (1, 40, 150):
+        a = _acts(m, k, seed=m)
+        check_gemm_close(layer(a.to(device)), o.gemm_ref(a, w_ref), f"gptq merged from shards m={m}")
+    # AWQ qkv_proj from q / k / v tensors
+    hf = dict(quant_method="awq", bits=4, group_size=128, zero_point=True)
+    qkv = QKVParallelLinear(k, 64, 4, 2, quant_config=get_quantization_config("awq_marlin").from_config(hf),
+                            params_dtype=torch.float16, return_bias=False).to(device)
+    cases = {sid: o.make_w4a16_case(k, n, 128, asym=True, dtype=torch.float16, seed=90 + i)
+             for i, (sid, n) in enumerate(zip("qkv", qkv.output_sizes))}
+    for sid, case in cases.items():
+        qkv.qweight.weight_loader(qkv.qweight, to_dev(o.awq_pack(case["q"], 4), device), sid)
+        qkv.qzeros.weight_loader(qkv.qzeros, to_dev(o.awq_pack(case["zp_vals"], 4), device), sid)
+        qkv.scales.weight_loader(qkv.scales, to_dev(case["scales"], device, torch.float16), sid)
+    qkv.process_weights_after_loading()
+    w_ref = torch.cat([o.case_w_ref(cases[sid]) for sid in "qkv"], dim=1)
+    for m in (2, 33):
+        a = _acts(m, k, torch.float16, seed=m)
+        check_gemm_close(qkv(a.to(device)), o.gemm_ref(a, w_ref), f"awq qkv from shards m={m}")
+    # FP8 serialized gate_up_proj: per-part weights and scalar scales; requantised to the largest scale after loading
+    fcfg = get_quantization_config("fp8").from_config(dict(quant_method="fp8", activation_scheme="dynamic"))
+    f8 = MergedColumnParallelLinear(k, sizes, quant_config=fcfg, params_dtype=torch.bfloat16, return_bias=False).to(device)
+    g = torch.Generator().manual_seed(6)
+    scales = [torch.tensor(0.013), torch.tensor(0.021)]
+    parts = [of.ref_static_quant(torch.randn(n, k, generator=g) * (0.5 + 0.6 * i), scales[i]) for i, n in enumerate(sizes)]
+    for i in (1, 0):
+        f8.weight.weight_loader(f8.weight, parts[i].to(device), i)
+        f8.weight_scale.weight_loader(f8.weight_scale, scales[i], i)
+    f8.process_weights_after_loading()
+    max_s = torch.stack(scales).max()
+    wq_ref = of.ref_static_quant(torch.cat([parts[i].float() * scales[i] for i in range(2)]), max_s)
+    assert torch.equal(f8.weight.t().contiguous().cpu().view(torch.uint8), wq_ref.view(torch.uint8))
+    a = _acts(20, k, seed=3)
+    aq, sa = of.ref_dynamic_per_token_quant(a)          # the dynamic scheme quantises activations per token
+    _fp8_close(f8(a.to(device)), of.scaled_mm_ref(aq, wq_ref.t(), sa, max_s.reshape(1), torch.float64, None),
+               "fp8 merged from shards")
+
+
 def test_ptpc_fp8_linear_method(device):
     """Per-token x per-channel (ptpc_fp8.py:82-137): bit-exact load-time weight quantisation, GEMM within tolerance."""
     from vllm_amd.layers.linear import LinearBase

@@ -1,18 +1,24 @@
 """Single-GPU linear layers that delegate to a quantization method -- the caller side of the plugin contract in the
 reference's ``vllm/model_executor/layers/linear.py`` (LinearBase :243-300; forward -> ``quant_method.apply`` at
-:399/:565/:1405).  Tensor-parallel sharding is out of scope: partition sizes equal full sizes."""
+:399/:565/:1405) -- and the checkpoint side: every parameter carries ``weight_loader`` = the layer's
+``weight_loader_v2``, which places a checkpoint tensor (the whole matrix, one logical part of a fused layer such as
+``gate_proj`` / ``"q"``, or an already fused tensor) inside the layer's parameters (linear.py:549,:784-866,:948-1060,
+:1379).  Tensor-parallel sharding is out of scope: partition sizes equal full sizes."""
 from __future__ import annotations
 
 import torch
 
+from ..parameter import BasevLLMParameter, PerTensorScaleParameter, _ColumnvLLMParameter
 from .quantization.base_config import LinearMethodBase, QuantizationConfig
 
 
 class UnquantizedLinearMethod(LinearMethodBase):
     def create_weights(self, layer, input_size_per_partition, output_partition_sizes, input_size, output_size,
                        params_dtype, **extra_weight_attrs):
-        layer.register_parameter("weight", torch.nn.Parameter(
-            torch.empty(sum(output_partition_sizes), input_size_per_partition, dtype=params_dtype), requires_grad=False))
+        from ..parameter import ModelWeightParameter
+        layer.register_parameter("weight", ModelWeightParameter(
+            data=torch.empty(sum(output_partition_sizes), input_size_per_partition, dtype=params_dtype), input_dim=1,
+            output_dim=0, weight_loader=extra_weight_attrs.get("weight_loader")))
 
     def apply(self, layer, x, bias=None):
         return torch.nn.functional.linear(x, layer.weight, bias)
@@ -39,11 +45,41 @@ class LinearBase(torch.nn.Module):
         if self.quant_method is None:
             self.quant_method = UnquantizedLinearMethod()
         self.quant_method.create_weights(self, input_size, self.output_sizes, input_size, output_size,
-                                         self.params_dtype)
+                                         self.params_dtype, weight_loader=self.weight_loader_v2)
         if bias:
-            self.bias = torch.nn.Parameter(torch.zeros(output_size, dtype=self.params_dtype), requires_grad=False)
+            self.bias = _ColumnvLLMParameter(data=torch.zeros(output_size, dtype=self.params_dtype), output_dim=0,
+                                             weight_loader=self.weight_loader_v2)
         else:
             self.register_parameter("bias", None)
+
+    # ---- checkpoint loading ------------------------------------------------------------------------------------------
+    def _part_offset_and_size(self, loaded_shard_id) -> tuple[int, int]:
+        """Where logical part `loaded_shard_id` (an index, or "q" / "k" / "v") sits along the output dimension."""
+        idx = {"q": 0, "k": 1, "v": 2}.get(loaded_shard_id, loaded_shard_id)
+        if not isinstance(idx, int) or not 0 <= idx < len(self.output_sizes):
+            raise ValueError(f"unknown shard id {loaded_shard_id!r} for a layer with {len(self.output_sizes)} parts")
+        return sum(self.output_sizes[:idx]), self.output_sizes[idx]
+
+    def weight_loader_v2(self, param: BasevLLMParameter, loaded_weight: torch.Tensor, loaded_shard_id=None) -> None:
+        """Copy one checkpoint tensor into `param`.  Without a shard id the tensor covers the whole layer: a fused
+        tensor is cut along the output dimension into the layer's logical parts (a per-tensor scale then belongs to all
+        of them and goes to entry 0, the maximum over the entries is taken after loading); with a shard id it is
+        one logical part."""
+        if loaded_shard_id is None:
+            if isinstance(param, PerTensorScaleParameter):
+                param.load_merged_column_weight(loaded_weight=loaded_weight, shard_id=0)
+            elif len(self.output_sizes) == 1 or param.output_dim is None:
+                param.load_column_parallel_weight(loaded_weight)
+            else:
+                for idx in range(len(self.output_sizes)):
+                    offset, size = self._part_offset_and_size(idx)
+                    if param.packed_dim is not None and param.packed_dim == param.output_dim:
+                        size, offset = param.adjust_shard_indexes_for_packing(size, offset)
+                    self.weight_loader_v2(param, loaded_weight.narrow(param.output_dim, offset, size), idx)
+            return
+        offset, size = self._part_offset_and_size(loaded_shard_id)
+        param.load_merged_column_weight(loaded_weight=loaded_weight, shard_id=loaded_shard_id, shard_offset=offset,
+                                        shard_size=size)
 
     def process_weights_after_loading(self) -> None:
         self.quant_method.process_weights_after_loading(self)

@@ -12,6 +12,7 @@ from typing import Any, Optional
 import torch
 
 from vllm_amd import _custom_ops as ops
+from vllm_amd.parameter import GroupQuantScaleParameter, PackedvLLMParameter
 from vllm_amd.scalar_type import scalar_types
 from .base_config import LinearMethodBase, QuantizationConfig, QuantizeMethodBase
 from .utils.marlin_utils import (apply_awq_marlin_linear, awq_to_marlin_zero_points, check_marlin_supported,
@@ -136,11 +137,17 @@ class AWQMarlinLinearMethod(LinearMethodBase):
                                      group_size=group_size)
         pf = self.quant_config.pack_factor
         num_groups = input_size_per_partition // group_size
-        P = lambda t: torch.nn.Parameter(t, requires_grad=False)   # noqa: E731
-        layer.register_parameter("qweight", P(torch.empty(input_size_per_partition, output_size_per_partition // pf,
-                                                          dtype=torch.int32)))
-        layer.register_parameter("qzeros", P(torch.empty(num_groups, output_size_per_partition // pf, dtype=torch.int32)))
-        layer.register_parameter("scales", P(torch.empty(num_groups, output_size_per_partition, dtype=params_dtype)))
+        loader = extra_weight_attrs.get("weight_loader")
+        # AutoAWQ checkpoint layout (awq_marlin.py:296-340): weights and zero points packed along the output dimension
+        layer.register_parameter("qweight", PackedvLLMParameter(
+            data=torch.empty(input_size_per_partition, output_size_per_partition // pf, dtype=torch.int32), input_dim=0,
+            output_dim=1, packed_dim=1, packed_factor=pf, weight_loader=loader))
+        layer.register_parameter("qzeros", PackedvLLMParameter(
+            data=torch.empty(num_groups, output_size_per_partition // pf, dtype=torch.int32), input_dim=0, output_dim=1,
+            packed_dim=1, packed_factor=pf, weight_loader=loader))
+        layer.register_parameter("scales", GroupQuantScaleParameter(
+            data=torch.empty(num_groups, output_size_per_partition, dtype=params_dtype), input_dim=0, output_dim=1,
+            weight_loader=loader))
         layer.input_size_per_partition = input_size_per_partition
         layer.output_size_per_partition = output_size_per_partition
         layer.num_groups = num_groups

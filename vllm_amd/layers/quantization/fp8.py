@@ -9,6 +9,7 @@ import torch
 from torch.nn import Parameter
 
 from vllm_amd import _custom_ops as ops
+from vllm_amd.parameter import ModelWeightParameter, PerTensorScaleParameter
 from .base_config import LinearMethodBase, QuantizationConfig, QuantizeMethodBase
 from .input_quant_fp8 import GroupShape
 from .utils.w8a8_utils import Fp8LinearOp
@@ -84,16 +85,20 @@ class Fp8LinearMethod(LinearMethodBase):
         layer.orig_dtype = params_dtype
         layer.weight_block_size = None
         weight_dtype = ops.FP8_DTYPE if self.quant_config.is_checkpoint_fp8_serialized else params_dtype
-        layer.register_parameter("weight", Parameter(torch.empty(output_size_per_partition, input_size_per_partition,
-                                                                  dtype=weight_dtype), requires_grad=False))
+        loader = extra_weight_attrs.get("weight_loader")
+        layer.register_parameter("weight", ModelWeightParameter(
+            data=torch.empty(output_size_per_partition, input_size_per_partition, dtype=weight_dtype), input_dim=1,
+            output_dim=0, weight_loader=loader))
         if self.quant_config.is_checkpoint_fp8_serialized:
-            scale = Parameter(torch.full((len(output_partition_sizes),), torch.finfo(torch.float32).min,
-                                         dtype=torch.float32), requires_grad=False)
-            layer.register_parameter("weight_scale", scale)
+            # one scale per logical matrix of a fused layer, initialised to the most negative float so that the maximum
+            # taken after loading ignores entries no checkpoint tensor filled (fp8.py:405-428)
+            def per_part():
+                return PerTensorScaleParameter(data=torch.full((len(output_partition_sizes),),
+                                                               torch.finfo(torch.float32).min, dtype=torch.float32),
+                                               weight_loader=loader)
+            layer.register_parameter("weight_scale", per_part())
             if self.act_q_static:
-                layer.register_parameter("input_scale", Parameter(torch.full((len(output_partition_sizes),),
-                                                                              torch.finfo(torch.float32).min,
-                                                                              dtype=torch.float32), requires_grad=False))
+                layer.register_parameter("input_scale", per_part())
             else:
                 layer.register_parameter("input_scale", None)
 

@@ -9,6 +9,8 @@ from typing import Any, Optional
 
 import torch
 
+from vllm_amd.parameter import (ChannelQuantScaleParameter, GroupQuantScaleParameter, PackedColumnParameter,
+                                PackedvLLMParameter, RowvLLMParameter)
 from vllm_amd.scalar_type import scalar_types
 from .base_config import LinearMethodBase, QuantizationConfig, QuantizeMethodBase
 from .kernels.mixed_precision import MPLinearLayerConfig, choose_mp_linear_kernel
@@ -140,14 +142,28 @@ class GPTQMarlinLinearMethod(LinearMethodBase):
             scales_and_zp_size = input_size_per_partition // group_size
 
         pf = self.quant_config.pack_factor
-        P = lambda t: torch.nn.Parameter(t, requires_grad=False)   # noqa: E731
-        layer.register_parameter("qweight", P(torch.empty(input_size_per_partition // pf, output_size_per_partition,
-                                                          dtype=torch.int32)))
-        layer.register_parameter("g_idx", P(torch.empty(input_size_per_partition, dtype=torch.int32)))
-        layer.register_parameter("scales", P(torch.empty(scales_and_zp_size, output_size_per_partition,
-                                                         dtype=params_dtype)))
-        layer.register_parameter("qzeros", P(torch.empty(scales_and_zp_size, output_size_per_partition // pf,
-                                                         dtype=torch.int32)))
+        loader = extra_weight_attrs.get("weight_loader")
+        # the checkpoint layout of gptq_marlin.py:380-440: qweight packed along the input dimension, qzeros along the
+        # output dimension, scales / zero points one row per group (channelwise: one row)
+        layer.register_parameter("qweight", PackedvLLMParameter(
+            data=torch.empty(input_size_per_partition // pf, output_size_per_partition, dtype=torch.int32), input_dim=0,
+            output_dim=1, packed_dim=0, packed_factor=pf, weight_loader=loader))
+        layer.register_parameter("g_idx", RowvLLMParameter(
+            data=torch.empty(input_size_per_partition, dtype=torch.int32), input_dim=0, weight_loader=loader))
+        scale_cls = ChannelQuantScaleParameter if scales_and_zp_size == 1 and self.quant_config.group_size == -1 \
+            else GroupQuantScaleParameter
+        dims = dict(output_dim=1) if scale_cls is ChannelQuantScaleParameter else dict(output_dim=1, input_dim=0)
+        layer.register_parameter("scales", scale_cls(
+            data=torch.empty(scales_and_zp_size, output_size_per_partition, dtype=params_dtype), weight_loader=loader,
+            **dims))
+        if scale_cls is ChannelQuantScaleParameter:
+            layer.register_parameter("qzeros", PackedColumnParameter(
+                data=torch.empty(scales_and_zp_size, output_size_per_partition // pf, dtype=torch.int32), output_dim=1,
+                packed_dim=1, packed_factor=pf, weight_loader=loader))
+        else:
+            layer.register_parameter("qzeros", PackedvLLMParameter(
+                data=torch.empty(scales_and_zp_size, output_size_per_partition // pf, dtype=torch.int32), input_dim=0,
+                output_dim=1, packed_dim=1, packed_factor=pf, weight_loader=loader))
         self.kernel = kernel_type(mp_linear_kernel_config, w_q_param_name="qweight", w_s_param_name="scales",
                                   w_zp_param_name="qzeros", w_gidx_param_name="g_idx")
 
