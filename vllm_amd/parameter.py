@@ -112,7 +112,7 @@ class BasevLLMParameter(torch.nn.Parameter):
         return self._marlin_tile_size
 
     def adjust_shard_indexes_for_packing(self, shard_size: int, shard_offset: int) -> tuple[int, int]:
-        """Sizes in logical elements -> sizes in stored words (parameter.py:608-627)."""
+        """Sizes in logical elements -> sizes in stored words (parameter.py:616-650)."""
         if self._packed_factor is None:
             return shard_size, shard_offset
         size, offset = shard_size // self._packed_factor, shard_offset // self._packed_factor
