@@ -340,7 +340,7 @@ def test_silu_and_mul_quant(device, tokens, hidden, dtype):
         assert torch.equal(out3.reshape(tokens, -1).view(torch.uint8), out.view(torch.uint8))
 
 
-@pytest.mark.parametrize("cfg", [1, 3, 4, 7, 13, 23, 14, 24, 17])
+@pytest.mark.parametrize("cfg", [1, 8, 3, 4, 7, 13, 23, 14, 24, 17])
 def test_scaled_mm_every_tile_shape_exact(device, cfg):
     """Every shape of the multi-stage tile kernel, forced through the tuning export (the automatic choice only reaches
     some of them at any one problem size), including the ones that take two k-slices per step: small-integer operands

@@ -55,11 +55,33 @@ constexpr int F8_PITCH = 144;    // LDS row pitch in bytes
 template <bool BF16_OUT, int WMB, int WNB>
 __device__ inline void tile_epilogue(const Fp8MMParams& p, v16f (&acc)[WMB][WNB], int m0, int n0, int wm, int wn, int lane) {
   using T = F16Traits<BF16_OUT>;
+  // Every scale and bias value this lane needs is requested before the first store: a load that follows a store to
+  // memory it might alias cannot be moved above it, and the epilogue would pay one memory latency per 8-byte store.
+  float sam[WMB];
+#pragma unroll
+  for (int i = 0; i < WMB; ++i) {
+    const int m = m0 + wm * 32 * WMB + i * 32 + (lane & 31);
+    sam[i] = m < p.M ? p.sa[p.sa_per_row ? m : 0] : 0.f;
+  }
+  v4f sbv[WNB][4];
+  v2u bv[WNB][4];
+#pragma unroll
+  for (int j = 0; j < WNB; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int n = n0 + wn * 32 * WNB + j * 32 + 8 * q + 4 * (lane >> 5);
+      sbv[j][q] = v4f{0.f, 0.f, 0.f, 0.f};
+      bv[j][q] = v2u{0u, 0u};
+      if (n < p.N) {
+        if (p.sb_per_col) sbv[j][q] = *reinterpret_cast<const v4f*>(p.sb + n);
+        else sbv[j][q] = v4f{p.sb[0], p.sb[0], p.sb[0], p.sb[0]};
+        if (p.bias) bv[j][q] = *reinterpret_cast<const v2u*>(p.bias + n);
+      }
+    }
 #pragma unroll
   for (int i = 0; i < WMB; ++i) {
     const int m = m0 + wm * 32 * WMB + i * 32 + (lane & 31);
     if (m >= p.M) continue;
-    const float sam = p.sa[p.sa_per_row ? m : 0];
     uint16_t* orow = p.out + (int64_t)m * p.ldc;
 #pragma unroll
     for (int j = 0; j < WNB; ++j) {
@@ -67,22 +89,14 @@ __device__ inline void tile_epilogue(const Fp8MMParams& p, v16f (&acc)[WMB][WNB]
       for (int q = 0; q < 4; ++q) {
         const int n = n0 + wn * 32 * WNB + j * 32 + 8 * q + 4 * (lane >> 5);
         if (n >= p.N) continue;
-        float sb4[4];
-        if (p.sb_per_col) {
-          const v4f t = *reinterpret_cast<const v4f*>(p.sb + n);
-          sb4[0] = t.x; sb4[1] = t.y; sb4[2] = t.z; sb4[3] = t.w;
-        } else {
-          sb4[0] = sb4[1] = sb4[2] = sb4[3] = p.sb[0];
-        }
         float o[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) o[r] = sam * (sb4[r] * acc[i][j][4 * q + r]);
+        for (int r = 0; r < 4; ++r) o[r] = sam[i] * (sbv[j][q][r] * acc[i][j][4 * q + r]);
         if (p.bias) {
-          const v2u bb = *reinterpret_cast<const v2u*>(p.bias + n);
-          o[0] += T::to_float((uint16_t)(bb.x & 0xffffu));
-          o[1] += T::to_float((uint16_t)(bb.x >> 16));
-          o[2] += T::to_float((uint16_t)(bb.y & 0xffffu));
-          o[3] += T::to_float((uint16_t)(bb.y >> 16));
+          o[0] += T::to_float((uint16_t)(bv[j][q].x & 0xffffu));
+          o[1] += T::to_float((uint16_t)(bv[j][q].x >> 16));
+          o[2] += T::to_float((uint16_t)(bv[j][q].y & 0xffffu));
+          o[3] += T::to_float((uint16_t)(bv[j][q].y >> 16));
         }
         v2u ov;
         ov.x = (uint32_t)T::from_float(o[0]) | ((uint32_t)T::from_float(o[1]) << 16);
@@ -90,6 +104,74 @@ __device__ inline void tile_epilogue(const Fp8MMParams& p, v16f (&acc)[WMB][WNB]
         *reinterpret_cast<v2u*>(orow + n) = ov;
       }
     }
+  }
+}
+
+// Epilogue of the multi-stage kernel: same arithmetic as tile_epilogue, but the 16-bit results cross a wavefront-private
+// piece of LDS (32 rows of WNB * 64 + 16 bytes) so that they leave as 16-byte stores, 8 or 16 lanes to a row.  With the
+// direct 8-byte stores every instruction touches 32 rows with 16 bytes each, and the write requests of a whole device
+// finishing its tiles at the same time (one 16-byte piece each) took 10-17 us per tile.
+// Requires: every wavefront of the workgroup has finished reading the operand ring, out 16-byte aligned.
+template <bool BF16_OUT, int WMB, int WNB>
+__device__ inline void tile_epilogue_lds(const Fp8MMParams& p, v16f (&acc)[WMB][WNB], int m0, int n0, int wm, int wn, int lane,
+                                         uint8_t* wave_lds) {
+  using T = F16Traits<BF16_OUT>;
+  constexpr int PITCH = WNB * 64 + 16;
+  constexpr int CPR = WNB * 4;                 // 16-byte chunks per row
+  float sam[WMB];
+#pragma unroll
+  for (int i = 0; i < WMB; ++i) {
+    const int m = m0 + wm * 32 * WMB + i * 32 + (lane & 31);
+    sam[i] = m < p.M ? p.sa[p.sa_per_row ? m : 0] : 0.f;
+  }
+  v4f sbv[WNB][4];
+  v2u bv[WNB][4];
+#pragma unroll
+  for (int j = 0; j < WNB; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int n = n0 + wn * 32 * WNB + j * 32 + 8 * q + 4 * (lane >> 5);
+      sbv[j][q] = v4f{0.f, 0.f, 0.f, 0.f};
+      bv[j][q] = v2u{0u, 0u};
+      if (n < p.N) {
+        if (p.sb_per_col) sbv[j][q] = *reinterpret_cast<const v4f*>(p.sb + n);
+        else sbv[j][q] = v4f{p.sb[0], p.sb[0], p.sb[0], p.sb[0]};
+        if (p.bias) bv[j][q] = *reinterpret_cast<const v2u*>(p.bias + n);
+      }
+    }
+#pragma unroll
+  for (int i = 0; i < WMB; ++i) {
+#pragma unroll
+    for (int j = 0; j < WNB; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float o[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = sam[i] * (sbv[j][q][r] * acc[i][j][4 * q + r]);
+        if (p.bias) {
+          o[0] += T::to_float((uint16_t)(bv[j][q].x & 0xffffu));
+          o[1] += T::to_float((uint16_t)(bv[j][q].x >> 16));
+          o[2] += T::to_float((uint16_t)(bv[j][q].y & 0xffffu));
+          o[3] += T::to_float((uint16_t)(bv[j][q].y >> 16));
+        }
+        v2u ov;
+        ov.x = (uint32_t)T::from_float(o[0]) | ((uint32_t)T::from_float(o[1]) << 16);
+        ov.y = (uint32_t)T::from_float(o[2]) | ((uint32_t)T::from_float(o[3]) << 16);
+        *reinterpret_cast<v2u*>(wave_lds + (lane & 31) * PITCH + (j * 32 + 8 * q + 4 * (lane >> 5)) * 2) = ov;
+      }
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_wave_barrier();           // lanes exchange data through LDS; its operations run in program order
+#pragma unroll
+    for (int it = 0; it < 32 * CPR / 64; ++it) {
+      const int idx = it * 64 + lane;
+      const int row = idx / CPR, ch = idx % CPR;
+      const v4u v = *reinterpret_cast<const v4u*>(wave_lds + row * PITCH + ch * 16);
+      const int m = m0 + wm * 32 * WMB + i * 32 + row;
+      const int n = n0 + wn * 32 * WNB + ch * 8;
+      if (m < p.M && n < p.N) *reinterpret_cast<v4u*>(p.out + (int64_t)m * p.ldc + n) = v;
+    }
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
   }
 }
 
@@ -315,7 +397,7 @@ __global__ __launch_bounds__(256) void fp8_mm_tile2_kernel(const Fp8MMParams p) 
 //  * WAVES_M x WAVES_N wavefronts; tiles are handed out in bands of 8 tile rows inside each XCD's contiguous range so
 //    that the tiles resident on one XCD share activation rows and weight columns in its L2.
 // Requires K % 64 == 0 (a partial last step would read the neighbouring row instead of zeros) and M*lda, N*ldb < 2^32.
-template <bool BF16_OUT, int BM, int BN, int WAVES_M, int WAVES_N, int NST, int KS = 1>
+template <bool BF16_OUT, int BM, int BN, int WAVES_M, int WAVES_N, int NST, int KS = 1, int PP = 0>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(const Fp8MMParams p) {
   // A step is KS k-slices of 64 bytes (KS = 2 for the small tiles, whose steps are otherwise shorter than the barrier
   // and the LDS round trip that every step pays); a stage holds the KS slices of one step, each as [A tile | B tile].
@@ -434,7 +516,66 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
   const int split = blockIdx.y;
   const int s_lo = (int)(((int64_t)all_steps * split) / p.SK), s_hi = (int)(((int64_t)all_steps * (split + 1)) / p.SK);
   const int steps = s_hi - s_lo;
-  if (steps >= NST) {
+  if (PP != 0 && steps >= NST) {
+    // Alternating phases: the two wavefronts that share a SIMD run half a step apart, so that one reads its fragments
+    // (and requests tiles) while the other one issues its MFMAs.  A step is [requests, fragment reads, wait] barrier
+    // [MFMAs] barrier; the late half of the workgroup passes one extra barrier first and skips its last one, so every
+    // wavefront passes the same number.  The tile of step s+1 must have landed at the END OF THE READ PHASE of step s
+    // (the early half reads it two barriers later, the late half three).
+    auto read_frags = [&](int stage, v8i (&af)[KS][WMB], v8i (&bf)[KS][WNB]) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const uint8_t* base = lds8 + (size_t)stage * STAGE + ks * SLICE;
+#pragma unroll
+        for (int j = 0; j < WNB; ++j) {
+          const v4i lo = *reinterpret_cast<const v4i*>(base + brow + j * 2048 + coff[0]);
+          const v4i hi = *reinterpret_cast<const v4i*>(base + brow + j * 2048 + coff[1]);
+          bf[ks][j] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        }
+#pragma unroll
+        for (int i = 0; i < WMB; ++i) {
+          const v4i lo = *reinterpret_cast<const v4i*>(base + arow + i * 2048 + coff[0]);
+          const v4i hi = *reinterpret_cast<const v4i*>(base + arow + i * 2048 + coff[1]);
+          af[ks][i] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        }
+      }
+    };
+    auto mfmas = [&](v8i (&af)[KS][WMB], v8i (&bf)[KS][WNB]) {
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int i = 0; i < WMB; ++i)
+#pragma unroll
+          for (int j = 0; j < WNB; ++j) acc[i][j] = mfma_fp8_32(bf[ks][j], af[ks][i], acc[i][j]);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    auto bare_barrier = [&]() { asm volatile("s_barrier" ::: "memory"); };
+    const bool late = wave >= NW / 2;     // wavefronts w and w + 4 share a SIMD (the other pairing measured 10-25 % slower)
+    v8i af[KS][WMB], bf[KS][WNB];
+#pragma unroll
+    for (int s0 = 0; s0 < NST - 1; ++s0) issue_loads(s_lo + s0, s0);
+    sync_step(WAIT_STEADY{});           // tile 0 landed
+    if (late) bare_barrier();
+    int cur = 0, dst = NST - 1;
+    int step = 0;
+    for (; step + NST - 1 < steps; ++step) {
+      issue_loads(s_lo + step + NST - 1, dst);
+      read_frags(cur, af, bf);
+      sync_step(WAIT_STEADY{});
+      mfmas(af, bf);
+      bare_barrier();
+      cur = cur + 1 == NST ? 0 : cur + 1;
+      dst = dst + 1 == NST ? 0 : dst + 1;
+    }
+    for (; step < steps; ++step) {      // nothing left to request: drain
+      read_frags(cur, af, bf);
+      sync_step(WAIT_NONE{});
+      mfmas(af, bf);
+      if (!(late && step == steps - 1)) bare_barrier();
+      cur = cur + 1 == NST ? 0 : cur + 1;
+    }
+  } else if (steps >= NST) {
 #pragma unroll
     for (int s0 = 0; s0 < NST - 1; ++s0) issue_loads(s_lo + s0, s0);
     sync_step(WAIT_STEADY{});           // tile 0 landed
@@ -505,7 +646,11 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
     if (lane == 0) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
-  tile_epilogue<BF16_OUT, WMB, WNB>(p, acc, m0, n0, wm, wn, lane);
+  static_assert(NST * STAGE >= NW * 32 * (WNB * 64 + 16), "operand ring too small for the epilogue staging");
+  if (((uintptr_t)p.out & 15) == 0)
+    tile_epilogue_lds<BF16_OUT, WMB, WNB>(p, acc, m0, n0, wm, wn, lane, lds8 + wave * (32 * (WNB * 64 + 16)));
+  else
+    tile_epilogue<BF16_OUT, WMB, WNB>(p, acc, m0, n0, wm, wn, lane);
 }
 
 // ----------------------------------------------------------------------------- stream kernel (M <= 32)
@@ -650,10 +795,10 @@ static int launch_tile2(const Fp8MMParams& p, hipStream_t s) {
   return VAQ_OK;
 }
 
-template <bool BF16_OUT, int BM, int BN, int WAVES_M, int WAVES_N, int NST, int KS = 1>
+template <bool BF16_OUT, int BM, int BN, int WAVES_M, int WAVES_N, int NST, int KS = 1, int PP = 0>
 static int launch_tile3(const Fp8MMParams& p, hipStream_t s) {
   const size_t lds = (size_t)NST * KS * (BM + BN) * 64;
-  auto kern = fp8_mm_tile3_kernel<BF16_OUT, BM, BN, WAVES_M, WAVES_N, NST, KS>;
+  auto kern = fp8_mm_tile3_kernel<BF16_OUT, BM, BN, WAVES_M, WAVES_N, NST, KS, PP>;
   static bool attr_done = false;
   if (!attr_done) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
@@ -728,7 +873,8 @@ static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t c
       pl.sk = 1;
     p.SK = pl.sk;
     switch (pl.cfg) {
-      case 1: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 5>(p, s);
+      case 1: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 5, 1, 1>(p, s);   // alternating phases (see the kernel)
+      case 8: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 5>(p, s);
       case 2: return launch_tile3<BF16_OUT, 256, 256, 2, 2, 5>(p, s);
       case 3: return launch_tile3<BF16_OUT, 128, 128, 2, 2, 5>(p, s);
       case 4: return launch_tile3<BF16_OUT, 64, 128, 2, 2, 5>(p, s);
