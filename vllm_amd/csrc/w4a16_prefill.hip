@@ -11,6 +11,7 @@ template <bool BF16, bool HAS_ZP>
 static int dispatch_tile(const PrefillParams& p, int tile, hipStream_t s) {
   switch (tile) {
     case 10: return launch_prefill2<BF16, 256, 256, 2, 4, HAS_ZP, 1>(p, s);   // 8 wavefronts, 128 x 64 each
+    case 20: return launch_prefill2<BF16, 256, 256, 2, 4, HAS_ZP, 1, false, true>(p, s);   // the same, alternating phases
     case 11: return launch_prefill2<BF16, 256, 256, 2, 2, HAS_ZP, 1>(p, s);   // 4 wavefronts, 128 x 128 each
     case 12: return launch_prefill2<BF16, 128, 128, 2, 2, HAS_ZP, 1>(p, s);   // 4 wavefronts, 64 x 64 each
     case 13: return launch_prefill2<BF16, 128, 256, 2, 4, HAS_ZP, 1>(p, s);   // 8 wavefronts, 64 x 64 each
@@ -58,7 +59,7 @@ static PrefillPlan plan_prefill(int M, int N, int K, bool direct_ok) {
   PrefillPlan pl;
   pl.tile = pick_tile(M, N, direct_ok);
   switch (pl.tile) {
-    case 10: pl.bm = 256; pl.bn = 256; pl.nw = 8; break;
+    case 10: case 20: pl.bm = 256; pl.bn = 256; pl.nw = 8; break;
     case 11: pl.bm = 256; pl.bn = 256; pl.nw = 4; break;
     case 12: pl.bm = 128; pl.bn = 128; pl.nw = 4; break;
     case 13: pl.bm = 128; pl.bn = 256; pl.nw = 8; break;

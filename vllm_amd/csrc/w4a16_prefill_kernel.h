@@ -51,65 +51,75 @@ static __device__ inline uint32_t pack2(float lo, float hi) {
   }
 }
 
-// One native weight word (8 codes of 8 consecutive k) -> 8 scaled 16-bit weights in k order.
+// float(byte B of x).  One instruction each; written as assembly because the compiler turns `(float)((x >> 8B) & 0xff)`
+// of a nibble-masked word into a bit-field extract plus a conversion (two instructions per weight, and the
+// dequantisation competes with the MFMAs for issue slots).  The results feed ordinary VALU instructions only.
+template <int B>
+static __device__ inline float cvt_ubyte(uint32_t x) {
+  float f;
+  if constexpr (B == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(x));
+  else if constexpr (B == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(x));
+  else if constexpr (B == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(x));
+  else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(x));
+  return f;
+}
+
+// Four bytes t (elements 0,4,1,5) and u (elements 2,6,3,7) of 8 consecutive k -> 8 scaled 16-bit weights in k order.
 template <bool BF16>
-static __device__ inline v4u dequant_scaled(uint32_t w, float s, float neg_zs) {
-  const uint32_t t = w & 0x0f0f0f0fu;          // nibble positions 0,2,4,6 -> elements 0,4,1,5
-  const uint32_t u = (w >> 4) & 0x0f0f0f0fu;   // nibble positions 1,3,5,7 -> elements 2,6,3,7
-  const float e0 = fmaf((float)(t & 0xffu), s, neg_zs);
-  const float e4 = fmaf((float)((t >> 8) & 0xffu), s, neg_zs);
-  const float e1 = fmaf((float)((t >> 16) & 0xffu), s, neg_zs);
-  const float e5 = fmaf((float)(t >> 24), s, neg_zs);
-  const float e2 = fmaf((float)(u & 0xffu), s, neg_zs);
-  const float e6 = fmaf((float)((u >> 8) & 0xffu), s, neg_zs);
-  const float e3 = fmaf((float)((u >> 16) & 0xffu), s, neg_zs);
-  const float e7 = fmaf((float)(u >> 24), s, neg_zs);
+static __device__ inline v4u scale_bytes(uint32_t t, uint32_t u, float s, float neg_zs) {
+  const float e0 = fmaf(cvt_ubyte<0>(t), s, neg_zs);
+  const float e4 = fmaf(cvt_ubyte<1>(t), s, neg_zs);
+  const float e1 = fmaf(cvt_ubyte<2>(t), s, neg_zs);
+  const float e5 = fmaf(cvt_ubyte<3>(t), s, neg_zs);
+  const float e2 = fmaf(cvt_ubyte<0>(u), s, neg_zs);
+  const float e6 = fmaf(cvt_ubyte<1>(u), s, neg_zs);
+  const float e3 = fmaf(cvt_ubyte<2>(u), s, neg_zs);
+  const float e7 = fmaf(cvt_ubyte<3>(u), s, neg_zs);
   v4u r;
   r.x = pack2<BF16>(e0, e1);
   r.y = pack2<BF16>(e2, e3);
   r.z = pack2<BF16>(e4, e5);
   r.w = pack2<BF16>(e6, e7);
   return r;
+}
+
+// One native weight word (8 codes of 8 consecutive k) -> 8 scaled 16-bit weights in k order.
+template <bool BF16>
+static __device__ inline v4u dequant_scaled(uint32_t w, float s, float neg_zs) {
+  // nibble positions 0,2,4,6 -> elements 0,4,1,5; nibble positions 1,3,5,7 -> elements 2,6,3,7
+  return scale_bytes<BF16>(w & 0x0f0f0f0fu, (w >> 4) & 0x0f0f0f0fu, s, neg_zs);
 }
 
 // 8-bit codes stored as two 4-bit planes: the words of the high and of the low nibbles of the same 8 codes.
 template <bool BF16>
 static __device__ inline v4u dequant_scaled8(uint32_t hi, uint32_t lo, float s, float neg_zs) {
-  const uint32_t t = ((hi & 0x0f0f0f0fu) << 4) | (lo & 0x0f0f0f0fu);          // bytes: elements 0,4,1,5
-  const uint32_t u = (hi & 0xf0f0f0f0u) | ((lo >> 4) & 0x0f0f0f0fu);           // bytes: elements 2,6,3,7
-  const float e0 = fmaf((float)(t & 0xffu), s, neg_zs);
-  const float e4 = fmaf((float)((t >> 8) & 0xffu), s, neg_zs);
-  const float e1 = fmaf((float)((t >> 16) & 0xffu), s, neg_zs);
-  const float e5 = fmaf((float)(t >> 24), s, neg_zs);
-  const float e2 = fmaf((float)(u & 0xffu), s, neg_zs);
-  const float e6 = fmaf((float)((u >> 8) & 0xffu), s, neg_zs);
-  const float e3 = fmaf((float)((u >> 16) & 0xffu), s, neg_zs);
-  const float e7 = fmaf((float)(u >> 24), s, neg_zs);
-  v4u r;
-  r.x = pack2<BF16>(e0, e1);
-  r.y = pack2<BF16>(e2, e3);
-  r.z = pack2<BF16>(e4, e5);
-  r.w = pack2<BF16>(e6, e7);
-  return r;
+  return scale_bytes<BF16>(((hi & 0x0f0f0f0fu) << 4) | (lo & 0x0f0f0f0fu), (hi & 0xf0f0f0f0u) | ((lo >> 4) & 0x0f0f0f0fu), s, neg_zs);
+}
+
+// Register t (0..3) of scale_bytes' result: elements 2t and 2t+1.
+template <bool BF16>
+static __device__ inline uint32_t scale_bytes_part(uint32_t tb, uint32_t ub, float s, float neg_zs, int t) {
+  const uint32_t x = (t & 1) ? ub : tb;
+  float l, h;
+  if (t >> 1) {
+    l = cvt_ubyte<1>(x);
+    h = cvt_ubyte<3>(x);
+  } else {
+    l = cvt_ubyte<0>(x);
+    h = cvt_ubyte<2>(x);
+  }
+  return pack2<BF16>(fmaf(l, s, neg_zs), fmaf(h, s, neg_zs));
 }
 
 template <bool BF16>
 static __device__ inline uint32_t dequant_part8(uint32_t hi, uint32_t lo, float s, float neg_zs, int t) {
-  const uint32_t x = (t & 1) ? ((hi & 0xf0f0f0f0u) | ((lo >> 4) & 0x0f0f0f0fu)) : (((hi & 0x0f0f0f0fu) << 4) | (lo & 0x0f0f0f0fu));
-  const int sh = (t >> 1) * 8;
-  const float l = fmaf((float)((x >> sh) & 0xffu), s, neg_zs);
-  const float h = fmaf((float)((x >> (sh + 16)) & 0xffu), s, neg_zs);
-  return pack2<BF16>(l, h);
+  return scale_bytes_part<BF16>(((hi & 0x0f0f0f0fu) << 4) | (lo & 0x0f0f0f0fu), (hi & 0xf0f0f0f0u) | ((lo >> 4) & 0x0f0f0f0fu), s, neg_zs, t);
 }
 
 // Quarter t of dequant_scaled: register t of its result (elements 2t and 2t+1).
 template <bool BF16>
 static __device__ inline uint32_t dequant_part(uint32_t w, float s, float neg_zs, int t) {
-  const uint32_t x = ((t & 1) ? (w >> 4) : w) & 0x0f0f0f0fu;
-  const int sh = (t >> 1) * 8;
-  const float lo = fmaf((float)((x >> sh) & 0xffu), s, neg_zs);
-  const float hi = fmaf((float)((x >> (sh + 16)) & 0xffu), s, neg_zs);
-  return pack2<BF16>(lo, hi);
+  return scale_bytes_part<BF16>(w & 0x0f0f0f0fu, (w >> 4) & 0x0f0f0f0fu, s, neg_zs, t);
 }
 
 // value of the sub-group that word j (0..3) of a tile belongs to
@@ -291,9 +301,11 @@ __global__ __launch_bounds__(256) void w4a16_prefill_kernel(const PrefillParams 
 //  * the MFMAs take the weight fragment as A operand, so four consecutive accumulator registers are four consecutive
 //    output columns of one row: packed 8-byte stores in the epilogue;
 //  * weight words of group g+1 are requested one K step before they are needed (two register sets, by group parity).
-template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP, int SUBG, bool W8 = false>
+template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP, int SUBG, bool W8 = false, bool PP = false>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(const PrefillParams p) {
   using T = F16Traits<BF16>;
+  static_assert(!PP || (!W8 && SUBG == 1 && (BM / (8 * WAVES_M * WAVES_N)) % 2 == 0 && WAVES_M * WAVES_N == 8),
+                "alternating phases: 8 wavefronts, groups of 128 rows, an even number of DMA instructions per step");
   static_assert(!W8 || (SUBG == 1 && !HAS_ZP), "8-bit codes: symmetric, one group per tile");
   constexpr int TPG = W8 ? 2 : 1;                 // 1 KiB weight blocks per tile (8-bit: high-nibble plane, low-nibble plane)
   constexpr int NW = WAVES_M * WAVES_N;
@@ -357,8 +369,12 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
   // scales, and for one group per tile -(zero * scale); with several groups per tile the zero points stay packed as one
   // byte per group (registers are short here) and the product is formed where it is used
   using ZT = std::conditional_t<SUBG == 1, float, uint32_t>;
-  float scur[W_LD][SUBG], snxt[W_LD][SUBG];
-  ZT zcur[W_LD], znxt[W_LD];
+  float scur[W_LD][SUBG];
+  ZT zcur[W_LD];
+  // the next group's scales and zero-point words as loaded; converted in advance_w, a K step after the request (a
+  // conversion next to the load makes the wavefront wait for the memory latency in the middle of the step)
+  uint16_t snxt_raw[W_LD][SUBG];
+  uint32_t znxt_raw[W_LD][SUBG];
   const int o = lane >> 4, r = lane & 15;
   auto load_w = [&](int g) {
 #pragma unroll
@@ -368,19 +384,12 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
       wnxt[i] = p.b[(((int64_t)nt * p.G + g) * TPG) * 64 + lane];
       if constexpr (W8) wnxt_lo[i] = p.b[(((int64_t)nt * p.G + g) * TPG + 1) * 64 + lane];
       const int n = nt * 16 + r;
-      if constexpr (SUBG > 1) znxt[i] = 0u;
 #pragma unroll
       for (int sj = 0; sj < SUBG; ++sj) {
         const int64_t row = (int64_t)g * SUBG + sj;
-        const float sv = T::to_float(p.scales[row * p.s_stride + n]);
-        uint32_t zc = W8 ? 128u : 8u;
-        if constexpr (HAS_ZP) {
-          const uint32_t zw = p.zeros[row * p.z_stride + (n >> 3)];
-          zc = (zw >> ((n & 7) * 4)) & 0xFu;
-        }
-        snxt[i][sj] = sv;
-        if constexpr (SUBG == 1) znxt[i] = -((float)zc * sv);   // exact: <= 4 + 11 significant bits
-        else if constexpr (HAS_ZP) znxt[i] |= zc << (8 * sj);
+        snxt_raw[i][sj] = p.scales[row * p.s_stride + n];
+        if constexpr (HAS_ZP) znxt_raw[i][sj] = p.zeros[row * p.z_stride + (n >> 3)];
+        else znxt_raw[i][sj] = 0u;
       }
     }
   };
@@ -389,9 +398,16 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
     for (int i = 0; i < W_LD; ++i) {
       wcur[i] = wnxt[i];
       if constexpr (W8) wcur_lo[i] = wnxt_lo[i];
-      zcur[i] = znxt[i];
+      if constexpr (SUBG > 1) zcur[i] = 0u;
 #pragma unroll
-      for (int sj = 0; sj < SUBG; ++sj) scur[i][sj] = snxt[i][sj];
+      for (int sj = 0; sj < SUBG; ++sj) {
+        const float sv = T::to_float(snxt_raw[i][sj]);
+        uint32_t zc = W8 ? 128u : 8u;
+        if constexpr (HAS_ZP) zc = (znxt_raw[i][sj] >> ((r & 7) * 4)) & 0xFu;    // column n = 16 * tile + r
+        scur[i][sj] = sv;
+        if constexpr (SUBG == 1) zcur[i] = -((float)zc * sv);   // exact: <= 4 + 11 significant bits
+        else if constexpr (HAS_ZP) zcur[i] |= zc << (8 * sj);
+      }
     }
   };
   // scale and -(zero * scale) for word j (0..3) of weight load i
@@ -552,6 +568,107 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
   auto sync_step = [&](auto n_c) {
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(decltype(n_c)::value) : "memory");
   };
+  if constexpr (PP) {
+    // Alternating phases.  A K step is two half steps of two MFMA k-slices; a half step is a READ phase (this
+    // wavefront's fragments of the two slices, its share of the DMA requests and of the dequantisation for the next
+    // step) and an MFMA phase (16 MFMAs), each ended by a workgroup barrier.  The wavefronts w and w + 4 share a SIMD;
+    // the second four pass one extra barrier first (and skip their last one), so on every SIMD one wavefront is in its
+    // READ phase while the other one keeps the matrix core busy.  Hazards, with the late half one phase behind: a
+    // weight stage written during step s is first read two barriers after its last write; the activation stage
+    // requested during step s was last read one barrier before the first request; the tile of step s+1 has landed at
+    // the end of the second READ phase of step s of every wavefront, at least one barrier before anyone reads it.
+    const bool late = wave >= NW / 2;
+    v4u af[2][WMB], bf[2][WNB];
+    auto read_phase = [&](int a_cur, int w_cur, auto stage_c, auto dma_c, int a_dst, int a_step, int half, auto h_c) {
+      constexpr bool stage_on = decltype(stage_c)::value;
+      constexpr bool dma_on = decltype(dma_c)::value;
+      constexpr int h = decltype(h_c)::value;
+      const uint8_t* base_a = lds8 + (size_t)a_cur * A_ST;
+      const uint8_t* base_b = lds8 + W_BASE + (size_t)w_cur * W_ST;
+      uint8_t* Bn = lds8 + W_BASE + (size_t)(w_cur ^ 1) * W_ST;
+      if constexpr (dma_on) {
+#pragma unroll
+        for (int i = h * (A_LD / 2); i < (h + 1) * (A_LD / 2); ++i) issue_a_one(a_step, a_dst, i);
+      }
+#pragma unroll
+      for (int k2 = 0; k2 < 2; ++k2) {
+#pragma unroll
+        for (int j = 0; j < WNB; ++j) bf[k2][j] = *reinterpret_cast<const v4u*>(base_b + brow + j * 4096 + coff[2 * h + k2]);
+#pragma unroll
+        for (int i = 0; i < WMB; ++i) af[k2][i] = *reinterpret_cast<const v4u*>(base_a + arow + i * 4096 + coff[2 * h + k2]);
+      }
+      __builtin_amdgcn_sched_barrier(0);        // the reads go out first; the dequantisation fills their latency
+      if constexpr (stage_on) {
+#pragma unroll
+        for (int pc = h * W_LD; pc < (h + 1) * W_LD; ++pc) {
+          const int i = pc >> 1, which = pc & 1;
+          const uint32_t wsel = half ? (which ? wcur[i].w : wcur[i].z) : (which ? wcur[i].y : wcur[i].x);
+          float sv, zv;
+          sub_vals(i, half * 2 + which, sv, zv);
+          const int row = (i * NW + wave) * 16 + r;
+          const int c0 = (row & 1) * 8 + o + which * 4, sw = (row >> 1) & 15;
+          *reinterpret_cast<v4u*>(Bn + (row >> 1) * 256 + ((c0 ^ sw) * 16)) = dequant_scaled<BF16>(wsel, sv, zv);
+        }
+      }
+    };
+    auto mfma_phase = [&]() {
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int k2 = 0; k2 < 2; ++k2)
+#pragma unroll
+        for (int i = 0; i < WMB; ++i)
+#pragma unroll
+          for (int j = 0; j < WNB; ++j) acc[i][j] = T::mfma32(bf[k2][j], af[k2][i], acc[i][j]);   // rows = n, columns = m
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    auto bare_barrier = [&]() { asm volatile("s_barrier" ::: "memory"); };
+    using H0 = std::integral_constant<int, 0>;
+    using H1 = std::integral_constant<int, 1>;
+    using LGKM_ONLY = std::integral_constant<int, 63>;     // no vector-memory wait in the first half of a step
+    if (late) bare_barrier();
+    for (int g = g_lo; g + 1 < g_hi; ++g) {
+      // even step 2g: dequantise (g, half 1) for step 2g+1; request the tile of step 2g+2 and the words of group g+1
+      load_w(g + 1);
+      read_phase(a_cur, 0, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 2, 1, H0{});
+      sync_step(LGKM_ONLY{});
+      mfma_phase();
+      bare_barrier();
+      read_phase(a_cur, 0, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 2, 1, H1{});
+      sync_step(std::integral_constant<int, A_LD + KW>{});
+      mfma_phase();
+      bare_barrier();
+      a_cur = nxt(a_cur);
+      // odd step 2g+1: dequantise (g+1, half 0) for step 2g+2; request the tile of step 2g+3
+      advance_w();
+      read_phase(a_cur, 1, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 3, 0, H0{});
+      sync_step(LGKM_ONLY{});
+      mfma_phase();
+      bare_barrier();
+      read_phase(a_cur, 1, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 3, 0, H1{});
+      sync_step(std::integral_constant<int, A_LD>{});
+      mfma_phase();
+      bare_barrier();
+      a_cur = nxt(a_cur);
+    }
+    // last group: its second half is still dequantised, nothing is requested any more
+    read_phase(a_cur, 0, TT{}, FF{}, 0, 0, 1, H0{});
+    sync_step(LGKM_ONLY{});
+    mfma_phase();
+    bare_barrier();
+    read_phase(a_cur, 0, TT{}, FF{}, 0, 0, 1, H1{});
+    sync_step(std::integral_constant<int, 0>{});
+    mfma_phase();
+    bare_barrier();
+    a_cur = nxt(a_cur);
+    read_phase(a_cur, 1, FF{}, FF{}, 0, 0, 0, H0{});
+    sync_step(LGKM_ONLY{});
+    mfma_phase();
+    bare_barrier();
+    read_phase(a_cur, 1, FF{}, FF{}, 0, 0, 0, H1{});
+    sync_step(LGKM_ONLY{});
+    mfma_phase();
+    if (!late) bare_barrier();
+  } else {
   for (int g = g_lo; g + 1 < g_hi; ++g) {
     // even step 2g: dequantise (g, half 1) for step 2g+1; request the tile of step 2g+2 and the words of group g+1
     load_w(g + 1);
@@ -569,6 +686,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
   sync_step(std::integral_constant<int, 0>{});
   a_cur = nxt(a_cur);
   fused_step(a_cur, 1, FF{}, FF{}, 0, 0, 0);
+  }
   // every wavefront is done with the operand stages: the epilogue reuses them
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
@@ -720,10 +838,10 @@ static int launch_prefill(const PrefillParams& p, hipStream_t s) {
   return VAQ_OK;
 }
 
-template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP, int SUBG, bool W8 = false>
+template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP, int SUBG, bool W8 = false, bool PP = false>
 static int launch_prefill2(const PrefillParams& p, hipStream_t s) {
   const size_t lds = (size_t)(3 * BM + 2 * BN) * 128;
-  auto kern = w4a16_prefill2_kernel<BF16, BM, BN, WAVES_M, WAVES_N, HAS_ZP, SUBG, W8>;
+  auto kern = w4a16_prefill2_kernel<BF16, BM, BN, WAVES_M, WAVES_N, HAS_ZP, SUBG, W8, PP>;
   static bool attr_done = false;
   if (!attr_done) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
