@@ -192,6 +192,36 @@ def test_prefill_gemm_split_k(device, k, n, m, asym):
     assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
 
 
+@pytest.mark.parametrize("asym", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_prefill_every_tile_shape(device, asym, dtype):
+    """Every tile shape of the prefill kernels, forced through the tuning export (the automatic choice only reaches some of
+    them at any one problem size), with and without K split over workgroups, against the oracle.  The direct-to-LDS
+    shapes (ids 10-15 and 20, the one with alternating phases) dequantise exactly and add the same MFMA products in the
+    same order, so without a K split they must agree with each other bit for bit."""
+    from vllm_amd import _lib
+    lib = _lib.load()
+    try:
+        for k, n, m in ((1024, 512, 300), (640, 320, 513), (384, 256, 257), (2048, 576, 70)):
+            case = o.make_w4a16_case(k, n, 128, asym=asym, seed=k + n + m)
+            layer = W4A16Layer(case, device, dtype)
+            a = _acts(m, k, device, dtype, seed=m)
+            ref = o.gemm_ref(a.cpu(), o.case_w_ref(case))
+            first = None
+            for tile in (10, 20, 11, 12, 13, 14, 15, 0, 1, 2):
+                for split in ((0, 2, 3) if tile >= 10 else (0,)):
+                    lib.vaq_debug_set_prefill_tile(tile + 100 * split)
+                    out = layer(a)
+                    check_gemm_close(out, ref, f"tile {tile} split {split} k={k} n={n} m={m}")
+                    if tile >= 10 and split == 0:
+                        if first is None:
+                            first = out
+                        assert torch.equal(out, first), f"tile {tile} differs from tile 10 (k={k} n={n} m={m})"
+            assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
+    finally:
+        lib.vaq_debug_set_prefill_tile(-1)
+
+
 @pytest.mark.parametrize("group_size", [-1, 32, 64])
 @pytest.mark.parametrize("k,n", [(128, 64), (1024, 192), (2048, 576), (14336 // 4, 128)])
 @pytest.mark.parametrize("m", [1, 4, 16, 17, 32, 33, 200, 257])

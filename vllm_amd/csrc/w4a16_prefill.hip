@@ -34,7 +34,7 @@ static int pick_tile(int M, int N, bool direct_ok) {
   auto tiles = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   if (direct_ok) {
     // measured: the 256x256 / 8-wavefront tile wins as soon as it fills ~60 % of the compute units
-    if (tiles(256, 256) * 10 >= cus * 6) return 10;
+    if (tiles(256, 256) * 10 >= cus * 6) return 20;      // 256 x 256, alternating phases
     if (tiles(128, 128) >= cus) return 12;
     // Few tiles: 64 x 128, or 128 x 64 once M fills more than one 64-row tile (the dequantisation of a weight tile is
     // then shared by twice as many rows: 7-15 % faster at M = 128 .. 768 on the narrow layers); K is split over
@@ -123,8 +123,9 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
   p.SK = pl.sk;
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
-  if (w8) rc = prefill_launch_w8(p, pl.tile, bf16, s);
-  else if (sub > 1) rc = prefill_launch_sub(p, sub, pl.tile, bf16, zp, s);
+  const int tile_other = pl.tile == 20 ? 10 : pl.tile;      // the alternating-phase variant exists for 4-bit codes, groups of 128
+  if (w8) rc = prefill_launch_w8(p, tile_other, bf16, s);
+  else if (sub > 1) rc = prefill_launch_sub(p, sub, tile_other, bf16, zp, s);
   else if (bf16) rc = zp ? dispatch_tile<true, true>(p, pl.tile, s) : dispatch_tile<true, false>(p, pl.tile, s);
   else rc = zp ? dispatch_tile<false, true>(p, pl.tile, s) : dispatch_tile<false, false>(p, pl.tile, s);
   if (rc != VAQ_OK) return rc;

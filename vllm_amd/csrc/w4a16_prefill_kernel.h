@@ -570,17 +570,37 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
   };
   if constexpr (PP) {
     // Alternating phases.  A K step is two half steps of two MFMA k-slices; a half step is a READ phase (this
-    // wavefront's fragments of the two slices, its share of the DMA requests and of the dequantisation for the next
-    // step) and an MFMA phase (16 MFMAs), each ended by a workgroup barrier.  The wavefronts w and w + 4 share a SIMD;
-    // the second four pass one extra barrier first (and skip their last one), so on every SIMD one wavefront is in its
-    // READ phase while the other one keeps the matrix core busy.  Hazards, with the late half one phase behind: a
-    // weight stage written during step s is first read two barriers after its last write; the activation stage
-    // requested during step s was last read one barrier before the first request; the tile of step s+1 has landed at
-    // the end of the second READ phase of step s of every wavefront, at least one barrier before anyone reads it.
+    // wavefront's fragments of the two slices, its share of the DMA requests, the LDS writes of two dequantised weight
+    // pieces) and an MFMA phase (16 MFMAs with the dequantisation of the next two pieces in their shadow: a wavefront's
+    // LDS traffic and its VALU work do not overlap each other, but both overlap the other wavefront's MFMAs), each
+    // ended by a workgroup barrier.  The wavefronts w and w + 4 share a SIMD; the second four pass one extra barrier
+    // first (and skip their last one), so on every SIMD one wavefront is in its READ phase while the other one keeps
+    // the matrix core busy.
+    // Weight pieces for step t+1 (four per wavefront): 0,1 dequantised in MFMA phase (t-1, 1), written in READ phase
+    // (t, 0); 2,3 dequantised in (t, 0), written in (t, 1).  The next group's words are requested a step and a half
+    // before their first use and become current in the middle of the even step.
+    // Hazards, with the late half one phase behind: a weight stage written during step t is first read two barriers
+    // after its last write; the activation stage requested during step t was last read one barrier before the first
+    // request; the tile of step t+1 has landed at the end of the second READ phase of step t of every wavefront, at
+    // least one barrier before anyone reads it.
     const bool late = wave >= NW / 2;
     v4u af[2][WMB], bf[2][WNB];
-    auto read_phase = [&](int a_cur, int w_cur, auto stage_c, auto dma_c, int a_dst, int a_step, int half, auto h_c) {
-      constexpr bool stage_on = decltype(stage_c)::value;
+    v4u dq[W_LD];
+    // pieces h*W_LD .. of weight half `half` of the current group -> dq
+    auto deq = [&](int half, auto h_c) {
+      constexpr int h = decltype(h_c)::value;
+#pragma unroll
+      for (int x = 0; x < W_LD; ++x) {
+        const int pc = h * W_LD + x;
+        const int i = pc >> 1, which = pc & 1;
+        const uint32_t wsel = half ? (which ? wcur[i].w : wcur[i].z) : (which ? wcur[i].y : wcur[i].x);
+        float sv, zv;
+        sub_vals(i, half * 2 + which, sv, zv);
+        dq[x] = dequant_scaled<BF16>(wsel, sv, zv);
+      }
+    };
+    auto read_phase = [&](int a_cur, int w_cur, auto write_c, auto dma_c, int a_dst, int a_step, auto h_c) {
+      constexpr bool write_on = decltype(write_c)::value;
       constexpr bool dma_on = decltype(dma_c)::value;
       constexpr int h = decltype(h_c)::value;
       const uint8_t* base_a = lds8 + (size_t)a_cur * A_ST;
@@ -597,21 +617,19 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
 #pragma unroll
         for (int i = 0; i < WMB; ++i) af[k2][i] = *reinterpret_cast<const v4u*>(base_a + arow + i * 4096 + coff[2 * h + k2]);
       }
-      __builtin_amdgcn_sched_barrier(0);        // the reads go out first; the dequantisation fills their latency
-      if constexpr (stage_on) {
+      if constexpr (write_on) {
+        __builtin_amdgcn_sched_barrier(0);        // the writes stay behind the reads (see sync_reads_only)
 #pragma unroll
-        for (int pc = h * W_LD; pc < (h + 1) * W_LD; ++pc) {
+        for (int x = 0; x < W_LD; ++x) {
+          const int pc = h * W_LD + x;
           const int i = pc >> 1, which = pc & 1;
-          const uint32_t wsel = half ? (which ? wcur[i].w : wcur[i].z) : (which ? wcur[i].y : wcur[i].x);
-          float sv, zv;
-          sub_vals(i, half * 2 + which, sv, zv);
           const int row = (i * NW + wave) * 16 + r;
           const int c0 = (row & 1) * 8 + o + which * 4, sw = (row >> 1) & 15;
-          *reinterpret_cast<v4u*>(Bn + (row >> 1) * 256 + ((c0 ^ sw) * 16)) = dequant_scaled<BF16>(wsel, sv, zv);
+          *reinterpret_cast<v4u*>(Bn + (row >> 1) * 256 + ((c0 ^ sw) * 16)) = dq[x];
         }
       }
     };
-    auto mfma_phase = [&]() {
+    auto mfma_phase = [&](auto deq_c, int half, auto h_c) {
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int k2 = 0; k2 < 2; ++k2)
@@ -619,54 +637,72 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
         for (int i = 0; i < WMB; ++i)
 #pragma unroll
           for (int j = 0; j < WNB; ++j) acc[i][j] = T::mfma32(bf[k2][j], af[k2][i], acc[i][j]);   // rows = n, columns = m
+      if constexpr (decltype(deq_c)::value) {
+        deq(half, h_c);
+#pragma unroll
+        for (int x = 0; x < 2 * WMB * WNB; ++x) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);     // three VALU instructions in its shadow
+        }
+      }
       __builtin_amdgcn_sched_barrier(0);
     };
     auto bare_barrier = [&]() { asm volatile("s_barrier" ::: "memory"); };
     using H0 = std::integral_constant<int, 0>;
     using H1 = std::integral_constant<int, 1>;
     using LGKM_ONLY = std::integral_constant<int, 63>;     // no vector-memory wait in the first half of a step
+    // End of the first READ phase of a step: the fragment reads are complete, the W_LD piece writes issued after them
+    // may still be queued (LDS operations complete in order); they are waited for at the end of the step's second READ
+    // phase, a barrier before the stage they fill is read.
+    auto sync_reads_only = [&]() {
+      asm volatile("s_waitcnt lgkmcnt(%0)\n\ts_barrier" ::"n"(W_LD) : "memory");
+    };
+    // (prologue, continued) the next group's words; pieces 0,1 of (g_lo, half 1)
+    if (g_lo + 1 < g_hi) load_w(g_lo + 1);
+    deq(1, H0{});
     if (late) bare_barrier();
     for (int g = g_lo; g + 1 < g_hi; ++g) {
-      // even step 2g: dequantise (g, half 1) for step 2g+1; request the tile of step 2g+2 and the words of group g+1
-      load_w(g + 1);
-      read_phase(a_cur, 0, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 2, 1, H0{});
-      sync_step(LGKM_ONLY{});
-      mfma_phase();
+      // even step 2g reads weight stage 0 and fills stage 1 with (g, half 1); requests the tile of step 2g+2
+      read_phase(a_cur, 0, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 2, H0{});
+      sync_reads_only();
+      mfma_phase(TT{}, 1, H1{});                     // pieces 2,3 of (g, half 1)
       bare_barrier();
-      read_phase(a_cur, 0, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 2, 1, H1{});
-      sync_step(std::integral_constant<int, A_LD + KW>{});
-      mfma_phase();
+      read_phase(a_cur, 0, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 2, H1{});
+      sync_step(std::integral_constant<int, A_LD>{});
+      advance_w();                                   // group g+1 becomes current
+      mfma_phase(TT{}, 0, H0{});                     // pieces 0,1 of (g+1, half 0)
       bare_barrier();
       a_cur = nxt(a_cur);
-      // odd step 2g+1: dequantise (g+1, half 0) for step 2g+2; request the tile of step 2g+3
-      advance_w();
-      read_phase(a_cur, 1, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 3, 0, H0{});
-      sync_step(LGKM_ONLY{});
-      mfma_phase();
+      // odd step 2g+1 reads stage 1 and fills stage 0 with (g+1, half 0); requests the tile of step 2g+3 and the words
+      // of group g+2 (clamped at the end of this workgroup's range: a repeated load keeps the wait counts uniform)
+      load_w(min(g + 2, g_hi - 1));
+      read_phase(a_cur, 1, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 3, H0{});
+      sync_reads_only();
+      mfma_phase(TT{}, 0, H1{});                     // pieces 2,3 of (g+1, half 0)
       bare_barrier();
-      read_phase(a_cur, 1, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 3, 0, H1{});
-      sync_step(std::integral_constant<int, A_LD>{});
-      mfma_phase();
+      read_phase(a_cur, 1, TT{}, TT{}, nxt(nxt(a_cur)), 2 * g + 3, H1{});
+      sync_step(std::integral_constant<int, A_LD + KW>{});
+      mfma_phase(TT{}, 1, H0{});                     // pieces 0,1 of (g+1, half 1)
       bare_barrier();
       a_cur = nxt(a_cur);
     }
     // last group: its second half is still dequantised, nothing is requested any more
-    read_phase(a_cur, 0, TT{}, FF{}, 0, 0, 1, H0{});
-    sync_step(LGKM_ONLY{});
-    mfma_phase();
+    read_phase(a_cur, 0, TT{}, FF{}, 0, 0, H0{});
+    sync_reads_only();
+    mfma_phase(TT{}, 1, H1{});
     bare_barrier();
-    read_phase(a_cur, 0, TT{}, FF{}, 0, 0, 1, H1{});
+    read_phase(a_cur, 0, TT{}, FF{}, 0, 0, H1{});
     sync_step(std::integral_constant<int, 0>{});
-    mfma_phase();
+    mfma_phase(FF{}, 0, H0{});
     bare_barrier();
     a_cur = nxt(a_cur);
-    read_phase(a_cur, 1, FF{}, FF{}, 0, 0, 0, H0{});
+    read_phase(a_cur, 1, FF{}, FF{}, 0, 0, H0{});
     sync_step(LGKM_ONLY{});
-    mfma_phase();
+    mfma_phase(FF{}, 0, H0{});
     bare_barrier();
-    read_phase(a_cur, 1, FF{}, FF{}, 0, 0, 0, H1{});
+    read_phase(a_cur, 1, FF{}, FF{}, 0, 0, H1{});
     sync_step(LGKM_ONLY{});
-    mfma_phase();
+    mfma_phase(FF{}, 0, H0{});
     if (!late) bare_barrier();
   } else {
   for (int g = g_lo; g + 1 < g_hi; ++g) {
