@@ -209,11 +209,11 @@ def test_prefill_every_tile_shape(device, asym, dtype):
             ref = o.gemm_ref(a.cpu(), o.case_w_ref(case))
             first = None
             for tile in (10, 20, 11, 12, 13, 14, 15, 0, 1, 2):
-                for split in ((0, 2, 3) if tile >= 10 else (0,)):
+                for split in ((1, 0, 2, 3) if tile >= 10 else (0,)):      # 0: the automatic split, 1: none
                     lib.vaq_debug_set_prefill_tile(tile + 100 * split)
                     out = layer(a)
                     check_gemm_close(out, ref, f"tile {tile} split {split} k={k} n={n} m={m}")
-                    if tile >= 10 and split == 0:
+                    if tile >= 10 and split == 1:
                         if first is None:
                             first = out
                         assert torch.equal(out, first), f"tile {tile} differs from tile 10 (k={k} n={n} m={m})"

@@ -28,13 +28,22 @@ static int dispatch_tile(const PrefillParams& p, int tile, hipStream_t s) {
 
 static int g_force_tile = -1, g_force_split = 0;
 
-static int pick_tile(int M, int N, bool direct_ok) {
+// Splits of K for the 256 x 256 tile (one workgroup per compute unit): as many as bring the workgroup count to one per
+// compute unit, every split at least 28 groups (3584 rows) long.
+static int splits_256(int64_t tiles256, int K, int cus) {
+  int sk = (int)(cus / (tiles256 > 0 ? tiles256 : 1));
+  if (sk > K / 128 / 28) sk = K / 128 / 28;
+  return sk < 1 ? 1 : (sk > 8 ? 8 : sk);
+}
+
+static int pick_tile(int M, int N, int K, bool direct_ok) {
   if (g_force_tile >= 0) return g_force_tile;
   const int cus = num_cus_current_device();
   auto tiles = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   if (direct_ok) {
-    // measured: the 256x256 / 8-wavefront tile wins as soon as it fills ~60 % of the compute units
-    if (tiles(256, 256) * 10 >= cus * 6) return 20;      // 256 x 256, alternating phases
+    // measured: the 256x256 / 8-wavefront tile wins as soon as it fills ~60 % of the compute units, also when it
+    // takes a split of a long K to get there (14336 x 4096 at M = 1024 / 2048: 4 % / 21 % faster than 128 x 128)
+    if (tiles(256, 256) * splits_256(tiles(256, 256), K, cus) * 10 >= cus * 6) return 20;      // 256 x 256, alternating phases
     if (tiles(128, 128) >= cus) return 12;
     // Few tiles: 64 x 128, or 128 x 64 once M fills more than one 64-row tile (the dequantisation of a weight tile is
     // then shared by twice as many rows: 7-15 % faster at M = 128 .. 768 on the narrow layers); K is split over
@@ -57,7 +66,7 @@ struct PrefillPlan {
 // shapes for M = 48 .. 512.
 static PrefillPlan plan_prefill(int M, int N, int K, bool direct_ok) {
   PrefillPlan pl;
-  pl.tile = pick_tile(M, N, direct_ok);
+  pl.tile = pick_tile(M, N, K, direct_ok);
   switch (pl.tile) {
     case 10: case 20: pl.bm = 256; pl.bn = 256; pl.nw = 8; break;
     case 11: pl.bm = 256; pl.bn = 256; pl.nw = 4; break;
@@ -74,7 +83,9 @@ static PrefillPlan plan_prefill(int M, int N, int K, bool direct_ok) {
   const int cus = num_cus_current_device();
   const int G = K / 128;
   int sk = 1;
-  if (pl.tiles < 2 * (int64_t)cus) {
+  if (pl.bm == 256 && pl.bn == 256 && pl.nw == 8) {
+    sk = splits_256(pl.tiles, K, cus);
+  } else if (pl.tiles < 2 * (int64_t)cus) {
     sk = (int)((2 * (int64_t)cus) / pl.tiles);
     if (sk > 8) sk = 8;
     const int min_groups = pl.tiles < cus ? 8 : 32;     // a device already full of tiles only splits a very long K
