@@ -825,7 +825,7 @@ struct Fp8TilePlan {
 };
 
 // Tile shape and K split of the multi-stage kernel.  K is split when the output tiles alone leave compute units idle:
-// about two workgroups per compute unit, at most 8 splits, each at least 64 steps (4096 bytes of K) long -- measured at
+// as many workgroups as fit the device at once (one or two per compute unit), at most 8 splits, each at least 64 steps (4096 bytes of K) long -- measured at
 // M = 256: the FP8 steps are short, so the hand-over only pays on a long K (1.35x on K = 14336, a loss on K = 4096).
 static Fp8TilePlan plan_tile3(int M, int N, int K) {
   const int cus = num_cus_current_device();
@@ -833,7 +833,9 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   Fp8TilePlan pl;
   pl.cfg = g_fp8_tile3_cfg;
   if (pl.cfg <= 0)
-    pl.cfg = tiles(256, 256) >= cus ? 1 : (tiles(128, 256) * 8 >= cus * 7 ? 7 : (tiles(128, 128) >= cus ? 3 : 4));
+    // the largest tile shape that fills 70 % of the compute units (measured on the Llama shapes, M = 256 .. 4096: a
+    // partly filled device of large tiles beats a full one of small tiles by 25-40 %)
+    pl.cfg = tiles(256, 256) * 10 >= cus * 7 ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (tiles(128, 128) * 10 >= cus * 7 ? 3 : 4));
   // the smallest tile with two k-slices per step: 5-8 % faster on a short K (half the barriers), no gain on a long one
   if (g_fp8_tile3_cfg <= 0 && pl.cfg == 4 && K % 128 == 0 && K <= 8192) pl.cfg = 14;
   if (pl.cfg >= 10 && K % 128 != 0) pl.cfg %= 10;      // two k-slices per step need K % 128 == 0
@@ -848,7 +850,8 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   int sk = 1;
   const int steps = K / 64;
   if (pl.tiles < cus) {
-    sk = (int)((2 * (int64_t)cus) / pl.tiles);
+    const int per_cu = pl.bm * pl.bn >= 128 * 256 ? 1 : 2;      // workgroups of this tile shape that share a compute unit
+    sk = (int)((per_cu * (int64_t)cus) / pl.tiles);
     if (sk > 8) sk = 8;
     if (sk > steps / 64) sk = steps / 64;
     if (sk < 1) sk = 1;
