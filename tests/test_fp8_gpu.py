@@ -340,6 +340,26 @@ def test_silu_and_mul_quant(device, tokens, hidden, dtype):
         assert torch.equal(out3.reshape(tokens, -1).view(torch.uint8), out.view(torch.uint8))
 
 
+@pytest.mark.parametrize("offset", [0, 4, 8])
+def test_scaled_mm_into_a_view_of_a_wider_buffer(device, offset):
+    """The registered op writes into the tensor it is given: a column range of a wider buffer (row stride a multiple of
+    16 elements).  An offset of 4 elements starts the rows 8 bytes off a 16-byte boundary, which takes the tile kernel's
+    8-byte store path instead of the LDS-staged 16-byte one; every element outside the view must stay untouched."""
+    import vllm_amd._custom_ops as ops
+    g = torch.Generator().manual_seed(offset)
+    for m, n, k in ((300, 384, 512), (70, 256, 1024), (4, 128, 256)):
+        a = torch.randint(-2, 3, (m, k), generator=g).float()
+        w = torch.randint(-1, 2, (n, k), generator=g).float()
+        big = torch.full((m, n + 32), 7.0, dtype=torch.bfloat16, device=device)
+        view = big[:, offset:offset + n]
+        torch.ops.vllm_amd.cutlass_scaled_mm(view, a.to(torch.float8_e4m3fn).to(device),
+                                             w.to(torch.float8_e4m3fn).to(device).t(), torch.ones(m, 1, device=device),
+                                             torch.ones(n, 1, device=device), None)
+        got = big.cpu().float()
+        assert torch.equal(got[:, offset:offset + n], a @ w.t()), (offset, m, n, k)
+        assert bool((got[:, :offset] == 7).all()) and bool((got[:, offset + n:] == 7).all()), "wrote outside the view"
+
+
 @pytest.mark.parametrize("cfg", [1, 8, 3, 4, 7, 13, 23, 14, 24, 17])
 def test_scaled_mm_every_tile_shape_exact(device, cfg):
     """Every shape of the multi-stage tile kernel, forced through the tuning export (the automatic choice only reaches
