@@ -760,16 +760,8 @@ static int launch_tile(const Fp8MMParams& p, hipStream_t s) {
   constexpr int BM = 64 * WMB, BN = 64 * WNB;
   const size_t lds = (size_t)2 * (BM + BN) * F8_PITCH;
   auto kern = fp8_mm_tile_kernel<BF16_OUT, WMB, WNB>;
-  static bool attr_done = false;
-  if (!attr_done) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
-        hipSuccess) {
-      set_error("fp8_scaled_mm: cannot reserve %zu bytes of LDS", lds);
-      (void)hipGetLastError();
-      return VAQ_ERR_LAUNCH;
-    }
-    attr_done = true;
-  }
+  static size_t reserved[VAQ_MAX_DEVICES];
+  if (const int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "fp8_scaled_mm"); rc != VAQ_OK) return rc;
   const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   hipLaunchKernelGGL(kern, dim3(tiles), dim3(256), lds, s, p);
   return VAQ_OK;
@@ -780,16 +772,8 @@ static int launch_tile2(const Fp8MMParams& p, hipStream_t s) {
   constexpr int BM = 64 * WMB, BN = 64 * WNB;
   const size_t lds = (size_t)2 * (BM + BN) * 128;
   auto kern = fp8_mm_tile2_kernel<BF16_OUT, WMB, WNB>;
-  static bool attr_done = false;
-  if (!attr_done) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
-        hipSuccess) {
-      set_error("fp8_scaled_mm: cannot reserve %zu bytes of LDS", lds);
-      (void)hipGetLastError();
-      return VAQ_ERR_LAUNCH;
-    }
-    attr_done = true;
-  }
+  static size_t reserved[VAQ_MAX_DEVICES];
+  if (const int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "fp8_scaled_mm"); rc != VAQ_OK) return rc;
   const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   hipLaunchKernelGGL(kern, dim3(tiles), dim3(256), lds, s, p);
   return VAQ_OK;
@@ -799,16 +783,8 @@ template <bool BF16_OUT, int BM, int BN, int WAVES_M, int WAVES_N, int NST, int 
 static int launch_tile3(const Fp8MMParams& p, hipStream_t s) {
   const size_t lds = (size_t)NST * KS * (BM + BN) * 64;
   auto kern = fp8_mm_tile3_kernel<BF16_OUT, BM, BN, WAVES_M, WAVES_N, NST, KS, PP>;
-  static bool attr_done = false;
-  if (!attr_done) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
-        hipSuccess) {
-      set_error("fp8_scaled_mm: cannot reserve %zu bytes of LDS", lds);
-      (void)hipGetLastError();
-      return VAQ_ERR_LAUNCH;
-    }
-    attr_done = true;
-  }
+  static size_t reserved[VAQ_MAX_DEVICES];
+  if (const int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "fp8_scaled_mm"); rc != VAQ_OK) return rc;
   const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   hipLaunchKernelGGL(kern, dim3(tiles, p.SK), dim3(WAVES_M * WAVES_N * 64), lds, s, p);
   return VAQ_OK;

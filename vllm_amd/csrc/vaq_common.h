@@ -40,6 +40,27 @@ void set_error(const char* fmt, ...);   // defined in api.hip (thread-local buff
 
 int num_cus_current_device();   // cached per device, api.hip
 
+// Dynamic LDS above the default limit has to be reserved per kernel and per device.  `reserved` is the calling launch
+// function's own static array (one per kernel instantiation, zero-initialised): bytes already reserved on each device.
+// The attribute is idempotent, so two threads racing here at worst set it twice.
+constexpr int VAQ_MAX_DEVICES = 64;
+inline int reserve_dynamic_lds(const void* kern, size_t lds, size_t (&reserved)[VAQ_MAX_DEVICES], const char* what) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= VAQ_MAX_DEVICES) {
+    set_error("%s: cannot identify the current device", what);
+    (void)hipGetLastError();
+    return VAQ_ERR_LAUNCH;
+  }
+  if (lds <= reserved[dev]) return VAQ_OK;
+  if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+    set_error("%s: cannot reserve %zu bytes of LDS", what, lds);
+    (void)hipGetLastError();
+    return VAQ_ERR_LAUNCH;
+  }
+  reserved[dev] = lds;
+  return VAQ_OK;
+}
+
 // ----------------------------------------------------------------------------- device: vector types
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));

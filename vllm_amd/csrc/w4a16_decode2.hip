@@ -82,26 +82,6 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8) 
   return c;
 }
 
-template <bool BF16, int GS, int MB, bool HAS_ZP, int MR>
-static int launch_decode2(const Decode2Params& p, hipStream_t s) {
-  const int WN = p.WN;
-  const size_t lds = (size_t)p.WKS * GS * 256 * MR * MB + (p.WKS > 1 ? (size_t)D2_WAVES * MB * 1024 : 16);
-  auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP, MR>;
-  static size_t attr_lds = 0;
-  if (lds > attr_lds) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
-        hipSuccess) {
-      set_error("w4a16_gemm(decode): cannot reserve %zu bytes of LDS", lds);
-      (void)hipGetLastError();
-      return VAQ_ERR_LAUNCH;
-    }
-    attr_lds = lds;
-  }
-  const int gx = (p.NT + WN - 1) / WN;
-  hipLaunchKernelGGL(kern, dim3(gx, p.SK), dim3(64, p.WKS * WN), lds, s, p);
-  return VAQ_OK;
-}
-
 template <bool BF16, int MB, bool HAS_ZP, int MR>
 static int dispatch_gs2(const Decode2Params& p, int gs, hipStream_t s) {
   switch (gs) {

@@ -389,16 +389,8 @@ static int launch_decode2(const Decode2Params& p, hipStream_t s) {
   const int WN = p.WN;
   const size_t lds = decode2_lds_bytes(p.WKS, GS / (W8 ? 2 : 1), MR, MB);
   auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP, MR, SUBG, W8>;
-  static size_t attr_lds = 0;
-  if (lds > attr_lds) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
-        hipSuccess) {
-      set_error("w4a16_gemm(decode): cannot reserve %zu bytes of LDS", lds);
-      (void)hipGetLastError();
-      return VAQ_ERR_LAUNCH;
-    }
-    attr_lds = lds;
-  }
+  static size_t reserved[VAQ_MAX_DEVICES];
+  if (const int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "w4a16_gemm(decode)"); rc != VAQ_OK) return rc;
   const int gx = (p.NT + WN - 1) / WN;
   hipLaunchKernelGGL(kern, dim3(gx, p.SK), dim3(64, p.WKS * WN), lds, s, p);
   return VAQ_OK;

@@ -859,16 +859,8 @@ static int launch_prefill(const PrefillParams& p, hipStream_t s) {
   constexpr int BM = 64 * WMB, BN = 64 * WNB;
   const size_t lds = (size_t)2 * (BM + BN) * PF_PITCH * sizeof(uint16_t);
   auto kern = w4a16_prefill_kernel<BF16, WMB, WNB, HAS_ZP, SUBG>;
-  static bool attr_done = false;   // idempotent attribute; a benign race sets it twice
-  if (!attr_done) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
-        hipSuccess) {
-      set_error("w4a16_gemm(prefill): cannot reserve %zu bytes of LDS", lds);
-      (void)hipGetLastError();
-      return VAQ_ERR_LAUNCH;
-    }
-    attr_done = true;
-  }
+  static size_t reserved[VAQ_MAX_DEVICES];
+  if (const int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "w4a16_gemm(prefill)"); rc != VAQ_OK) return rc;
   const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   hipLaunchKernelGGL(kern, dim3(tiles), dim3(256), lds, s, p);
   return VAQ_OK;
@@ -878,16 +870,8 @@ template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP, int 
 static int launch_prefill2(const PrefillParams& p, hipStream_t s) {
   const size_t lds = (size_t)(3 * BM + 2 * BN) * 128;
   auto kern = w4a16_prefill2_kernel<BF16, BM, BN, WAVES_M, WAVES_N, HAS_ZP, SUBG, W8, PP>;
-  static bool attr_done = false;
-  if (!attr_done) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
-        hipSuccess) {
-      set_error("w4a16_gemm(prefill): cannot reserve %zu bytes of LDS", lds);
-      (void)hipGetLastError();
-      return VAQ_ERR_LAUNCH;
-    }
-    attr_done = true;
-  }
+  static size_t reserved[VAQ_MAX_DEVICES];
+  if (const int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "w4a16_gemm(prefill)"); rc != VAQ_OK) return rc;
   const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   hipLaunchKernelGGL(kern, dim3(tiles, p.SK), dim3(WAVES_M * WAVES_N * 64), lds, s, p);
   return VAQ_OK;
