@@ -98,7 +98,7 @@ int vaq_w4a16_gemm_workspace(int64_t size_m, int64_t size_n, int64_t size_k, int
  *   bias     [N] activation dtype or NULL
  *   c        [M, N] activation dtype, contiguous
  *   group_size  128, 64, 32, or -1 / K for channelwise scales (the reference's MARLIN_SUPPORTED_GROUP_SIZES,
- *               marlin_utils.py:24); anything else returns VAQ_ERR_UNSUPPORTED, and so do 64 / 32 with U8B128
+ *               marlin_utils.py:24), for every wtype; anything else returns VAQ_ERR_UNSUPPORTED
  * M == 0 is a no-op.  Kernel choice (decode: M <= 32, up to 64 for 4-bit codes in groups of 128 rows or channelwise,
  * MFMA GEMV with in-register dequant; prefill: LDS-staged MFMA)
  * is internal; `force_path` = 0 auto, 1 decode, 2 prefill (tests / benchmarks).

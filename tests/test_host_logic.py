@@ -143,9 +143,10 @@ def test_shape_and_type_support_checks():
     assert mu.check_marlin_supported(st.uint4b8, 128) and not mu.check_marlin_supported(st.uint4b8, 256)
     assert all(mu.check_marlin_supported(st.uint4b8, g) for g in (-1, 32, 64))
     assert mu.check_marlin_supported(st.uint4, 128, has_zp=True) and not mu.check_marlin_supported(st.uint4, 128)
-    mu.verify_marlin_supported(st.uint8b128, 128)
+    for g in (-1, 32, 64, 128):
+        mu.verify_marlin_supported(st.uint8b128, g)
     with pytest.raises(ValueError):
-        mu.verify_marlin_supported(st.uint8b128, 64)
+        mu.verify_marlin_supported(st.uint8b128, 256)
     with pytest.raises(ValueError):
         mu.verify_marlin_supported(st.uint8, 128, has_zp=True)
 
@@ -271,7 +272,8 @@ def test_plugin_surface_contract():
     assert shapes == {"qweight": (512, 6144), "g_idx": (4096,), "scales": (32, 6144), "qzeros": (32, 768)}
     assert GPTQMarlinConfig.is_gptq_marlin_compatible(dict(quant_method="gptq", bits=4, group_size=128, sym=True, desc_act=False))
     assert GPTQMarlinConfig.is_gptq_marlin_compatible(dict(quant_method="gptq", bits=8, group_size=128, sym=True, desc_act=False))
-    assert not GPTQMarlinConfig.is_gptq_marlin_compatible(dict(quant_method="gptq", bits=8, group_size=32, sym=True, desc_act=False))
+    assert GPTQMarlinConfig.is_gptq_marlin_compatible(dict(quant_method="gptq", bits=8, group_size=32, sym=True, desc_act=False))
+    assert not GPTQMarlinConfig.is_gptq_marlin_compatible(dict(quant_method="gptq", bits=8, group_size=256, sym=True, desc_act=False))
     assert not GPTQMarlinConfig.is_gptq_marlin_compatible(dict(quant_method="gptq", bits=4, group_size=128, sym=False, desc_act=False))
     assert GPTQMarlinConfig.override_quantization_method(dict(quant_method="gptq", bits=4, group_size=128, sym=True, desc_act=False), None) == "gptq_marlin"
     mp = MPLinearLayerConfig((4096, 4096), (4096, 4096), st.uint4, torch.bfloat16, 128, True, False)

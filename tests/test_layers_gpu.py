@@ -172,7 +172,7 @@ def test_gptq_and_awq_methods_other_group_sizes(device, group_size):
         check_gemm_close(layer(a.to(device)), o.gemm_ref(a, w_ref), f"awq g={group_size} m={m}")
 
 
-@pytest.mark.parametrize("group_size,desc_act", [(128, False), (128, True), (-1, False)])
+@pytest.mark.parametrize("group_size,desc_act", [(128, False), (128, True), (-1, False), (64, True), (32, False)])
 def test_gptq_8bit_method_end_to_end(device, group_size, desc_act):
     """A GPTQ 8-bit checkpoint (bits = 8, sym: the uint8b128 type, gptq_marlin.py:96-99) through GPTQMarlinConfig and
     the linear method: qweight packs 4 codes per int32 along K."""

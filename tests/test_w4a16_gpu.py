@@ -271,7 +271,7 @@ def test_gemm_other_group_sizes_llama_shape(device):
         assert bool((layer.workspace == 0).all())
 
 
-@pytest.mark.parametrize("group_size", [128, -1])
+@pytest.mark.parametrize("group_size", [128, -1, 64, 32])
 @pytest.mark.parametrize("k,n", [(128, 64), (1024, 192), (2048, 576), (14336 // 4, 128), (14336, 256)])
 @pytest.mark.parametrize("m", [1, 4, 16, 17, 32, 33, 200, 257])
 @pytest.mark.parametrize("act_order", [False, True])
@@ -288,12 +288,13 @@ def test_gemm_8bit_weights(device, group_size, k, n, m, act_order):
     assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
 
 
+@pytest.mark.parametrize("group_size", [128, 64, 32])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("m", [1, 4, 16, 32, 48])
-def test_one_hot_activation_8bit_exact(device, dtype, m):
+def test_one_hot_activation_8bit_exact(device, group_size, dtype, m):
     """One-hot rows of A with 8-bit weights: rn16((q - 128) * s) bit for bit, on every kernel variant by M."""
     k, n = 512, 128
-    case = o.make_w4a16_case(k, n, 128, dtype=dtype, seed=21, num_bits=8)
+    case = o.make_w4a16_case(k, n, group_size, dtype=dtype, seed=21 + group_size, num_bits=8)
     layer = W4A16Layer(case, device, dtype)
     w = o.case_w_ref(case)
     rows = [(37 * i + 5) % k for i in range(m)]
@@ -325,7 +326,7 @@ def test_gemm_random_shapes_and_formats(device, seed):
         n = 64 * int(rng.integers(1, 20))
         m = int(rng.choice([1, 2, 3, 5, 8, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 100, 129, 300]))
         fmt = rng.choice(["u4b8", "u4", "u8b128"])
-        group_size = int(rng.choice([128, -1] if fmt == "u8b128" else [128, 64, 32, -1]))
+        group_size = int(rng.choice([128, 64, 32, -1]))
         act_order = bool(rng.integers(0, 2)) and group_size != -1 and k // group_size > 1
         dtype = torch.bfloat16 if rng.integers(0, 2) else torch.float16
         case = o.make_w4a16_case(k, n, group_size, asym=fmt == "u4", act_order=act_order, dtype=dtype,

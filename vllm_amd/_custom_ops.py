@@ -246,9 +246,6 @@ def _check_gemm_args(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, 
     _check(size_k % GPTQ_MARLIN_MIN_THREAD_K == 0,
            f"size_k = {size_k}, is not divisible by min_thread_k = {GPTQ_MARLIN_MIN_THREAD_K}")
     if b_q_type == scalar_types.uint8b128:
-        if group_size not in (-1, 128):
-            raise NotImplementedError(f"gptq_marlin_gemm: uint8b128 weights with group_size = {group_size} are not built "
-                                      "for gfx950 (only -1, 128)")
         wtype = _lib.VAQ_WTYPE_U8B128
     else:
         wtype = _lib.VAQ_WTYPE_U4 if has_zp else _lib.VAQ_WTYPE_U4B8

@@ -160,7 +160,8 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
   }
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
-  if (w8) rc = decode2_launch_w8(p, cfg.gs, MB, cfg.mr, bf16, s);
+  if (w8 && sub > 1) rc = decode2_launch_w8sub(p, sub, cfg.gs, MB, cfg.mr, bf16, s);
+  else if (w8) rc = decode2_launch_w8(p, cfg.gs, MB, cfg.mr, bf16, s);
   else if (sub == 2) rc = decode2_launch_sub2(p, cfg.gs, MB, cfg.mr, bf16, zp, s);
   else if (sub == 4) rc = decode2_launch_sub4(p, cfg.gs, MB, cfg.mr, bf16, zp, s);
   else if (MB > 2) rc = decode2_launch_mb34(p, cfg.gs, MB, bf16, zp, s);

@@ -63,7 +63,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   using T = F16Traits<BF16>;
   static_assert(SUBG == 1 || SUBG == 2 || SUBG == 4, "quantisation groups per 128-row tile");
   constexpr int TPG = W8 ? 2 : 1;                      // weight tiles per 128 rows of K
-  static_assert(!W8 || (SUBG == 1 && !HAS_ZP && GS % 2 == 0), "8-bit codes: two planes per group, symmetric, one group per tile");
+  static_assert(!W8 || (!HAS_ZP && GS % 2 == 0), "8-bit codes: two planes per 128 rows, symmetric");
   static_assert(MR == 16 || MB == 1, "compact row staging is for a single m-block");
   // Ring slots.  Two tiles in flight per wavefront measured best: a wavefront does not get past its load instructions
   // until the memory pipeline has accepted them, and with deeper rings (every wavefront of the device asking for
@@ -402,7 +402,9 @@ int decode2_launch_sub2(const Decode2Params& p, int gs, int MB, int mr, bool bf1
 int decode2_launch_sub4(const Decode2Params& p, int gs, int MB, int mr, bool bf16, bool zp, hipStream_t s);
 // Three and four m-blocks (32 < M <= 64), groups of 128 rows / channelwise; defined in w4a16_decode2_mb34.hip.
 int decode2_launch_mb34(const Decode2Params& p, int gs, int MB, bool bf16, bool zp, hipStream_t s);
-// 8-bit codes; defined in w4a16_decode2_w8.hip: gs in {2, 4, 8, 14, 16}, staged rows mr in {1, 4, 16} (16 when MB == 2).
+// 8-bit codes; defined in w4a16_decode2_w8.hip (groups of 128 rows / channelwise: gs in {2, 4, 8, 14, 16}) and
+// w4a16_decode2_w8sub.hip (sub = 2 / 4 groups per 128 rows: gs in {2, 4, 8, 16}); staged rows mr in {1, 4, 16} (16 when MB == 2).
 int decode2_launch_w8(const Decode2Params& p, int gs, int MB, int mr, bool bf16, hipStream_t s);
+int decode2_launch_w8sub(const Decode2Params& p, int sub, int gs, int MB, int mr, bool bf16, hipStream_t s);
 
 }  // namespace vaq

@@ -112,8 +112,6 @@ extern "C" int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, cons
                       "w4a16_gemm: group_size = %d is not built (only -1, 32, 64, 128)", group_size);
   const int sub = channelwise ? 1 : 128 / group_size;
   VAQ_CHECK_ARG(!w8 || size_k * size_n < (1ll << 32), "w4a16_gemm: problem too large for 8-bit weights");
-  VAQ_CHECK_SUPPORTED(!w8 || sub == 1, "w4a16_gemm: 8-bit weights with group_size = %d are not built (only -1, 128)",
-                      group_size);
   VAQ_CHECK_ARG(force_path >= 0 && force_path <= 2, "w4a16_gemm: force_path = %d", force_path);
   if (size_m == 0) return VAQ_OK;
   VAQ_CHECK_ARG(a && b && scales && c, "w4a16_gemm: null pointer");

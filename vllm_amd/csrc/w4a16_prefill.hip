@@ -135,7 +135,7 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
   const int tile_other = pl.tile == 20 ? 10 : pl.tile;      // the alternating-phase variant exists for 4-bit codes, groups of 128
-  if (w8) rc = prefill_launch_w8(p, tile_other, bf16, s);
+  if (w8) rc = prefill_launch_w8(p, sub, tile_other, bf16, s);
   else if (sub > 1) rc = prefill_launch_sub(p, sub, tile_other, bf16, zp, s);
   else if (bf16) rc = zp ? dispatch_tile<true, true>(p, pl.tile, s) : dispatch_tile<true, false>(p, pl.tile, s);
   else rc = zp ? dispatch_tile<false, true>(p, pl.tile, s) : dispatch_tile<false, false>(p, pl.tile, s);

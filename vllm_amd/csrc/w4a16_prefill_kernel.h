@@ -306,7 +306,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
   using T = F16Traits<BF16>;
   static_assert(!PP || (!W8 && SUBG == 1 && (BM / (8 * WAVES_M * WAVES_N)) % 2 == 0 && WAVES_M * WAVES_N == 8),
                 "alternating phases: 8 wavefronts, groups of 128 rows, an even number of DMA instructions per step");
-  static_assert(!W8 || (SUBG == 1 && !HAS_ZP), "8-bit codes: symmetric, one group per tile");
+  static_assert(!W8 || !HAS_ZP, "8-bit codes: symmetric");
   constexpr int TPG = W8 ? 2 : 1;                 // 1 KiB weight blocks per tile (8-bit: high-nibble plane, low-nibble plane)
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;
@@ -419,7 +419,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
       const int sj = (j * SUBG) >> 2;
       zv = -((float)((zcur[i] >> (8 * sj)) & 0xffu) * sv);
     } else {
-      zv = -8.f * sv;
+      zv = -(W8 ? 128.f : 8.f) * sv;
     }
   };
   // Prologue only: dequantise half 0 of the current group into weight stage 0.
@@ -880,7 +880,8 @@ static int launch_prefill2(const PrefillParams& p, hipStream_t s) {
 // Groups of 64 / 32 rows (sub = 2 / 4 per tile); defined in w4a16_prefill_sub.hip for the tile ids the automatic choice
 // uses (10, 12, 14, 15 and 0, 1, 2).
 int prefill_launch_sub(const PrefillParams& p, int sub, int tile, bool bf16, bool zp, hipStream_t s);
-// 8-bit codes; defined in w4a16_prefill_w8.hip for the direct-to-LDS tile ids 10, 12, 14, 15.
-int prefill_launch_w8(const PrefillParams& p, int tile, bool bf16, hipStream_t s);
+// 8-bit codes; defined in w4a16_prefill_w8.hip for the direct-to-LDS tile ids 10, 12, 14, 15 (sub = 1, 2 or 4 groups per
+// 128 rows).
+int prefill_launch_w8(const PrefillParams& p, int sub, int tile, bool bf16, hipStream_t s);
 
 }  // namespace vaq

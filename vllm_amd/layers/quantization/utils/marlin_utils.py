@@ -23,7 +23,7 @@ GPTQ_MARLIN_MAX_PARALLEL = 16
 MARLIN_SUPPORTED_GROUP_SIZES = [-1, 32, 64, 128]
 # what the gfx950 kernels implement out of the above (marlin_utils.py:24)
 HIP_W4A16_SUPPORTED_GROUP_SIZES = [-1, 32, 64, 128]
-HIP_W8A16_SUPPORTED_GROUP_SIZES = [-1, 128]      # uint8b128 weights
+HIP_W8A16_SUPPORTED_GROUP_SIZES = [-1, 32, 64, 128]      # uint8b128 weights
 
 USE_FP32_REDUCE_DEFAULT = True
 
