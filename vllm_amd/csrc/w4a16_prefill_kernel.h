@@ -299,7 +299,7 @@ __global__ __launch_bounds__(256) void w4a16_prefill_kernel(const PrefillParams 
 //  * WAVES_M x WAVES_N wavefronts per workgroup (8 = two per SIMD lets one wavefront dequantise while the other one
 //    issues MFMAs);
 //  * the MFMAs take the weight fragment as A operand, so four consecutive accumulator registers are four consecutive
-//    output columns of one row: packed 8-byte stores in the epilogue;
+//    output columns of one row: 8 bytes per lane into the epilogue's LDS staging (16-byte global stores from there);
 //  * weight words of group g+1 are requested one K step before they are needed (two register sets, by group parity).
 template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP, int SUBG, bool W8 = false, bool PP = false>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(const PrefillParams p) {
