@@ -394,7 +394,7 @@ __global__ __launch_bounds__(256) void fp8_mm_tile2_kernel(const Fp8MMParams p) 
 //  * LDS rows are 64 bytes; four rows form one 256-byte line of 16 chunks (chunk index (row & 3) * 4 + c) and the chunk
 //    index is XOR-ed with (row >> 2) & 3.  The LDS has 64 banks (256 bytes per cycle): 16 lanes reading 16 consecutive
 //    rows at the same k chunk touch 16 different 16-byte bank groups;
-//  * WAVES_M x WAVES_N wavefronts; tiles are handed out in bands of 8 tile rows inside each XCD's contiguous range so
+//  * WAVES_M x WAVES_N wavefronts; tiles are handed out in bands of 4 tile rows inside each XCD's contiguous range so
 //    that the tiles resident on one XCD share activation rows and weight columns in its L2.
 // Requires K % 64 == 0 (a partial last step would read the neighbouring row instead of zeros) and M*lda, N*ldb < 2^32.
 template <bool BF16_OUT, int BM, int BN, int WAVES_M, int WAVES_N, int NST, int KS = 1, int PP = 0>
@@ -420,7 +420,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
   const int total = tiles_m * tiles_n;
   int t = blockIdx.x;
   if (total % 8 == 0) t = (t & 7) * (total / 8) + (t >> 3);          // one contiguous range of tile ids per XCD
-  constexpr int GM = 8;                                              // band height in tiles
+  constexpr int GM = 4;                                              // band height in tiles (2 .. 16 measured: 4 is 1-2 % ahead of 8)
   const int band = t / (GM * tiles_n);
   const int first_m = band * GM;
   const int gsz = min(tiles_m - first_m, GM);
