@@ -178,7 +178,6 @@ __device__ inline void tile_epilogue_lds(const Fp8MMParams& p, v16f (&acc)[WMB][
 // ----------------------------------------------------------------------------- tile kernel
 template <bool BF16_OUT, int WMB, int WNB>
 __global__ __launch_bounds__(256) void fp8_mm_tile_kernel(const Fp8MMParams p) {
-  using T = F16Traits<BF16_OUT>;
   constexpr int BM = 64 * WMB, BN = 64 * WNB;
   constexpr int A_CH = BM / 32, B_CH = BN / 32;   // 16-byte chunks per thread per step
   extern __shared__ __attribute__((aligned(16))) uint8_t lds8[];
@@ -288,7 +287,6 @@ __global__ __launch_bounds__(256) void fp8_mm_tile_kernel(const Fp8MMParams p) {
 // Requires K % 128 == 0 (a partial last step would read the neighbouring row instead of zeros).
 template <bool BF16_OUT, int WMB, int WNB>
 __global__ __launch_bounds__(256) void fp8_mm_tile2_kernel(const Fp8MMParams p) {
-  using T = F16Traits<BF16_OUT>;
   constexpr int BM = 64 * WMB, BN = 64 * WNB;
   constexpr int STAGE = (BM + BN) * 128;          // bytes per stage
   extern __shared__ __attribute__((aligned(16))) uint8_t lds8[];

@@ -111,52 +111,43 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   };
 
   const int KO = slab_groups / TPG * 16;             // k-octets in the slab
-  // 16 bytes behind the activations for lanes without a chunk (the start of the reduction buffer, unused until the K
-  // loop is over, when there is one)
-  const uint32_t dummy_slot = (uint32_t)(KO * MR * MB);
+  // LDS image of the slab's activations: row-major, slot (16 bytes) of (row m, k-octet ko) = m*KO + (ko ^ (m & (MR-1))).
+  // A row is contiguous like in global memory, so 64 consecutive slots are one coalesced 1 KiB piece of a row (the XOR
+  // permutes 16-byte chunks inside aligned 256-byte blocks) and a direct-to-LDS load can fill them; the operand reads
+  // of 16 lanes (16 rows, one k-octet) hit 16 different bank groups because the row pitch is a multiple of 256 bytes.
   {
-    // chunk c = m * KO + ko (16 bytes: row m, k-octet ko); thread tid handles c = tid, tid + NTHR, ...  The (m, ko)
-    // pair is advanced incrementally: one scalar division per kernel instead of one vector division per chunk.
     const int tid = w * 64 + lane;
     const int chunks = KO * MR * MB;
     const int64_t k_slab0 = (int64_t)(slab_g0 / TPG) * 128;
     const int NTHR = WKS * WN * 64;
     const int step_m = NTHR / KO, step_ko = NTHR - step_m * KO;     // scalar
+    // chunk c = m * KO + ko' (LDS slot c); thread tid handles c = tid, tid + NTHR, ...  The (m, ko') pair is advanced
+    // incrementally: one scalar division per kernel instead of one vector division per chunk.
     int m = tid / KO, ko = tid - m * KO;
     if (p.perm == nullptr) {
-      // Straight-line code, no branch between the loads and the LDS writes (at a join the compiler's wait-count
-      // bookkeeping falls back to draining every load): the rows are read through a buffer descriptor that ends with
-      // the last valid element, chunks that do not exist get an out-of-range offset and come back as zeros, and
-      // their lanes write to a dummy slot.  FB chunks per thread cover a full-size slab in the first pass.
-      constexpr int FB = MR == 1 ? 2 : 8;
+      // Direct-to-LDS loads (no registers, no LDS write instructions): wavefront instruction q fills slots 64q .. 64q+63,
+      // lane l fetching the chunk that belongs in slot 64q + l.  Rows past M, k past K and slots past the image get an
+      // out-of-range offset of the buffer descriptor (which ends with the last valid element) and arrive as zeros; the
+      // image is padded to a multiple of 1 KiB for the last instruction.  The weight tiles are requested after these
+      // loads (loads retire in order as far as the wait counter is concerned) and stay in flight across the barrier.
       const __amdgpu_buffer_rsrc_t ra = d2_rsrc(p.a, ((uint64_t)(p.M - 1) * (uint64_t)p.lda + (uint64_t)p.K) * 2);
-      auto fill_pass = [&](auto first) {
-        v4u v[FB];
-        uint32_t slot[FB];
-#pragma unroll
-        for (int i = 0; i < FB; ++i) {
-          const int64_t k = k_slab0 + (int64_t)ko * 8;
-          const bool ok = m < MR * MB && m < p.M && k < p.K;
-          const uint32_t off = ok ? (uint32_t)(((int64_t)m * p.lda + k) * 2) : 0x80000000u;
-          v[i] = __builtin_amdgcn_raw_buffer_load_b128(ra, (int)off, 0, 0);
-          const int mb = m / MR, ml = m % MR;
-          slot[i] = m < MR * MB ? (uint32_t)(mb * KO * MR + ko * MR + (ml ^ (ko & (MR - 1)))) : dummy_slot;
-          m += step_m;
-          ko += step_ko;
-          if (ko >= KO) {
-            ko -= KO;
-            m += 1;
-          }
+      typedef __attribute__((address_space(3))) void* lds_ptr_t;
+      for (int c0 = w * 64; c0 < chunks; c0 += NTHR) {
+        const int64_t k = k_slab0 + (int64_t)(ko ^ (m & (MR - 1))) * 8;
+        const bool ok = m < MR * MB && m < p.M && k < p.K;
+        const uint32_t off = ok ? (uint32_t)(((int64_t)m * p.lda + k) * 2) : 0x80000000u;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(lds + (size_t)c0 * 16), 16, (int)off, 0, 0, 0);
+        m += step_m;
+        ko += step_ko;
+        if (ko >= KO) {
+          ko -= KO;
+          m += 1;
         }
-        if constexpr (decltype(first)::value) {
+      }
 #pragma unroll
-          for (int s = 0; s < R; ++s) issue_load(s, s);
-        }
-#pragma unroll
-        for (int i = 0; i < FB; ++i) *reinterpret_cast<v4u*>(lds + (size_t)slot[i] * 16) = v[i];
-      };
-      fill_pass(std::true_type{});
-      for (int c0 = NTHR * FB; c0 < chunks; c0 += NTHR * FB) fill_pass(std::false_type{});
+      for (int s = 0; s < R; ++s) issue_load(s, s);
+      constexpr int W_LOADS = R * (1 + SUBG * (HAS_ZP ? 2 : 1));      // vector-memory instructions of the weight requests
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(W_LOADS) : "memory");
     } else {
       // act_order: the columns of A are gathered through `perm`; two dependent levels of loads, weights requested first
 #pragma unroll
@@ -168,7 +159,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
         for (int i = 0; i < 4; ++i) {
           mm[i] = m;
           kk[i] = ko;
-          const int64_t k = k_slab0 + (int64_t)ko * 8;
+          const int64_t k = k_slab0 + (int64_t)(ko ^ (m & (MR - 1))) * 8;
           v[i] = v4u{0u, 0u, 0u, 0u};
           if (m < MR * MB && m < p.M && k < p.K) {
             const uint16_t* row = p.a + (int64_t)m * p.lda;
@@ -188,16 +179,12 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          if (mm[i] < MR * MB) {
-            const int mb = mm[i] / MR, ml = mm[i] % MR;
-            const int slot = mb * KO * MR + kk[i] * MR + (ml ^ (kk[i] & (MR - 1)));
-            *reinterpret_cast<v4u*>(lds + (size_t)slot * 16) = v[i];
-          }
+          if (mm[i] < MR * MB) *reinterpret_cast<v4u*>(lds + ((size_t)mm[i] * KO + kk[i]) * 16) = v[i];
         }
       }
+      __syncthreads();
     }
   }
-  __syncthreads();
 
   // ---- 3. the K loop of this wavefront: GS tiles, fully unrolled ----
   // operand read of MFMA jj of local group gl: k-octet = gl*16 + jj*4 + o  ->  (ko & 15) = jj*4 + o
@@ -205,7 +192,8 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
 #pragma unroll
   for (int jj = 0; jj < 4; ++jj) {
     const int kol = jj * 4 + o;
-    abase[jj] = (uint32_t)(((wks * (GS / TPG) * 16 + kol) * MR + ((r16 ^ kol) & (MR - 1))) * 16);
+    const int ml = r16 & (MR - 1);
+    abase[jj] = (uint32_t)((ml * KO + wks * (GS / TPG) * 16 + (kol ^ ml)) * 16);
   }
   uint32_t ex;     // kept in a vector register so that (x & MSK) | ex is a legal single VOP3 instruction (one scalar operand)
   asm volatile("v_mov_b32 %0, %1" : "=v"(ex) : "s"(p.k_ex));
@@ -248,7 +236,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
         aop.w = d2_and_or(wj[jj] >> 12, MSK, ex);
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
-          const v4u bop = *reinterpret_cast<const v4u*>(lds + abase[jj] + (uint32_t)(mb * KO * MR * 16) + (uint32_t)((gi / TPG) * 256 * MR));
+          const v4u bop = *reinterpret_cast<const v4u*>(lds + abase[jj] + (uint32_t)(mb * KO * MR * 16) + (uint32_t)((gi / TPG) * 256));
           P[mb] = T::mfma16(aop, bop, P[mb]);
           P[mb] = T::mfma16(zop, bop, P[mb]);
         }
@@ -298,7 +286,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   // [16 waves][MB][64] partial tiles: behind the activations, or -- with three or four m-blocks, where both would not
   // fit -- on top of them once every wavefront is through its K loop
   constexpr bool RED_ALIAS = MB > 2;
-  v4f* red = reinterpret_cast<v4f*>(RED_ALIAS ? lds : lds + (size_t)KO * MR * MB * 16);
+  v4f* red = reinterpret_cast<v4f*>(RED_ALIAS ? lds : lds + (((size_t)KO * MR * MB * 16 + 1023) & ~(size_t)1023));
   if (WKS > 1) {
     if constexpr (RED_ALIAS) __syncthreads();
 #pragma unroll
@@ -378,10 +366,10 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
 // LDS of a workgroup: activations of `groups` = WKS * (groups per wavefront) quantisation groups for MR x MB rows, 16
 // spare bytes, and the reduction buffer of the K slices (on top of the activations for MB > 2, see the kernel).
 static inline size_t decode2_lds_bytes(int wks, int groups_per_wave, int mr, int mb) {
-  const size_t act = (size_t)wks * groups_per_wave * 256 * mr * mb;
+  const size_t act = ((size_t)wks * groups_per_wave * 256 * mr * mb + 1023) & ~(size_t)1023;     // padded to 1 KiB (see the fill)
   const size_t red = wks > 1 ? (size_t)D2_WAVES * mb * 1024 : 0;
-  if (mb > 2) return act + 16 > red ? act + 16 : red;
-  return act + (red ? red : 16);
+  if (mb > 2) return act > red ? act : red;
+  return act + red;
 }
 
 template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, bool W8 = false>
