@@ -36,7 +36,8 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8) 
   const int cus = num_cus_current_device();
   // K slices wanted: about 16 wavefronts per compute unit, 8 when few rows are staged (measured: with little LDS to
   // fill, longer per-wavefront tile streams beat more wavefronts on layers with few n-tiles)
-  int want = (cus * (c.mr <= 4 && NT <= 2 * cus ? 8 : D2_WAVES)) / (NT * c.sk);
+  // (also with 16 staged rows when there is at most one workgroup per compute unit: 4096 x 4096 at M = 16, 6.60 -> 6.34 us)
+  int want = (cus * ((c.mr <= 4 && NT <= 2 * cus) || NT * c.sk <= cus ? 8 : D2_WAVES)) / (NT * c.sk);
   int wks = 1;
   while (wks * 2 <= want && wks < 16) wks *= 2;
   while (wks > 1 && wks > gslab) wks /= 2;
