@@ -4,10 +4,10 @@
 //  * A workgroup is WKS slices of K  x  WN n-tiles (16 columns each) = up to 16 wavefronts.  Wavefront (wks, wn)
 //    streams the GS consecutive 1 KiB weight tiles (= quantisation groups) of its slice for its n-tile through a
 //    register ring of min(GS, 2) slots; no wavefront ever waits for another one inside the K loop.
-//  * The activations of the workgroup's K slab (WKS*GS groups) are written once to LDS in MFMA-B-operand order
-//    ([k-octet][m] 16-byte slots, rows m >= M zero, XOR-swizzled so that both the row-contiguous fill and the
-//    operand reads are bank-conflict free) and read back with one ds_read_b128 per MFMA.  The activation loads are
-//    issued before the first weight loads, in branch-free code (see step 1).  Only MR rows per m-block are staged
+//  * The activations of the workgroup's K slab (WKS*GS groups) are staged once in LDS by direct-to-LDS loads, row-major
+//    with the 16-byte chunks XOR-swizzled inside aligned 256-byte blocks (rows m >= M zero; both the 1 KiB fill
+//    pieces and the operand reads are bank-conflict free) and read back with one ds_read_b128 per MFMA.  The activation
+//    loads are issued before the first weight loads (see step 1).  Only MR rows per m-block are staged
 //    (MR = 1, 4 or 16, the smallest that holds M): MFMA columns are independent, so lanes of the columns m >= MR read
 //    the slot of row m mod MR and their results are never stored.  With few rows a whole K = 14336 slab fits LDS and
 //    K need not be split over workgroups.
@@ -85,10 +85,9 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   const int nt = nt_ok ? nt_raw : p.NT - 1;
   const int g_first = slab_g0 + wks * GS;           // this wavefront's first group
 
-  // ---- 1. activations of the K slab -> LDS, with the first R weight tiles requested in between ----
+  // ---- 1. activations of the K slab -> LDS, then the first R weight tiles requested ----
   // Loads retire in issue order as far as the wait counter is concerned, so the activation loads go out FIRST: the
-  // wait before the LDS writes then leaves the weight tiles in flight instead of draining them.
-  // slot (16 bytes) of (m-block mb, row ml, k-octet ko):  mb*KO*MR + ko*MR + (ml ^ (ko & (MR-1)))
+  // wait before the barrier then leaves the weight tiles in flight instead of draining them.
   const __amdgpu_buffer_rsrc_t rb = d2_rsrc(p.b, (uint64_t)p.K * p.N / 2 * TPG);
   const __amdgpu_buffer_rsrc_t rs = d2_rsrc(p.scales, (uint64_t)p.GR * p.N * 2);
   const __amdgpu_buffer_rsrc_t rz = d2_rsrc(HAS_ZP ? (const void*)p.zeros : (const void*)p.scales, (uint64_t)p.GR * (p.N / 8) * 4);
