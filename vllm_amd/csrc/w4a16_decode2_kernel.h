@@ -68,8 +68,10 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   // Ring slots.  Two tiles in flight per wavefront measured best: a wavefront does not get past its load instructions
   // until the memory pipeline has accepted them, and with deeper rings (every wavefront of the device asking for
   // 7-8 KiB at once) the first MFMA of each wavefront starts when most of the stream has already been served, so the
-  // arithmetic no longer overlaps it.
-  constexpr int R = GS < 2 ? GS : 2;
+  // arithmetic no longer overlaps it.  Exception: 16 staged rows and a long stream (K = 14336 at M = 5 .. 16) -- the
+  // activation fill then takes 2 us during which nothing else is requested, and four tiles in flight fill that gap
+  // (the 12-GEMM decode step 1.4 % faster; four slots for 1 or 4 staged rows: 0.8 % slower).
+  constexpr int R = (MR == 16 && MB == 1 && GS >= 7) ? 4 : (GS < 2 ? GS : 2);
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
   const int lane = threadIdx.x;
