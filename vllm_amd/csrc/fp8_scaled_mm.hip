@@ -54,6 +54,7 @@ constexpr int F8_PITCH = 144;    // LDS row pitch in bytes
 // 8-byte store, one scale load per row, one 16-byte load of the channel scales.
 template <bool BF16_OUT, int WMB, int WNB>
 __device__ inline void tile_epilogue(const Fp8MMParams& p, v16f (&acc)[WMB][WNB], int m0, int n0, int wm, int wn, int lane) {
+#pragma clang fp contract(off)      // sa * (sb * acc), then + bias: two fp32 roundings, like the oracle's separate operations
   using T = F16Traits<BF16_OUT>;
   // Every scale and bias value this lane needs is requested before the first store: a load that follows a store to
   // memory it might alias cannot be moved above it, and the epilogue would pay one memory latency per 8-byte store.
@@ -115,6 +116,7 @@ __device__ inline void tile_epilogue(const Fp8MMParams& p, v16f (&acc)[WMB][WNB]
 template <bool BF16_OUT, int WMB, int WNB>
 __device__ inline void tile_epilogue_lds(const Fp8MMParams& p, v16f (&acc)[WMB][WNB], int m0, int n0, int wm, int wn, int lane,
                                          uint8_t* wave_lds) {
+#pragma clang fp contract(off)      // sa * (sb * acc), then + bias: two fp32 roundings, like the oracle's separate operations
   using T = F16Traits<BF16_OUT>;
   constexpr int PITCH = WNB * 64 + 16;
   constexpr int CPR = WNB * 4;                 // 16-byte chunks per row
@@ -729,6 +731,7 @@ __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p,
         const v4f val = (WK > 1) ? tot : acc[mb];
         const int m = mb * 16 + r16;
         if (m < p.M) {
+#pragma clang fp contract(off)      // sa * (sb * acc), then + bias: two fp32 roundings, like the tile kernels
           const int n = nt * 16 + q * 4;
           const float sam = p.sa[p.sa_per_row ? m : 0];
           float o[4];
