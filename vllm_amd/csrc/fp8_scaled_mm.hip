@@ -802,8 +802,10 @@ struct Fp8TilePlan {
 };
 
 // Tile shape and K split of the multi-stage kernel.  K is split when the output tiles alone leave compute units idle:
-// as many workgroups as fit the device at once (one or two per compute unit), at most 8 splits, each at least 64 steps (4096 bytes of K) long -- measured at
-// M = 256: the FP8 steps are short, so the hand-over only pays on a long K (1.35x on K = 14336, a loss on K = 4096).
+// as many workgroups as fit the device at once (one or two per compute unit), at most 8 splits, each at least 64 steps
+// (4096 bytes of K) long, 32 steps when the tiles leave three quarters of the device idle -- measured with cold weights:
+// 14336 x 4096 at M = 48 / 128 47.7 -> 34.7 / 35.5 us with 4 splits, 4096 x 4096 at M = 48 .. 128 24.4 -> 20.6 us with
+// 2; with more tiles the shorter parts lose (14336 x 4096 at M = 256: 4 splits 50.5 us, 2 splits 48.7 us).
 static Fp8TilePlan plan_tile3(int M, int N, int K) {
   const int cus = num_cus_current_device();
   auto tiles = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
@@ -828,9 +830,10 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   const int steps = K / 64;
   if (pl.tiles < cus) {
     const int per_cu = pl.bm * pl.bn >= 128 * 256 ? 1 : 2;      // workgroups of this tile shape that share a compute unit
+    const int min_steps = pl.tiles * 4 <= cus ? 32 : 64;        // shorter parts only when the tiles leave 3/4 of the device idle
     sk = (int)((per_cu * (int64_t)cus) / pl.tiles);
     if (sk > 8) sk = 8;
-    if (sk > steps / 64) sk = steps / 64;
+    if (sk > steps / min_steps) sk = steps / min_steps;
     if (sk < 1) sk = 1;
     while (sk & (sk - 1)) --sk;       // a power of two (3 splits measured slower than 2)
   }
@@ -891,16 +894,23 @@ static void launch_stream(const Fp8MMParams& p, int wk, int gx, hipStream_t s) {
   hipLaunchKernelGGL((fp8_mm_stream_kernel<BF16_OUT, KS, MB>), dim3(gx), dim3(64, wk), lds, s, p, wk);
 }
 
+// K steps (of 128) per wavefront of the stream kernel for a problem, 0 if the kernel does not take it (the activations of
+// a wavefront's K slab live in registers: at most 8 wavefronts along K, 14 steps each for one m-block, 8 for two).
+static int stream_steps_per_wave(int64_t M, int64_t K) {
+  const int64_t steps = (K + 127) / 128;
+  if (M > 32) return 0;
+  if (steps <= 8 * 4) return 4;
+  if (steps <= 8 * 8) return 8;
+  if (steps <= 8 * 14 && M <= 16) return 14;
+  return 0;
+}
+
 template <bool BF16_OUT>
 static bool dispatch_stream(const Fp8MMParams& p, hipStream_t s) {
   const int steps = (p.K + 127) / 128;
   const int MB = p.M <= 16 ? 1 : 2;
-  // wavefronts along K: at most 8; per-wave slab of KS steps
-  int ks;
-  if (steps <= 8 * 4) ks = 4;
-  else if (steps <= 8 * 8) ks = 8;
-  else if (steps <= 8 * 14 && MB == 1) ks = 14;
-  else return false;
+  const int ks = stream_steps_per_wave(p.M, p.K);
+  if (ks == 0) return false;
   const int wk = (steps + ks - 1) / ks;
   const int NT = p.N / 16;
   int gx = g_force_fp8_gx > 0 ? g_force_fp8_gx : 2 * num_cus_current_device();
@@ -927,7 +937,8 @@ extern "C" int vaq_fp8_scaled_mm_workspace(int64_t size_m, int64_t size_n, int64
                 (long long)size_n, (long long)size_k);
   *c_tmp_bytes = 0;
   *counter_ints = 0;
-  if (size_m <= 32 || size_k % 64 != 0 || g_fp8_tile_impl != 0 || g_fp8_tile3_cfg < 0) return VAQ_OK;
+  const bool stream = g_force_fp8_path != 2 && stream_steps_per_wave(size_m, size_k) != 0;      // needs no scratch
+  if (stream || size_k % 64 != 0 || g_fp8_tile_impl != 0 || g_fp8_tile3_cfg < 0) return VAQ_OK;
   const Fp8TilePlan pl = plan_tile3((int)size_m, (int)size_n, (int)size_k);
   if (pl.sk > 1) {
     *c_tmp_bytes = (size_t)pl.sk * (size_t)pl.tiles * pl.bm * pl.bn * sizeof(float);
