@@ -7,7 +7,7 @@
 //  * tile kernel (any M): one workgroup of 4 wavefronts (2 x 2) per BM x BN output tile, K walked in steps of 128
 //    bytes through double-buffered, padded LDS (pitch 144 B), v_mfma_f32_32x32x64_f8f6f4 (the full-rate gfx950 FP8
 //    instruction, 32 bytes per lane per operand);
-//  * stream kernel (M <= 32): weight-streaming GEMV-like kernel, weights are the A operand of
+//  * stream kernel (M <= 32; M <= 64 on narrow layers with K <= 4096): weight-streaming GEMV-like kernel, weights are the A operand of
 //    v_mfma_f32_16x16x128_f8f6f4 straight from global memory, activations stay in registers, the wavefronts of a
 //    workgroup split K and reduce through LDS.
 //
@@ -653,7 +653,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
     tile_epilogue<BF16_OUT, WMB, WNB>(p, acc, m0, n0, wm, wn, lane);
 }
 
-// ----------------------------------------------------------------------------- stream kernel (M <= 32)
+// ----------------------------------------------------------------------------- stream kernel (M <= 32, narrow layers M <= 64)
 // blockDim = (64, WK).  Wavefront w owns K steps [w*KS, (w+1)*KS) of 128 bytes; activations of that slab live in
 // registers for the whole kernel; the workgroup walks a contiguous range of 16-row weight tiles.
 template <bool BF16_OUT, int KS, int MB>
@@ -896,9 +896,12 @@ static void launch_stream(const Fp8MMParams& p, int wk, int gx, hipStream_t s) {
 
 // K steps (of 128) per wavefront of the stream kernel for a problem, 0 if the kernel does not take it (the activations of
 // a wavefront's K slab live in registers: at most 8 wavefronts along K, 14 steps each for one m-block, 8 for two).
-static int stream_steps_per_wave(int64_t M, int64_t K) {
+static int stream_steps_per_wave(int64_t M, int64_t N, int64_t K) {
   const int64_t steps = (K + 127) / 128;
-  if (M > 32) return 0;
+  // three and four m-blocks: K = 1664 .. 4096 (4 steps per wavefront keep the registers, and the workgroup must have a
+  // wavefront per m-block for the reduction), and only where a workgroup gets one n-tile (measured, cold weights, M = 48 /
+  // 64: 4096 x 4096 21.0 / 21.4 -> 11.6 / 13.4 us; 4096 x 6144 no gain / a loss, 4096 x 28672 36 -> 43 / 47 us)
+  if (M > 32) return (M <= 64 && steps <= 8 * 4 && steps >= 13 && N / 16 <= num_cus_current_device()) ? 4 : 0;
   if (steps <= 8 * 4) return 4;
   if (steps <= 8 * 8) return 8;
   if (steps <= 8 * 14 && M <= 16) return 14;
@@ -908,8 +911,8 @@ static int stream_steps_per_wave(int64_t M, int64_t K) {
 template <bool BF16_OUT>
 static bool dispatch_stream(const Fp8MMParams& p, hipStream_t s) {
   const int steps = (p.K + 127) / 128;
-  const int MB = p.M <= 16 ? 1 : 2;
-  const int ks = stream_steps_per_wave(p.M, p.K);
+  const int MB = (p.M + 15) / 16;
+  const int ks = stream_steps_per_wave(p.M, p.N, p.K);
   if (ks == 0) return false;
   const int wk = (steps + ks - 1) / ks;
   const int NT = p.N / 16;
@@ -919,9 +922,13 @@ static bool dispatch_stream(const Fp8MMParams& p, hipStream_t s) {
     if (ks == 4) launch_stream<BF16_OUT, 4, 1>(p, wk, gx, s);
     else if (ks == 8) launch_stream<BF16_OUT, 8, 1>(p, wk, gx, s);
     else launch_stream<BF16_OUT, 14, 1>(p, wk, gx, s);
-  } else {
+  } else if (MB == 2) {
     if (ks == 4) launch_stream<BF16_OUT, 4, 2>(p, wk, gx, s);
     else launch_stream<BF16_OUT, 8, 2>(p, wk, gx, s);
+  } else if (MB == 3) {
+    launch_stream<BF16_OUT, 4, 3>(p, wk, gx, s);
+  } else {
+    launch_stream<BF16_OUT, 4, 4>(p, wk, gx, s);
   }
   return true;
 }
@@ -937,7 +944,7 @@ extern "C" int vaq_fp8_scaled_mm_workspace(int64_t size_m, int64_t size_n, int64
                 (long long)size_n, (long long)size_k);
   *c_tmp_bytes = 0;
   *counter_ints = 0;
-  const bool stream = g_force_fp8_path != 2 && stream_steps_per_wave(size_m, size_k) != 0;      // needs no scratch
+  const bool stream = g_force_fp8_path != 2 && stream_steps_per_wave(size_m, size_n, size_k) != 0;      // needs no scratch
   if (stream || size_k % 64 != 0 || g_fp8_tile_impl != 0 || g_fp8_tile3_cfg < 0) return VAQ_OK;
   const Fp8TilePlan pl = plan_tile3((int)size_m, (int)size_n, (int)size_k);
   if (pl.sk > 1) {
@@ -996,8 +1003,8 @@ extern "C" int vaq_fp8_scaled_mm_ws(const uint8_t* a, int64_t lda, const uint8_t
   hipStream_t s = (hipStream_t)stream;
   const bool bf16 = out_dtype == VAQ_BF16;
   bool done = false;
-  const bool want_stream = g_force_fp8_path == 1 || (g_force_fp8_path == 0 && size_m <= 32);
-  if (want_stream && size_m <= 32) done = bf16 ? dispatch_stream<true>(p, s) : dispatch_stream<false>(p, s);
+  const bool want_stream = g_force_fp8_path != 2 && stream_steps_per_wave(size_m, size_n, size_k) != 0;
+  if (want_stream) done = bf16 ? dispatch_stream<true>(p, s) : dispatch_stream<false>(p, s);
   if (!done) {
     int rc = bf16 ? dispatch_tile<true>(p, c_tmp_bytes, counter_ints, s) : dispatch_tile<false>(p, c_tmp_bytes, counter_ints, s);
     if (rc != VAQ_OK) return rc;
