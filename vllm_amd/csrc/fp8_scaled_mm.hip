@@ -36,6 +36,7 @@ struct Fp8MMParams {
   float* c_tmp = nullptr;        // fp32 partial tiles when K is split over workgroups (SK > 1)
   int32_t* counters = nullptr;   // arrival counters, zero on entry, left zero
   int SK = 1;
+  int rotate_k = 0;              // multi-stage tile kernel: tile rows start their K loop at different places (see the kernel)
 };
 
 __device__ inline v16f mfma_fp8_32(v8i a, v8i b, v16f c) {
@@ -438,7 +439,21 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
   const uint32_t voff_b = (uint32_t)lrow * (uint32_t)p.ldb + (uint32_t)(c16 & 3) * 16u;
 
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
-  auto issue_loads = [&](int step, int stage) {
+  // K may be split over blockIdx.y: this workgroup covers the steps [s_lo, s_hi)
+  const int all_steps = p.K / (64 * KS);
+  const int split = blockIdx.y;
+  const int s_lo = (int)(((int64_t)all_steps * split) / p.SK), s_hi = (int)(((int64_t)all_steps * (split + 1)) / p.SK);
+  const int steps = s_hi - s_lo;
+  // Few tile rows (M at most 4 tiles high) on a device that the tiles do not fill: the tiles of one column would read
+  // the same weight rows at the same time, which leaves only (ring depth x 64 KS) bytes per weight row in flight --
+  // with cold weights the kernel then runs at a fraction of the memory bandwidth.  Tile row tm starts its K loop
+  // tm / tiles_m of the way into its range and wraps around: the rows are read at tiles_m places at once, and the later
+  // readers find them in the L2 (4096 x 4096 at M = 256, cold: 24.4 -> 18.3 us).
+  const int rot = p.rotate_k ? (tm * steps) / tiles_m : 0;
+  auto issue_loads = [&](int step_in, int stage) {
+    int step = step_in - s_lo + rot;
+    if (step >= steps) step -= steps;
+    step += s_lo;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       uint8_t* Ab = lds8 + (size_t)stage * STAGE + ks * SLICE;
@@ -511,11 +526,6 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
 
   // Invariant at the start of step s: the tile of step s complete in LDS, the tiles of steps s+1 .. s+NST-2 requested,
   // stage (s-1) % NST free.  The requests of step s+NST-1 go out first thing in step s.
-  // K may be split over blockIdx.y: this workgroup covers the steps [s_lo, s_hi)
-  const int all_steps = p.K / (64 * KS);
-  const int split = blockIdx.y;
-  const int s_lo = (int)(((int64_t)all_steps * split) / p.SK), s_hi = (int)(((int64_t)all_steps * (split + 1)) / p.SK);
-  const int steps = s_hi - s_lo;
   if (PP != 0 && steps >= NST) {
     // Alternating phases: the two wavefronts that share a SIMD run half a step apart, so that one reads its fragments
     // (and requests tiles) while the other one issues its MFMAs.  A step is [requests, fragment reads, wait] barrier
@@ -855,6 +865,11 @@ static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t c
                       c_tmp_bytes < (int64_t)pl.sk * pl.tiles * pl.bm * pl.bn * 4))
       pl.sk = 1;
     p.SK = pl.sk;
+    {
+      const int64_t tiles_m = (p.M + pl.bm - 1) / pl.bm;
+      // (with K split over workgroups the rotation gains nothing on cold weights and costs 20-30 % on cached ones)
+      p.rotate_k = pl.sk == 1 && tiles_m > 1 && tiles_m <= 4 && pl.tiles * 5 < (int64_t)num_cus_current_device() * 4;
+    }
     switch (pl.cfg) {
       case 1: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 5, 1, 1>(p, s);   // alternating phases (see the kernel)
       case 8: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 5>(p, s);
