@@ -821,10 +821,12 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   auto tiles = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   Fp8TilePlan pl;
   pl.cfg = g_fp8_tile3_cfg;
+  // the largest tile shape that fills 70 % of the compute units (measured on the Llama shapes, M = 256 .. 4096: a
+  // partly filled device of large tiles beats a full one of small tiles by 25-40 %); for 128 x 128 also when two
+  // parts of a long K get it there (14336 x 4096 at M = 512, cold, 73 -> 62 us)
+  const int parts128 = K / 64 >= 128 ? 2 : 1;
   if (pl.cfg <= 0)
-    // the largest tile shape that fills 70 % of the compute units (measured on the Llama shapes, M = 256 .. 4096: a
-    // partly filled device of large tiles beats a full one of small tiles by 25-40 %)
-    pl.cfg = tiles(256, 256) * 10 >= cus * 7 ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (tiles(128, 128) * 10 >= cus * 7 ? 3 : 4));
+    pl.cfg = tiles(256, 256) * 10 >= cus * 7 ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (tiles(128, 128) * parts128 * 10 >= cus * 7 ? 3 : 4));
   // the smallest tile with two k-slices per step: 5-8 % faster on a short K (half the barriers), no gain on a long one
   if (g_fp8_tile3_cfg <= 0 && pl.cfg == 4 && K % 128 == 0 && K <= 8192) pl.cfg = 14;
   if (pl.cfg >= 10 && K % 128 != 0) pl.cfg %= 10;      // two k-slices per step need K % 128 == 0
