@@ -21,16 +21,17 @@ constexpr int64_t DECODE_MAX_M = 64;          // up to four m-blocks of 16 rows 
 constexpr int64_t DECODE_MAX_M_2BLK = 32;     // the register-resident kernel, groups below 128 rows and 8-bit codes: two
 static int g_decode_impl = -1;  // -1: automatic, 0: LDS-staged activations (w4a16_decode2.hip), 1: register-resident (w4a16_decode.hip)
 
-// Measured on MI355X (Llama-3-8B shapes): staging the activations once per workgroup in LDS (one independent task
-// per wavefront, no barrier in the K loop) wins everywhere except for 2 < M <= 16 on wide layers (many n-tiles per compute
-// unit), where the register-resident kernel, whose wavefronts walk over n-tiles with their slice of the activations
-// held in registers, is slightly ahead.
+// Measured on MI355X (cold weights): staging the activations once per workgroup in LDS (one independent task per
+// wavefront, no barrier in the K loop) wins on every Llama-3-8B projection and on 8192 x 28672 (30 us against 43.5 us
+// for 3 <= M <= 16).  The register-resident kernel, whose wavefronts walk over n-tiles with their slice of the
+// activations held in registers, stays ahead only on a vocabulary-sized layer (4096 x 128256, 3 <= M <= 16: 55 us
+// against 62 us).
 static int decode_impl_for(int64_t size_m, int64_t size_n, int64_t lda, int sub, bool w8) {
   // the LDS-staged kernel addresses A through a 32-bit buffer offset
   if (size_m * lda * 2 >= (1ll << 31)) return 1;
   if (sub > 1 || w8) return 0;    // groups below 128 rows and 8-bit codes are built for the LDS-staged kernel only
   if (g_decode_impl >= 0) return g_decode_impl;
-  return (size_n <= 8192 || size_m <= 2 || size_m > 16) ? 0 : 1;
+  return (size_n >= 65536 && size_m > 2 && size_m <= 16) ? 1 : 0;
 }
 
 static int check_shape(int64_t size_m, int64_t size_n, int64_t size_k) {
