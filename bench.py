@@ -37,10 +37,10 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes moved per algorithmic byte over the 12 headline GEMMs, from two hardware-counter runs of
 # `bench.py --counter-pass` (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same counter reads for the 256 MiB
 # copy in that run (FETCH_SIZE reads 131083.5 for 262144 KiB -> x2.000, WRITE_SIZE reads 262144.0 -> x1.000):
-# fetch 361.56 MB + write 2.90 MB = 364.46 MB against 340.30 MB algorithmic.  The excess is about 10 % on the fetch
+# fetch 361.52 MB + write 2.90 MB = 364.42 MB against 340.30 MB algorithmic.  The excess is about 10 % on the fetch
 # side of every small layer (its size matches a 128-byte line of a scale row, which spans four 16-column tiles, being
 # fetched by each of the four XCDs those tiles' workgroups run on), the fp32 split-K partials of the K=14336, M=16 case, and activation re-reads at M=16.
-MEASURED_TRAFFIC_PER_ALGORITHMIC_BYTE = 364.46 / 340.30
+MEASURED_TRAFFIC_PER_ALGORITHMIC_BYTE = 364.42 / 340.30
 BF16_PEAK_TFLOPS = 2500.0
 FP8_PEAK_TFLOPS = 5000.0
 GROUP = 128
@@ -551,7 +551,7 @@ def main():
                                "(14336,4096)} x M in {1,4,16}, group 128, symmetric int4, bf16 act, fp32 acc; one step = "
                                "12 GEMMs in a HIP graph, weights cold (650 MB cycling)",
                    "launches_per_step": launches},
-        "roofline": {"bound": "hbm", "kernel": "vaq::w4a16_decode2_kernel / vaq::w4a16_decode_kernel", "achieved": round(value, 2), "peak": HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": "vaq::w4a16_decode2_kernel", "achieved": round(value, 2), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(value / HBM_PEAK_GBS, 4),
                      "traffic": int(MEASURED_TRAFFIC_PER_ALGORITHMIC_BYTE * step_bytes / launches),
                      "avg_launch_us": round(sec * 1e6 / launches, 3),
