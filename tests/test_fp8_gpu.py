@@ -243,17 +243,23 @@ def test_scaled_mm_exact_small_integers(device):
 @pytest.mark.parametrize("m", [17, 32, 33, 40, 48, 49, 64, 65])
 def test_scaled_mm_small_m_every_route_exact(device, m):
     """M around the switch points of the small-M routes: the weight-streaming kernel with one to four blocks of 16
-    rows (three and four only for K = 1664 .. 4096 on narrow layers), the tile kernel with K split over workgroups for
-    a K beyond it (also at M <= 32) and without a split.  Small-integer operands: the result must equal the integer GEMM;
-    the arrival counters of the splits must be back at zero."""
+    rows (three for K = 1664 .. 4096, four only up to two rounds of workgroups), with one and with several n-tiles per
+    workgroup, the tile kernel with K split over workgroups for a K beyond it (also at M <= 32) and without a split.
+    Small-integer operands, power-of-two scales and an integer bias: the result must equal the integer GEMM, scaled and
+    shifted, rounded once to bf16; the arrival counters of the splits must be back at zero."""
     import vllm_amd._custom_ops as ops
     g = torch.Generator().manual_seed(m)
-    for n, k in ((128, 1664), (256, 4096), (4096, 2048), (4112, 2048), (64, 1536), (128, 14336), (4096, 8192 + 128), (48, 4224)):
+    for n, k in ((128, 1664), (256, 4096), (4096, 2048), (4112, 2048), (8208, 1664), (64, 1536), (128, 14336),
+                 (4096, 8192 + 128), (48, 4224)):
         a = torch.randint(-2, 3, (m, k), generator=g).float()
         w = torch.randint(-1, 2, (n, k), generator=g).float()
+        sa = torch.pow(2.0, -(torch.arange(m) % 2).float()).reshape(m, 1)
+        sb = torch.pow(2.0, (torch.arange(n) % 3).float()).reshape(n, 1)
+        bias = (torch.arange(n) % 5).float()
         out = ops.cutlass_scaled_mm(a.to(torch.float8_e4m3fn).to(device), w.to(torch.float8_e4m3fn).to(device).t(),
-                                    torch.ones(m, 1, device=device), torch.ones(n, 1, device=device), torch.bfloat16)
-        assert torch.equal(out.cpu().float(), (a @ w.t()).to(torch.bfloat16).float()), (m, n, k)
+                                    sa.to(device), sb.to(device), torch.bfloat16, bias.to(torch.bfloat16).to(device))
+        want = (sa * (sb.t() * (a @ w.t())) + bias).to(torch.bfloat16)
+        assert torch.equal(out.cpu().float(), want.float()), (m, n, k)
     assert bool((ops._fp8_counters(torch.device(device)) == 0).all()), "arrival counters not restored to zero"
 
 

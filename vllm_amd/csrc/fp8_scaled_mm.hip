@@ -709,11 +709,38 @@ __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p,
     for (int s = 0; s < KS; ++s) issue(nt0, s);
   }
 
+  // Epilogue operands are requested ahead of their use (a load issued after the reduction would stall the reducing
+  // wavefront, and through the next barrier the whole workgroup, for a memory round trip per n-tile): the activation
+  // scales once per kernel, the weight scales and the bias of an n-tile before its MFMAs.  With 14 steps per wavefront
+  // there are no registers to spare for that and a workgroup has a single n-tile anyway.
+  constexpr bool AHEAD = KS < 14;
+  const bool reducer_wave = WK > 1 ? w < MB : true;
+  float sam_mb[MB];
+  if constexpr (AHEAD) {
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int m = mb * 16 + r16;
+      sam_mb[mb] = (reducer_wave && m < p.M) ? p.sa[p.sa_per_row ? m : 0] : 0.f;
+    }
+  }
+
   int parity = 0;
   for (int nt = nt0; nt < nt1; ++nt) {
     v4f acc[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[mb] = v4f{0.f, 0.f, 0.f, 0.f};
+    float sb_r[4] = {0.f, 0.f, 0.f, 0.f};
+    uint16_t bias_r[4] = {0, 0, 0, 0};
+    if constexpr (AHEAD) {
+      if (reducer_wave) {
+        const int n = nt * 16 + q * 4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          sb_r[r] = p.sb[p.sb_per_col ? n + r : 0];
+          if (p.bias) bias_r[r] = p.bias[n + r];
+        }
+      }
+    }
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       const v8i aop = v8i{wlo[s].x, wlo[s].y, wlo[s].z, wlo[s].w, whi[s].x, whi[s].y, whi[s].z, whi[s].w};
@@ -737,24 +764,48 @@ __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p,
     }
     if (reducer) {
       const int mb_lo = (WK > 1) ? w : 0, mb_hi = (WK > 1) ? w + 1 : MB;
-      for (int mb = mb_lo; mb < mb_hi; ++mb) {
+      auto emit = [&](int mb, float sam, const float* sbv, const uint16_t* bsv) {
         const v4f val = (WK > 1) ? tot : acc[mb];
         const int m = mb * 16 + r16;
         if (m < p.M) {
 #pragma clang fp contract(off)      // sa * (sb * acc), then + bias: two fp32 roundings, like the tile kernels
           const int n = nt * 16 + q * 4;
-          const float sam = p.sa[p.sa_per_row ? m : 0];
           float o[4];
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const float sbn = p.sb[p.sb_per_col ? n + r : 0];
-            o[r] = sam * (sbn * val[r]);
-            if (p.bias) o[r] += T::to_float(p.bias[n + r]);
+            o[r] = sam * (sbv[r] * val[r]);
+            if (p.bias) o[r] += T::to_float(bsv[r]);
           }
           v2u ov;
           ov.x = (uint32_t)T::from_float(o[0]) | ((uint32_t)T::from_float(o[1]) << 16);
           ov.y = (uint32_t)T::from_float(o[2]) | ((uint32_t)T::from_float(o[3]) << 16);
           *reinterpret_cast<v2u*>(p.out + (int64_t)m * p.ldc + n) = ov;
+        }
+      };
+      if constexpr (AHEAD) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)       // unrolled: sam_mb stays in registers
+          if (mb >= mb_lo && mb < mb_hi) emit(mb, sam_mb[mb], sb_r, bias_r);
+      } else {
+        for (int mb = mb_lo; mb < mb_hi; ++mb) {
+          const v4f val = (WK > 1) ? tot : acc[mb];
+          const int m = mb * 16 + r16;
+          if (m < p.M) {
+#pragma clang fp contract(off)
+            const int n = nt * 16 + q * 4;
+            const float sam = p.sa[p.sa_per_row ? m : 0];
+            float o[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const float sbn = p.sb[p.sb_per_col ? n + r : 0];
+              o[r] = sam * (sbn * val[r]);
+              if (p.bias) o[r] += T::to_float(p.bias[n + r]);
+            }
+            v2u ov;
+            ov.x = (uint32_t)T::from_float(o[0]) | ((uint32_t)T::from_float(o[1]) << 16);
+            ov.y = (uint32_t)T::from_float(o[2]) | ((uint32_t)T::from_float(o[3]) << 16);
+            *reinterpret_cast<v2u*>(p.out + (int64_t)m * p.ldc + n) = ov;
+          }
         }
       }
     }
@@ -916,9 +967,13 @@ static void launch_stream(const Fp8MMParams& p, int wk, int gx, hipStream_t s) {
 static int stream_steps_per_wave(int64_t M, int64_t N, int64_t K) {
   const int64_t steps = (K + 127) / 128;
   // three and four m-blocks: K = 1664 .. 4096 (4 steps per wavefront keep the registers, and the workgroup must have a
-  // wavefront per m-block for the reduction), and only where a workgroup gets one n-tile (measured, cold weights, M = 48 /
-  // 64: 4096 x 4096 21.0 / 21.4 -> 11.6 / 13.4 us; 4096 x 6144 no gain / a loss, 4096 x 28672 36 -> 43 / 47 us)
-  if (M > 32) return (M <= 64 && steps <= 8 * 4 && steps >= 13 && N / 16 <= num_cus_current_device()) ? 4 : 0;
+  // wavefront per m-block for the reduction).  Measured against the tile kernel with K split, cold weights, M = 48 / 64:
+  // 4096 x 4096 21.0 / 21.4 -> 11.6 / 13.4 us, 4096 x 6144 22.7 / 22.9 -> 14.6 / 16.5 us, 4096 x 28672 36.3 / 37.3 ->
+  // 35.9 / 38.7 us: four m-blocks only up to two rounds of workgroups.
+  if (M > 32) {
+    const bool fits = steps <= 8 * 4 && steps >= 13;
+    return (fits && (M <= 48 || (M <= 64 && N / 16 <= 2 * num_cus_current_device()))) ? 4 : 0;
+  }
   if (steps <= 8 * 4) return 4;
   if (steps <= 8 * 8) return 8;
   if (steps <= 8 * 14 && M <= 16) return 14;
@@ -933,7 +988,13 @@ static bool dispatch_stream(const Fp8MMParams& p, hipStream_t s) {
   if (ks == 0) return false;
   const int wk = (steps + ks - 1) / ks;
   const int NT = p.N / 16;
-  int gx = g_force_fp8_gx > 0 ? g_force_fp8_gx : 2 * num_cus_current_device();
+  // one workgroup per compute unit, the n-tiles dealt out evenly over the fewest rounds: every workgroup loads all the
+  // activations of its K slabs, so more workgroups than compute units only multiply that traffic (measured, cold weights,
+  // against two workgroups per compute unit: 4096 x 6144 at M = 16 / 32 11.9 / 16.4 -> 10.4 / 12.4 us, 4096 x 28672
+  // 31.8 / 38.0 -> 30.4 / 31.9 us, M = 1 unchanged or 3 % faster)
+  const int cus = num_cus_current_device();
+  const int rounds = (NT + cus - 1) / cus;
+  int gx = g_force_fp8_gx > 0 ? g_force_fp8_gx : (NT + rounds - 1) / rounds;
   if (gx > NT) gx = NT;
   if (MB == 1) {
     if (ks == 4) launch_stream<BF16_OUT, 4, 1>(p, wk, gx, s);
