@@ -187,8 +187,8 @@ int vaq_silu_and_mul_fp8_quant(uint8_t* out, const void* input, const float* sca
 
 /*
  * The same GEMM with caller-provided scratch, which lets the tile kernel split K over workgroups when M and N alone
- * leave compute units idle (up to a few hundred tokens on the narrow layers; also 17 .. 32 tokens when K is beyond
- * 8192, which the weight-streaming kernel does not take).  Sizes come from the query; both may be 0.
+ * leave compute units idle (up to a few hundred tokens on the narrow layers), and the weight-streaming kernel run
+ * 17 .. 32 tokens with K beyond 8192 (up to 16384) as two halves of K.  Sizes come from the query; both may be 0.
  *   c_tmp     fp32 partial tiles, 16-byte aligned, contents irrelevant on entry
  *   counters  int32 arrival counters that must be ZERO on entry and are left zero (calls sharing them must not overlap)
  * With NULL / too small scratch the call behaves exactly like vaq_fp8_scaled_mm.  (The reference's cutlass_scaled_mm has

@@ -240,17 +240,18 @@ def test_scaled_mm_exact_small_integers(device):
         assert torch.equal(out.cpu().float(), a @ w.t()), (m, n, k)
 
 
-@pytest.mark.parametrize("m", [17, 32, 33, 40, 48, 49, 64, 65])
+@pytest.mark.parametrize("m", [1, 16, 17, 32, 33, 40, 48, 49, 64, 65])
 def test_scaled_mm_small_m_every_route_exact(device, m):
     """M around the switch points of the small-M routes: the weight-streaming kernel with one to four blocks of 16
     rows (three for K = 1664 .. 4096, four only up to two rounds of workgroups), with one and with several n-tiles per
-    workgroup, the tile kernel with K split over workgroups for a K beyond it (also at M <= 32) and without a split.
+    workgroup, the same kernel over two halves of K with a hand-over (16 < M <= 32 up to K = 16384),
+    the tile kernel with K split over workgroups for a K beyond it (also at M <= 32) and without a split.
     Small-integer operands, power-of-two scales and an integer bias: the result must equal the integer GEMM, scaled and
     shifted, rounded once to bf16; the arrival counters of the splits must be back at zero."""
     import vllm_amd._custom_ops as ops
     g = torch.Generator().manual_seed(m)
     for n, k in ((128, 1664), (256, 4096), (4096, 2048), (4112, 2048), (8208, 1664), (64, 1536), (128, 14336),
-                 (4096, 8192 + 128), (48, 4224)):
+                 (4096, 8192 + 128), (48, 4224), (128, 28672), (4112, 14336 + 256), (64, 16384 + 128)):
         a = torch.randint(-2, 3, (m, k), generator=g).float()
         w = torch.randint(-1, 2, (n, k), generator=g).float()
         sa = torch.pow(2.0, -(torch.arange(m) % 2).float()).reshape(m, 1)

@@ -672,7 +672,9 @@ __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p,
   extern __shared__ v4f red[];   // [2][WK][MB][64]
   const int lane = threadIdx.x, w = threadIdx.y;
   const int q = lane >> 4, r16 = lane & 15;
-  const int kbase = w * KS * 128 + q * 32;
+  // gridDim.y = 2: the K range is split over two workgroups (the second starts where the slabs of the first end);
+  // their partial tiles are summed by whichever arrives last (see the hand-over below)
+  const int kbase = ((int)blockIdx.y * WK + w) * KS * 128 + q * 32;
 
   v8i breg[KS][MB];
 #pragma unroll
@@ -778,6 +780,34 @@ __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p,
     } else {
       reducer = true;
     }
+    if (gridDim.y > 1 && reducer) {
+      // Hand-over as in the tile kernel: the partial tile goes out in device-scope 16-byte stores, one arrival counter
+      // per (n-tile, m-block); the workgroup that arrives last adds the parts in the order of the K halves and returns the
+      // counter to zero.  (WK > 1 always here: the host splits only a long K.)
+      constexpr int SC1 = 16;
+      const uint32_t units = (uint32_t)NT * (uint32_t)MB;
+      const uint32_t unit = (uint32_t)nt * (uint32_t)MB + (uint32_t)w;
+      const __amdgpu_buffer_rsrc_t rt =
+          __builtin_amdgcn_make_buffer_rsrc(p.c_tmp, 0, (int)(units * gridDim.y * 1024u), 0x00020000);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, tot), rt, lane * 16,
+                                             (int)((blockIdx.y * units + unit) * 1024u), SC1);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // partial tile acknowledged before the counter moves
+      int32_t* ctr = p.counters + unit;
+      int old = 0;
+      if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      old = __shfl(old, 0);
+      if (old != (int)gridDim.y - 1) {
+        reducer = false;
+      } else {
+        v4f sum = {0.f, 0.f, 0.f, 0.f};
+        for (uint32_t h = 0; h < gridDim.y; ++h) {
+          const v4u r = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)((h * units + unit) * 1024u), SC1);
+          sum += __builtin_bit_cast(v4f, r);
+        }
+        tot = sum;
+        if (lane == 0) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
     if (reducer) {
       const int mb_lo = (WK > 1) ? w : 0, mb_hi = (WK > 1) ? w + 1 : MB;
       auto emit = [&](int mb, float sam, const float* sbv, const uint16_t* bsv) {
@@ -808,6 +838,7 @@ __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p,
 // ----------------------------------------------------------------------------- host side
 
 static int g_force_fp8_path = 0;   // 0 auto, 1 stream, 2 tile
+static int g_fp8_stream_split = 0;   // -1: the stream kernel over two K halves is off (benchmarking)
 static int g_force_fp8_gx = 0;
 
 template <bool BF16_OUT, int WMB, int WNB>
@@ -950,9 +981,9 @@ static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t c
 }
 
 template <bool BF16_OUT, int KS, int MB>
-static void launch_stream(const Fp8MMParams& p, int wk, int gx, hipStream_t s) {
+static void launch_stream(const Fp8MMParams& p, int wk, int gx, hipStream_t s, int halves = 1) {
   const size_t lds = wk > 1 ? (size_t)2 * wk * MB * 64 * sizeof(v4f) : 0;
-  hipLaunchKernelGGL((fp8_mm_stream_kernel<BF16_OUT, KS, MB>), dim3(gx), dim3(64, wk), lds, s, p, wk);
+  hipLaunchKernelGGL((fp8_mm_stream_kernel<BF16_OUT, KS, MB>), dim3(gx, halves), dim3(64, wk), lds, s, p, wk);
 }
 
 // K steps (of 128) per wavefront of the stream kernel for a problem, 0 if the kernel does not take it (the activations of
@@ -971,6 +1002,35 @@ static int stream_steps_per_wave(int64_t M, int64_t N, int64_t K) {
   if (steps <= 8 * 8) return 8;
   if (steps <= 8 * 14 && M <= 16) return 14;
   return 0;
+}
+
+// The stream kernel over two halves of K (two workgroups per n-tile range, partial tiles handed over through the caller's
+// scratch): K steps per wavefront, 0 if this route does not take the problem.  It covers what the registers of one
+// workgroup cannot at two m-blocks: 16 < M <= 32 up to K = 16384 (cold weights, against the tile kernel with K split:
+// 14336 x 4096 at M = 17 / 32 34.5 / 35.3 -> 22.0 / 24.4 us, 16384 x 4096 at M = 32 37.1 -> 27.4 us).  For M <= 16 beyond
+// K = 14336 (14 steps per wavefront and half) the tile kernel stays ahead: 28672 x 8192 72 against 85 us.
+static int stream_split_steps_per_wave(int64_t M, int64_t N, int64_t K) {
+  if (g_fp8_stream_split < 0 || M <= 16 || M > 32 || stream_steps_per_wave(M, N, K) != 0) return 0;
+  const int64_t half = ((K + 127) / 128 + 1) / 2;
+  return half <= 8 * 8 ? 8 : 0;
+}
+
+template <bool BF16_OUT>
+static bool dispatch_stream_split(const Fp8MMParams& p, int64_t c_tmp_bytes, int64_t counter_ints, hipStream_t s) {
+  const int ks = stream_split_steps_per_wave(p.M, p.N, p.K);
+  if (ks == 0) return false;
+  const int MB = (p.M + 15) / 16, NT = p.N / 16;
+  if (p.c_tmp == nullptr || p.counters == nullptr || counter_ints < (int64_t)NT * MB ||
+      c_tmp_bytes < (int64_t)2 * NT * MB * 1024 || (int64_t)2 * NT * MB * 1024 >= (1ll << 31))
+    return false;                                   // without the scratch the tile kernel still gives the result
+  const int half = ((p.K + 127) / 128 + 1) / 2;
+  const int wk = (half + ks - 1) / ks;              // >= 5: the K range of this route starts above one workgroup's
+  const int cus = num_cus_current_device();
+  const int rounds = (2 * NT + cus - 1) / cus;
+  int gx = g_force_fp8_gx > 0 ? g_force_fp8_gx : (NT + rounds - 1) / rounds;
+  if (gx > NT) gx = NT;
+  launch_stream<BF16_OUT, 8, 2>(p, wk, gx, s, 2);
+  return true;
 }
 
 template <bool BF16_OUT>
@@ -1016,7 +1076,14 @@ extern "C" int vaq_fp8_scaled_mm_workspace(int64_t size_m, int64_t size_n, int64
   *c_tmp_bytes = 0;
   *counter_ints = 0;
   const bool stream = g_force_fp8_path != 2 && stream_steps_per_wave(size_m, size_n, size_k) != 0;      // needs no scratch
-  if (stream || size_k % 64 != 0 || g_fp8_tile_impl != 0 || g_fp8_tile3_cfg < 0) return VAQ_OK;
+  if (stream) return VAQ_OK;
+  if (g_force_fp8_path != 2 && stream_split_steps_per_wave(size_m, size_n, size_k) != 0) {
+    const size_t units = (size_t)(size_n / 16) * (size_t)((size_m + 15) / 16);
+    *c_tmp_bytes = 2 * units * 1024;
+    *counter_ints = units;
+    return VAQ_OK;
+  }
+  if (size_k % 64 != 0 || g_fp8_tile_impl != 0 || g_fp8_tile3_cfg < 0) return VAQ_OK;
   const Fp8TilePlan pl = plan_tile3((int)size_m, (int)size_n, (int)size_k);
   if (pl.sk > 1) {
     *c_tmp_bytes = (size_t)pl.sk * (size_t)pl.tiles * pl.bm * pl.bn * sizeof(float);
@@ -1076,6 +1143,9 @@ extern "C" int vaq_fp8_scaled_mm_ws(const uint8_t* a, int64_t lda, const uint8_t
   bool done = false;
   const bool want_stream = g_force_fp8_path != 2 && stream_steps_per_wave(size_m, size_n, size_k) != 0;
   if (want_stream) done = bf16 ? dispatch_stream<true>(p, s) : dispatch_stream<false>(p, s);
+  if (!done && g_force_fp8_path != 2)
+    done = bf16 ? dispatch_stream_split<true>(p, c_tmp_bytes, counter_ints, s)
+                : dispatch_stream_split<false>(p, c_tmp_bytes, counter_ints, s);
   if (!done) {
     int rc = bf16 ? dispatch_tile<true>(p, c_tmp_bytes, counter_ints, s) : dispatch_tile<false>(p, c_tmp_bytes, counter_ints, s);
     if (rc != VAQ_OK) return rc;
@@ -1085,6 +1155,8 @@ extern "C" int vaq_fp8_scaled_mm_ws(const uint8_t* a, int64_t lda, const uint8_t
 }
 
 // Benchmark / tuning aid, not part of the drop-in surface.  path: 0 auto, 1 stream, 2 tile; gx: stream-kernel grid.
+extern "C" void vaq_debug_set_fp8_stream_split(int mode) { vaq::g_fp8_stream_split = mode; }
+
 extern "C" void vaq_debug_set_fp8_tile_cfg(int cfg, int split) {     // cfg: 0 = automatic, -1 = off; split: 0 = automatic
   vaq::g_fp8_tile3_cfg = cfg;
   vaq::g_fp8_force_split = split;
