@@ -666,15 +666,16 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
 // ----------------------------------------------------------------------------- stream kernel (M <= 32, narrow layers M <= 64)
 // blockDim = (64, WK).  Wavefront w owns K steps [w*KS, (w+1)*KS) of 128 bytes; activations of that slab live in
 // registers for the whole kernel; the workgroup walks a contiguous range of 16-row weight tiles.
-template <bool BF16_OUT, int KS, int MB>
+template <bool BF16_OUT, int KS, int MB, bool HALVES = false>
 __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p, int WK) {
   using T = F16Traits<BF16_OUT>;
   extern __shared__ v4f red[];   // [2][WK][MB][64]
   const int lane = threadIdx.x, w = threadIdx.y;
   const int q = lane >> 4, r16 = lane & 15;
-  // gridDim.y = 2: the K range is split over two workgroups (the second starts where the slabs of the first end);
-  // their partial tiles are summed by whichever arrives last (see the hand-over below)
-  const int kbase = ((int)blockIdx.y * WK + w) * KS * 128 + q * 32;
+  // HALVES (gridDim.y = 2): the K range is split over two workgroups (the second starts where the slabs of the first
+  // end); their partial tiles are summed by whichever arrives last (see the hand-over below).  A template parameter,
+  // because the extra live values cost the other instances registers they do not have (14 steps: 12 -> 260 bytes spilled).
+  const int kbase = ((HALVES ? (int)blockIdx.y * WK : 0) + w) * KS * 128 + q * 32;
 
   v8i breg[KS][MB];
 #pragma unroll
@@ -780,7 +781,7 @@ __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p,
     } else {
       reducer = true;
     }
-    if (gridDim.y > 1 && reducer) {
+    if (HALVES && reducer) {
       // Hand-over as in the tile kernel: the partial tile goes out in device-scope 16-byte stores, one arrival counter
       // per (n-tile, m-block); the workgroup that arrives last adds the parts in the order of the K halves and returns the
       // counter to zero.  (WK > 1 always here: the host splits only a long K.)
@@ -980,10 +981,10 @@ static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t c
   return launch_tile<BF16_OUT, 1, 2>(p, s);
 }
 
-template <bool BF16_OUT, int KS, int MB>
-static void launch_stream(const Fp8MMParams& p, int wk, int gx, hipStream_t s, int halves = 1) {
+template <bool BF16_OUT, int KS, int MB, bool HALVES = false>
+static void launch_stream(const Fp8MMParams& p, int wk, int gx, hipStream_t s) {
   const size_t lds = wk > 1 ? (size_t)2 * wk * MB * 64 * sizeof(v4f) : 0;
-  hipLaunchKernelGGL((fp8_mm_stream_kernel<BF16_OUT, KS, MB>), dim3(gx, halves), dim3(64, wk), lds, s, p, wk);
+  hipLaunchKernelGGL((fp8_mm_stream_kernel<BF16_OUT, KS, MB, HALVES>), dim3(gx, HALVES ? 2 : 1), dim3(64, wk), lds, s, p, wk);
 }
 
 // K steps (of 128) per wavefront of the stream kernel for a problem, 0 if the kernel does not take it (the activations of
@@ -1007,7 +1008,7 @@ static int stream_steps_per_wave(int64_t M, int64_t N, int64_t K) {
 // The stream kernel over two halves of K (two workgroups per n-tile range, partial tiles handed over through the caller's
 // scratch): K steps per wavefront, 0 if this route does not take the problem.  It covers what the registers of one
 // workgroup cannot at two m-blocks: 16 < M <= 32 up to K = 16384 (cold weights, against the tile kernel with K split:
-// 14336 x 4096 at M = 17 / 32 34.5 / 35.3 -> 22.0 / 24.4 us, 16384 x 4096 at M = 32 37.1 -> 27.4 us).  For M <= 16 beyond
+// 14336 x 4096 at M = 24 / 32 34.7 / 35.1 -> 21.6 / 22.5 us, 16384 x 4096 at M = 32 37.1 -> 27.4 us).  For M <= 16 beyond
 // K = 14336 (14 steps per wavefront and half) the tile kernel stays ahead: 28672 x 8192 72 against 85 us.
 static int stream_split_steps_per_wave(int64_t M, int64_t N, int64_t K) {
   if (g_fp8_stream_split < 0 || M <= 16 || M > 32 || stream_steps_per_wave(M, N, K) != 0) return 0;
@@ -1029,7 +1030,7 @@ static bool dispatch_stream_split(const Fp8MMParams& p, int64_t c_tmp_bytes, int
   const int rounds = (2 * NT + cus - 1) / cus;
   int gx = g_force_fp8_gx > 0 ? g_force_fp8_gx : (NT + rounds - 1) / rounds;
   if (gx > NT) gx = NT;
-  launch_stream<BF16_OUT, 8, 2>(p, wk, gx, s, 2);
+  launch_stream<BF16_OUT, 8, 2, true>(p, wk, gx, s);
   return true;
 }
 
