@@ -37,6 +37,7 @@ struct Fp8MMParams {
   int32_t* counters = nullptr;   // arrival counters, zero on entry, left zero
   int SK = 1;
   int rotate_k = 0;              // multi-stage tile kernel: tile rows start their K loop at different places (see the kernel)
+  int nt_base = 0, nt_rem = 0;   // stream kernel: n-tiles per workgroup = nt_base, one more for the first nt_rem (N/16 split on the host)
 };
 
 __device__ inline v16f mfma_fp8_32(v8i a, v8i b, v16f c) {
@@ -695,8 +696,9 @@ __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p,
   }
 
   const int NT = p.N / 16;
-  const int nt0 = (int)(((int64_t)NT * blockIdx.x) / gridDim.x);
-  const int nt1 = (int)(((int64_t)NT * (blockIdx.x + 1)) / gridDim.x);
+  const int bx = blockIdx.x;
+  const int nt0 = bx * p.nt_base + (bx < p.nt_rem ? bx : p.nt_rem);
+  const int nt1 = nt0 + p.nt_base + (bx < p.nt_rem ? 1 : 0);
 
   v4i wlo[KS], whi[KS];
   auto issue = [&](int nt, int s) {
@@ -982,7 +984,10 @@ static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t c
 }
 
 template <bool BF16_OUT, int KS, int MB, bool HALVES = false>
-static void launch_stream(const Fp8MMParams& p, int wk, int gx, hipStream_t s) {
+static void launch_stream(const Fp8MMParams& p_in, int wk, int gx, hipStream_t s) {
+  Fp8MMParams p = p_in;
+  p.nt_base = (p.N / 16) / gx;
+  p.nt_rem = (p.N / 16) % gx;
   const size_t lds = wk > 1 ? (size_t)2 * wk * MB * 64 * sizeof(v4f) : 0;
   hipLaunchKernelGGL((fp8_mm_stream_kernel<BF16_OUT, KS, MB, HALVES>), dim3(gx, HALVES ? 2 : 1), dim3(64, wk), lds, s, p, wk);
 }

@@ -44,6 +44,12 @@ struct Decode2Params {
   int GR;                  // rows of the scale / zero-point tensors (G * SUBG, or 1 for channelwise scales)
   int s_stride, z_stride;  // elements between consecutive rows of scales (N) / zeros (N/8); 0 for channelwise
   uint32_t k_mask, k_ex;   // 0x000f000f and the exponent pattern, passed as run-time values (see and_or)
+  // Set by the launcher (it knows the template arguments): the divisions of the kernel's first instructions, done on
+  // the host.  x / WN = (x * wn_magic) >> 16 for a wavefront index, x / KO = umulhi(x, ko_magic) for a thread index (KO =
+  // k-octets of the staged slab; both exact in those ranges); step_m, step_ko = (threads / KO, threads % KO).
+  uint32_t wn_magic, ko_magic;
+  int step_m, step_ko;
+  uint32_t b_bytes, s_bytes, z_bytes, a_bytes;   // extents of the buffer descriptors (saturated to 4 GiB - 1)
 };
 
 // (x & mask) | ex.  mask and ex reach the kernel as run-time arguments: with literal constants the compiler emits two
@@ -55,6 +61,10 @@ static __device__ inline __amdgpu_buffer_rsrc_t d2_rsrc(const void* base, uint64
   const uint32_t n = bytes > 0xffffffffull ? 0xffffffffu : (uint32_t)bytes;
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)n, 0x00020000);
 }
+static __device__ inline __amdgpu_buffer_rsrc_t d2_rsrc32(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+static inline uint32_t d2_sat32(uint64_t bytes) { return bytes > 0xffffffffull ? 0xffffffffu : (uint32_t)bytes; }
 
 constexpr int D2_WAVES = 16;
 
@@ -78,7 +88,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   const int w = __builtin_amdgcn_readfirstlane(threadIdx.y);
   const int o = lane >> 4, r16 = lane & 15;
   const int WKS = p.WKS, WN = p.WN;
-  const int wks = w / WN, wn = w - wks * WN;
+  const int wks = (int)(((uint32_t)w * p.wn_magic) >> 16), wn = w - wks * WN;
   const int sk = blockIdx.y;
   const int slab_groups = WKS * GS;                 // tiles in this workgroup's K slab
   const int slab_g0 = sk * slab_groups;             // first tile of the slab
@@ -90,9 +100,9 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   // ---- 1. activations of the K slab -> LDS, then the first R weight tiles requested ----
   // Loads retire in issue order as far as the wait counter is concerned, so the activation loads go out FIRST: the
   // wait before the barrier then leaves the weight tiles in flight instead of draining them.
-  const __amdgpu_buffer_rsrc_t rb = d2_rsrc(p.b, (uint64_t)p.K * p.N / 2 * TPG);
-  const __amdgpu_buffer_rsrc_t rs = d2_rsrc(p.scales, (uint64_t)p.GR * p.N * 2);
-  const __amdgpu_buffer_rsrc_t rz = d2_rsrc(HAS_ZP ? (const void*)p.zeros : (const void*)p.scales, (uint64_t)p.GR * (p.N / 8) * 4);
+  const __amdgpu_buffer_rsrc_t rb = d2_rsrc32(p.b, p.b_bytes);
+  const __amdgpu_buffer_rsrc_t rs = d2_rsrc32(p.scales, p.s_bytes);
+  const __amdgpu_buffer_rsrc_t rz = d2_rsrc32(HAS_ZP ? (const void*)p.zeros : (const void*)p.scales, p.z_bytes);
   const int vo_b = lane * 16, vo_s = o * 8, vo_z = (r16 >> 3) * 4;
   v4u wq[R];
   v2u sc[R][SUBG];
@@ -121,17 +131,17 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
     const int chunks = KO * MR * MB;
     const int64_t k_slab0 = (int64_t)(slab_g0 / TPG) * 128;
     const int NTHR = WKS * WN * 64;
-    const int step_m = NTHR / KO, step_ko = NTHR - step_m * KO;     // scalar
+    const int step_m = p.step_m, step_ko = p.step_ko;               // NTHR / KO, NTHR % KO
     // chunk c = m * KO + ko' (LDS slot c); thread tid handles c = tid, tid + NTHR, ...  The (m, ko') pair is advanced
     // incrementally: one scalar division per kernel instead of one vector division per chunk.
-    int m = tid / KO, ko = tid - m * KO;
+    int m = (int)__umulhi((uint32_t)tid, p.ko_magic), ko = tid - m * KO;
     if (p.perm == nullptr) {
       // Direct-to-LDS loads (no registers, no LDS write instructions): wavefront instruction q fills slots 64q .. 64q+63,
       // lane l fetching the chunk that belongs in slot 64q + l.  Rows past M, k past K and slots past the image get an
       // out-of-range offset of the buffer descriptor (which ends with the last valid element) and arrive as zeros; the
       // image is padded to a multiple of 1 KiB for the last instruction.  The weight tiles are requested after these
       // loads (loads retire in order as far as the wait counter is concerned) and stay in flight across the barrier.
-      const __amdgpu_buffer_rsrc_t ra = d2_rsrc(p.a, ((uint64_t)(p.M - 1) * (uint64_t)p.lda + (uint64_t)p.K) * 2);
+      const __amdgpu_buffer_rsrc_t ra = d2_rsrc32(p.a, p.a_bytes);
       typedef __attribute__((address_space(3))) void* lds_ptr_t;
       for (int c0 = w * 64; c0 < chunks; c0 += NTHR) {
         const int64_t k = k_slab0 + (int64_t)(ko ^ (m & (MR - 1))) * 8;
@@ -374,8 +384,20 @@ static inline size_t decode2_lds_bytes(int wks, int groups_per_wave, int mr, int
 }
 
 template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, bool W8 = false>
-static int launch_decode2(const Decode2Params& p, hipStream_t s) {
+static int launch_decode2(const Decode2Params& p_in, hipStream_t s) {
+  Decode2Params p = p_in;
   const int WN = p.WN;
+  {
+    const int ko = p.WKS * GS / (W8 ? 2 : 1) * 16, nthr = p.WKS * WN * 64;
+    p.wn_magic = (uint32_t)((65536 + WN - 1) / WN);
+    p.ko_magic = (uint32_t)(((1ull << 32) + (uint64_t)ko - 1) / (uint64_t)ko);
+    p.step_m = nthr / ko;
+    p.step_ko = nthr - p.step_m * ko;
+    p.b_bytes = d2_sat32((uint64_t)p.K * p.N / 2 * (W8 ? 2 : 1));
+    p.s_bytes = d2_sat32((uint64_t)p.GR * p.N * 2);
+    p.z_bytes = d2_sat32((uint64_t)p.GR * (p.N / 8) * 4);
+    p.a_bytes = d2_sat32(((uint64_t)(p.M - 1) * (uint64_t)p.lda + (uint64_t)p.K) * 2);
+  }
   const size_t lds = decode2_lds_bytes(p.WKS, GS / (W8 ? 2 : 1), MR, MB);
   auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP, MR, SUBG, W8>;
   static size_t reserved[VAQ_MAX_DEVICES];
