@@ -280,7 +280,7 @@ __global__ __launch_bounds__(MAXW * 64) void w4a16_decode_kernel(const DecodePar
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // partial tile acknowledged before the counter moves
             int old = 0;
             if (lane == 0) old = __hip_atomic_fetch_add(&p.counters[nt * MB + mb], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            old = __shfl(old, 0);
+            old = __builtin_amdgcn_readfirstlane(old);      // lane 0 holds it; a scalar keeps what depends on it scalar
             write_out = (old == p.SK - 1);
             if (write_out) {
               val = v4f{0.f, 0.f, 0.f, 0.f};

@@ -129,7 +129,8 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   {
     const int tid = w * 64 + lane;
     const int chunks = KO * MR * MB;
-    const int64_t k_slab0 = (int64_t)(slab_g0 / TPG) * 128;
+    const int k_slab0 = (slab_g0 / TPG) * 128;          // 32-bit arithmetic: the launcher checks that A ends below 2 GiB
+    const int lda32 = (int)p.lda;
     const int NTHR = WKS * WN * 64;
     const int step_m = p.step_m, step_ko = p.step_ko;               // NTHR / KO, NTHR % KO
     // chunk c = m * KO + ko' (LDS slot c); thread tid handles c = tid, tid + NTHR, ...  The (m, ko') pair is advanced
@@ -144,9 +145,9 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
       const __amdgpu_buffer_rsrc_t ra = d2_rsrc32(p.a, p.a_bytes);
       typedef __attribute__((address_space(3))) void* lds_ptr_t;
       for (int c0 = w * 64; c0 < chunks; c0 += NTHR) {
-        const int64_t k = k_slab0 + (int64_t)(ko ^ (m & (MR - 1))) * 8;
+        const int k = k_slab0 + (ko ^ (m & (MR - 1))) * 8;
         const bool ok = m < MR * MB && m < p.M && k < p.K;
-        const uint32_t off = ok ? (uint32_t)(((int64_t)m * p.lda + k) * 2) : 0x80000000u;
+        const uint32_t off = ok ? (uint32_t)(m * lda32 + k) * 2u : 0x80000000u;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(lds + (size_t)c0 * 16), 16, (int)off, 0, 0, 0);
         m += step_m;
         ko += step_ko;
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
         for (int i = 0; i < 4; ++i) {
           mm[i] = m;
           kk[i] = ko;
-          const int64_t k = k_slab0 + (int64_t)(ko ^ (m & (MR - 1))) * 8;
+          const int64_t k = (int64_t)k_slab0 + (int64_t)(ko ^ (m & (MR - 1))) * 8;
           v[i] = v4u{0u, 0u, 0u, 0u};
           if (m < MR * MB && m < p.M && k < p.K) {
             const uint16_t* row = p.a + (int64_t)m * p.lda;
@@ -329,7 +330,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // partial tiles acknowledged before the counter moves
     int old = 0;
     if (lane == 0) old = __hip_atomic_fetch_add(&p.counters[nt * MB], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    old = __shfl(old, 0);
+    old = __builtin_amdgcn_readfirstlane(old);      // lane 0 holds it; a scalar keeps what depends on it scalar
     if (old != p.SK - 1) return;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[mb] = v4f{0.f, 0.f, 0.f, 0.f};
@@ -397,6 +398,10 @@ static int launch_decode2(const Decode2Params& p_in, hipStream_t s) {
     p.s_bytes = d2_sat32((uint64_t)p.GR * p.N * 2);
     p.z_bytes = d2_sat32((uint64_t)p.GR * (p.N / 8) * 4);
     p.a_bytes = d2_sat32(((uint64_t)(p.M - 1) * (uint64_t)p.lda + (uint64_t)p.K) * 2);
+    if (p.a_bytes >= 0x80000000u) {
+      set_error("w4a16_gemm(decode): activations beyond 2 GiB (M = %d, row stride %lld)", p.M, (long long)p.lda);
+      return VAQ_ERR_UNSUPPORTED;
+    }
   }
   const size_t lds = decode2_lds_bytes(p.WKS, GS / (W8 ? 2 : 1), MR, MB);
   auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP, MR, SUBG, W8>;

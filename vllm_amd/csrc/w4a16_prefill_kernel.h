@@ -781,7 +781,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
     int32_t* ctr = p.counters + (int64_t)t * NW + wave;
     int old = 0;
     if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    old = __shfl(old, 0);
+    old = __builtin_amdgcn_readfirstlane(old);      // lane 0 holds it; a scalar keeps what depends on it scalar
     if (old != p.SK - 1) return;
 #pragma unroll
     for (int i = 0; i < WMB; ++i)
