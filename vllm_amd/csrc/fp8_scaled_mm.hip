@@ -37,6 +37,7 @@ struct Fp8MMParams {
   int32_t* counters = nullptr;   // arrival counters, zero on entry, left zero
   int SK = 1;
   int rotate_k = 0;              // multi-stage tile kernel: tile rows start their K loop at different places (see the kernel)
+  uint32_t a_extent = 0, b_extent = 0;   // stream kernel: bytes up to the end of the last row of a / b (below 2 GiB)
   int nt_base = 0, nt_rem = 0;   // stream kernel: n-tiles per workgroup = nt_base, one more for the first nt_rem (N/16 split on the host)
 };
 
@@ -667,7 +668,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
 // ----------------------------------------------------------------------------- stream kernel (M <= 32, narrow layers M <= 64)
 // blockDim = (64, WK).  Wavefront w owns K steps [w*KS, (w+1)*KS) of 128 bytes; activations of that slab live in
 // registers for the whole kernel; the workgroup walks a contiguous range of 16-row weight tiles.
-template <bool BF16_OUT, int KS, int MB, bool HALVES = false>
+template <bool BF16_OUT, int KS, int MB, bool HALVES = false, bool PF = true>
 __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p, int WK) {
   using T = F16Traits<BF16_OUT>;
   extern __shared__ v4f red[];   // [2][WK][MB][64]
@@ -678,6 +679,12 @@ __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p,
   // because the extra live values cost the other instances registers they do not have (14 steps: 12 -> 260 bytes spilled).
   const int kbase = ((HALVES ? (int)blockIdx.y * WK : 0) + w) * KS * 128 + q * 32;
 
+  // Operand loads go through buffer descriptors (the host checks that both operands end below 2 GiB): a 16-byte piece
+  // past K or past the last row gets an offset beyond the descriptor's extent and arrives as zeros -- one compare and
+  // one select per load instead of a branch and eight zeroed registers.
+  constexpr uint32_t OOB = 0x80000000u;
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.a), 0, (int)p.a_extent, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.b), 0, (int)p.b_extent, 0x00020000);
   v8i breg[KS][MB];
 #pragma unroll
   for (int s = 0; s < KS; ++s) {
@@ -685,12 +692,10 @@ __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p,
     for (int mb = 0; mb < MB; ++mb) {
       const int m = mb * 16 + r16;
       const int k = kbase + s * 128;
-      v4i lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
-      if (m < p.M) {
-        const uint8_t* row = p.a + (int64_t)m * p.lda;
-        if (k < p.K) lo = *reinterpret_cast<const v4i*>(row + k);
-        if (k + 16 < p.K) hi = *reinterpret_cast<const v4i*>(row + k + 16);
-      }
+      const uint32_t base = (uint32_t)m * (uint32_t)p.lda + (uint32_t)k;
+      const uint32_t o_lo = (m < p.M && k < p.K) ? base : OOB, o_hi = (m < p.M && k + 16 < p.K) ? base + 16u : OOB;
+      const v4i lo = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ra, (int)o_lo, 0, 0));
+      const v4i hi = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ra, (int)o_hi, 0, 0));
       breg[s][mb] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     }
   }
@@ -701,18 +706,18 @@ __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p,
   const int nt1 = nt0 + p.nt_base + (bx < p.nt_rem ? 1 : 0);
 
   v4i wlo[KS], whi[KS];
-  auto issue = [&](int nt, int s) {
+  // `live` = false requests nothing (offsets beyond the extent): the request for the tile after the last one stays in
+  // the instruction stream, so that the count of loads in flight -- which the waits are derived from -- is the same on
+  // every path (behind a branch the compiler assumes the shorter path and waits for the next tile's loads as well).
+  auto issue = [&](int nt, int s, bool live) {
     const int k = kbase + s * 128;
-    const uint8_t* row = p.b + (int64_t)(nt * 16 + r16) * p.ldb;
-    wlo[s] = v4i{0, 0, 0, 0};
-    whi[s] = v4i{0, 0, 0, 0};
-    if (k < p.K) wlo[s] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(row + k));
-    if (k + 16 < p.K) whi[s] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(row + k + 16));
+    const uint32_t base = (uint32_t)(nt * 16 + r16) * (uint32_t)p.ldb + (uint32_t)k;
+    const uint32_t o_lo = (live && k < p.K) ? base : OOB, o_hi = (live && k + 16 < p.K) ? base + 16u : OOB;
+    wlo[s] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rb, (int)o_lo, 0, 2));     // 2: streamed once
+    whi[s] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rb, (int)o_hi, 0, 2));
   };
-  if (nt0 < nt1) {
 #pragma unroll
-    for (int s = 0; s < KS; ++s) issue(nt0, s);
-  }
+  for (int s = 0; s < KS; ++s) issue(nt0, s, nt0 < nt1);
 
   // Epilogue operands are requested ahead of their use (a load issued after the reduction would stall the reducing
   // wavefront, and through the next barrier the whole workgroup, for a memory round trip per n-tile): the activation
@@ -732,7 +737,12 @@ __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p,
   }
 
   int parity = 0;
-  for (int nt = nt0; nt < nt1; ++nt) {
+  // One n-tile.  PF: request the next tile's weights behind each step's MFMAs.  Launches in which every workgroup has a
+  // single tile use the instance without those requests (they would be 2 KS loads that fetch nothing but still pass
+  // through the load path: 14336 x 4096 at M = 1 / 16 15.4 / 19.2 -> 16.0 / 20.2 us); as a run-time condition the compiler
+  // would derive the waits of the multi-tile case from the shorter path and wait for the next tile's loads too, and
+  // both variants in one kernel cost registers (spills with 8 steps and two m-blocks).
+  auto do_tile = [&](int nt) {
     v4f acc[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[mb] = v4f{0.f, 0.f, 0.f, 0.f};
@@ -751,9 +761,14 @@ __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p,
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       const v8i aop = v8i{wlo[s].x, wlo[s].y, wlo[s].z, wlo[s].w, whi[s].x, whi[s].y, whi[s].z, whi[s].w};
-      if (nt + 1 < nt1) issue(nt + 1, s);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) acc[mb] = mfma_fp8_16(aop, breg[s][mb], acc[mb]);
+      // the step's registers are free once its MFMAs have issued: request the next tile's step into them right away
+      // (the fence keeps the compiler from collecting these requests behind the tile's last MFMA)
+      if constexpr (PF) {
+        issue(nt + 1, s, nt + 1 < nt1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
 
     if constexpr (!AHEAD) {
@@ -835,6 +850,11 @@ __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p,
       for (int mb = 0; mb < MB; ++mb)       // unrolled: sam_mb stays in registers
         if (mb >= mb_lo && mb < mb_hi) emit(mb, sam_mb[mb], sb_r, bias_r);
     }
+  };
+  if constexpr (PF) {
+    for (int nt = nt0; nt < nt1; ++nt) do_tile(nt);
+  } else {
+    if (nt0 < nt1) do_tile(nt0);       // the launcher picks this instance only for one tile per workgroup
   }
 }
 
@@ -988,8 +1008,19 @@ static void launch_stream(const Fp8MMParams& p_in, int wk, int gx, hipStream_t s
   Fp8MMParams p = p_in;
   p.nt_base = (p.N / 16) / gx;
   p.nt_rem = (p.N / 16) % gx;
+  p.a_extent = (uint32_t)((int64_t)(p.M - 1) * p.lda + p.K);
+  p.b_extent = (uint32_t)((int64_t)(p.N - 1) * p.ldb + p.K);
   const size_t lds = wk > 1 ? (size_t)2 * wk * MB * 64 * sizeof(v4f) : 0;
-  hipLaunchKernelGGL((fp8_mm_stream_kernel<BF16_OUT, KS, MB, HALVES>), dim3(gx, HALVES ? 2 : 1), dim3(64, wk), lds, s, p, wk);
+  if (p.nt_base == 1 && p.nt_rem == 0)
+    hipLaunchKernelGGL((fp8_mm_stream_kernel<BF16_OUT, KS, MB, HALVES, false>), dim3(gx, HALVES ? 2 : 1), dim3(64, wk), lds, s, p, wk);
+  else
+    hipLaunchKernelGGL((fp8_mm_stream_kernel<BF16_OUT, KS, MB, HALVES, true>), dim3(gx, HALVES ? 2 : 1), dim3(64, wk), lds, s, p, wk);
+}
+
+// The stream kernel addresses its operands with 32-bit offsets from buffer descriptors: both must end below 2 GiB
+// (otherwise the tile kernels take the problem).
+static bool stream_offsets_fit(const Fp8MMParams& p) {
+  return (int64_t)(p.M - 1) * p.lda + p.K < (1ll << 31) && (int64_t)(p.N - 1) * p.ldb + p.K < (1ll << 31);
 }
 
 // K steps (of 128) per wavefront of the stream kernel for a problem, 0 if the kernel does not take it (the activations of
@@ -1024,7 +1055,7 @@ static int stream_split_steps_per_wave(int64_t M, int64_t N, int64_t K) {
 template <bool BF16_OUT>
 static bool dispatch_stream_split(const Fp8MMParams& p, int64_t c_tmp_bytes, int64_t counter_ints, hipStream_t s) {
   const int ks = stream_split_steps_per_wave(p.M, p.N, p.K);
-  if (ks == 0) return false;
+  if (ks == 0 || !stream_offsets_fit(p)) return false;
   const int MB = (p.M + 15) / 16, NT = p.N / 16;
   if (p.c_tmp == nullptr || p.counters == nullptr || counter_ints < (int64_t)NT * MB ||
       c_tmp_bytes < (int64_t)2 * NT * MB * 1024 || (int64_t)2 * NT * MB * 1024 >= (1ll << 31))
@@ -1044,7 +1075,7 @@ static bool dispatch_stream(const Fp8MMParams& p, hipStream_t s) {
   const int steps = (p.K + 127) / 128;
   const int MB = (p.M + 15) / 16;
   const int ks = stream_steps_per_wave(p.M, p.N, p.K);
-  if (ks == 0) return false;
+  if (ks == 0 || !stream_offsets_fit(p)) return false;
   const int wk = (steps + ks - 1) / ks;
   const int NT = p.N / 16;
   // one workgroup per compute unit, the n-tiles dealt out evenly over the fewest rounds: every workgroup loads all the
