@@ -102,11 +102,13 @@ int vaq_w4a16_gemm_workspace(int64_t size_m, int64_t size_n, int64_t size_k, int
  * M == 0 is a no-op.  Kernel choice (decode: M <= 32, up to 64 for 4-bit codes in groups of 128 rows or channelwise,
  * MFMA GEMV with in-register dequant; prefill: LDS-staged MFMA)
  * is internal; `force_path` = 0 auto, 1 decode, 2 prefill (tests / benchmarks).
+ * Scratch: `c_tmp` holds at least `c_tmp_bytes` bytes and `counters` at least `counter_ints` zeroed ints; a call whose
+ * kernel needs more than it was given returns VAQ_ERR_INVALID_ARG (sizes: vaq_w4a16_gemm_workspace) and launches nothing.
  */
 int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
-                   const int32_t* perm, const void* bias, void* c, float* c_tmp, void* a_tmp, int32_t* counters,
-                   int64_t counter_ints, int64_t size_m, int64_t size_n, int64_t size_k, int group_size, int dtype,
-                   int wtype, int force_path, void* stream);
+                   const int32_t* perm, const void* bias, void* c, float* c_tmp, int64_t c_tmp_bytes, void* a_tmp,
+                   int32_t* counters, int64_t counter_ints, int64_t size_m, int64_t size_n, int64_t size_k,
+                   int group_size, int dtype, int wtype, int force_path, void* stream);
 
 /*
  * out[m, k] = a[m, perm[k]] for 16-bit elements.  Replaces `permute_cols(Tensor A, Tensor perm) -> Tensor`
@@ -200,6 +202,51 @@ int vaq_fp8_scaled_mm_ws(const uint8_t* a, int64_t lda, const uint8_t* b, int64_
                          const float* sb, int64_t sb_count, const void* bias, void* out, int64_t ldc, int out_dtype,
                          int64_t size_m, int64_t size_n, int64_t size_k, float* c_tmp, int64_t c_tmp_bytes,
                          int32_t* counters, int64_t counter_ints, void* stream);
+
+/*
+ * Kernel-variant overrides for tests and benchmarks.  No counterpart in the reference (its kernels take no such
+ * argument); the drop-in surface never passes one.  A VaqTuning applies to the ONE call it is handed to, on the calling
+ * thread only: the library keeps no tuning state between calls.  Every field: 0 = the automatic choice.
+ */
+typedef struct VaqTuning {
+  int decode_impl;      /* W4A16 decode kernel: 1 LDS-staged activations, 2 register-resident activations          */
+  int decode2_gs;       /* LDS-staged kernel: weight tiles per wavefront                                             */
+  int decode2_wks;      /*   K slices per workgroup                                                                  */
+  int decode2_wn;       /*   n-tiles per workgroup                                                                   */
+  int decode_tg;        /* register-resident kernel: groups per wavefront                                            */
+  int decode_wk;        /*   wavefronts along K per workgroup                                                        */
+  int decode_gx;        /*   workgroups along N                                                                      */
+  int decode_depth;     /*   prefetch depth                                                                          */
+  int prefill_tile;     /* W4A16 tile kernel: tile id + 1                                                            */
+  int prefill_split;    /*   K split                                                                                 */
+  int fp8_path;         /* FP8 GEMM: 1 weight-streaming kernel, 2 tile kernel                                        */
+  int fp8_tile_impl;    /*   1 register-staged tile kernel                                                           */
+  int fp8_tile_cfg;     /*   multi-stage tile shape id, -1 = two-stage kernel                                        */
+  int fp8_split;        /*   K split of the tile kernel                                                              */
+  int fp8_gx;           /*   workgroups of the weight-streaming kernel                                               */
+  int fp8_stream_split; /*   -1 = never run the weight-streaming kernel over two halves of K                         */
+  int quant_wg_per_row; /* per-token FP8 quant: 1 = always one workgroup per row                                     */
+  int exp[15];          /* experiment switches of development builds; ignored by released kernels                    */
+} VaqTuning;
+
+/* The entry points of the same name without `_tuned`, with `tuning` (may be NULL) applied to this call. */
+int vaq_w4a16_gemm_workspace_tuned(int64_t size_m, int64_t size_n, int64_t size_k, int has_perm, int device,
+                                   size_t* c_tmp_bytes, size_t* a_tmp_bytes, size_t* counter_ints,
+                                   const VaqTuning* tuning);
+int vaq_w4a16_gemm_tuned(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
+                         const int32_t* perm, const void* bias, void* c, float* c_tmp, int64_t c_tmp_bytes, void* a_tmp,
+                         int32_t* counters, int64_t counter_ints, int64_t size_m, int64_t size_n, int64_t size_k,
+                         int group_size, int dtype, int wtype, int force_path, void* stream, const VaqTuning* tuning);
+int vaq_fp8_scaled_mm_workspace_tuned(int64_t size_m, int64_t size_n, int64_t size_k, size_t* c_tmp_bytes,
+                                      size_t* counter_ints, const VaqTuning* tuning);
+int vaq_fp8_scaled_mm_ws_tuned(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t ldb, const float* sa,
+                               int64_t sa_count, const float* sb, int64_t sb_count, const void* bias, void* out,
+                               int64_t ldc, int out_dtype, int64_t size_m, int64_t size_n, int64_t size_k, float* c_tmp,
+                               int64_t c_tmp_bytes, int32_t* counters, int64_t counter_ints, void* stream,
+                               const VaqTuning* tuning);
+int vaq_fp8_quant_per_token_tuned(const void* in, int in_dtype, int64_t in_row_stride, uint8_t* out,
+                                  int64_t out_row_stride, float* scales, const float* scale_ub, int64_t rows,
+                                  int64_t hidden, void* stream, const VaqTuning* tuning);
 
 #ifdef __cplusplus
 }

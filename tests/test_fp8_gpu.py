@@ -223,7 +223,7 @@ def test_scaled_mm_random_shapes(device, seed):
         out = ops.cutlass_scaled_mm(a_q.to(device), w_q.to(device).t(), sa.to(device), sb.to(device), out_dtype,
                                     None if b is None else b.to(device))
         _check_mm(out, ref, f"m={m} n={n} k={k} per_token={per_token} per_channel={per_channel} bias={bias} {out_dtype}")
-    assert bool((ops._fp8_counters(torch.device(device)) == 0).all())
+    assert all(bool((t == 0).all()) for t in ops._FP8_COUNTERS.values())
 
 
 def test_scaled_mm_exact_small_integers(device):
@@ -261,7 +261,7 @@ def test_scaled_mm_small_m_every_route_exact(device, m):
                                     sa.to(device), sb.to(device), torch.bfloat16, bias.to(torch.bfloat16).to(device))
         want = (sa * (sb.t() * (a @ w.t())) + bias).to(torch.bfloat16)
         assert torch.equal(out.cpu().float(), want.float()), (m, n, k)
-    assert bool((ops._fp8_counters(torch.device(device)) == 0).all()), "arrival counters not restored to zero"
+    assert all(bool((t == 0).all()) for t in ops._FP8_COUNTERS.values()), "arrival counters not restored to zero"
 
 
 @pytest.mark.parametrize("tokens,hidden", [(1, 17), (11, 1024), (1, 2), (4096, 64), (7, 5120), (83, 4096), (3, 17000)])
@@ -386,25 +386,22 @@ def test_scaled_mm_into_a_view_of_a_wider_buffer(device, offset):
 
 @pytest.mark.parametrize("cfg", [1, 8, 3, 4, 7, 13, 23, 14, 24, 17])
 def test_scaled_mm_every_tile_shape_exact(device, cfg):
-    """Every shape of the multi-stage tile kernel, forced through the tuning export (the automatic choice only reaches
+    """Every shape of the multi-stage tile kernel, forced through a per-call tuning override (the automatic choice only reaches
     some of them at any one problem size), including the ones that take two k-slices per step: small-integer operands
     make the fp32 accumulation exact, so the result must equal the integer GEMM, also with K split over workgroups."""
     import vllm_amd._custom_ops as ops
-    from vllm_amd import _lib
-    lib = _lib.load()
+    from vllm_amd import _tuning
     g = torch.Generator().manual_seed(cfg)
-    try:
-        for m, n, k, split in ((300, 384, 1024, 0), (64, 256, 8192 + 128, 2), (513, 512, 640, 0), (257, 272, 384, 0),
-                               (100, 128, 448, 0), (520, 256, 64 * 13, 3)):
-            a = torch.randint(-2, 3, (m, k), generator=g).float()
-            w = torch.randint(-1, 2, (n, k), generator=g).float()
-            lib.vaq_debug_set_fp8_tile_cfg(cfg, split)
+    for m, n, k, split in ((300, 384, 1024, 0), (64, 256, 8192 + 128, 2), (513, 512, 640, 0), (257, 272, 384, 0),
+                           (100, 128, 448, 0), (520, 256, 64 * 13, 3)):
+        a = torch.randint(-2, 3, (m, k), generator=g).float()
+        w = torch.randint(-1, 2, (n, k), generator=g).float()
+        with _tuning.override(fp8_tile_cfg=cfg, fp8_split=split):
             out = ops.cutlass_scaled_mm(a.to(torch.float8_e4m3fn).to(device), w.to(torch.float8_e4m3fn).to(device).t(),
                                         torch.ones(m, 1, device=device), torch.ones(n, 1, device=device), torch.float16)
-            assert torch.equal(out.cpu().float(), a @ w.t()), (cfg, m, n, k)
-    finally:
-        lib.vaq_debug_set_fp8_tile_cfg(0, 0)
-    assert bool((ops._fp8_counters(torch.device(device)) == 0).all()), "arrival counters not restored to zero"
+        assert torch.equal(out.cpu().float(), a @ w.t()), (cfg, m, n, k)
+    for t in ops._FP8_COUNTERS.values():
+        assert bool((t == 0).all()), "arrival counters not restored to zero"
 
 
 def test_scaled_mm_split_k_exact_and_deterministic(device):
@@ -421,7 +418,7 @@ def test_scaled_mm_split_k_exact_and_deterministic(device):
         out = ops.cutlass_scaled_mm(*args)
         assert torch.equal(out.cpu().float(), a @ w.t()), (m, n, k)
         assert torch.equal(out, ops.cutlass_scaled_mm(*args))
-        assert bool((ops._fp8_counters(torch.device(device)) == 0).all()), "arrival counters not restored to zero"
+        assert all(bool((t == 0).all()) for t in ops._FP8_COUNTERS.values()), "arrival counters not restored to zero"
 
 
 @pytest.mark.parametrize("k,n", LLAMA_SHAPES)
@@ -443,3 +440,56 @@ def test_config4_llama_shapes(device, k, n):
         ref = f.scaled_mm_ref(a_ref, w_q.t(), sa_ref, sb, torch.bfloat16, bias)
         _check_mm(out[rows], ref, f"config 4 k={k} n={n} m={m}")
         assert torch.isfinite(out.float()).all()
+
+
+def test_scaled_mm_split_k_on_two_streams_at_once(device):
+    """Two split-K GEMMs in flight on two streams: each stream has its own arrival counters, so the results must equal the
+    ones computed one after the other (small-integer operands: every partial sum is exact, any lost or doubled partial
+    tile changes the result)."""
+    import vllm_amd._custom_ops as ops
+    g = torch.Generator().manual_seed(21)
+    probs = []
+    for m, n, k in ((200, 256, 14336), (96, 384, 16384)):
+        a = torch.randint(-2, 3, (m, k), generator=g).float()
+        w = torch.randint(-1, 2, (n, k), generator=g).float()
+        probs.append(((a.to(torch.float8_e4m3fn).to(device), w.to(torch.float8_e4m3fn).to(device).t(),
+                       torch.ones(m, 1, device=device), torch.ones(n, 1, device=device), torch.float16), a @ w.t()))
+    serial = [ops.cutlass_scaled_mm(*args) for args, _ in probs]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[], []]
+    for _ in range(20):
+        for i, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                outs[i].append(ops.cutlass_scaled_mm(*probs[i][0]))
+    torch.cuda.synchronize()
+    keys = {key for key in ops._FP8_COUNTERS if key[1] in (streams[0].cuda_stream, streams[1].cuda_stream)}
+    assert len(keys) == 2, "each stream must own its arrival counters"
+    for i in range(2):
+        assert torch.equal(serial[i].cpu().float(), probs[i][1])
+        for o_ in outs[i]:
+            assert torch.equal(o_, serial[i]), f"stream {i}: concurrent result differs from the serial one"
+    assert all(bool((t == 0).all()) for t in ops._FP8_COUNTERS.values()), "arrival counters not restored to zero"
+
+
+def test_scaled_mm_split_k_first_call_under_graph_capture(device):
+    """A stream whose first split-K GEMM happens inside a HIP graph capture: the op takes zeroed counters from the
+    capture's own pool (a fill kernel, no memset node), and every replay gives the eager result."""
+    import vllm_amd._custom_ops as ops
+    g = torch.Generator().manual_seed(22)
+    m, n, k = 200, 256, 14336
+    a = torch.randint(-2, 3, (m, k), generator=g).float()
+    w = torch.randint(-1, 2, (n, k), generator=g).float()
+    args = (a.to(torch.float8_e4m3fn).to(device), w.to(torch.float8_e4m3fn).to(device).t(),
+            torch.ones(m, 1, device=device), torch.ones(n, 1, device=device), torch.float16)
+    eager = ops.cutlass_scaled_mm(*args)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):          # runs on a fresh side stream that has no cached counters
+        out = ops.cutlass_scaled_mm(*args)
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager) and torch.equal(out.cpu().float(), a @ w.t())
+        assert torch.equal(ops.cutlass_scaled_mm(*args), eager)      # eager work between the replays

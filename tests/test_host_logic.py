@@ -47,10 +47,10 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
         _lib.check(rc)
     rc = lib.vaq_w4a16_repack(None, None, None, 144, 64, 4, _lib.VAQ_LAYOUT_NATIVE, None)
     assert rc == _lib.VAQ_ERR_INVALID_ARG and b"128" in lib.vaq_last_error()
-    rc = lib.vaq_w4a16_gemm(None, 4096, None, None, None, None, None, None, None, None, None, 0, 16, 4096 + 32, 4096,
+    rc = lib.vaq_w4a16_gemm(None, 4096, None, None, None, None, None, None, None, 0, None, None, 0, 16, 4096 + 32, 4096,
                             128, _lib.VAQ_BF16, _lib.VAQ_WTYPE_U4B8, 0, None)
     assert rc == _lib.VAQ_ERR_INVALID_ARG and b"min_thread_n" in lib.vaq_last_error()
-    rc = lib.vaq_w4a16_gemm(None, 4096, None, None, None, None, None, None, None, None, None, 0, 16, 4096, 4096, 256,
+    rc = lib.vaq_w4a16_gemm(None, 4096, None, None, None, None, None, None, None, 0, None, None, 0, 16, 4096, 4096, 256,
                             _lib.VAQ_BF16, _lib.VAQ_WTYPE_U4B8, 0, None)
     assert rc == _lib.VAQ_ERR_UNSUPPORTED and b"group_size" in lib.vaq_last_error()
     rc = lib.vaq_fp8_scaled_mm(None, 100, None, 128, None, 1, None, 1, None, None, 128, _lib.VAQ_BF16, 4, 128, 128, None)
@@ -65,7 +65,7 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert rc == _lib.VAQ_ERR_INVALID_ARG and b"dtype" in lib.vaq_last_error()
     assert lib.vaq_silu_and_mul_fp8_quant(None, None, None, _lib.VAQ_BF16, 0, 16, None) == _lib.VAQ_OK
     # M == 0 is a no-op that touches nothing
-    assert lib.vaq_w4a16_gemm(None, 4096, None, None, None, None, None, None, None, None, None, 0, 0, 4096, 4096, 128,
+    assert lib.vaq_w4a16_gemm(None, 4096, None, None, None, None, None, None, None, 0, None, None, 0, 0, 4096, 4096, 128,
                               _lib.VAQ_BF16, _lib.VAQ_WTYPE_U4B8, 0, None) == _lib.VAQ_OK
 
 
@@ -388,3 +388,61 @@ def test_weight_loaders_place_checkpoint_tensors_in_fused_layers():
     row.weight_scale.weight_loader(row.weight_scale, torch.tensor(0.125))
     assert torch.equal(row.weight.data.view(torch.uint8), w.view(torch.uint8)) and row.weight_scale.data.tolist() == [0.125]
 
+
+
+def test_fp8_module_fused_on_disk_keeps_its_weight():
+    """A qkv / gate_up module that is already fused in an FP8 checkpoint brings ONE weight scale: `weight_loader_v2`
+    puts it in entry 0 and the other entries keep their initial value (the most negative float).  The method must then
+    keep the weight as loaded and use that one scale -- requantising the shards with the untouched entries would turn
+    them into +-448 (the reference skips it the same way: w8a8_utils.py:108-136)."""
+    from vllm_amd.layers.linear import MergedColumnParallelLinear
+    from vllm_amd.layers.quantization.fp8 import Fp8Config
+    k, sizes = 64, [32, 48]
+    cfg = Fp8Config(is_checkpoint_fp8_serialized=True, activation_scheme="dynamic")
+    layer = MergedColumnParallelLinear(k, sizes, quant_config=cfg, params_dtype=torch.bfloat16, return_bias=False)
+    g = torch.Generator().manual_seed(11)
+    w = torch.randint(0, 0x7E, (sum(sizes), k), dtype=torch.uint8, generator=g).view(torch.float8_e4m3fn)
+    layer.weight.weight_loader(layer.weight, w)                              # no shard id: fused on disk
+    layer.weight_scale.weight_loader(layer.weight_scale, torch.tensor(0.0375))
+    assert layer.weight_scale.data[0] == torch.tensor(0.0375) and layer.weight_scale.data[1] == torch.finfo(torch.float32).min
+    layer.process_weights_after_loading()                                    # no device work on this branch
+    assert torch.equal(layer.weight.t().contiguous().view(torch.uint8), w.view(torch.uint8)), "weight was requantised"
+    assert layer.weight_scale.dim() == 0 and float(layer.weight_scale) == float(torch.tensor(0.0375))
+    assert layer.input_scale is None
+
+
+def test_tuning_override_applies_to_one_call_only():
+    """A VaqTuning travels with the call it is passed to: the `_tuned` workspace query sees the forced K split, the plain
+    query right after it sees the automatic choice again (the library keeps no tuning state)."""
+    import ctypes
+    from vllm_amd import _lib
+    lib = _lib.load()
+
+    def query(tuning=None):
+        t, a, n = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+        args = (8, 320, 2048, 0, 0, ctypes.byref(t), ctypes.byref(a), ctypes.byref(n))
+        rc = lib.vaq_w4a16_gemm_workspace(*args) if tuning is None else lib.vaq_w4a16_gemm_workspace_tuned(*args, tuning)
+        assert rc == _lib.VAQ_OK
+        return t.value, n.value
+
+    auto = query()
+    assert auto == (0, 0)                      # K = 2048 fits one workgroup's LDS: no split, no scratch
+    forced = _lib.VaqTuning(decode_impl=1, decode2_gs=2, decode2_wks=2, decode2_wn=1)     # slabs of 4 groups: 4 splits
+    t, n = query(ctypes.byref(forced))
+    assert n == 320 // 16 and t >= 4 * (320 // 16) * 1024      # (the query covers whichever decode kernel may run)
+    assert query() == auto and query(None) == auto
+
+
+def test_workspace_from_the_helper_covers_every_batch_size():
+    """`marlin_make_workspace_new` must satisfy the GEMM's counter request for every M on the layer it was sized for, and
+    its default size must do so on a vocabulary-sized layer (N = 128256: three m-blocks at M = 40 need 24048 counters)."""
+    import ctypes
+    from vllm_amd import _lib
+    from vllm_amd.layers.quantization.utils.marlin_utils import marlin_workspace_ints
+    lib = _lib.load()
+    for n, k in ((128256, 4096), (4096, 14336), (28672, 4096), (64, 128)):
+        for m in (1, 16, 17, 32, 33, 40, 48, 49, 64, 65, 100, 256, 1024, 4096):
+            t, a, c = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+            assert lib.vaq_w4a16_gemm_workspace(m, n, k, 0, 0, ctypes.byref(t), ctypes.byref(a), ctypes.byref(c)) == _lib.VAQ_OK
+            assert c.value <= marlin_workspace_ints(n), (n, k, m, c.value)
+            assert c.value <= marlin_workspace_ints(None), (n, k, m, c.value)

@@ -270,6 +270,30 @@ def test_fp8_linear_method_serialized_static_fused_shards(device):
         _fp8_close(out, ref, f"fp8 static fused m={m}")
 
 
+def test_fp8_linear_method_module_fused_on_disk(device):
+    """An FP8 checkpoint whose qkv module is already fused: one weight tensor and ONE scalar scale arrive without a
+    shard id.  The weight must be used as loaded with that scale (w8a8_utils.py:108-136 skips the requantisation)."""
+    from vllm_amd.layers.linear import QKVParallelLinear
+    from vllm_amd.layers.quantization import get_quantization_config
+    k = 512
+    cfg = get_quantization_config("fp8").from_config(dict(quant_method="fp8", activation_scheme="dynamic"))
+    layer = QKVParallelLinear(k, 64, 4, 2, quant_config=cfg, params_dtype=torch.bfloat16, return_bias=False).to(device)
+    n = sum(layer.output_sizes)
+    g = torch.Generator().manual_seed(9)
+    scale = torch.tensor(0.019)
+    wq = of.ref_static_quant(torch.randn(n, k, generator=g) * 0.8, scale)
+    layer.weight.weight_loader(layer.weight, wq.to(device))
+    layer.weight_scale.weight_loader(layer.weight_scale, scale)
+    layer.process_weights_after_loading()
+    assert torch.equal(layer.weight.t().contiguous().cpu().view(torch.uint8), wq.view(torch.uint8)), "weight was requantised"
+    assert float(layer.weight_scale) == float(scale)
+    for m in (2, 50):
+        a = _acts(m, k, seed=m)
+        aq, sa = of.ref_dynamic_per_token_quant(a)
+        ref = of.scaled_mm_ref(aq, wq.t(), sa, scale.reshape(1), torch.float64, None)
+        _fp8_close(layer(a.to(device)), ref, f"fp8 fused on disk m={m}")
+
+
 def test_layers_loaded_shard_by_shard_through_weight_loaders(device):
     """Checkpoint tensors enter the layers the way a model loader delivers them -- `param.weight_loader(param, tensor,
     shard_id)` per logical part, on a layer that already lives on the device (linear.py:820-866,:1009-1060) -- then

@@ -22,11 +22,9 @@ def _acts(m, k, device, dtype=torch.bfloat16, seed=0):
 def decode_kernel(request):
     """Runs a test once with the library's own choice of decode kernel and once with each of the two kernels forced, so
     that both are checked on every shape whichever one the selection rule would pick."""
-    from vllm_amd import _lib
-    lib = _lib.load()
-    lib.vaq_debug_set_decode_impl({"auto": -1, "lds_staged": 0, "register_resident": 1}[request.param])
-    yield request.param
-    lib.vaq_debug_set_decode_impl(-1)
+    from vllm_amd import _tuning
+    with _tuning.override(decode_impl={"auto": 0, "lds_staged": 1, "register_resident": 2}[request.param]):
+        yield request.param
 
 
 # ------------------------------------------------------------------------------------------------ repack
@@ -138,30 +136,23 @@ def test_decode_gemm_small(device, decode_kernel, k, n, m, asym, act_order):
 @pytest.mark.parametrize("kernel", ["lds_staged", "register_resident"])
 @pytest.mark.parametrize("m", [1, 5, 16, 29])
 def test_decode_gemm_forced_split_k(device, kernel, m):
-    """K split over several workgroups on both decode kernels (forced through the tuning exports: the automatic choice
-    only splits a long K): partial tiles through `c_tmp`, arrival counters in `workspace`.  Against the oracle, twice for
-    determinism, counters left zero."""
-    from vllm_amd import _lib
-    lib = _lib.load()
+    """K split over several workgroups on both decode kernels (forced through a per-call tuning override: the automatic
+    choice only splits a long K): partial tiles through `c_tmp`, arrival counters in `workspace`.  Against the oracle,
+    twice for determinism, counters left zero."""
+    from vllm_amd import _tuning
     k, n = 2048, 320
     case = o.make_w4a16_case(k, n, 128, asym=True, seed=90 + m)
     layer = W4A16Layer(case, device)
     a = _acts(m, k, device, seed=m)
-    try:
-        if kernel == "lds_staged":
-            lib.vaq_debug_set_decode_impl(0)
-            lib.vaq_debug_set_decode2_config(2, 2 + 100 * 1)      # slabs of 4 groups: 4 splits
-        else:
-            lib.vaq_debug_set_decode_impl(1)
-            lib.vaq_debug_set_decode_config(1, 4, 0)              # 4 wavefronts of 1 group: 4 (M <= 16) splits
+    if kernel == "lds_staged":
+        forced = dict(decode_impl=1, decode2_gs=2, decode2_wks=2, decode2_wn=1)      # slabs of 4 groups: 4 splits
+    else:
+        forced = dict(decode_impl=2, decode_tg=1, decode_wk=4)      # 4 wavefronts of 1 group: 4 (M <= 16) splits
+    with _tuning.override(**forced):
         out = layer(a)
         check_gemm_close(out, o.gemm_ref(a.cpu(), o.case_w_ref(case)), f"forced split-K {kernel} m={m}")
         assert torch.equal(out, layer(a)), "split-K result is not deterministic run to run"
-        assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
-    finally:
-        lib.vaq_debug_set_decode_impl(-1)
-        lib.vaq_debug_set_decode2_config(0, 0)
-        lib.vaq_debug_set_decode_config(0, 0, 0)
+    assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
 
 
 @pytest.mark.parametrize("k,n", SMALL)
@@ -195,31 +186,27 @@ def test_prefill_gemm_split_k(device, k, n, m, asym):
 @pytest.mark.parametrize("asym", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_prefill_every_tile_shape(device, asym, dtype):
-    """Every tile shape of the prefill kernels, forced through the tuning export (the automatic choice only reaches some of
+    """Every tile shape of the prefill kernels, forced through a per-call tuning override (the automatic choice only reaches some of
     them at any one problem size), with and without K split over workgroups, against the oracle.  The direct-to-LDS
     shapes (ids 10-15 and 20, the one with alternating phases) dequantise exactly and add the same MFMA products in the
     same order, so without a K split they must agree with each other bit for bit."""
-    from vllm_amd import _lib
-    lib = _lib.load()
-    try:
-        for k, n, m in ((1024, 512, 300), (640, 320, 513), (384, 256, 257), (2048, 576, 70)):
-            case = o.make_w4a16_case(k, n, 128, asym=asym, seed=k + n + m)
-            layer = W4A16Layer(case, device, dtype)
-            a = _acts(m, k, device, dtype, seed=m)
-            ref = o.gemm_ref(a.cpu(), o.case_w_ref(case))
-            first = None
-            for tile in (10, 20, 11, 12, 13, 14, 15, 0, 1, 2):
-                for split in ((1, 0, 2, 3) if tile >= 10 else (0,)):      # 0: the automatic split, 1: none
-                    lib.vaq_debug_set_prefill_tile(tile + 100 * split)
+    from vllm_amd import _tuning
+    for k, n, m in ((1024, 512, 300), (640, 320, 513), (384, 256, 257), (2048, 576, 70)):
+        case = o.make_w4a16_case(k, n, 128, asym=asym, seed=k + n + m)
+        layer = W4A16Layer(case, device, dtype)
+        a = _acts(m, k, device, dtype, seed=m)
+        ref = o.gemm_ref(a.cpu(), o.case_w_ref(case))
+        first = None
+        for tile in (10, 20, 11, 12, 13, 14, 15, 0, 1, 2):
+            for split in ((1, 0, 2, 3) if tile >= 10 else (0,)):      # 0: the automatic split, 1: none
+                with _tuning.override(prefill_tile=tile + 1, prefill_split=split):
                     out = layer(a)
-                    check_gemm_close(out, ref, f"tile {tile} split {split} k={k} n={n} m={m}")
-                    if tile >= 10 and split == 1:
-                        if first is None:
-                            first = out
-                        assert torch.equal(out, first), f"tile {tile} differs from tile 10 (k={k} n={n} m={m})"
-            assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
-    finally:
-        lib.vaq_debug_set_prefill_tile(-1)
+                check_gemm_close(out, ref, f"tile {tile} split {split} k={k} n={n} m={m}")
+                if tile >= 10 and split == 1:
+                    if first is None:
+                        first = out
+                    assert torch.equal(out, first), f"tile {tile} differs from tile 10 (k={k} n={n} m={m})"
+        assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
 
 
 @pytest.mark.parametrize("group_size", [-1, 32, 64])
@@ -455,12 +442,12 @@ def test_decode_three_and_four_m_blocks(device, k, n, m):
 @pytest.mark.parametrize("k,n", LLAMA_SHAPES)
 @pytest.mark.parametrize("group_level", [False, True])
 def test_config3_prefill_llama_shapes_sampled(device, k, n, group_level):
-    """Asymmetric + act_order at M=4096 (also 512): the oracle is evaluated on 24 sampled rows (the full fp64 GEMM
+    """Asymmetric + act_order at M in {512, 2048, 4096}: the oracle is evaluated on 24 sampled rows (the full fp64 GEMM
     would take minutes on the CPU); rows are independent in a GEMM, so a wrong tile shows up in its rows."""
     case = o.make_w4a16_case(k, n, 128, asym=True, act_order=True, group_level_perm=group_level, seed=2)
     layer = W4A16Layer(case, device)
     w_ref = o.case_w_ref(case)
-    for m in (512, 4096):
+    for m in (512, 2048, 4096):
         a = _acts(m, k, device, seed=m)
         out = layer(a)
         rows = np.random.default_rng(m).choice(m, size=24, replace=False)
@@ -471,3 +458,15 @@ def test_config3_prefill_llama_shapes_sampled(device, k, n, group_level):
         assert torch.isfinite(out).all()
         col_norm = out.float().norm(dim=1)
         assert bool((col_norm > 0).all())
+
+
+@pytest.mark.parametrize("k,n", LLAMA_SHAPES)
+def test_config5_decode_step_gemm_llama_shapes(device, decode_kernel, k, n):
+    """The GEMM of BASELINE.json config 5: symmetric 4-bit, groups of 128, batch 32 (two 16-row blocks) at the four
+    Llama-3-8B projection shapes, full fp64 oracle."""
+    case = o.make_w4a16_case(k, n, 128, seed=5)
+    layer = W4A16Layer(case, device)
+    a = _acts(32, k, device, seed=32)
+    out = layer(a)
+    check_gemm_close(out, o.gemm_ref(a.cpu(), o.case_w_ref(case)), f"config 5 GEMM k={k} n={n} m=32")
+    assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"

@@ -15,7 +15,7 @@ import ctypes
 
 import torch
 
-from . import _lib
+from . import _lib, _tuning
 from .scalar_type import ScalarType, scalar_types
 
 FP8_DTYPE = torch.float8_e4m3fn        # gfx950 is an OCP part (reference: vllm/platforms/rocm.py:447-452)
@@ -268,19 +268,22 @@ def _gemm_impl(a: torch.Tensor, c_or_none: torch.Tensor | None, b_q_weight: torc
         c = c_or_none if c_or_none is not None else torch.empty((size_m, size_n), dtype=a.dtype, device=dev)
         if size_m == 0:
             return c
+        # Scratch for this problem: split-K partials and permuted activations from the caching allocator (safe under
+        # graph capture), arrival counters from the caller's `workspace`.  The library checks what it is handed against
+        # what the kernel it picks needs and reports a workspace that is too small (gptq_marlin.cu:899-902).
+        tune = _tuning.current_ref()
         n_ctmp, n_atmp, n_cnt = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
-        _lib.check(lib.vaq_w4a16_gemm_workspace(size_m, size_n, size_k, int(has_act_order), dev.index or 0,
-                                                ctypes.byref(n_ctmp), ctypes.byref(n_atmp), ctypes.byref(n_cnt)))
-        # decode sizes need their counters; the tile kernel falls back to an unsplit K when the array is too small
-        _check(size_m > 64 or workspace.numel() >= n_cnt.value,
-               f"workspace.numel = {workspace.numel()} is below min_workspace_size = {n_cnt.value}")
+        q_args = (size_m, size_n, size_k, int(has_act_order), dev.index or 0, ctypes.byref(n_ctmp), ctypes.byref(n_atmp),
+                  ctypes.byref(n_cnt))
+        _lib.check(lib.vaq_w4a16_gemm_workspace(*q_args) if tune is None
+                   else lib.vaq_w4a16_gemm_workspace_tuned(*q_args, tune))
         c_tmp = torch.empty((n_ctmp.value // 4,), dtype=torch.float32, device=dev) if n_ctmp.value else None
         a_tmp = torch.empty((n_atmp.value // 2,), dtype=a.dtype, device=dev) if n_atmp.value else None
-        _lib.check(lib.vaq_w4a16_gemm(
-            _ptr(a), a.stride(0), _ptr(b_q_weight), _ptr(b_scales), _ptr(b_zeros_or_none) if has_zp else None,
-            _ptr(perm_or_none) if has_act_order else None, _ptr(b_bias_or_none), _ptr(c), _ptr(c_tmp), _ptr(a_tmp),
-            _ptr(workspace), workspace.numel(), size_m, size_n, size_k, group_size, _dtype_tag(a.dtype), wtype, 0,
-            _stream(dev)))
+        g_args = (_ptr(a), a.stride(0), _ptr(b_q_weight), _ptr(b_scales), _ptr(b_zeros_or_none) if has_zp else None,
+                  _ptr(perm_or_none) if has_act_order else None, _ptr(b_bias_or_none), _ptr(c), _ptr(c_tmp),
+                  n_ctmp.value, _ptr(a_tmp), _ptr(workspace), workspace.numel(), size_m, size_n, size_k, group_size,
+                  _dtype_tag(a.dtype), wtype, 0, _stream(dev))
+        _lib.check(lib.vaq_w4a16_gemm(*g_args) if tune is None else lib.vaq_w4a16_gemm_tuned(*g_args, tune))
     return c
 
 
@@ -361,9 +364,10 @@ def _per_token_quant_impl(result: torch.Tensor, input: torch.Tensor, scale: torc
         return
     lib = _lib.load()
     with torch.cuda.device(input.device):
-        _lib.check(lib.vaq_fp8_quant_per_token(_ptr(input), _dtype_tag(input.dtype), input.stride(0), _ptr(result),
-                                               result.stride(0), _ptr(scale), _ptr(scale_ub), tokens, hidden,
-                                               _stream(input.device)))
+        args = (_ptr(input), _dtype_tag(input.dtype), input.stride(0), _ptr(result), result.stride(0), _ptr(scale),
+                _ptr(scale_ub), tokens, hidden, _stream(input.device))
+        tune = _tuning.current_ref()
+        _lib.check(lib.vaq_fp8_quant_per_token(*args) if tune is None else lib.vaq_fp8_quant_per_token_tuned(*args, tune))
 
 
 # ============================================================================ FP8 scaled GEMM
@@ -401,35 +405,43 @@ def _scaled_mm_impl(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor, a_scale
     dev = a.device
     with torch.cuda.device(dev):
         # scratch for the K split of mid-sized M: partial tiles from the caching allocator (capture-safe), arrival
-        # counters from one zeroed per-device array that the kernel leaves zero
+        # counters that are zero on entry and left zero, one array per (device, stream)
+        tune = _tuning.current_ref()
         n_ctmp, n_cnt = ctypes.c_size_t(), ctypes.c_size_t()
-        _lib.check(lib.vaq_fp8_scaled_mm_workspace(a.size(0), b.size(1), a.size(1), ctypes.byref(n_ctmp),
-                                                   ctypes.byref(n_cnt)))
+        q_args = (a.size(0), b.size(1), a.size(1), ctypes.byref(n_ctmp), ctypes.byref(n_cnt))
+        _lib.check(lib.vaq_fp8_scaled_mm_workspace(*q_args) if tune is None
+                   else lib.vaq_fp8_scaled_mm_workspace_tuned(*q_args, tune))
         c_tmp = counters = None
         if n_ctmp.value:
-            counters = _fp8_counters(dev)
-            if counters.numel() >= n_cnt.value:
-                c_tmp = torch.empty((n_ctmp.value // 4,), dtype=torch.float32, device=dev)
-            else:
-                counters = None
-        _lib.check(lib.vaq_fp8_scaled_mm_ws(_ptr(a), a.stride(0), _ptr(b), b.stride(1), _ptr(a_scales), a_scales.numel(),
-                                            _ptr(b_scales), b_scales.numel(), _ptr(bias), _ptr(out), out.stride(0),
-                                            _dtype_tag(out.dtype), a.size(0), b.size(1), a.size(1), _ptr(c_tmp),
-                                            n_ctmp.value if c_tmp is not None else 0, _ptr(counters),
-                                            counters.numel() if counters is not None else 0, _stream(dev)))
+            counters = _fp8_counters(dev, n_cnt.value)
+            c_tmp = torch.empty((n_ctmp.value // 4,), dtype=torch.float32, device=dev)
+        args = (_ptr(a), a.stride(0), _ptr(b), b.stride(1), _ptr(a_scales), a_scales.numel(), _ptr(b_scales),
+                b_scales.numel(), _ptr(bias), _ptr(out), out.stride(0), _dtype_tag(out.dtype), a.size(0), b.size(1),
+                a.size(1), _ptr(c_tmp), n_ctmp.value if c_tmp is not None else 0, _ptr(counters),
+                counters.numel() if counters is not None else 0, _stream(dev))
+        _lib.check(lib.vaq_fp8_scaled_mm_ws(*args) if tune is None else lib.vaq_fp8_scaled_mm_ws_tuned(*args, tune))
 
 
-_FP8_COUNTERS: dict[int, torch.Tensor] = {}
+_FP8_COUNTERS: dict[tuple[int, int], torch.Tensor] = {}
+_FP8_COUNTER_INTS = 16384
 
 
-def _fp8_counters(dev: torch.device) -> torch.Tensor:
-    """One zeroed int32 array per device for the FP8 GEMM's K split (the reference's CUTLASS path owns its workspace
-    too).  Created on first use; calls that use it must not overlap on different streams."""
+def _fp8_counters(dev: torch.device, need: int) -> torch.Tensor:
+    """Zeroed int32 arrival counters for the FP8 GEMM's K split (the op has no workspace argument; the reference's
+    CUTLASS path owns its workspace too).  One array per (device, stream): GEMMs on one stream run one after the other
+    and each leaves the counters zero, GEMMs on different streams never share an array.  An array is created on a
+    stream's first split-K call outside graph capture; a call that finds none while its stream is being captured, or
+    that needs more counters than the array holds, takes a fresh zeroed one for that call alone (an allocation of the
+    capture's own pool and a fill kernel, both legal inside a capture, replayed with the graph)."""
     idx = dev.index if dev.index is not None else torch.cuda.current_device()
-    t = _FP8_COUNTERS.get(idx)
-    if t is None:
-        t = torch.zeros(16384, dtype=torch.int32, device=dev)
-        _FP8_COUNTERS[idx] = t
+    key = (idx, torch.cuda.current_stream(dev).cuda_stream)
+    t = _FP8_COUNTERS.get(key)
+    if t is not None and t.numel() >= need:
+        return t
+    if torch.cuda.is_current_stream_capturing() or need > _FP8_COUNTER_INTS:
+        return torch.zeros(need, dtype=torch.int32, device=dev)
+    t = torch.zeros(_FP8_COUNTER_INTS, dtype=torch.int32, device=dev)
+    _FP8_COUNTERS[key] = t
     return t
 
 

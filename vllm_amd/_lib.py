@@ -30,8 +30,8 @@ _SIGNATURES = {
     "vaq_w4a16_gemm_workspace": (c_int, [c_int64, c_int64, c_int64, c_int, c_int, POINTER(c_size_t), POINTER(c_size_t),
                                          POINTER(c_size_t)]),
     "vaq_w4a16_gemm": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                               c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int,
-                               c_void_p]),
+                               c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int,
+                               c_int, c_void_p]),
     "vaq_permute_cols": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
     "vaq_fp8_quant_per_token": (c_int, [c_void_p, c_int, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
                                         c_int64, c_void_p]),
@@ -51,16 +51,19 @@ _SIGNATURES = {
                                      c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p,
                                      c_int64, c_void_p]),
 }
-# tuning aids exported by the library but not part of the drop-in header
-_DEBUG_SIGNATURES = {
-    "vaq_debug_set_decode_config": (None, [c_int, c_int, c_int]),
-    "vaq_debug_set_prefill_tile": (None, [c_int]),
-    "vaq_debug_set_decode_impl": (None, [c_int]),
-    "vaq_debug_set_decode2_config": (None, [c_int, c_int]),
-    "vaq_debug_set_fp8_config": (None, [c_int, c_int]),
-    "vaq_debug_set_fp8_tile_cfg": (None, [c_int, c_int]),
-    "vaq_debug_set_quant_row_per_wave": (None, [c_int]),
-}
+class VaqTuning(ctypes.Structure):
+    """``VaqTuning`` of the header: kernel-variant overrides for ONE call (tests, benchmarks); all zero = automatic."""
+    _fields_ = [(n, c_int) for n in (
+        "decode_impl", "decode2_gs", "decode2_wks", "decode2_wn", "decode_tg", "decode_wk", "decode_gx", "decode_depth",
+        "prefill_tile", "prefill_split", "fp8_path", "fp8_tile_impl", "fp8_tile_cfg", "fp8_split", "fp8_gx",
+        "fp8_stream_split", "quant_wg_per_row")] + [("exp", c_int * 15)]
+
+
+_TUNING_P = POINTER(VaqTuning)
+for _name in ("vaq_w4a16_gemm_workspace", "vaq_w4a16_gemm", "vaq_fp8_scaled_mm_workspace", "vaq_fp8_scaled_mm_ws",
+              "vaq_fp8_quant_per_token"):
+    _res, _args = _SIGNATURES[_name]
+    _SIGNATURES[_name + "_tuned"] = (_res, [*_args, _TUNING_P])
 
 _lib = None
 
@@ -79,12 +82,10 @@ def load() -> ctypes.CDLL:
             f"{LIB_PATH} is missing: the gfx950 kernels are not built (run `python -m vllm_amd.build`). "
             "vllm_amd has no fallback path.")
     lib = ctypes.CDLL(str(LIB_PATH))
-    for name, (res, args) in {**_SIGNATURES, **_DEBUG_SIGNATURES}.items():
+    for name, (res, args) in _SIGNATURES.items():
         try:
             fn = getattr(lib, name)
         except AttributeError:
-            if name in _DEBUG_SIGNATURES:
-                continue
             raise RuntimeError(f"{LIB_PATH} does not export {name}; rebuild it") from None
         fn.restype = res
         fn.argtypes = args

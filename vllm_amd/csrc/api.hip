@@ -14,6 +14,13 @@ void set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
+static thread_local const VaqTuning* g_tuning = nullptr;
+static const VaqTuning g_no_tuning = {};
+
+const VaqTuning& tuning() { return g_tuning ? *g_tuning : g_no_tuning; }
+TuningScope::TuningScope(const VaqTuning* t) : prev_(g_tuning) { g_tuning = t; }
+TuningScope::~TuningScope() { g_tuning = prev_; }
+
 // Immutable per-device cache (the only host-visible state of the library).
 static int g_cus[64];
 static std::once_flag g_cus_once[64];

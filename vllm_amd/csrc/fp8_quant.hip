@@ -18,7 +18,6 @@ namespace vaq {
 constexpr float FP8_MAX = 448.0f;
 constexpr int QT = 256;         // threads per workgroup
 constexpr int QV = 8;           // cached 8-element vectors per thread
-static int g_quant_row_per_wave = 1;    // tuning aid: 0 = always one workgroup per row
 
 template <typename T>
 __device__ inline float load_as_float(const T* p);
@@ -267,14 +266,22 @@ static int check_quant(const char* who, const void* in, int64_t in_stride, const
 extern "C" int vaq_fp8_quant_per_token(const void* in, int in_dtype, int64_t in_row_stride, uint8_t* out,
                                        int64_t out_row_stride, float* scales, const float* scale_ub, int64_t rows,
                                        int64_t hidden, void* stream) {
+  return vaq_fp8_quant_per_token_tuned(in, in_dtype, in_row_stride, out, out_row_stride, scales, scale_ub, rows, hidden,
+                                       stream, nullptr);
+}
+
+extern "C" int vaq_fp8_quant_per_token_tuned(const void* in, int in_dtype, int64_t in_row_stride, uint8_t* out,
+                                             int64_t out_row_stride, float* scales, const float* scale_ub, int64_t rows,
+                                             int64_t hidden, void* stream, const VaqTuning* tuning_or_null) {
   using namespace vaq;
+  const TuningScope scope(tuning_or_null);
   int rc = check_quant("fp8_quant_per_token", in, in_row_stride, out, out_row_stride, scales, rows, hidden);
   if (rc != VAQ_OK || rows == 0) return rc;
   // Measured: a row per wavefront is 1.1-1.6x faster for short rows in large batches; with few rows a whole workgroup
   // per row has the shorter latency, and from 4096 elements on the 64 registers of row data per lane cost more than the
   // barriers saved.
   const bool many_short_rows = hidden <= 1024 ? rows >= 512 : (hidden <= 2048 && rows >= 2048);
-  if (g_quant_row_per_wave && many_short_rows &&
+  if (tuning().quant_wg_per_row == 0 && many_short_rows &&
       row_per_wave_ok(in, in_dtype, in_row_stride, out, out_row_stride, hidden)) {
     if (in_dtype == VAQ_BF16)
       launch_row_per_wave<bf16_t>(in, in_row_stride, out, out_row_stride, scales, scale_ub, rows, hidden, (hipStream_t)stream);
@@ -318,6 +325,3 @@ extern "C" int vaq_fp8_quant_dynamic(const void* in, int in_dtype, int64_t in_ro
   VAQ_CHECK_LAUNCH("fp8_quant_dynamic");
   return VAQ_OK;
 }
-
-// Benchmark / tuning aid, not part of the drop-in surface: 0 = per-token quantisation always with one workgroup per row.
-extern "C" void vaq_debug_set_quant_row_per_wave(int on) { vaq::g_quant_row_per_wave = on; }

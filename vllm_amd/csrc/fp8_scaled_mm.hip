@@ -860,9 +860,9 @@ __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p,
 
 // ----------------------------------------------------------------------------- host side
 
-static int g_force_fp8_path = 0;   // 0 auto, 1 stream, 2 tile
-static int g_fp8_stream_split = 0;   // -1: the stream kernel over two K halves is off (benchmarking)
-static int g_force_fp8_gx = 0;
+// Overrides for tests and benchmarks come through tuning() (all zero = automatic): fp8_path 1 stream / 2 tile,
+// fp8_tile_impl 1 = register-staged tile kernel, fp8_tile_cfg = fixed multi-stage tile shape (-1: two-stage kernel),
+// fp8_split = K split of the tile kernel, fp8_gx = stream-kernel grid, fp8_stream_split -1 = no two-halves stream route.
 
 template <bool BF16_OUT, int WMB, int WNB>
 static int launch_tile(const Fp8MMParams& p, hipStream_t s) {
@@ -899,11 +899,6 @@ static int launch_tile3(const Fp8MMParams& p, hipStream_t s) {
   return VAQ_OK;
 }
 
-static int g_fp8_tile3_cfg = 0;    // 0: automatic, -1: off (two-stage kernel), >0: a fixed tile shape (benchmarking)
-static int g_fp8_tile_impl = 0;   // 0: direct-to-LDS kernel when its preconditions hold, 1: always the register-staged kernel
-
-static int g_fp8_force_split = 0;
-
 struct Fp8TilePlan {
   int cfg, sk, bm, bn, nw;
   int64_t tiles;
@@ -918,7 +913,7 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   const int cus = num_cus_current_device();
   auto tiles = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   Fp8TilePlan pl;
-  pl.cfg = g_fp8_tile3_cfg;
+  pl.cfg = tuning().fp8_tile_cfg;
   // the largest tile shape that fills 70 % of the compute units (measured on the Llama shapes, M = 256 .. 4096: a
   // partly filled device of large tiles beats a full one of small tiles by 25-40 %); for 128 x 128 also when two
   // parts of a long K get it there (14336 x 4096 at M = 512, cold, 73 -> 62 us)
@@ -926,7 +921,7 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   if (pl.cfg <= 0)
     pl.cfg = tiles(256, 256) * 10 >= cus * 7 ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (tiles(128, 128) * parts128 * 10 >= cus * 7 ? 3 : 4));
   // the smallest tile with two k-slices per step: 5-8 % faster on a short K (half the barriers), no gain on a long one
-  if (g_fp8_tile3_cfg <= 0 && pl.cfg == 4 && K % 128 == 0 && K <= 8192) pl.cfg = 14;
+  if (tuning().fp8_tile_cfg <= 0 && pl.cfg == 4 && K % 128 == 0 && K <= 8192) pl.cfg = 14;
   if (pl.cfg >= 10 && K % 128 != 0) pl.cfg %= 10;      // two k-slices per step need K % 128 == 0
   switch (pl.cfg) {
     case 3: case 13: case 23: pl.bm = 128; pl.bn = 128; pl.nw = 4; break;
@@ -947,7 +942,7 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
     if (sk < 1) sk = 1;
     while (sk & (sk - 1)) --sk;       // a power of two (3 splits measured slower than 2)
   }
-  if (g_fp8_force_split > 0) sk = g_fp8_force_split <= steps ? g_fp8_force_split : steps;
+  if (tuning().fp8_split > 0) sk = tuning().fp8_split <= steps ? tuning().fp8_split : steps;
   while (sk > 1 && (uint64_t)sk * (uint64_t)pl.tiles * pl.bm * pl.bn * 4 >= (1ull << 32)) --sk;   // 32-bit buffer offsets
   pl.sk = sk;
   return pl;
@@ -956,9 +951,9 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
 template <bool BF16_OUT>
 static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t counter_ints, hipStream_t s) {
   Fp8MMParams p = p_in;
-  const bool direct_ok = g_fp8_tile_impl == 0 && p.K % 64 == 0 && (uint64_t)p.M * (uint64_t)p.lda < (1ull << 32) &&
+  const bool direct_ok = tuning().fp8_tile_impl == 0 && p.K % 64 == 0 && (uint64_t)p.M * (uint64_t)p.lda < (1ull << 32) &&
                          (uint64_t)p.N * (uint64_t)p.ldb < (1ull << 32);
-  if (direct_ok && g_fp8_tile_impl == 0 && g_fp8_tile3_cfg >= 0) {
+  if (direct_ok && tuning().fp8_tile_impl == 0 && tuning().fp8_tile_cfg >= 0) {
     Fp8TilePlan pl = plan_tile3(p.M, p.N, p.K);
     // without (enough) scratch from the caller the unsplit kernel still gives the result
     if (pl.sk > 1 && (p.c_tmp == nullptr || p.counters == nullptr || counter_ints < pl.tiles * pl.nw ||
@@ -1047,7 +1042,7 @@ static int stream_steps_per_wave(int64_t M, int64_t N, int64_t K) {
 // 14336 x 4096 at M = 24 / 32 34.7 / 35.1 -> 21.6 / 22.5 us, 16384 x 4096 at M = 32 37.1 -> 27.4 us).  For M <= 16 beyond
 // K = 14336 (14 steps per wavefront and half) the tile kernel stays ahead: 28672 x 8192 72 against 85 us.
 static int stream_split_steps_per_wave(int64_t M, int64_t N, int64_t K) {
-  if (g_fp8_stream_split < 0 || M <= 16 || M > 32 || stream_steps_per_wave(M, N, K) != 0) return 0;
+  if (tuning().fp8_stream_split < 0 || M <= 16 || M > 32 || stream_steps_per_wave(M, N, K) != 0) return 0;
   const int64_t half = ((K + 127) / 128 + 1) / 2;
   return half <= 8 * 8 ? 8 : 0;
 }
@@ -1064,7 +1059,7 @@ static bool dispatch_stream_split(const Fp8MMParams& p, int64_t c_tmp_bytes, int
   const int wk = (half + ks - 1) / ks;              // >= 5: the K range of this route starts above one workgroup's
   const int cus = num_cus_current_device();
   const int rounds = (2 * NT + cus - 1) / cus;
-  int gx = g_force_fp8_gx > 0 ? g_force_fp8_gx : (NT + rounds - 1) / rounds;
+  int gx = tuning().fp8_gx > 0 ? tuning().fp8_gx : (NT + rounds - 1) / rounds;
   if (gx > NT) gx = NT;
   launch_stream<BF16_OUT, 8, 2, true>(p, wk, gx, s);
   return true;
@@ -1084,7 +1079,7 @@ static bool dispatch_stream(const Fp8MMParams& p, hipStream_t s) {
   // 31.8 / 38.0 -> 30.4 / 31.9 us, M = 1 unchanged or 3 % faster)
   const int cus = num_cus_current_device();
   const int rounds = (NT + cus - 1) / cus;
-  int gx = g_force_fp8_gx > 0 ? g_force_fp8_gx : (NT + rounds - 1) / rounds;
+  int gx = tuning().fp8_gx > 0 ? tuning().fp8_gx : (NT + rounds - 1) / rounds;
   if (gx > NT) gx = NT;
   if (MB == 1) {
     if (ks == 4) launch_stream<BF16_OUT, 4, 1>(p, wk, gx, s);
@@ -1105,22 +1100,28 @@ static bool dispatch_stream(const Fp8MMParams& p, hipStream_t s) {
 
 extern "C" int vaq_fp8_scaled_mm_workspace(int64_t size_m, int64_t size_n, int64_t size_k, size_t* c_tmp_bytes,
                                            size_t* counter_ints) {
+  return vaq_fp8_scaled_mm_workspace_tuned(size_m, size_n, size_k, c_tmp_bytes, counter_ints, nullptr);
+}
+
+extern "C" int vaq_fp8_scaled_mm_workspace_tuned(int64_t size_m, int64_t size_n, int64_t size_k, size_t* c_tmp_bytes,
+                                                 size_t* counter_ints, const VaqTuning* tuning_or_null) {
   using namespace vaq;
+  const TuningScope scope(tuning_or_null);
   VAQ_CHECK_ARG(c_tmp_bytes && counter_ints, "fp8_scaled_mm_workspace: null output pointer");
   VAQ_CHECK_ARG(size_m >= 0 && size_n > 0 && size_k > 0 && size_m < (1ll << 31) && size_n < (1ll << 31) &&
                     size_k < (1ll << 31), "fp8_scaled_mm_workspace: bad shape M=%lld N=%lld K=%lld", (long long)size_m,
                 (long long)size_n, (long long)size_k);
   *c_tmp_bytes = 0;
   *counter_ints = 0;
-  const bool stream = g_force_fp8_path != 2 && stream_steps_per_wave(size_m, size_n, size_k) != 0;      // needs no scratch
+  const bool stream = tuning().fp8_path != 2 && stream_steps_per_wave(size_m, size_n, size_k) != 0;      // needs no scratch
   if (stream) return VAQ_OK;
-  if (g_force_fp8_path != 2 && stream_split_steps_per_wave(size_m, size_n, size_k) != 0) {
+  if (tuning().fp8_path != 2 && stream_split_steps_per_wave(size_m, size_n, size_k) != 0) {
     const size_t units = (size_t)(size_n / 16) * (size_t)((size_m + 15) / 16);
     *c_tmp_bytes = 2 * units * 1024;
     *counter_ints = units;
     return VAQ_OK;
   }
-  if (size_k % 64 != 0 || g_fp8_tile_impl != 0 || g_fp8_tile3_cfg < 0) return VAQ_OK;
+  if (size_k % 64 != 0 || tuning().fp8_tile_impl != 0 || tuning().fp8_tile_cfg < 0) return VAQ_OK;
   const Fp8TilePlan pl = plan_tile3((int)size_m, (int)size_n, (int)size_k);
   if (pl.sk > 1) {
     *c_tmp_bytes = (size_t)pl.sk * (size_t)pl.tiles * pl.bm * pl.bn * sizeof(float);
@@ -1142,7 +1143,17 @@ extern "C" int vaq_fp8_scaled_mm_ws(const uint8_t* a, int64_t lda, const uint8_t
                                     int64_t ldc, int out_dtype, int64_t size_m, int64_t size_n, int64_t size_k,
                                     float* c_tmp, int64_t c_tmp_bytes, int32_t* counters, int64_t counter_ints,
                                     void* stream) {
+  return vaq_fp8_scaled_mm_ws_tuned(a, lda, b, ldb, sa, sa_count, sb, sb_count, bias, out, ldc, out_dtype, size_m, size_n,
+                                    size_k, c_tmp, c_tmp_bytes, counters, counter_ints, stream, nullptr);
+}
+
+extern "C" int vaq_fp8_scaled_mm_ws_tuned(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t ldb, const float* sa,
+                                          int64_t sa_count, const float* sb, int64_t sb_count, const void* bias,
+                                          void* out, int64_t ldc, int out_dtype, int64_t size_m, int64_t size_n,
+                                          int64_t size_k, float* c_tmp, int64_t c_tmp_bytes, int32_t* counters,
+                                          int64_t counter_ints, void* stream, const VaqTuning* tuning_or_null) {
   using namespace vaq;
+  const TuningScope scope(tuning_or_null);
   VAQ_CHECK_ARG(size_m >= 0 && size_n > 0 && size_k > 0, "fp8_scaled_mm: bad shape M=%lld N=%lld K=%lld",
                 (long long)size_m, (long long)size_n, (long long)size_k);
   VAQ_CHECK_ARG(size_m < (1ll << 31) && size_n < (1ll << 31) && size_k < (1ll << 31), "fp8_scaled_mm: shape too large");
@@ -1178,9 +1189,9 @@ extern "C" int vaq_fp8_scaled_mm_ws(const uint8_t* a, int64_t lda, const uint8_t
   hipStream_t s = (hipStream_t)stream;
   const bool bf16 = out_dtype == VAQ_BF16;
   bool done = false;
-  const bool want_stream = g_force_fp8_path != 2 && stream_steps_per_wave(size_m, size_n, size_k) != 0;
+  const bool want_stream = tuning().fp8_path != 2 && stream_steps_per_wave(size_m, size_n, size_k) != 0;
   if (want_stream) done = bf16 ? dispatch_stream<true>(p, s) : dispatch_stream<false>(p, s);
-  if (!done && g_force_fp8_path != 2)
+  if (!done && tuning().fp8_path != 2)
     done = bf16 ? dispatch_stream_split<true>(p, c_tmp_bytes, counter_ints, s)
                 : dispatch_stream_split<false>(p, c_tmp_bytes, counter_ints, s);
   if (!done) {
@@ -1189,19 +1200,4 @@ extern "C" int vaq_fp8_scaled_mm_ws(const uint8_t* a, int64_t lda, const uint8_t
   }
   VAQ_CHECK_LAUNCH("fp8_scaled_mm");
   return VAQ_OK;
-}
-
-// Benchmark / tuning aid, not part of the drop-in surface.  path: 0 auto, 1 stream, 2 tile; gx: stream-kernel grid.
-extern "C" void vaq_debug_set_fp8_stream_split(int mode) { vaq::g_fp8_stream_split = mode; }
-
-extern "C" void vaq_debug_set_fp8_tile_cfg(int cfg, int split) {     // cfg: 0 = automatic, -1 = off; split: 0 = automatic
-  vaq::g_fp8_tile3_cfg = cfg;
-  vaq::g_fp8_force_split = split;
-}
-extern "C" void vaq_debug_set_fp8_config(int path, int gx) {
-  vaq::g_force_fp8_path = path % 10;
-  vaq::g_fp8_tile_impl = (path / 10) % 10;     // tens digit: 1 = force the register-staged tile kernel
-  vaq::g_fp8_tile3_cfg = (path / 100) % 10 == 9 ? -1 : (path / 100) % 10;   // hundreds digit: multi-stage tile shape (9 = off)
-  vaq::g_fp8_force_split = path / 1000;                     // thousands: forced K split (0 = automatic)
-  vaq::g_force_fp8_gx = gx;
 }

@@ -40,6 +40,21 @@ void set_error(const char* fmt, ...);   // defined in api.hip (thread-local buff
 
 int num_cus_current_device();   // cached per device, api.hip
 
+// Kernel-variant overrides of the `_tuned` entry points (tests, benchmarks).  An entry point opens a TuningScope with
+// the caller's struct; the host code below it reads `tuning()`, which is all zeros (= automatic) outside a scope.  The
+// pointer lives in a thread-local for the duration of that one call: nothing persists between calls or crosses threads.
+const VaqTuning& tuning();
+class TuningScope {
+ public:
+  explicit TuningScope(const VaqTuning* t);
+  ~TuningScope();
+  TuningScope(const TuningScope&) = delete;
+  TuningScope& operator=(const TuningScope&) = delete;
+
+ private:
+  const VaqTuning* prev_;
+};
+
 // Dynamic LDS above the default limit has to be reserved per kernel and per device.  `reserved` is the calling launch
 // function's own static array (one per kernel instantiation, zero-initialised): bytes already reserved on each device.
 // The attribute is idempotent, so two threads racing here at worst set it twice.

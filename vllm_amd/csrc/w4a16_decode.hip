@@ -324,14 +324,13 @@ struct DecodeConfig {
   int tg, wk, sk, gx, maxw, d;
 };
 
-static int g_force_tg = 0, g_force_wk = 0, g_force_gx = 0, g_force_d = 0;
-
 // `wk` wavefronts of a workgroup x `sk` workgroups cover the K/128 groups, TG groups per wavefront.
 static DecodeConfig pick_decode_config(int M, int N, int K) {
   const int G = K / 128, NT = N / 16;
   const int MB = M <= 16 ? 1 : 2;
+  const VaqTuning& tn = tuning();
   DecodeConfig c;
-  if (g_force_tg > 0) c.tg = g_force_tg;
+  if (tn.decode_tg > 0) c.tg = tn.decode_tg;
   else if (MB == 2) c.tg = 1;
   else if (G % 7 == 0 && G >= 56) c.tg = 7;      // K = 14336: 7 groups per wavefront, 8 wavefronts, 2 workgroups
   else c.tg = G >= 2 ? 2 : 1;
@@ -340,16 +339,16 @@ static DecodeConfig pick_decode_config(int M, int N, int K) {
   const int kw = (G + c.tg - 1) / c.tg;          // wavefronts needed along K
   int wk_max = (c.tg >= 4 || (MB == 2 && c.tg == 2)) ? 8 : 16;
   c.maxw = wk_max > 8 ? 16 : 8;                  // the instantiated launch bound; fewer wavefronts may run under it
-  if (g_force_wk > 0 && g_force_wk < wk_max) wk_max = g_force_wk;
+  if (tn.decode_wk > 0 && tn.decode_wk < wk_max) wk_max = tn.decode_wk;
   c.sk = (kw + wk_max - 1) / wk_max;
   c.wk = (kw + c.sk - 1) / c.sk;
   const int cus = num_cus_current_device();
-  int gx = g_force_gx > 0 ? g_force_gx : cus / c.sk;
+  int gx = tn.decode_gx > 0 ? tn.decode_gx : cus / c.sk;
   if (gx < 1) gx = 1;
   if (gx > NT) gx = NT;
   c.gx = gx;
   const int per = (NT + gx - 1) / gx;           // n-tiles per workgroup
-  c.d = g_force_d > 0 ? g_force_d : (per >= 2 ? 2 : 1);   // depth 3 spills in the 128-register shapes
+  c.d = tn.decode_depth > 0 ? tn.decode_depth : (per >= 2 ? 2 : 1);   // depth 3 spills in the 128-register shapes
   if (c.tg == 7) c.d = 1;
   if (c.d > 3) c.d = 3;
   if (c.d < 1) c.d = 1;
@@ -401,8 +400,9 @@ int w4a16_decode_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* cou
 }
 
 int w4a16_decode_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
-                        const int32_t* perm, const void* bias, void* c, float* c_tmp, int32_t* counters,
-                        int64_t counter_ints, int M, int N, int K, bool channelwise, int dtype, hipStream_t s) {
+                        const int32_t* perm, const void* bias, void* c, float* c_tmp, int64_t c_tmp_bytes,
+                        int32_t* counters, int64_t counter_ints, int M, int N, int K, bool channelwise, int dtype,
+                        hipStream_t s) {
   DecodeParams p;
   p.a = (const uint16_t*)a;
   p.lda = lda;
@@ -433,6 +433,8 @@ int w4a16_decode_launch(const void* a, int64_t lda, const int32_t* b, const void
     VAQ_CHECK_ARG(counter_ints >= (int64_t)p.NT * MB,
                   "w4a16_gemm: workspace.numel = %lld is below min_workspace_size = %lld", (long long)counter_ints,
                   (long long)p.NT * MB);
+    VAQ_CHECK_ARG(c_tmp_bytes >= (int64_t)cfg.sk * p.NT * MB * 1024, "w4a16_gemm: c_tmp holds %lld bytes, the K split needs %lld",
+                  (long long)c_tmp_bytes, (long long)cfg.sk * p.NT * MB * 1024);
   }
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
@@ -449,12 +451,3 @@ int w4a16_decode_launch(const void* a, int64_t lda, const int32_t* b, const void
 }
 
 }  // namespace vaq
-
-// Benchmark / tuning aid, not part of the drop-in surface: override the decode launch shape
-// (0 = automatic).  Process-global and not thread-safe.
-extern "C" void vaq_debug_set_decode_config(int tg, int wk, int gx) {
-  vaq::g_force_tg = tg;
-  vaq::g_force_wk = wk;
-  vaq::g_force_gx = gx % 100000;
-  vaq::g_force_d = gx / 100000;     // prefetch depth rides in the upper digits: gx = depth * 100000 + grid
-}

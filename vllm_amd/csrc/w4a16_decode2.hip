@@ -10,8 +10,6 @@ struct Decode2Config {
   int gs, wks, wn, sk, mr;
 };
 
-static int g2_force_gs = 0, g2_force_wks = 0, g2_force_wn = 0;
-
 static int round_gs(int x, int sub, bool w8) {
   const int opts[] = {1, 2, 4, 7, 8, 14, 16};
   for (int o : opts) {
@@ -41,9 +39,10 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8) 
   int wks = 1;
   while (wks * 2 <= want && wks < 16) wks *= 2;
   while (wks > 1 && wks > gslab) wks /= 2;
-  if (g2_force_wks > 0) wks = g2_force_wks;
+  const VaqTuning& tn = tuning();
+  if (tn.decode2_wks > 0) wks = tn.decode2_wks;
   int gs = round_gs((gslab + wks - 1) / wks, sub, w8);
-  if (g2_force_gs > 0) gs = g2_force_gs;
+  if (tn.decode2_gs > 0) gs = tn.decode2_gs;
   while (wks * gs > slab_max && wks > 1) wks /= 2;     // respect the LDS limit
   if (gs > slab_max) {                                 // rounding up went past it: largest instantiated size below
     const int opts[] = {8, 7, 4, 2, 1};
@@ -78,7 +77,7 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8) 
       best_wn = wn;
     }
   }
-  c.wn = g2_force_wn > 0 ? g2_force_wn : best_wn;
+  c.wn = tn.decode2_wn > 0 ? tn.decode2_wn : best_wn;
   if (c.wn * wks > D2_WAVES) c.wn = D2_WAVES / wks;
   return c;
 }
@@ -124,9 +123,9 @@ int w4a16_decode2_workspace(int M, int N, int K, int sub, bool w8, size_t* c_tmp
 }
 
 int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
-                         const int32_t* perm, const void* bias, void* c, float* c_tmp, int32_t* counters,
-                         int64_t counter_ints, int M, int N, int K, int sub, bool channelwise, bool w8, int dtype,
-                         hipStream_t s) {
+                         const int32_t* perm, const void* bias, void* c, float* c_tmp, int64_t c_tmp_bytes,
+                         int32_t* counters, int64_t counter_ints, int M, int N, int K, int sub, bool channelwise,
+                         bool w8, int dtype, hipStream_t s) {
   Decode2Params p;
   p.a = (const uint16_t*)a;
   p.lda = lda;
@@ -158,6 +157,8 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
     VAQ_CHECK_ARG(counter_ints >= (int64_t)p.NT * MB,
                   "w4a16_gemm: workspace.numel = %lld is below min_workspace_size = %lld", (long long)counter_ints,
                   (long long)p.NT * MB);
+    VAQ_CHECK_ARG(c_tmp_bytes >= (int64_t)cfg.sk * p.NT * MB * 1024, "w4a16_gemm: c_tmp holds %lld bytes, the K split needs %lld",
+                  (long long)c_tmp_bytes, (long long)cfg.sk * p.NT * MB * 1024);
   }
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
@@ -174,10 +175,3 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
 }
 
 }  // namespace vaq
-
-// Benchmark / tuning aid, not part of the drop-in surface (0 = automatic).  Process-global, not thread-safe.
-extern "C" void vaq_debug_set_decode2_config(int gs, int wks) {
-  vaq::g2_force_gs = gs;
-  vaq::g2_force_wks = wks % 100;      // wks + 100 * (n-tiles per workgroup)
-  vaq::g2_force_wn = wks / 100;
-}

@@ -5,21 +5,22 @@ namespace vaq {
 // `sub` = quantisation groups per 128-row weight tile (1, 2, 4); `channelwise` = one scale row for all of K (sub == 1)
 int w4a16_decode_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* counter_ints);
 int w4a16_decode_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
-                        const int32_t* perm, const void* bias, void* c, float* c_tmp, int32_t* counters,
-                        int64_t counter_ints, int M, int N, int K, bool channelwise, int dtype, hipStream_t s);
+                        const int32_t* perm, const void* bias, void* c, float* c_tmp, int64_t c_tmp_bytes,
+                        int32_t* counters, int64_t counter_ints, int M, int N, int K, bool channelwise, int dtype,
+                        hipStream_t s);
 int w4a16_decode2_workspace(int M, int N, int K, int sub, bool w8, size_t* c_tmp_bytes, size_t* counter_ints);
 int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
-                         const int32_t* perm, const void* bias, void* c, float* c_tmp, int32_t* counters,
-                         int64_t counter_ints, int M, int N, int K, int sub, bool channelwise, bool w8, int dtype,
-                         hipStream_t s);
+                         const int32_t* perm, const void* bias, void* c, float* c_tmp, int64_t c_tmp_bytes,
+                         int32_t* counters, int64_t counter_ints, int M, int N, int K, int sub, bool channelwise,
+                         bool w8, int dtype, hipStream_t s);
 int w4a16_prefill_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* counter_ints);
 int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
-                         const void* bias, void* c, float* c_tmp, int32_t* counters, int64_t counter_ints, int M, int N,
-                         int K, int sub, bool channelwise, bool w8, int dtype, hipStream_t s);
+                         const void* bias, void* c, float* c_tmp, int64_t c_tmp_bytes, int32_t* counters,
+                         int64_t counter_ints, int M, int N, int K, int sub, bool channelwise, bool w8, int dtype,
+                         hipStream_t s);
 
 constexpr int64_t DECODE_MAX_M = 64;          // up to four m-blocks of 16 rows on the LDS-staged kernel
 constexpr int64_t DECODE_MAX_M_2BLK = 32;     // the register-resident kernel, groups below 128 rows and 8-bit codes: two
-static int g_decode_impl = -1;  // -1: automatic, 0: LDS-staged activations (w4a16_decode2.hip), 1: register-resident (w4a16_decode.hip)
 
 // Measured on MI355X (cold weights): staging the activations once per workgroup in LDS (one independent task per
 // wavefront, no barrier in the K loop) wins on every Llama-3-8B projection and on 8192 x 28672 (30 us against 43.5 us
@@ -30,7 +31,7 @@ static int decode_impl_for(int64_t size_m, int64_t size_n, int64_t lda, int sub,
   // the LDS-staged kernel addresses A through a 32-bit buffer offset
   if (size_m * lda * 2 >= (1ll << 31)) return 1;
   if (sub > 1 || w8) return 0;    // groups below 128 rows and 8-bit codes are built for the LDS-staged kernel only
-  if (g_decode_impl >= 0) return g_decode_impl;
+  if (tuning().decode_impl > 0) return tuning().decode_impl - 1;   // tests / benchmarks: 1 LDS-staged, 2 register-resident
   return (size_n >= 65536 && size_m > 2 && size_m <= 16) ? 1 : 0;
 }
 
@@ -49,8 +50,16 @@ static int check_shape(int64_t size_m, int64_t size_n, int64_t size_k) {
 
 extern "C" int vaq_w4a16_gemm_workspace(int64_t size_m, int64_t size_n, int64_t size_k, int has_perm, int device,
                                         size_t* c_tmp_bytes, size_t* a_tmp_bytes, size_t* counter_ints) {
+  return vaq_w4a16_gemm_workspace_tuned(size_m, size_n, size_k, has_perm, device, c_tmp_bytes, a_tmp_bytes, counter_ints,
+                                        nullptr);
+}
+
+extern "C" int vaq_w4a16_gemm_workspace_tuned(int64_t size_m, int64_t size_n, int64_t size_k, int has_perm, int device,
+                                              size_t* c_tmp_bytes, size_t* a_tmp_bytes, size_t* counter_ints,
+                                              const VaqTuning* tuning_or_null) {
   using namespace vaq;
   (void)device;
+  const TuningScope scope(tuning_or_null);
   VAQ_CHECK_ARG(c_tmp_bytes && a_tmp_bytes && counter_ints, "w4a16_gemm_workspace: null output pointer");
   int rc = check_shape(size_m, size_n, size_k);
   if (rc != VAQ_OK) return rc;
@@ -95,10 +104,21 @@ extern "C" int vaq_w4a16_gemm_workspace(int64_t size_m, int64_t size_n, int64_t 
 }
 
 extern "C" int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
-                              const int32_t* perm, const void* bias, void* c, float* c_tmp, void* a_tmp,
-                              int32_t* counters, int64_t counter_ints, int64_t size_m, int64_t size_n, int64_t size_k,
-                              int group_size, int dtype, int wtype, int force_path, void* stream) {
+                              const int32_t* perm, const void* bias, void* c, float* c_tmp, int64_t c_tmp_bytes,
+                              void* a_tmp, int32_t* counters, int64_t counter_ints, int64_t size_m, int64_t size_n,
+                              int64_t size_k, int group_size, int dtype, int wtype, int force_path, void* stream) {
+  return vaq_w4a16_gemm_tuned(a, lda, b, scales, zeros, perm, bias, c, c_tmp, c_tmp_bytes, a_tmp, counters, counter_ints,
+                              size_m, size_n, size_k, group_size, dtype, wtype, force_path, stream, nullptr);
+}
+
+extern "C" int vaq_w4a16_gemm_tuned(const void* a, int64_t lda, const int32_t* b, const void* scales,
+                                    const int32_t* zeros, const int32_t* perm, const void* bias, void* c, float* c_tmp,
+                                    int64_t c_tmp_bytes, void* a_tmp, int32_t* counters, int64_t counter_ints,
+                                    int64_t size_m, int64_t size_n, int64_t size_k, int group_size, int dtype, int wtype,
+                                    int force_path, void* stream, const VaqTuning* tuning_or_null) {
   using namespace vaq;
+  const TuningScope scope(tuning_or_null);
+  VAQ_CHECK_ARG(c_tmp_bytes >= 0 && counter_ints >= 0, "w4a16_gemm: negative scratch size");
   int rc = check_shape(size_m, size_n, size_k);
   if (rc != VAQ_OK) return rc;
   VAQ_CHECK_ARG(dtype == VAQ_F16 || dtype == VAQ_BF16, "w4a16_gemm: only supports bfloat16 and float16 (dtype tag %d)",
@@ -138,12 +158,12 @@ extern "C" int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, cons
     decode = false;
   }
   if (decode && decode_impl_for(size_m, size_n, lda, sub, w8) == 0)
-    return w4a16_decode2_launch(a, lda, b, scales, zeros, perm, bias, c, c_tmp, counters, counter_ints, (int)size_m,
+    return w4a16_decode2_launch(a, lda, b, scales, zeros, perm, bias, c, c_tmp, c_tmp_bytes, counters, counter_ints, (int)size_m,
                                 (int)size_n, (int)size_k, sub, channelwise, w8, dtype, s);
   if (decode) {
     VAQ_CHECK_SUPPORTED(sub == 1 && !w8, "w4a16_gemm: group_size = %d / 8-bit weights with an A of 2 GiB or more are not built",
                         group_size);
-    return w4a16_decode_launch(a, lda, b, scales, zeros, perm, bias, c, c_tmp, counters, counter_ints, (int)size_m,
+    return w4a16_decode_launch(a, lda, b, scales, zeros, perm, bias, c, c_tmp, c_tmp_bytes, counters, counter_ints, (int)size_m,
                                (int)size_n, (int)size_k, channelwise, dtype, s);
   }
 
@@ -157,10 +177,6 @@ extern "C" int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, cons
     a_eff = a_tmp;
     lda_eff = size_k;
   }
-  return w4a16_prefill_launch(a_eff, lda_eff, b, scales, zeros, bias, c, c_tmp, counters, counter_ints, (int)size_m,
+  return w4a16_prefill_launch(a_eff, lda_eff, b, scales, zeros, bias, c, c_tmp, c_tmp_bytes, counters, counter_ints, (int)size_m,
                               (int)size_n, (int)size_k, sub, channelwise, w8, dtype, s);
 }
-
-// Benchmark / tuning aid, not part of the drop-in surface: choose the decode implementation (-1 = automatic, 0 = LDS-staged
-// activations, 1 = register-resident activations).  Process-global, not thread-safe.
-extern "C" void vaq_debug_set_decode_impl(int impl) { vaq::g_decode_impl = impl; }

@@ -26,8 +26,6 @@ static int dispatch_tile(const PrefillParams& p, int tile, hipStream_t s) {
   return VAQ_ERR_UNSUPPORTED;
 }
 
-static int g_force_tile = -1, g_force_split = 0;
-
 // Splits of K for the 256 x 256 tile (one workgroup per compute unit): as many as bring the workgroup count to one per
 // compute unit, every split at least 28 groups (3584 rows) long.
 static int splits_256(int64_t tiles256, int K, int cus) {
@@ -37,7 +35,7 @@ static int splits_256(int64_t tiles256, int K, int cus) {
 }
 
 static int pick_tile(int M, int N, int K, bool direct_ok) {
-  if (g_force_tile >= 0) return g_force_tile;
+  if (tuning().prefill_tile > 0) return tuning().prefill_tile - 1;
   const int cus = num_cus_current_device();
   auto tiles = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   if (direct_ok) {
@@ -92,7 +90,7 @@ static PrefillPlan plan_prefill(int M, int N, int K, bool direct_ok) {
     if (sk > G / min_groups) sk = G / min_groups;
     if (sk < 1) sk = 1;
   }
-  if (g_force_split > 0) sk = g_force_split <= G ? g_force_split : G;
+  if (tuning().prefill_split > 0) sk = tuning().prefill_split <= G ? tuning().prefill_split : G;
   while (sk > 1 && (uint64_t)sk * (uint64_t)pl.tiles * pl.bm * pl.bn * 4 >= (1ull << 32)) --sk;   // 32-bit buffer offsets
   pl.sk = sk;
   return pl;
@@ -106,8 +104,9 @@ int w4a16_prefill_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* co
 }
 
 int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
-                         const void* bias, void* c, float* c_tmp, int32_t* counters, int64_t counter_ints, int M, int N,
-                         int K, int sub, bool channelwise, bool w8, int dtype, hipStream_t s) {
+                         const void* bias, void* c, float* c_tmp, int64_t c_tmp_bytes, int32_t* counters,
+                         int64_t counter_ints, int M, int N, int K, int sub, bool channelwise, bool w8, int dtype,
+                         hipStream_t s) {
   PrefillParams p;
   p.a = (const uint16_t*)a;
   p.lda = lda;
@@ -129,8 +128,17 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
     return VAQ_ERR_UNSUPPORTED;
   }
   PrefillPlan pl = plan_prefill(M, N, K, direct_ok);
-  // without scratch from the caller (or with too small a counter array) the unsplit kernel still gives the result
-  if (pl.sk > 1 && (c_tmp == nullptr || counters == nullptr || counter_ints < pl.tiles * pl.nw)) pl.sk = 1;
+  // A caller that passes no scratch at all gets the unsplit kernel (same result, no K split); scratch that is there but
+  // too small is the caller's mistake and is reported, not worked around.
+  if (pl.sk > 1 && c_tmp == nullptr && counters == nullptr) pl.sk = 1;
+  if (pl.sk > 1) {
+    const int64_t need_tmp = (int64_t)pl.sk * pl.tiles * pl.bm * pl.bn * 4, need_cnt = pl.tiles * pl.nw;
+    VAQ_CHECK_ARG(c_tmp != nullptr && counters != nullptr, "w4a16_gemm: split-K needs both c_tmp and counters");
+    VAQ_CHECK_ARG(counter_ints >= need_cnt, "w4a16_gemm: workspace.numel = %lld is below min_workspace_size = %lld",
+                  (long long)counter_ints, (long long)need_cnt);
+    VAQ_CHECK_ARG(c_tmp_bytes >= need_tmp, "w4a16_gemm: c_tmp holds %lld bytes, the K split needs %lld",
+                  (long long)c_tmp_bytes, (long long)need_tmp);
+  }
   p.SK = pl.sk;
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
@@ -145,11 +153,3 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
 }
 
 }  // namespace vaq
-
-// Benchmark / tuning aid, not part of the drop-in surface: force the prefill tile (-1 = automatic,
-// 0 = 256x256, 1 = 128x128, 2 = 64x128).  Process-global and not thread-safe.
-extern "C" void vaq_debug_set_prefill_tile(int tile) {
-  // tile < 0: automatic; otherwise tile id + 100 * (forced K split, 0 = automatic)
-  vaq::g_force_tile = tile < 0 ? -1 : tile % 100;
-  vaq::g_force_split = tile < 0 ? 0 : tile / 100;
-}

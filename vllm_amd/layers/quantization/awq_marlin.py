@@ -155,7 +155,7 @@ class AWQMarlinLinearMethod(LinearMethodBase):
     def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
         device = layer.qweight.device
         P = lambda t: torch.nn.Parameter(t, requires_grad=False)   # noqa: E731
-        layer.workspace = marlin_make_workspace_new(device)
+        layer.workspace = marlin_make_workspace_new(device, size_n=layer.output_size_per_partition)
         num_bits = self.quant_config.quant_type.size_bits
         layer.qweight = P(ops.awq_marlin_repack(layer.qweight.data, size_k=layer.input_size_per_partition,
                                                 size_n=layer.output_size_per_partition, num_bits=num_bits))

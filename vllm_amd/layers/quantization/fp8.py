@@ -112,15 +112,22 @@ class Fp8LinearMethod(LinearMethodBase):
             weight = layer.weight
             weight_scale = layer.weight_scale
             if weight_scale.numel() > 1:
-                # fused module with one scale per logical shard: requantise every shard to the largest scale
-                # (fp8_utils.py:1086-1111 process_fp8_weight_tensor_strategy / requantize_with_max_scale)
+                # fused module with one scale per logical shard (fp8_utils.py:1086-1111
+                # process_fp8_weight_tensor_strategy; w8a8_utils.py:108-136 requantize_with_max_scale)
                 max_w_scale = weight_scale.max()
-                start = 0
-                deq = torch.empty_like(weight, dtype=torch.float32)
-                for idx, width in enumerate(layer.logical_widths):
-                    deq[start:start + width] = weight[start:start + width].to(torch.float32) * weight_scale[idx]
-                    start += width
-                weight, _ = ops.scaled_fp8_quant(deq, max_w_scale.reshape(1))
+                # A module that is already fused on disk brings ONE scale: it sits in entry 0 and the last entry still
+                # holds its initial value.  Its weight is quantised with that single scale already and stays as it is.
+                unfused_in_checkpoint = bool(weight_scale[-1] > torch.finfo(torch.float8_e4m3fn).min)
+                if unfused_in_checkpoint:
+                    # one scale per shard: requantise every shard to the largest one
+                    start = 0
+                    deq = torch.zeros_like(weight, dtype=torch.float32)
+                    for idx, width in enumerate(layer.logical_widths):
+                        if width == 0:
+                            continue
+                        deq[start:start + width] = weight[start:start + width].to(torch.float32) * weight_scale[idx]
+                        start += width
+                    weight, _ = ops.scaled_fp8_quant(deq, max_w_scale.reshape(1))
                 weight_scale = max_w_scale
             if self.act_q_static:
                 input_scale = layer.input_scale.max()

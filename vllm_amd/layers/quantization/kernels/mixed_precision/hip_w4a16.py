@@ -45,7 +45,7 @@ class HipW4A16LinearKernel(MPLinearKernel):
 
         row_parallel = c.partition_weight_shape[0] != c.full_weight_shape[0]
         self.is_k_full = marlin_is_k_full(c.has_g_idx, row_parallel)
-        self.workspace = marlin_make_workspace_new(device)
+        self.workspace = marlin_make_workspace_new(device, size_n=size_n)
 
         if self.w_gidx_name is None:
             self.w_gidx_name = "g_idx"
@@ -74,6 +74,13 @@ class HipW4A16LinearKernel(MPLinearKernel):
             layer.g_idx_sort_indices = marlin_make_empty_g_idx(device)
         elif c.has_g_idx:
             g_idx, g_idx_sort_indices = marlin_sort_g_idx(getattr(layer, self.w_gidx_name))
+            # The kernels take the group of sorted row r to be r // group_size (the reference's kernel looks g_idx up
+            # per row instead): every group id must label exactly group_size rows.
+            group_len = c.group_size if c.group_size > 0 else size_k
+            expect = torch.arange(size_k, device=g_idx.device, dtype=g_idx.dtype) // group_len
+            if g_idx.numel() != size_k or not bool((g_idx == expect).all()):
+                raise NotImplementedError("act_order: g_idx must assign exactly group_size rows to each group 0 .. K / "
+                                          "group_size - 1; uneven groups are not built for gfx950")
             self._transform_param(layer, self.w_gidx_name, lambda _: g_idx)
             layer.g_idx_sort_indices = g_idx_sort_indices
         else:

@@ -28,7 +28,7 @@ HIP_W8A16_SUPPORTED_GROUP_SIZES = [-1, 32, 64, 128]      # uint8b128 weights
 USE_FP32_REDUCE_DEFAULT = True
 
 # int32 arrival counters handed to the GEMM: one per 16-column tile and m-block of the largest layer served.
-_WORKSPACE_INTS = 16384
+_WORKSPACE_INTS = 65536
 
 _INTERLEAVE4 = (0, 2, 4, 6, 1, 3, 5, 7)
 
@@ -95,10 +95,21 @@ def check_marlin_supports_shape(output_size_per_partition: int, input_size_per_p
     return True, None
 
 
-def marlin_make_workspace_new(device: torch.device, max_blocks_per_sm: int = 1) -> torch.Tensor:
+def marlin_workspace_ints(size_n: int | None = None) -> int:
+    """Arrival counters the GEMM can ask for on a layer with `size_n` output columns, whatever the batch size: the decode
+    kernels use one per 16-column tile and 16-row block (up to four blocks: size_n / 4), the tile kernel at most 4096.
+    Without a width: enough for 262144 columns."""
+    if size_n is None:
+        return _WORKSPACE_INTS
+    return max(size_n // 4, 4096)
+
+
+def marlin_make_workspace_new(device: torch.device, max_blocks_per_sm: int = 1, size_n: int | None = None) -> torch.Tensor:
     """Zeroed int32 counters for the GEMM's split-K hand-off (marlin_utils.py:237-245).  The GEMM requires them zero
-    on entry and leaves them zero."""
-    return torch.zeros(_WORKSPACE_INTS * max_blocks_per_sm, dtype=torch.int, device=device, requires_grad=False)
+    on entry and leaves them zero, and reports a workspace that is too small for the kernel it runs.  `size_n` (not in
+    the reference, whose count depends on the device only) sizes the array for one layer."""
+    return torch.zeros(marlin_workspace_ints(size_n) * max_blocks_per_sm, dtype=torch.int, device=device,
+                       requires_grad=False)
 
 
 def marlin_is_k_full(act_order: bool, is_row_parallel: bool) -> bool:
