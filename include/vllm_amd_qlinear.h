@@ -111,6 +111,24 @@ int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, const void* sca
                    int group_size, int dtype, int wtype, int force_path, void* stream);
 
 /*
+ * vaq_w4a16_gemm on scratch the library owns, for callers that cannot allocate device memory (code under HIP graph
+ * capture, serving loops and harnesses that forbid hipMalloc).  No counterpart in the reference, whose GEMM allocates its
+ * scratch through the torch allocator (gptq_marlin.cu:752-763, :799).  Same arguments, results and kernels as
+ * vaq_w4a16_gemm with force_path 0; the partial tiles, permuted activations and arrival counters live in one
+ * file-scope device array of VAQ_STATIC_SCRATCH_COUNTER_INTS ints + VAQ_STATIC_SCRATCH_DATA_BYTES bytes per GPU, which
+ * a GPU holds from the library's first use on it until the process ends.  The call allocates and frees nothing.
+ * A problem whose scratch (vaq_w4a16_gemm_workspace) exceeds that returns VAQ_ERR_INVALID_ARG and launches nothing.
+ * Every call on a GPU uses that GPU's one array: calls that may overlap in time on one GPU (different streams or
+ * threads) race on it and must be serialised by the caller.  The first call on a GPU looks the array's address up
+ * (hipGetSymbolAddress); make it outside any graph capture.
+ */
+#define VAQ_STATIC_SCRATCH_COUNTER_INTS 65536
+#define VAQ_STATIC_SCRATCH_DATA_BYTES (16u << 20)
+int vaq_w4a16_gemm_static(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
+                          const int32_t* perm, const void* bias, void* c, int64_t size_m, int64_t size_n, int64_t size_k,
+                          int group_size, int dtype, int wtype, void* stream);
+
+/*
  * out[m, k] = a[m, perm[k]] for 16-bit elements.  Replaces `permute_cols(Tensor A, Tensor perm) -> Tensor`
  * (csrc/torch_bindings.cpp:304; csrc/permute_cols.cu:13-87).
  */

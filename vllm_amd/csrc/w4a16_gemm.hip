@@ -1,6 +1,8 @@
 // C-ABI entry of the W4A16 GEMM: argument validation and the decode / prefill dispatch.
 #include "vaq_common.h"
 
+#include <mutex>
+
 namespace vaq {
 // `sub` = quantisation groups per 128-row weight tile (1, 2, 4); `channelwise` = one scale row for all of K (sub == 1)
 int w4a16_decode_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* counter_ints);
@@ -179,4 +181,68 @@ extern "C" int vaq_w4a16_gemm_tuned(const void* a, int64_t lda, const int32_t* b
   }
   return w4a16_prefill_launch(a_eff, lda_eff, b, scales, zeros, bias, c, c_tmp, c_tmp_bytes, counters, counter_ints, (int)size_m,
                               (int)size_n, (int)size_k, sub, channelwise, w8, dtype, s);
+}
+
+// ----------------------------------------------------------------------------- the GEMM on library-owned scratch
+namespace vaq {
+
+// Scratch of vaq_w4a16_gemm_static: arrival counters (zero when the module is loaded, left zero by every kernel), then
+// the split-K partial tiles, then the permuted activations.  One copy per GPU, held from the first use of the library
+// on that GPU until the process ends.
+constexpr size_t STATIC_COUNTER_INTS = VAQ_STATIC_SCRATCH_COUNTER_INTS;
+constexpr size_t STATIC_DATA_BYTES = VAQ_STATIC_SCRATCH_DATA_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_COUNTER_INTS * 4 + STATIC_DATA_BYTES];
+
+// `scratch` above is the host-side handle of the array, not an address a kernel can use: the device address is looked up
+// once per device, with that device current, and kept here.
+static unsigned char* g_scratch_ptr[VAQ_MAX_DEVICES];
+static hipError_t g_scratch_err[VAQ_MAX_DEVICES];
+static std::once_flag g_scratch_once[VAQ_MAX_DEVICES];
+
+static int static_scratch_of_current_device(unsigned char** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= VAQ_MAX_DEVICES) {
+    (void)hipGetLastError();
+    set_error("w4a16_gemm_static: cannot identify the current device");
+    return VAQ_ERR_LAUNCH;
+  }
+  std::call_once(g_scratch_once[dev], [dev] {
+    void* p = nullptr;
+    g_scratch_err[dev] = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    g_scratch_ptr[dev] = g_scratch_err[dev] == hipSuccess ? static_cast<unsigned char*>(p) : nullptr;
+    if (g_scratch_err[dev] != hipSuccess) (void)hipGetLastError();
+  });
+  if (g_scratch_ptr[dev] == nullptr) {
+    set_error("w4a16_gemm_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(g_scratch_err[dev]));
+    return VAQ_ERR_LAUNCH;
+  }
+  *out = g_scratch_ptr[dev];
+  return VAQ_OK;
+}
+
+}  // namespace vaq
+
+extern "C" int vaq_w4a16_gemm_static(const void* a, int64_t lda, const int32_t* b, const void* scales,
+                                     const int32_t* zeros, const int32_t* perm, const void* bias, void* c, int64_t size_m,
+                                     int64_t size_n, int64_t size_k, int group_size, int dtype, int wtype, void* stream) {
+  using namespace vaq;
+  size_t c_tmp_bytes = 0, a_tmp_bytes = 0, counter_ints = 0;
+  int rc = vaq_w4a16_gemm_workspace(size_m, size_n, size_k, perm != nullptr, 0, &c_tmp_bytes, &a_tmp_bytes, &counter_ints);
+  if (rc != VAQ_OK) return rc;
+  const size_t c_tmp_span = (c_tmp_bytes + 255) & ~(size_t)255;
+  VAQ_CHECK_ARG(counter_ints <= STATIC_COUNTER_INTS && c_tmp_span + a_tmp_bytes <= STATIC_DATA_BYTES,
+                "w4a16_gemm_static: M=%lld N=%lld K=%lld needs %zu counters and %zu + %zu bytes of scratch, the "
+                "library-owned scratch holds %zu counters and %zu bytes; use vaq_w4a16_gemm with caller scratch",
+                (long long)size_m, (long long)size_n, (long long)size_k, counter_ints, c_tmp_bytes, a_tmp_bytes,
+                STATIC_COUNTER_INTS, STATIC_DATA_BYTES);
+  unsigned char* base = nullptr;
+  if (size_m > 0) {
+    rc = static_scratch_of_current_device(&base);
+    if (rc != VAQ_OK) return rc;
+  }
+  int32_t* counters = reinterpret_cast<int32_t*>(base);
+  unsigned char* data = base ? base + STATIC_COUNTER_INTS * 4 : nullptr;
+  return vaq_w4a16_gemm(a, lda, b, scales, zeros, perm, bias, c, c_tmp_bytes ? reinterpret_cast<float*>(data) : nullptr,
+                        (int64_t)c_tmp_bytes, a_tmp_bytes ? data + c_tmp_span : nullptr, counters,
+                        (int64_t)STATIC_COUNTER_INTS, size_m, size_n, size_k, group_size, dtype, wtype, 0, stream);
 }
