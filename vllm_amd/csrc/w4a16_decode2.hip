@@ -8,6 +8,7 @@ namespace vaq {
 
 struct Decode2Config {
   int gs, wks, wn, sk, mr;
+  int rc;      // ring variant of long streams (see the kernel): 0 two slots refilled early, 1 / 2 four / three slots refilled late
 };
 
 static int round_gs(int x, int sub, bool w8) {
@@ -79,19 +80,40 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8) 
   }
   c.wn = tn.decode2_wn > 0 ? tn.decode2_wn : best_wn;
   if (c.wn * wks > D2_WAVES) c.wn = D2_WAVES / wks;
+  // ring variant of long streams (instances exist for 4-bit codes in groups of 128 rows / channelwise, up to two
+  // m-blocks): by the wavefronts that share a compute unit
+  c.rc = 0;
+  if (sub == 1 && !w8 && MB <= 2 && gs >= 7) {
+    long slots = D2_WAVES / (wks * c.wn);
+    const long lds_slots = (long)((size_t)(160 * 1024) / lds_wg);
+    if (slots > lds_slots) slots = lds_slots;
+    if (slots < 1) slots = 1;
+    const long per_cu = ((long)((NT + c.wn - 1) / c.wn) * c.sk + cus - 1) / cus;
+    const long waves_cu = (per_cu < slots ? per_cu : slots) * wks * c.wn;
+    if (waves_cu <= 8) c.rc = 1;
+    else if (c.mr == 16) c.rc = 2;
+  }
+  if (tn.exp[1] > 0) c.rc = tn.exp[1] - 1;      // (development switch: forced ring variant + 1)
   return c;
 }
 
+template <bool BF16, int MB, bool HAS_ZP, int MR, int GS>
+static int dispatch_rc2(const Decode2Params& p, int rc, hipStream_t s) {
+  if (rc == 1) return launch_decode2<BF16, GS, MB, HAS_ZP, MR, 1, false, 1>(p, s);
+  if (rc == 2) return launch_decode2<BF16, GS, MB, HAS_ZP, MR, 1, false, 2>(p, s);
+  return launch_decode2<BF16, GS, MB, HAS_ZP, MR, 1>(p, s);
+}
+
 template <bool BF16, int MB, bool HAS_ZP, int MR>
-static int dispatch_gs2(const Decode2Params& p, int gs, hipStream_t s) {
+static int dispatch_gs2(const Decode2Params& p, int gs, int rc, hipStream_t s) {
   switch (gs) {
     case 1: return launch_decode2<BF16, 1, MB, HAS_ZP, MR, 1>(p, s);
     case 2: return launch_decode2<BF16, 2, MB, HAS_ZP, MR, 1>(p, s);
     case 4: return launch_decode2<BF16, 4, MB, HAS_ZP, MR, 1>(p, s);
-    case 7: return launch_decode2<BF16, 7, MB, HAS_ZP, MR, 1>(p, s);
-    case 8: return launch_decode2<BF16, 8, MB, HAS_ZP, MR, 1>(p, s);
-    case 14: return launch_decode2<BF16, 14, MB, HAS_ZP, MR, 1>(p, s);
-    case 16: return launch_decode2<BF16, 16, MB, HAS_ZP, MR, 1>(p, s);
+    case 7: return dispatch_rc2<BF16, MB, HAS_ZP, MR, 7>(p, rc, s);
+    case 8: return dispatch_rc2<BF16, MB, HAS_ZP, MR, 8>(p, rc, s);
+    case 14: return dispatch_rc2<BF16, MB, HAS_ZP, MR, 14>(p, rc, s);
+    case 16: return dispatch_rc2<BF16, MB, HAS_ZP, MR, 16>(p, rc, s);
     default: break;
   }
   set_error("w4a16_gemm(decode): unsupported groups per wavefront %d", gs);
@@ -99,17 +121,17 @@ static int dispatch_gs2(const Decode2Params& p, int gs, hipStream_t s) {
 }
 
 template <int MB, int MR>
-static int dispatch_types2(const Decode2Params& p, int gs, bool bf16, bool zp, hipStream_t s) {
-  if (bf16) return zp ? dispatch_gs2<true, MB, true, MR>(p, gs, s) : dispatch_gs2<true, MB, false, MR>(p, gs, s);
-  return zp ? dispatch_gs2<false, MB, true, MR>(p, gs, s) : dispatch_gs2<false, MB, false, MR>(p, gs, s);
+static int dispatch_types2(const Decode2Params& p, int gs, int rc, bool bf16, bool zp, hipStream_t s) {
+  if (bf16) return zp ? dispatch_gs2<true, MB, true, MR>(p, gs, rc, s) : dispatch_gs2<true, MB, false, MR>(p, gs, rc, s);
+  return zp ? dispatch_gs2<false, MB, true, MR>(p, gs, rc, s) : dispatch_gs2<false, MB, false, MR>(p, gs, rc, s);
 }
 
 template <int MB>
 static int dispatch_mr2(const Decode2Params& p, const Decode2Config& c, bool bf16, bool zp, hipStream_t s) {
   switch (c.mr) {
-    case 1: return dispatch_types2<MB, 1>(p, c.gs, bf16, zp, s);
-    case 4: return dispatch_types2<MB, 4>(p, c.gs, bf16, zp, s);
-    default: return dispatch_types2<MB, 16>(p, c.gs, bf16, zp, s);
+    case 1: return dispatch_types2<MB, 1>(p, c.gs, c.rc, bf16, zp, s);
+    case 4: return dispatch_types2<MB, 4>(p, c.gs, c.rc, bf16, zp, s);
+    default: return dispatch_types2<MB, 16>(p, c.gs, c.rc, bf16, zp, s);
   }
 }
 
@@ -149,6 +171,9 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
   p.SK = cfg.sk;
   p.WKS = cfg.wks;
   p.WN = cfg.wn;
+  // private activation fill (see the kernel): measured ahead only on short streams with few staged rows (4096 x 4096 at
+  // M = 1 / 4: 4.53 / 4.83 -> 4.38 / 4.52 us; 14336 x 4096 at M = 4: 9.1 -> 9.3 us)
+  p.PRIV = (cfg.wn == 1 && perm == nullptr && cfg.mr <= 4 && cfg.gs <= 8 && tuning().exp[0] != 1) ? 1 : 0;
   const int MB = (M + 15) / 16;
   if (cfg.sk > 1) {
     VAQ_CHECK_ARG(c_tmp != nullptr && counters != nullptr, "w4a16_gemm: split-K needs c_tmp and counters");
@@ -168,7 +193,7 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
   else if (sub == 4) rc = decode2_launch_sub4(p, cfg.gs, MB, cfg.mr, bf16, zp, s);
   else if (MB > 2) rc = decode2_launch_mb34(p, cfg.gs, MB, bf16, zp, s);
   else if (MB == 1) rc = dispatch_mr2<1>(p, cfg, bf16, zp, s);
-  else rc = dispatch_types2<2, 16>(p, cfg.gs, bf16, zp, s);
+  else rc = dispatch_types2<2, 16>(p, cfg.gs, cfg.rc, bf16, zp, s);
   if (rc != VAQ_OK) return rc;
   VAQ_CHECK_LAUNCH("w4a16_gemm(decode)");
   return VAQ_OK;

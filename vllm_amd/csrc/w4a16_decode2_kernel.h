@@ -40,7 +40,7 @@ struct Decode2Params {
   uint16_t* c;
   float* c_tmp;
   int32_t* counters;
-  int M, N, K, G, NT, SK, WKS, WN;   // G: weight tiles along K per 16-column strip (K/128, twice that for 8-bit codes)
+  int M, N, K, G, NT, SK, WKS, WN, PRIV;   // PRIV: private activation fill (see the kernel; needs WN == 1, no perm); G: weight tiles along K per 16-column strip (K/128, twice that for 8-bit codes)
   int GR;                  // rows of the scale / zero-point tensors (G * SUBG, or 1 for channelwise scales)
   int s_stride, z_stride;  // elements between consecutive rows of scales (N) / zeros (N/8); 0 for channelwise
   uint32_t k_mask, k_ex;   // 0x000f000f and the exponent pattern, passed as run-time values (see and_or)
@@ -68,20 +68,35 @@ static inline uint32_t d2_sat32(uint64_t bytes) { return bytes > 0xffffffffull ?
 
 constexpr int D2_WAVES = 16;
 
-template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, bool W8 = false>
+template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, bool W8 = false, int RC = 0>
 __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Decode2Params p) {
   using T = F16Traits<BF16>;
   static_assert(SUBG == 1 || SUBG == 2 || SUBG == 4, "quantisation groups per 128-row tile");
   constexpr int TPG = W8 ? 2 : 1;                      // weight tiles per 128 rows of K
   static_assert(!W8 || (!HAS_ZP && GS % 2 == 0), "8-bit codes: two planes per 128 rows, symmetric");
   static_assert(MR == 16 || MB == 1, "compact row staging is for a single m-block");
-  // Ring slots.  Two tiles in flight per wavefront measured best: a wavefront does not get past its load instructions
-  // until the memory pipeline has accepted them, and with deeper rings (every wavefront of the device asking for
-  // 7-8 KiB at once) the first MFMA of each wavefront starts when most of the stream has already been served, so the
-  // arithmetic no longer overlaps it.  Exception: 16 staged rows and a long stream (K = 14336 at M = 5 .. 16) -- the
-  // activation fill then takes 2 us during which nothing else is requested, and four tiles in flight fill that gap
-  // (the 12-GEMM decode step 1.4 % faster; four slots for 1 or 4 staged rows: 0.8 % slower).
-  constexpr int R = (MR == 16 && MB == 1 && GS >= 7) ? 4 : (GS < 2 ? GS : 2);
+  // Ring of weight tiles in flight per wavefront.
+  //  * Short streams with few staged rows (up to 8 tiles per wavefront, M <= 4) request everything up front: the whole
+  //    layer is then in flight within the first microsecond, which is what a layer of a few megabytes needs to come near
+  //    the memory system's rate (4096 x 6144 at M = 1: 5.9 -> 5.4 us; with 16 staged rows the same depth competes with
+  //    the activation fill and loses 0.2-1 us).
+  //  * Long streams, RC = 0: two slots, each refilled as soon as its tile's registers have been copied.  The wavefront
+  //    then waits for both tiles at the top of every trip, so it overlaps little by itself: right when 14-16 wavefronts
+  //    share a compute unit and overlap each other (about 28 KiB in flight per unit; deeper rings measured 2-6 % slower
+  //    on 4096 x 28672).  (Four slots with 16 staged rows: the activation fill takes 2 us during which nothing else is
+  //    requested, and four tiles in flight fill that gap.)
+  //  * Long streams, RC = 1 / 2: four / three slots, each refilled only after its tile's arithmetic has been issued: no
+  //    register copies, and the wait in front of a tile leaves the other R - 1 tiles in flight.  For launches with at
+  //    most 8 wavefronts per compute unit, which are latency-bound with two slots (14336 x 4096 at M = 1: 9.2 -> 8.0 us
+  //    with four slots; six slots 8.7 us; 16 wavefronts of two slots 10.3 us), and, with three slots, for 16 staged rows
+  //    (4096 x 28672 at M = 16: 15.2 -> 14.8 us).
+  constexpr int LPT = 1 + SUBG * (HAS_ZP ? 2 : 1);              // vector-memory instructions per tile request
+  constexpr int R_SHORT = (GS < 63 / LPT ? GS : 63 / LPT) & (W8 ? ~1 : ~0);      // (8-bit codes: whole plane pairs)
+  constexpr bool SHORT = MR <= 4 && GS <= 8 && GS >= 2;
+  constexpr bool LATE = RC != 0 && !SHORT;
+  constexpr int R_LATE = RC == 1 ? 4 : 3;
+  static_assert(!(W8 && RC != 0), "8-bit codes take the plane from the slot parity: even rings only");
+  constexpr int R = SHORT ? R_SHORT : (LATE ? (GS < R_LATE ? GS : R_LATE) : ((MR == 16 && MB == 1 && GS >= 7) ? 4 : (GS < 2 ? GS : 2)));
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
   const int lane = threadIdx.x;
@@ -136,7 +151,34 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
     // chunk c = m * KO + ko' (LDS slot c); thread tid handles c = tid, tid + NTHR, ...  The (m, ko') pair is advanced
     // incrementally: one scalar division per kernel instead of one vector division per chunk.
     int m = (int)__umulhi((uint32_t)tid, p.ko_magic), ko = tid - m * KO;
-    if (p.perm == nullptr) {
+    if (p.PRIV != 0) {
+      // Private fill (one n-tile per workgroup, so no two wavefronts read the same k-octets): every wavefront fetches the
+      // k-octets of its own K slice, row by row, and waits for nobody -- the same bytes travel as in the shared fill, but
+      // a wavefront starts on its first tile as soon as ITS activations and ITS first weight tile are there instead of
+      // when the slowest wavefront's activations are.  An instruction whose 64 slots reach past the slice covers part of
+      // the next wavefront's slice (or of the next row) and writes there exactly what its owner writes.  The first
+      // weight tile is requested before the activations, the others after them: the wait below then leaves R - 1 tiles
+      // in flight.
+      const __amdgpu_buffer_rsrc_t ra = d2_rsrc32(p.a, p.a_bytes);
+      typedef __attribute__((address_space(3))) void* lds_ptr_t;
+      issue_load(0, 0);
+      const int own = (GS / TPG) * 16;                         // k-octets of this wavefront's slice
+      for (int mrow = 0; mrow < MR * MB; ++mrow) {
+        for (int q0 = 0; q0 < own; q0 += 64) {
+          const int c0 = mrow * KO + wks * own + q0;           // first slot of this instruction (wave-uniform)
+          const int sl = c0 + lane;
+          const int m2 = (int)__umulhi((uint32_t)sl, p.ko_magic), ko2 = sl - m2 * KO;
+          const int k = k_slab0 + (ko2 ^ (m2 & (MR - 1))) * 8;
+          const bool ok = m2 < MR * MB && m2 < p.M && k < p.K;
+          const uint32_t off = ok ? (uint32_t)(m2 * lda32 + k) * 2u : 0x80000000u;
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(lds + (size_t)c0 * 16), 16, (int)off, 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int s = 1; s < R; ++s) issue_load(s, s);
+      constexpr int W_LATER = (R - 1) * LPT;      // vector-memory instructions requested after the activations
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(W_LATER) : "memory");
+    } else if (p.perm == nullptr) {
       // Direct-to-LDS loads (no registers, no LDS write instructions): wavefront instruction q fills slots 64q .. 64q+63,
       // lane l fetching the chunk that belongs in slot 64q + l.  Rows past M, k past K and slots past the image get an
       // out-of-range offset of the buffer descriptor (which ends with the last valid element) and arrive as zeros; the
@@ -158,7 +200,8 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
       }
 #pragma unroll
       for (int s = 0; s < R; ++s) issue_load(s, s);
-      constexpr int W_LOADS = R * (1 + SUBG * (HAS_ZP ? 2 : 1));      // vector-memory instructions of the weight requests
+      constexpr int W_LOADS = R * LPT;      // vector-memory instructions of the weight requests
+      static_assert(W_LOADS < 64, "the wait counter holds 6 bits");
       asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(W_LOADS) : "memory");
     } else {
       // act_order: the columns of A are gathered through `perm`; two dependent levels of loads, weights requested first
@@ -225,7 +268,9 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
       sct[sj] = sc[slot][sj];
       zqt[sj] = zq[slot][sj];
     }
-    if (reissue) issue_load(slot, gi + R);
+    if constexpr (!LATE) {
+      if (reissue) issue_load(slot, gi + R);
+    }
 
 #pragma unroll
     for (int sj = 0; sj < SUBG; ++sj) {
@@ -236,9 +281,12 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
       const uint32_t z2 = zbits | (zbits << 16);
       const v4u zop = {z2, z2, z2, z2};
 
-      v4f P[MB];
+      // Two accumulation chains per m-block -- the products with the codes in P, the bias / zero-point correction in Q --
+      // issued alternately: an MFMA that accumulates on the previous one's result waits for it, and one chain of eight
+      // left the matrix core idle most of the time when few wavefronts share a SIMD.
+      v4f P[MB], Q[MB];
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) P[mb] = v4f{0.f, 0.f, 0.f, 0.f};
+      for (int mb = 0; mb < MB; ++mb) P[mb] = Q[mb] = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int jj = sj * (4 / SUBG); jj < (sj + 1) * (4 / SUBG); ++jj) {
         v4u aop;
@@ -250,7 +298,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
         for (int mb = 0; mb < MB; ++mb) {
           const v4u bop = *reinterpret_cast<const v4u*>(lds + abase[jj] + (uint32_t)(mb * KO * MR * 16) + (uint32_t)((gi / TPG) * 256));
           P[mb] = T::mfma16(aop, bop, P[mb]);
-          P[mb] = T::mfma16(zop, bop, P[mb]);
+          Q[mb] = T::mfma16(zop, bop, Q[mb]);
         }
       }
       float s[4];
@@ -274,7 +322,10 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[mb][r] = fmaf(s[r], P[mb][r], acc[mb][r]);
+        for (int r = 0; r < 4; ++r) acc[mb][r] = fmaf(s[r], P[mb][r] + Q[mb][r], acc[mb][r]);
+    }
+    if constexpr (LATE) {
+      if (reissue) issue_load(slot, gi + R);
     }
   };
   if constexpr (GS <= 4) {
@@ -305,10 +356,23 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
     for (int mb = 0; mb < MB; ++mb) red[(w * MB + mb) * 64 + lane] = acc[mb];
     __syncthreads();
     if (wks != 0) return;
+    // the partial tiles of the other slices, added in slice order; with many slices, seven reads in flight at a time
+    // (one by one, each read waits out the LDS latency: 0.3 us for eight slices)
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       v4f t = acc[mb];
-      for (int s2 = 1; s2 < WKS; ++s2) t += red[((s2 * WN + wn) * MB + mb) * 64 + lane];
+      if (WKS <= 4) {
+        for (int s2 = 1; s2 < WKS; ++s2) t += red[((s2 * WN + wn) * MB + mb) * 64 + lane];
+      } else {
+        for (int s0 = 1; s0 < WKS; s0 += 7) {
+          v4f part[7];
+#pragma unroll
+          for (int i = 0; i < 7; ++i) part[i] = red[((min(s0 + i, WKS - 1) * WN + wn) * MB + mb) * 64 + lane];
+#pragma unroll
+          for (int i = 0; i < 7; ++i)
+            if (s0 + i < WKS) t += part[i];
+        }
+      }
       acc[mb] = t;
     }
   }
@@ -384,13 +448,14 @@ static inline size_t decode2_lds_bytes(int wks, int groups_per_wave, int mr, int
   return act + red;
 }
 
-template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, bool W8 = false>
+template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, bool W8 = false, int RC = 0>
 static int launch_decode2(const Decode2Params& p_in, hipStream_t s) {
   Decode2Params p = p_in;
   const int WN = p.WN;
   {
     const int ko = p.WKS * GS / (W8 ? 2 : 1) * 16, nthr = p.WKS * WN * 64;
     p.wn_magic = (uint32_t)((65536 + WN - 1) / WN);
+    if (WN != 1 || p.perm != nullptr) p.PRIV = 0;
     p.ko_magic = (uint32_t)(((1ull << 32) + (uint64_t)ko - 1) / (uint64_t)ko);
     p.step_m = nthr / ko;
     p.step_ko = nthr - p.step_m * ko;
@@ -404,7 +469,7 @@ static int launch_decode2(const Decode2Params& p_in, hipStream_t s) {
     }
   }
   const size_t lds = decode2_lds_bytes(p.WKS, GS / (W8 ? 2 : 1), MR, MB);
-  auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP, MR, SUBG, W8>;
+  auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP, MR, SUBG, W8, RC>;
   static size_t reserved[VAQ_MAX_DEVICES];
   if (const int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "w4a16_gemm(decode)"); rc != VAQ_OK) return rc;
   const int gx = (p.NT + WN - 1) / WN;
