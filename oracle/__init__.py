@@ -21,6 +21,14 @@ Pinning status (what fixes each function besides its own formula):
 * ``w4a16.dequantize / gemm_ref``   special cases that reduce to closed forms
   (s=1,q-z=1 -> row sums; one-hot A picks a dequantised row; zp==8 with uint4
   equals uint4b8; act_order == plain GEMM on A[:, perm]).
+* ``w4a16.awq_pack``   one word packed by hand + inverse round trip.
+* ``quantize.quantize_weights / gptq_quantize_weights / sort_weights / marlin_quantize /
+  awq_marlin_quantize / scaled_quantize / scaled_dequantize / group_broadcast`` (the reference's weight quantisers,
+  which its GEMM tests feed with random normal weights)   error bound of uniform quantisation (half a step; one step
+  with a rounded zero point), textbook scales, extreme codes reached in every group, ranges, block-constant weights
+  returned exactly, act_order bookkeeping (a permutation that ``sort_weights`` undoes group-wise, GEMM identity),
+  hand-computed tiny groups, fp8 round trip; the case built from float weights dequantises through
+  ``w4a16.dequantize`` to the quantiser's own ``w_ref`` bit for bit.
 * ``fp8.ref_dynamic_per_token_quant``   torch CPU float8_e4m3fn cast versus an
   independent bit-level e4m3fn encoder brute-forced over all 65 536 bf16
   inputs; edge cases (zero row -> 1/(448*512), amax -> 0x7E, ties-to-even,

@@ -470,3 +470,33 @@ def test_config5_decode_step_gemm_llama_shapes(device, decode_kernel, k, n):
     out = layer(a)
     check_gemm_close(out, o.gemm_ref(a.cpu(), o.case_w_ref(case)), f"config 5 GEMM k={k} n={n} m=32")
     assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("mnk", [(1, 1, 1), (1, 4, 8), (26, 37, 13), (257, 13, 11)])
+@pytest.mark.parametrize("n_chunk", [64, 256])
+@pytest.mark.parametrize("quant_type,act_order", [("uint4b8", False), ("uint4b8", True), ("uint4", False), ("uint8b128", False)])
+def test_gemm_reference_grid_weights_quantized_from_float(device, quant_type, act_order, n_chunk, mnk, dtype):
+    """The reference's own GEMM test (tests/kernels/quantization/test_marlin_gemm.py:228-361): random normal activations
+    and weights, the weights pushed through the reference's quantisers (oracle/quantize.py) -- realistic scale spread,
+    extreme codes at every group's maximum, zero points at both ends of their range -- on its size grid (k_chunk 128,
+    n_chunk 64 / 256, its (M, N, K) factors) for every group size, against `a @ w_ref` of the quantiser's own
+    dequantised weight."""
+    from oracle import quantize as oq
+    m, nf, kf = mnk
+    k, n = 128 * kf, n_chunk * nf
+    g = torch.Generator().manual_seed(1000 * kf + nf + m)
+    for group_size in (-1, 32, 64, 128):
+        if act_order and (group_size == -1 or group_size == k):
+            continue                                  # needs more than one group (test_marlin_gemm.py:247-252)
+        if k % max(group_size, 1) != 0:
+            continue
+        w = torch.randn(k, n, generator=g).to(dtype)
+        a = torch.randn(m, k, generator=g).to(dtype)
+        case = oq.quantized_case(w, quant_type, group_size, act_order=act_order, seed=kf)
+        layer = W4A16Layer(case, device, dtype)
+        out = layer(a.to(device))
+        check_gemm_close(out, o.gemm_ref(a, case["w_ref"]), f"{quant_type} g={group_size} act_order={act_order} m={m} n={n} k={k}")
+        # the reference's own pass criterion, against its own 16-bit matmul
+        ref16 = o.gemm_ref_like_reference(a.float(), case["w_ref"].float())
+        assert o.rel_err_mean(out.cpu().float(), ref16) < 0.04

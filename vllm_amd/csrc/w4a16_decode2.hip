@@ -91,7 +91,7 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8) 
     const long per_cu = ((long)((NT + c.wn - 1) / c.wn) * c.sk + cus - 1) / cus;
     const long waves_cu = (per_cu < slots ? per_cu : slots) * wks * c.wn;
     if (waves_cu <= 8) c.rc = 1;
-    else if (c.mr == 16) c.rc = 2;
+    else if (c.mr == 16 && gs >= 14) c.rc = 2;      // (7 tiles per wavefront, 14336 x 4096 at M = 16: three slots 11.5 us, two 11.2 us)
   }
   if (tn.exp[1] > 0) c.rc = tn.exp[1] - 1;      // (development switch: forced ring variant + 1)
   return c;
@@ -101,6 +101,7 @@ template <bool BF16, int MB, bool HAS_ZP, int MR, int GS>
 static int dispatch_rc2(const Decode2Params& p, int rc, hipStream_t s) {
   if (rc == 1) return launch_decode2<BF16, GS, MB, HAS_ZP, MR, 1, false, 1>(p, s);
   if (rc == 2) return launch_decode2<BF16, GS, MB, HAS_ZP, MR, 1, false, 2>(p, s);
+  if (rc == 3) return launch_decode2<BF16, GS, MB, HAS_ZP, MR, 1, false, 3>(p, s);
   return launch_decode2<BF16, GS, MB, HAS_ZP, MR, 1>(p, s);
 }
 

@@ -94,7 +94,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   constexpr int R_SHORT = (GS < 63 / LPT ? GS : 63 / LPT) & (W8 ? ~1 : ~0);      // (8-bit codes: whole plane pairs)
   constexpr bool SHORT = MR <= 4 && GS <= 8 && GS >= 2;
   constexpr bool LATE = RC != 0 && !SHORT;
-  constexpr int R_LATE = RC == 1 ? 4 : 3;
+  constexpr int R_LATE = RC == 1 ? 4 : (RC == 2 ? 3 : 2);
   static_assert(!(W8 && RC != 0), "8-bit codes take the plane from the slot parity: even rings only");
   constexpr int R = SHORT ? R_SHORT : (LATE ? (GS < R_LATE ? GS : R_LATE) : ((MR == 16 && MB == 1 && GS >= 7) ? 4 : (GS < 2 ? GS : 2)));
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
