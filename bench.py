@@ -320,17 +320,36 @@ def vendor_ceiling_section(dev):
 
 
 def decode_step_section(dev):
-    """BASELINE.json config 5: one decode step of a random-init Llama-3-8B-architecture model, batch 32, context 1024.  All
-    32 x 4 linear layers run on the W4A16 GEMM (M = 32, distinct weights per layer: 3.6 GB); norms, rotary-free
-    attention over a bf16 KV cache, SiLU-mul, embedding and the bf16 lm_head are plain torch ops standing in for the
-    rest of the model.  Reports the step time, the share of it spent in the quantized GEMMs and tokens/s."""
+    """BASELINE.json config 5: one decode step of a random-init Llama-3-8B-architecture model, batch 32, context 1024.  The
+    32 x 4 linear layers are `QKVParallelLinear` / `RowParallelLinear` / `MergedColumnParallelLinear` modules carrying
+    `GPTQMarlinLinearMethod` (random int4 codes and scales written into the checkpoint-format parameters, then
+    `process_weights_after_loading`), called through `layer(x)` -> `quant_method.apply`: M = 32, distinct weights per
+    layer (3.6 GB).  Norms, rotary-free attention over a bf16 KV cache, SiLU-mul, embedding and the bf16 lm_head are plain
+    torch ops standing in for the rest of the model.  Reports the step time, tokens/s, and the time share of the
+    quantized GEMMs per projection type: each type's 32 layers replayed as their own HIP graph (cold weights), the way
+    the reference's layerwise profiler (vllm/profiler/layerwise_profile.py:365) attributes kernel time to modules."""
     import torch.nn.functional as F
+    from vllm_amd.layers.linear import MergedColumnParallelLinear, QKVParallelLinear, RowParallelLinear
+    from vllm_amd.layers.quantization import get_quantization_config
     gen = torch.Generator(device=dev).manual_seed(5)
     B, CTX, H, NQ, NKV, HD, FF, V, L = 32, 1024, 4096, 32, 8, 128, 14336, 128256, 32
+    cfg = get_quantization_config("gptq_marlin").from_config(dict(bits=4, group_size=GROUP, desc_act=False, sym=True))
+
+    def quantized(layer):
+        layer = layer.to(dev)
+        layer.qweight.data.random_(-2 ** 31, 2 ** 31 - 1, generator=gen)       # uniform int4 codes
+        layer.scales.data.copy_((torch.randn(layer.scales.shape, device=dev, generator=gen).abs() * 0.01 + 1e-3)
+                                .to(torch.float16).to(torch.bfloat16))
+        layer.g_idx.data.copy_(torch.arange(layer.input_size, device=dev, dtype=torch.int32) // GROUP)
+        layer.process_weights_after_loading()
+        return layer
+
+    kw = dict(quant_config=cfg, params_dtype=torch.bfloat16, return_bias=False)
     layers = []
     for _ in range(L):
-        layers.append(dict(qkv=W4Layer(H, (NQ + 2 * NKV) * HD, dev, gen), o=W4Layer(H, H, dev, gen),
-                           gate_up=W4Layer(H, 2 * FF, dev, gen), down=W4Layer(FF, H, dev, gen),
+        layers.append(dict(qkv=quantized(QKVParallelLinear(H, HD, NQ, NKV, **kw)), o=quantized(RowParallelLinear(H, H, **kw)),
+                           gate_up=quantized(MergedColumnParallelLinear(H, [FF, FF], **kw)),
+                           down=quantized(RowParallelLinear(FF, H, **kw)),
                            kc=torch.randn(B, NKV, CTX, HD, device=dev, generator=gen).to(torch.bfloat16),
                            vc=torch.randn(B, NKV, CTX, HD, device=dev, generator=gen).to(torch.bfloat16),
                            n1=torch.ones(H, device=dev, dtype=torch.bfloat16), n2=torch.ones(H, device=dev, dtype=torch.bfloat16)))
@@ -338,29 +357,36 @@ def decode_step_section(dev):
     lm_head = (torch.randn(V, H, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
     ids = torch.randint(0, V, (B,), device=dev, generator=gen)
 
-    def step(linear_only=False):
+    def step():
         x = emb[ids]
         for ly in layers:
-            h = x if linear_only else F.rms_norm(x, (H,), ly["n1"], 1e-5)
-            qkv = ly["qkv"](h)
-            if linear_only:
-                att = qkv[:, :H]
-            else:
-                q = qkv[:, :NQ * HD].view(B, NQ, 1, HD)
-                att = F.scaled_dot_product_attention(q, ly["kc"], ly["vc"], enable_gqa=True).reshape(B, H)
-            x = x + ly["o"](att.contiguous()) if not linear_only else ly["o"](att.contiguous())
-            h = x if linear_only else F.rms_norm(x, (H,), ly["n2"], 1e-5)
-            gu = ly["gate_up"](h)
-            act = gu[:, :FF].contiguous() if linear_only else F.silu(gu[:, :FF]) * gu[:, FF:]
-            x = ly["down"](act) if linear_only else x + ly["down"](act)
-        return x if linear_only else torch.matmul(x, lm_head.t())
+            qkv = ly["qkv"](F.rms_norm(x, (H,), ly["n1"], 1e-5))
+            q = qkv[:, :NQ * HD].view(B, NQ, 1, HD)
+            att = F.scaled_dot_product_attention(q, ly["kc"], ly["vc"], enable_gqa=True).reshape(B, H)
+            x = x + ly["o"](att)
+            gu = ly["gate_up"](F.rms_norm(x, (H,), ly["n2"], 1e-5))
+            x = x + ly["down"](F.silu(gu[:, :FF]) * gu[:, FF:])
+        return torch.matmul(x, lm_head.t())
 
-    t_full = time_graph(lambda: step(False), iters=5, warmup=2)
-    t_lin = time_graph(lambda: step(True), iters=5, warmup=2)
+    t_full = time_graph(step, iters=5, warmup=2)
+    x_h = torch.randn(B, H, device=dev, generator=gen).to(torch.bfloat16)
+    x_f = torch.randn(B, FF, device=dev, generator=gen).to(torch.bfloat16)
+    shapes = dict(qkv=(H, (NQ + 2 * NKV) * HD), o=(H, H), gate_up=(H, 2 * FF), down=(FF, H))
+    per_type = {}
+    for name, (k, n) in shapes.items():
+        xin = x_f if k == FF else x_h
+        t = time_graph(lambda: [ly[name](xin) for ly in layers], iters=5, warmup=2)
+        b = L * w4a16_bytes(B, k, n)
+        per_type[name] = dict(K=k, N=n, us_per_layer=t * 1e6 / L, us_per_step=t * 1e6, share_of_step=t / t_full,
+                              GBps=b / t / 1e9, hbm_frac=b / t / 1e9 / HBM_PEAK_GBS)
+        log(f"[decode step ] {name:8s} {k:5d}x{n:5d} M={B}: {t * 1e6 / L:6.2f} us per layer, {100 * t / t_full:4.1f}% of the step, "
+            f"{b / t / 1e9:5.0f} GB/s ({100 * b / t / 1e9 / HBM_PEAK_GBS:4.1f}% of 8 TB/s)")
+    t_lin = sum(v["us_per_step"] for v in per_type.values()) * 1e-6
     gemm_bytes = L * sum(w4a16_bytes(B, k, n) for (k, n) in LLAMA_SHAPES)
-    row = dict(kind="llama3_8b_decode_step", batch=B, context=CTX, layers=L, step_us=t_full * 1e6, linear_us=t_lin * 1e6,
-               linear_share=t_lin / t_full, tokens_per_s=B / t_full, tokens_per_s_linear_only=B / t_lin,
-               linear_GBps=gemm_bytes / t_lin / 1e9, linear_hbm_frac=gemm_bytes / t_lin / 1e9 / HBM_PEAK_GBS)
+    row = dict(kind="llama3_8b_decode_step", batch=B, context=CTX, layers=L, surface="GPTQMarlinLinearMethod.apply",
+               step_us=t_full * 1e6, linear_us=t_lin * 1e6, linear_share=t_lin / t_full, tokens_per_s=B / t_full,
+               tokens_per_s_linear_only=B / t_lin, linear_GBps=gemm_bytes / t_lin / 1e9,
+               linear_hbm_frac=gemm_bytes / t_lin / 1e9 / HBM_PEAK_GBS, per_projection=per_type)
     log(f"[decode step ] batch {B} ctx {CTX}: {t_full * 1e6:.0f} us/step = {B / t_full:.0f} tok/s; the 128 W4A16 GEMMs (M=32) take "
         f"{t_lin * 1e6:.0f} us = {100 * t_lin / t_full:.0f}% of the step, {gemm_bytes / t_lin / 1e9:.0f} GB/s "
         f"({100 * gemm_bytes / t_lin / 1e9 / HBM_PEAK_GBS:.1f}% of 8 TB/s)")
@@ -493,6 +519,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-extra", action="store_true", help="skip the prefill / FP8 sections")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--sections", default="", help="comma-separated subset of the extra sections to run (default: all)")
     ap.add_argument("--counter-pass", action="store_true",
                     help="for `rocprofv3 --pmc`: three eager passes of [256 MiB device copy, the 12 headline GEMMs], no timing")
     args = ap.parse_args()
@@ -527,6 +554,8 @@ def main():
                          ("variants", variants_section),
                          ("vendor_ceiling", vendor_ceiling_section),
                          ("decode_step", decode_step_section)):
+            if args.sections and name not in args.sections.split(","):
+                continue
             try:
                 extra[name] = fn(dev)
             except Exception as e:
