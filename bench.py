@@ -184,6 +184,44 @@ def per_shape_decode(dev, sets, acts):
     return rows
 
 
+def stream_ceiling_section(dev):
+    """What a kernel that only READS a layer's bytes achieves on this machine, launch to launch in the same kind of HIP
+    graph as the decode GEMMs and on buffers that have left the caches (600 MB of copies cycling): launch gap +
+    first-byte latency + streaming.  `vaq_stream_read_probe` (16-byte loads, every load of a wavefront in flight at
+    once), best of a few wavefront counts and depths per size.  The sum over the 12 headline GEMMs is the practical
+    ceiling the headline is also priced against."""
+    import ctypes
+    from vllm_amd import _lib
+    lib = _lib.load()
+    rows = []
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    pool = torch.empty(640 << 20, dtype=torch.uint8, device=dev).random_()
+    stream = lambda: ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)      # noqa: E731
+    for (k, n) in LLAMA_SHAPES:
+        nbytes = k * n // 2 + (k // GROUP) * n * 2                   # what every GEMM on this layer must read
+        copies = max(2, pool.numel() // nbytes)
+        best = None
+        for waves in (1024, 2048, 4096):
+            for depth in (4, 8):
+                if nbytes // 1024 // waves < depth:
+                    continue
+
+                def fn():
+                    for c in range(copies):
+                        _lib.check(lib.vaq_stream_read_probe(ctypes.c_void_p(pool.data_ptr() + c * (nbytes & ~1023)), nbytes, waves,
+                                                             depth, ctypes.c_void_p(sink.data_ptr()), stream()))
+                t = time_graph(fn, iters=5, warmup=2, inner=copies)
+                read = (nbytes // 1024 // waves) * waves * 1024
+                t_full = t * nbytes / read                                  # (the probe reads whole KiB per wavefront)
+                if best is None or t_full < best[0]:
+                    best = (t_full, waves, depth)
+        rows.append(dict(kind="stream_read_ceiling", K=k, N=n, bytes=nbytes, us=best[0] * 1e6, GBps=nbytes / best[0] / 1e9,
+                         waves=best[1], depth=best[2]))
+        log(f"[read ceiling] {nbytes / 1e6:6.2f} MB (K={k} N={n}): {best[0] * 1e6:6.2f} us launch to launch = {nbytes / best[0] / 1e9:5.0f} GB/s "
+            f"({best[1]} wavefronts, {best[2]} loads in flight)")
+    return rows
+
+
 def prefill_section(dev):
     """BASELINE.json config 3: asymmetric uint4 + act_order, both readings of its act_order wording.  `rows`: g_idx from a
     random permutation of the K rows (the reference's generator): activations are reordered on every call.  `groups`:
@@ -431,6 +469,50 @@ def fp8_section(dev):
     return rows
 
 
+def roofline_mfma(extra):
+    """The compute-bound kernels against the dense MFMA peaks, from the M = 4096 rows of the prefill and FP8 sections
+    (HIP-graph timings of this run): per kernel the FLOPs of one launch, its average duration and the fraction of peak."""
+    out = []
+    for r in extra.get("prefill", []):
+        if r["M"] == 4096 and r["kind"].endswith("groups"):
+            out.append(dict(kernel="vaq::w4a16_prefill2_kernel", K=r["K"], N=r["N"], M=r["M"], flops_per_launch=2.0 * r["M"] * r["N"] * r["K"],
+                            avg_ns=round(r["us"] * 1e3), peak_TFLOPs=BF16_PEAK_TFLOPS, frac=round(r["mfma_frac"], 4)))
+    for r in extra.get("fp8", []):
+        if r["M"] == 4096:
+            out.append(dict(kernel="vaq::fp8_mm_tile3_kernel", K=r["K"], N=r["N"], M=r["M"], flops_per_launch=2.0 * r["M"] * r["N"] * r["K"],
+                            avg_ns=round(r["us"] * 1e3), peak_TFLOPs=FP8_PEAK_TFLOPS, frac=round(r["mfma_frac"], 4)))
+    return out or None
+
+
+def mfma_pass(dev):
+    """Workload for a matrix-core counter run (`rocprofv3 --pmc`): the vendor library's plain bf16 GEMM at 4096^3 (the
+    calibration: a kernel whose FLOPs are known) followed by the W4A16 and FP8 GEMMs at M = 4096 on the four Llama-3-8B
+    shapes, eagerly, three times; the last repetition's dispatches are the ones to read."""
+    import vllm_amd._custom_ops as ops
+    gen = torch.Generator(device=dev).manual_seed(0)
+    m = 4096
+    a_cal = torch.randn(m, 4096, device=dev, generator=gen).to(torch.bfloat16)
+    w_cal = torch.randn(4096, 4096, device=dev, generator=gen).to(torch.bfloat16)
+    w4 = [W4Layer(k, n, dev, gen, asym=True) for (k, n) in LLAMA_SHAPES]
+    acts = {k: torch.randn(m, k, device=dev, generator=gen).to(torch.bfloat16) for (k, _) in LLAMA_SHAPES}
+    f8 = []
+    for (k, n) in LLAMA_SHAPES:
+        wq, ws = ops.scaled_fp8_quant((torch.randn(n, k, device=dev, generator=gen) * 0.02).to(torch.bfloat16),
+                                      use_per_token_if_dynamic=True)
+        aq, sa = ops.scaled_fp8_quant(acts[k], use_per_token_if_dynamic=True)
+        f8.append((aq, wq.t(), sa, ws))
+    torch.cuda.synchronize()
+    for _ in range(3):
+        torch.matmul(a_cal, w_cal.t())
+        for layer in w4:
+            layer(acts[layer.k])
+        for aq, wt, sa, ws in f8:
+            ops.cutlass_scaled_mm(aq, wt, sa, ws, torch.bfloat16, None)
+    torch.cuda.synchronize()
+    log(f"[mfma pass] calibration GEMM: {2.0 * m * 4096 * 4096:.0f} FLOP; GEMMs: " +
+        ", ".join(f"{k}x{n}: {2.0 * m * n * k:.0f}" for (k, n) in LLAMA_SHAPES))
+
+
 def counter_pass(dev):
     """Workload for a hardware-counter run: a plain 256 MiB device-to-device copy (the calibration kernel: it reads and
     writes exactly 262144 KiB) followed by one eager pass over the 12 headline GEMMs, three times; the last repetition's
@@ -519,6 +601,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-extra", action="store_true", help="skip the prefill / FP8 sections")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--mfma-pass", action="store_true",
+                    help="for `rocprofv3 --pmc`: three eager passes of [vendor bf16 GEMM 4096^3, W4A16 and FP8 GEMMs at M = 4096], no timing")
     ap.add_argument("--sections", default="", help="comma-separated subset of the extra sections to run (default: all)")
     ap.add_argument("--counter-pass", action="store_true",
                     help="for `rocprofv3 --pmc`: three eager passes of [256 MiB device copy, the 12 headline GEMMs], no timing")
@@ -538,6 +622,9 @@ def main():
     if args.counter_pass:
         counter_pass(dev)
         return
+    if args.mfma_pass:
+        mfma_pass(dev)
+        return
     sec, step_bytes, sets, acts = headline(dev, args.steps, args.warmup)
     value = step_bytes / sec / 1e9
     launches = len(LLAMA_SHAPES) * len(DECODE_MS)
@@ -548,6 +635,16 @@ def main():
     except Exception as e:   # extras never invalidate the headline
         log(f"[decode per shape] failed: {e}")
     del sets
+    torch.cuda.empty_cache()
+    practical = None
+    try:
+        extra["stream_read_ceiling"] = stream_ceiling_section(dev)
+        t_floor = len(DECODE_MS) * sum(r["us"] for r in extra["stream_read_ceiling"]) * 1e-6
+        practical = step_bytes / t_floor / 1e9
+        log(f"[read ceiling] 12 reads of the headline layers: {t_floor * 1e6:.1f} us -> practical ceiling {practical:.0f} GB/s; "
+            f"the headline is at {100 * value / practical:.1f}% of it")
+    except Exception as e:
+        log(f"[read ceiling] failed: {e}")
     torch.cuda.empty_cache()
     if not args.no_extra:
         for name, fn in (("prefill", prefill_section), ("fp8", fp8_section), ("fused_norm_quant", fused_norm_quant_section),
@@ -584,7 +681,11 @@ def main():
                      "unit": "GB/s", "frac": round(value / HBM_PEAK_GBS, 4),
                      "traffic": int(MEASURED_TRAFFIC_PER_ALGORITHMIC_BYTE * step_bytes / launches),
                      "avg_launch_us": round(sec * 1e6 / launches, 3),
-                     "algorithmic_bytes_per_launch": step_bytes // launches},
+                     "algorithmic_bytes_per_launch": step_bytes // launches,
+                     # what a read-only kernel reaches on the same layers in the same kind of graph (cold buffers)
+                     "practical_peak": None if practical is None else round(practical, 1),
+                     "practical_frac": None if practical is None else round(value / practical, 4)},
+        "roofline_mfma": roofline_mfma(extra),
         "cpu_baseline": cpu,
         "extra": extra,
     }

@@ -266,6 +266,14 @@ int vaq_fp8_quant_per_token_tuned(const void* in, int in_dtype, int64_t in_row_s
                                   int64_t out_row_stride, float* scales, const float* scale_ub, int64_t rows,
                                   int64_t hidden, void* stream, const VaqTuning* tuning);
 
+/*
+ * Measurement aid (no counterpart in the reference): a kernel that only reads `bytes` (rounded down to whole KiB per
+ * wavefront) from `src`, `waves` wavefronts (a multiple of 4) with `depth` (2, 4 or 8) 16-byte loads per lane in flight.
+ * The benchmark times it on cold buffers of each layer's size to report the practical ceiling of the memory-bound
+ * kernels beside the nominal HBM peak.  `sink` is a device word that is practically never written.
+ */
+int vaq_stream_read_probe(const void* src, int64_t bytes, int waves, int depth, void* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
