@@ -36,11 +36,15 @@ extern "C" {
 /* Weight layouts produced by vaq_w4a16_repack (both are int32 [K/16, 2N], same bytes). */
 #define VAQ_LAYOUT_MARLIN 0 /* the reference's Marlin tile order, bit-exact with gptq_marlin_repack   */
 #define VAQ_LAYOUT_NATIVE 1 /* wavefront tile order consumed by vaq_w4a16_gemm (K % 128 == 0 needed) */
+#define VAQ_LAYOUT_NATIVE_BYTES 2 /* num_bits 8 only: the same tiles with whole bytes, for wtype FE4M3    */
 
 /* Weight code types (what b_q_type.id selects in the reference, vllm/scalar_type.py:327-351). */
 #define VAQ_WTYPE_U4B8 0 /* symmetric: code - 8            */
 #define VAQ_WTYPE_U4 1   /* asymmetric: code - zeros[g][n] */
 #define VAQ_WTYPE_U8B128 2 /* 8-bit symmetric: code - 128 (weights from vaq_w4a16_repack with num_bits = 8) */
+#define VAQ_WTYPE_FE4M3 3  /* FP8 e4m3fn weights, 16-bit activations (the reference's weight-only FP8 path,
+                              marlin_utils_fp8.py); weights from vaq_w4a16_repack with num_bits = 8 and
+                              VAQ_LAYOUT_NATIVE_BYTES; group_size -1 or 128, no zero points, no act_order */
 
 /* Text of the last error on the calling thread ("" if none). */
 const char* vaq_last_error(void);

@@ -69,3 +69,42 @@ def native_unpack8(packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
     hi = native_unpack(planes[:, 0].reshape(size_k // 16, 2 * size_n), size_k, size_n)
     lo = native_unpack(planes[:, 1].reshape(size_k // 16, 2 * size_n), size_k, size_n)
     return (hi << 4) | lo
+
+
+def _byte_index_maps(size_k: int, size_n: int):
+    """For every output word of the byte layout the rows of its four bytes (low byte first) and its column."""
+    assert size_k % 128 == 0 and size_n % 16 == 0
+    k_tiles = size_k // 128
+    idx = np.arange(size_k * size_n // 4, dtype=np.int64)
+    q = idx & 3
+    lane = (idx >> 2) & 63
+    h = (idx >> 8) & 1
+    tile = idx >> 9
+    nt, kt = tile // k_tiles, tile % k_tiles
+    o, r = lane >> 4, lane & 15
+    j = 2 * h + (q >> 1)
+    k0 = kt * 128 + j * 32 + o * 8 + (q & 1) * 4
+    return k0[:, None] + np.arange(4)[None, :], nt * 16 + r
+
+
+def native_pack8_bytes(q: np.ndarray) -> np.ndarray:
+    """Logical 8-bit codes int[K, N] -> int32 [K/16, 4N], whole bytes (the layout of FP8 weights): per tile two 1 KiB
+    blocks; block h gives lane L = 16*o + r the 16 bytes of rows 128*kt + 32*j + 8*o + e, j = 2h (bytes 0..7) and
+    j = 2h + 1 (bytes 8..15), column 16*nt + r."""
+    size_k, size_n = q.shape
+    rows, n = _byte_index_maps(size_k, size_n)
+    codes = np.asarray(q).astype(np.uint32)[rows, n[:, None]]
+    shifts = (np.arange(4, dtype=np.uint32) * 8)[None, :]
+    words = np.bitwise_or.reduce(codes << shifts, axis=1).astype(np.uint32)
+    return words.view(np.int32).reshape(size_k // 16, 4 * size_n)
+
+
+def native_unpack8_bytes(packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    """Inverse of :func:`native_pack8_bytes`."""
+    words = np.asarray(packed).reshape(-1).view(np.uint32)
+    rows, n = _byte_index_maps(size_k, size_n)
+    shifts = (np.arange(4, dtype=np.uint32) * 8)[None, :]
+    codes = (words[:, None] >> shifts) & np.uint32(0xFF)
+    q = np.zeros((size_k, size_n), dtype=np.int32)
+    q[rows, n[:, None]] = codes.astype(np.int32)
+    return q

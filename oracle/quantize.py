@@ -229,3 +229,28 @@ def scaled_dequantize(x_q: torch.Tensor, x_s: torch.Tensor, group_shape=None, ou
     if group_shape is not None:
         assert x_s.shape[-1] == x_q.shape[-1] // group_shape[1] and x_s.shape[-2] == x_q.shape[-2] // group_shape[0]
     return (x_q.to(torch.float32) * group_broadcast(x_s.to(torch.float32), x_q.shape)).to(out_dtype)
+
+
+# --------------------------------------------------------------------------- weight-only FP8 (e4m3 weights, 16-bit activations)
+
+def marlin_quant_fp8_torch(weight: torch.Tensor, group_size: int):
+    """marlin_utils_fp8.py:316-351 without the Marlin re-ordering: ``weight`` [N, K] float ->
+    ``(w_ref [K, N] in weight.dtype, fp8 codes uint8 [K, N], scales [G, N] in weight.dtype)`` with
+    ``scale = amax(group) / 448``, ``fp8 = (weight / scale).to(float8_e4m3fn)``, ``w_ref = fp8.to(dtype) * scale``
+    (one group spanning K for ``group_size == -1``)."""
+    n, k = weight.shape
+    g = k if group_size == -1 else group_size
+    scales = weight.view(n, k // g, g).abs().max(-1)[0] / 448
+    rep = scales.repeat_interleave(g, 1)
+    fp8 = (weight / rep).to(torch.float8_e4m3fn)
+    w_ref = fp8.to(weight.dtype) * rep
+    return w_ref.T.contiguous(), fp8.view(torch.uint8).T.contiguous(), scales.T.contiguous()
+
+
+def fp8_weight_case(weight: torch.Tensor, group_size: int) -> dict:
+    """A weight-only FP8 layer in the GPTQ-style container the repack takes (int32 [K/4, N], four consecutive k per
+    word, low byte first: marlin_utils_fp8.py:299-313 ``pack_fp8_to_int32``), plus the codes, scales and ``w_ref``."""
+    w_ref, codes, scales = marlin_quant_fp8_torch(weight, group_size)
+    k, n = codes.shape
+    qn = codes.numpy().astype(np.int32)
+    return dict(q=qn, qweight=ow.gptq_pack(qn, 8), scales=scales, group_size=group_size, w_ref=w_ref)

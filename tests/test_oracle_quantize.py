@@ -206,3 +206,45 @@ def test_awq_pack_brute_force_one_word():
         want.append(np.uint32(word).astype(np.uint32).view(np.int32) if False else word)
     assert [int(np.uint32(v)) for v in packed.view(np.uint32)[0]] == want
     assert want[0] == 0x86427531                      # 1,3,5,7 in the low nibbles, then 2,4,6,8
+
+
+@pytest.mark.parametrize("group_size", [-1, 128])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fp8_weight_quantiser_pins(dtype, group_size):
+    """marlin_quant_fp8_torch restated: every group's largest magnitude maps to +-448 (code 0x7E / 0xFE), the
+    dequantised weight is within the e4m3 step (2^-4 relative, plus the 16-bit roundings) of the input, and the codes
+    decode (independent bit-level decoder of oracle/fp8.py) to w_ref / scale."""
+    from oracle import fp8 as of
+    n, k = 48, 256
+    w = torch.randn(n, k, generator=torch.Generator().manual_seed(3)).to(dtype)
+    w_ref, codes, scales = oq.marlin_quant_fp8_torch(w, group_size)
+    g = k if group_size == -1 else group_size
+    assert w_ref.shape == (k, n) and codes.shape == (k, n) and scales.shape == (k // g, n) and codes.dtype == torch.uint8
+    mags = (codes & 0x7F).reshape(k // g, g, n).amax(dim=1)
+    assert bool((mags == 0x7E).all()), "a group's maximum must land on 448"
+    eps = torch.finfo(dtype).eps
+    s_full = scales.repeat_interleave(g, 0).double()
+    err = (w.T.double() - w_ref.double()).abs()
+    assert bool((err <= w.T.double().abs() * (2.0 ** -4 + 8 * eps) + s_full * 2.0 ** -10).all())
+    dec = torch.from_numpy(of.e4m3fn_decode(codes.numpy())).double()
+    assert bool(((w_ref.double() - dec * s_full).abs() <= eps * w_ref.double().abs() + 1e-30).all())
+    case = oq.fp8_weight_case(w, group_size)
+    assert np.array_equal(ow.unpack_rows(case["qweight"], 8), case["q"])
+
+
+def test_native_byte_layout_round_trip_and_first_words():
+    from oracle import native_layout as nl
+    k, n = 256, 32
+    q = np.random.default_rng(0).integers(0, 256, size=(k, n), dtype=np.int32)
+    packed = nl.native_pack8_bytes(q)
+    assert packed.shape == (k // 16, 4 * n) and packed.dtype == np.int32
+    assert np.array_equal(nl.native_unpack8_bytes(packed, k, n), q)
+    words = packed.reshape(-1).view(np.uint32)
+    # by hand: word 0 = rows 0..3 of column 0; word 2 = rows 32..35 (j = 1); word 4 = lane 1 -> column 1;
+    # word 64 = lane 16 (o = 1) -> rows 8..11; word 256 = block 1 -> rows 64..67 (j = 2); word 512 = next K tile
+    def word(rows, col):
+        return sum(int(q[r, col]) << (8 * i) for i, r in enumerate(rows))
+    assert int(words[0]) == word(range(0, 4), 0) and int(words[1]) == word(range(4, 8), 0)
+    assert int(words[2]) == word(range(32, 36), 0) and int(words[4]) == word(range(0, 4), 1)
+    assert int(words[64]) == word(range(8, 12), 0) and int(words[256]) == word(range(64, 68), 0)
+    assert int(words[512]) == word(range(128, 132), 0) and int(words[1024]) == word(range(0, 4), 16)

@@ -23,7 +23,7 @@ GPTQ_MARLIN_TILE = 16
 GPTQ_MARLIN_MIN_THREAD_N = 64
 GPTQ_MARLIN_MIN_THREAD_K = 128
 
-_LAYOUTS = {"marlin": _lib.VAQ_LAYOUT_MARLIN, "native": _lib.VAQ_LAYOUT_NATIVE}
+_LAYOUTS = {"marlin": _lib.VAQ_LAYOUT_MARLIN, "native": _lib.VAQ_LAYOUT_NATIVE, "native_bytes": _lib.VAQ_LAYOUT_NATIVE_BYTES}
 
 
 def _check(cond: bool, msg: str) -> None:
@@ -229,9 +229,9 @@ def _check_gemm_args(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, 
     _check(b_scales.dtype == a.dtype, f"b_scales dtype {b_scales.dtype} must equal the activation dtype {a.dtype}")
 
     # what this build implements out of everything the reference accepts
-    if b_q_type not in (scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8b128):
+    if b_q_type not in (scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8b128, scalar_types.float8_e4m3fn):
         raise NotImplementedError(f"gptq_marlin_gemm: weight type {b_q_type} is not built for gfx950 "
-                                  "(uint4b8 / uint4 / uint8b128)")
+                                  "(uint4b8 / uint4 / uint8b128 / float8_e4m3fn)")
     if is_zp_float:
         raise NotImplementedError("gptq_marlin_gemm: float zero points (is_zp_float) are not built for gfx950")
     if has_act_order and not is_k_full:
@@ -245,7 +245,12 @@ def _check_gemm_args(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, 
                                       "(only -1, 32, 64, 128)")
     _check(size_k % GPTQ_MARLIN_MIN_THREAD_K == 0,
            f"size_k = {size_k}, is not divisible by min_thread_k = {GPTQ_MARLIN_MIN_THREAD_K}")
-    if b_q_type == scalar_types.uint8b128:
+    if b_q_type == scalar_types.float8_e4m3fn:
+        # weight-only FP8 (marlin_utils_fp8.py): channelwise scales or groups of 128 rows, no act_order
+        if group_size not in (-1, 128) or has_act_order:
+            raise NotImplementedError("gptq_marlin_gemm: float8_e4m3fn weights take group_size -1 or 128 and no act_order")
+        wtype = _lib.VAQ_WTYPE_FE4M3
+    elif b_q_type == scalar_types.uint8b128:
         wtype = _lib.VAQ_WTYPE_U8B128
     else:
         wtype = _lib.VAQ_WTYPE_U4 if has_zp else _lib.VAQ_WTYPE_U4B8
@@ -590,7 +595,8 @@ def gptq_marlin_repack(b_q_weight: torch.Tensor, perm: torch.Tensor, size_k: int
     """GPTQ int32[K/8, N] -> repacked int32[K/16, 2N].
 
     ``layout="native"`` (default) is the wavefront tile order ``gptq_marlin_gemm`` consumes; ``layout="marlin"``
-    reproduces the reference's Marlin order bit-for-bit.  Callers treat the result as opaque either way.
+    reproduces the reference's Marlin order bit-for-bit; ``layout="native_bytes"`` (``num_bits = 8`` only) keeps whole
+    bytes in the native tiles, for FP8 weights (``b_q_type = float8_e4m3fn``).  Callers treat the result as opaque.
     """
     return _ops.gptq_marlin_repack(b_q_weight, perm, size_k, size_n, num_bits, _LAYOUTS[layout])
 

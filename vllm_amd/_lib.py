@@ -17,8 +17,8 @@ VAQ_ERR_UNSUPPORTED = -2
 VAQ_ERR_LAUNCH = -3
 
 VAQ_F16, VAQ_BF16, VAQ_F32 = 0, 1, 2
-VAQ_LAYOUT_MARLIN, VAQ_LAYOUT_NATIVE = 0, 1
-VAQ_WTYPE_U4B8, VAQ_WTYPE_U4, VAQ_WTYPE_U8B128 = 0, 1, 2
+VAQ_LAYOUT_MARLIN, VAQ_LAYOUT_NATIVE, VAQ_LAYOUT_NATIVE_BYTES = 0, 1, 2
+VAQ_WTYPE_U4B8, VAQ_WTYPE_U4, VAQ_WTYPE_U8B128, VAQ_WTYPE_FE4M3 = 0, 1, 2, 3
 
 # name -> (restype, argtypes); must list every symbol the header declares (tests check this against the header)
 _SIGNATURES = {

@@ -99,9 +99,9 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8) 
 
 template <bool BF16, int MB, bool HAS_ZP, int MR, int GS>
 static int dispatch_rc2(const Decode2Params& p, int rc, hipStream_t s) {
-  if (rc == 1) return launch_decode2<BF16, GS, MB, HAS_ZP, MR, 1, false, 1>(p, s);
-  if (rc == 2) return launch_decode2<BF16, GS, MB, HAS_ZP, MR, 1, false, 2>(p, s);
-  if (rc == 3) return launch_decode2<BF16, GS, MB, HAS_ZP, MR, 1, false, 3>(p, s);
+  if (rc == 1) return launch_decode2<BF16, GS, MB, HAS_ZP, MR, 1, 0, 1>(p, s);
+  if (rc == 2) return launch_decode2<BF16, GS, MB, HAS_ZP, MR, 1, 0, 2>(p, s);
+  if (rc == 3) return launch_decode2<BF16, GS, MB, HAS_ZP, MR, 1, 0, 3>(p, s);
   return launch_decode2<BF16, GS, MB, HAS_ZP, MR, 1>(p, s);
 }
 
@@ -148,7 +148,8 @@ int w4a16_decode2_workspace(int M, int N, int K, int sub, bool w8, size_t* c_tmp
 int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
                          const int32_t* perm, const void* bias, void* c, float* c_tmp, int64_t c_tmp_bytes,
                          int32_t* counters, int64_t counter_ints, int M, int N, int K, int sub, bool channelwise,
-                         bool w8, int dtype, hipStream_t s) {
+                         int wt, int dtype, hipStream_t s) {
+  const bool w8 = wt != 0;      // 8-bit weights of either kind (1: nibble planes, 2: FP8 bytes): two blocks per 128 rows
   Decode2Params p;
   p.a = (const uint16_t*)a;
   p.lda = lda;
@@ -188,7 +189,8 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
   }
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
-  if (w8 && sub > 1) rc = decode2_launch_w8sub(p, sub, cfg.gs, MB, cfg.mr, bf16, s);
+  if (wt == 2) rc = decode2_launch_f8(p, cfg.gs, MB, cfg.mr, bf16, s);
+  else if (w8 && sub > 1) rc = decode2_launch_w8sub(p, sub, cfg.gs, MB, cfg.mr, bf16, s);
   else if (w8) rc = decode2_launch_w8(p, cfg.gs, MB, cfg.mr, bf16, s);
   else if (sub == 2) rc = decode2_launch_sub2(p, cfg.gs, MB, cfg.mr, bf16, zp, s);
   else if (sub == 4) rc = decode2_launch_sub4(p, cfg.gs, MB, cfg.mr, bf16, zp, s);

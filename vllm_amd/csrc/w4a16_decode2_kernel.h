@@ -19,6 +19,8 @@
 //  * 8-bit codes (W8, symmetric, bias 128): the weights come as two 4-bit planes per tile (high nibbles, then low
 //    nibbles), code - 128 = 16 * (hi - 8) + lo.  Each plane is one tile of the stream, multiplied with the same
 //    activations; the high plane uses the constant operand -(BIAS + 8) and 16 * scale, the low plane -(BIAS + 0).
+//  * FP8 e4m3 weights (WT = 2, 16-bit activations): whole bytes, two 1 KiB blocks per tile (MFMAs 0,1 and 2,3), each byte
+//    pair turned into two 16-bit numbers by one packed conversion; no bias or zero point, so one MFMA per operand.
 //  * WKS > 1: one LDS reduction at the end (wavefronts wks == 0 sum their column's slices).  K slabs that do not fit
 //    LDS (SK > 1 workgroups per n-tile) hand partial tiles over through device-scope write-through stores and an
 //    arrival counter, summed in fixed order by the last arriver.
@@ -68,12 +70,14 @@ static inline uint32_t d2_sat32(uint64_t bytes) { return bytes > 0xffffffffull ?
 
 constexpr int D2_WAVES = 16;
 
-template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, bool W8 = false, int RC = 0>
+template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, int WT = 0, int RC = 0>
 __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Decode2Params p) {
   using T = F16Traits<BF16>;
   static_assert(SUBG == 1 || SUBG == 2 || SUBG == 4, "quantisation groups per 128-row tile");
-  constexpr int TPG = W8 ? 2 : 1;                      // weight tiles per 128 rows of K
-  static_assert(!W8 || (!HAS_ZP && GS % 2 == 0), "8-bit codes: two planes per 128 rows, symmetric");
+  constexpr bool W8 = WT == 1, F8 = WT == 2;           // 8-bit codes as two nibble planes / FP8 e4m3 bytes (see the head comment)
+  constexpr int TPG = WT != 0 ? 2 : 1;                 // 1 KiB weight blocks per 128 rows of K
+  static_assert(WT == 0 || (!HAS_ZP && GS % 2 == 0), "8-bit weights: two blocks per 128 rows, no zero points");
+  static_assert(!F8 || SUBG == 1, "FP8 weights: channelwise scales or groups of 128 rows");
   static_assert(MR == 16 || MB == 1, "compact row staging is for a single m-block");
   // Ring of weight tiles in flight per wavefront.
   //  * Short streams with few staged rows (up to 8 tiles per wavefront, M <= 4) request everything up front: the whole
@@ -91,11 +95,11 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   //    with four slots; six slots 8.7 us; 16 wavefronts of two slots 10.3 us), and, with three slots, for 16 staged rows
   //    (4096 x 28672 at M = 16: 15.2 -> 14.8 us).
   constexpr int LPT = 1 + SUBG * (HAS_ZP ? 2 : 1);              // vector-memory instructions per tile request
-  constexpr int R_SHORT = (GS < 63 / LPT ? GS : 63 / LPT) & (W8 ? ~1 : ~0);      // (8-bit codes: whole plane pairs)
+  constexpr int R_SHORT = (GS < 63 / LPT ? GS : 63 / LPT) & (WT != 0 ? ~1 : ~0);      // (8-bit weights: whole block pairs)
   constexpr bool SHORT = MR <= 4 && GS <= 8 && GS >= 2;
   constexpr bool LATE = RC != 0 && !SHORT;
   constexpr int R_LATE = RC == 1 ? 4 : (RC == 2 ? 3 : 2);
-  static_assert(!(W8 && RC != 0), "8-bit codes take the plane from the slot parity: even rings only");
+  static_assert(!(WT != 0 && RC != 0), "8-bit weights take the block of a tile from the slot parity: even rings only");
   constexpr int R = SHORT ? R_SHORT : (LATE ? (GS < R_LATE ? GS : R_LATE) : ((MR == 16 && MB == 1 && GS >= 7) ? 4 : (GS < 2 ? GS : 2)));
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
@@ -287,6 +291,34 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
       v4f P[MB], Q[MB];
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) P[mb] = Q[mb] = v4f{0.f, 0.f, 0.f, 0.f};
+      if constexpr (F8) {
+        // FP8 bytes: block h = slot parity holds the 8-byte operands of MFMAs 2h and 2h + 1 (words 0,1 and 2,3); a packed
+        // conversion turns two bytes into two 16-bit numbers exactly (every e4m3 value is a bf16 and an fp16 value; the
+        // instruction's scale operand only contributes its power of two, 1.0 here).  No bias, no zero point: P and Q are
+        // the two MFMAs' own chains.
+#pragma unroll
+        for (int j2 = 0; j2 < 2; ++j2) {
+          const uint32_t wa = wj[2 * j2], wb = wj[2 * j2 + 1];
+          v4u aop;
+          if constexpr (BF16) {
+            aop.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wa, 1.0f, false));
+            aop.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wa, 1.0f, true));
+            aop.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wb, 1.0f, false));
+            aop.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(wb, 1.0f, true));
+          } else {
+            aop.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(wa, 1.0f, false));
+            aop.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(wa, 1.0f, true));
+            aop.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(wb, 1.0f, false));
+            aop.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(wb, 1.0f, true));
+          }
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) {
+            const v4u bop = *reinterpret_cast<const v4u*>(lds + abase[2 * (slot & 1) + j2] + (uint32_t)(mb * KO * MR * 16) + (uint32_t)((gi / TPG) * 256));
+            if (j2 == 0) P[mb] = T::mfma16(aop, bop, P[mb]);
+            else Q[mb] = T::mfma16(aop, bop, Q[mb]);
+          }
+        }
+      } else {
 #pragma unroll
       for (int jj = sj * (4 / SUBG); jj < (sj + 1) * (4 / SUBG); ++jj) {
         v4u aop;
@@ -300,6 +332,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
           P[mb] = T::mfma16(aop, bop, P[mb]);
           Q[mb] = T::mfma16(zop, bop, Q[mb]);
         }
+      }
       }
       float s[4];
       if constexpr (BF16) {
@@ -448,18 +481,18 @@ static inline size_t decode2_lds_bytes(int wks, int groups_per_wave, int mr, int
   return act + red;
 }
 
-template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, bool W8 = false, int RC = 0>
+template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, int WT = 0, int RC = 0>
 static int launch_decode2(const Decode2Params& p_in, hipStream_t s) {
   Decode2Params p = p_in;
   const int WN = p.WN;
   {
-    const int ko = p.WKS * GS / (W8 ? 2 : 1) * 16, nthr = p.WKS * WN * 64;
+    const int ko = p.WKS * GS / (WT != 0 ? 2 : 1) * 16, nthr = p.WKS * WN * 64;
     p.wn_magic = (uint32_t)((65536 + WN - 1) / WN);
     if (WN != 1 || p.perm != nullptr) p.PRIV = 0;
     p.ko_magic = (uint32_t)(((1ull << 32) + (uint64_t)ko - 1) / (uint64_t)ko);
     p.step_m = nthr / ko;
     p.step_ko = nthr - p.step_m * ko;
-    p.b_bytes = d2_sat32((uint64_t)p.K * p.N / 2 * (W8 ? 2 : 1));
+    p.b_bytes = d2_sat32((uint64_t)p.K * p.N / 2 * (WT != 0 ? 2 : 1));
     p.s_bytes = d2_sat32((uint64_t)p.GR * p.N * 2);
     p.z_bytes = d2_sat32((uint64_t)p.GR * (p.N / 8) * 4);
     p.a_bytes = d2_sat32(((uint64_t)(p.M - 1) * (uint64_t)p.lda + (uint64_t)p.K) * 2);
@@ -468,8 +501,8 @@ static int launch_decode2(const Decode2Params& p_in, hipStream_t s) {
       return VAQ_ERR_UNSUPPORTED;
     }
   }
-  const size_t lds = decode2_lds_bytes(p.WKS, GS / (W8 ? 2 : 1), MR, MB);
-  auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP, MR, SUBG, W8, RC>;
+  const size_t lds = decode2_lds_bytes(p.WKS, GS / (WT != 0 ? 2 : 1), MR, MB);
+  auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP, MR, SUBG, WT, RC>;
   static size_t reserved[VAQ_MAX_DEVICES];
   if (const int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "w4a16_gemm(decode)"); rc != VAQ_OK) return rc;
   const int gx = (p.NT + WN - 1) / WN;
@@ -487,5 +520,8 @@ int decode2_launch_mb34(const Decode2Params& p, int gs, int MB, bool bf16, bool 
 // w4a16_decode2_w8sub.hip (sub = 2 / 4 groups per 128 rows: gs in {2, 4, 8, 16}); staged rows mr in {1, 4, 16} (16 when MB == 2).
 int decode2_launch_w8(const Decode2Params& p, int gs, int MB, int mr, bool bf16, hipStream_t s);
 int decode2_launch_w8sub(const Decode2Params& p, int sub, int gs, int MB, int mr, bool bf16, hipStream_t s);
+// FP8 e4m3 weights (bytes), channelwise scales or groups of 128 rows; defined in w4a16_decode2_f8.hip: gs in {2, 4, 8, 14, 16},
+// staged rows mr in {1, 4, 16} (16 when MB == 2).
+int decode2_launch_f8(const Decode2Params& p, int gs, int MB, int mr, bool bf16, hipStream_t s);
 
 }  // namespace vaq

@@ -14,11 +14,11 @@ int w4a16_decode2_workspace(int M, int N, int K, int sub, bool w8, size_t* c_tmp
 int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
                          const int32_t* perm, const void* bias, void* c, float* c_tmp, int64_t c_tmp_bytes,
                          int32_t* counters, int64_t counter_ints, int M, int N, int K, int sub, bool channelwise,
-                         bool w8, int dtype, hipStream_t s);
+                         int wt, int dtype, hipStream_t s);      // wt: 0 4-bit codes, 1 8-bit codes, 2 FP8 e4m3 bytes
 int w4a16_prefill_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* counter_ints);
 int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
                          const void* bias, void* c, float* c_tmp, int64_t c_tmp_bytes, int32_t* counters,
-                         int64_t counter_ints, int M, int N, int K, int sub, bool channelwise, bool w8, int dtype,
+                         int64_t counter_ints, int M, int N, int K, int sub, bool channelwise, int wt, int dtype,
                          hipStream_t s);
 
 constexpr int64_t DECODE_MAX_M = 64;          // up to four m-blocks of 16 rows on the LDS-staged kernel
@@ -125,15 +125,18 @@ extern "C" int vaq_w4a16_gemm_tuned(const void* a, int64_t lda, const int32_t* b
   if (rc != VAQ_OK) return rc;
   VAQ_CHECK_ARG(dtype == VAQ_F16 || dtype == VAQ_BF16, "w4a16_gemm: only supports bfloat16 and float16 (dtype tag %d)",
                 dtype);
-  VAQ_CHECK_ARG(wtype == VAQ_WTYPE_U4B8 || wtype == VAQ_WTYPE_U4 || wtype == VAQ_WTYPE_U8B128,
+  VAQ_CHECK_ARG(wtype == VAQ_WTYPE_U4B8 || wtype == VAQ_WTYPE_U4 || wtype == VAQ_WTYPE_U8B128 || wtype == VAQ_WTYPE_FE4M3,
                 "w4a16_gemm: unknown weight type tag %d", wtype);
   VAQ_CHECK_ARG((wtype == VAQ_WTYPE_U4) == (zeros != nullptr),
-                "w4a16_gemm: b_q_type must be uint4 when has_zp = True and uint4b8 or uint8b128 when has_zp = False");
-  const bool w8 = wtype == VAQ_WTYPE_U8B128;
+                "w4a16_gemm: b_q_type must be uint4 when has_zp = True and uint4b8, uint8b128 or float8_e4m3fn when has_zp = False");
+  const int wt = wtype == VAQ_WTYPE_U8B128 ? 1 : (wtype == VAQ_WTYPE_FE4M3 ? 2 : 0);
+  const bool w8 = wt != 0;
   const bool channelwise = group_size == -1 || (group_size == size_k && size_k != 128);
   VAQ_CHECK_SUPPORTED(channelwise || group_size == 128 || group_size == 64 || group_size == 32,
                       "w4a16_gemm: group_size = %d is not built (only -1, 32, 64, 128)", group_size);
   const int sub = channelwise ? 1 : 128 / group_size;
+  VAQ_CHECK_SUPPORTED(wt != 2 || (sub == 1 && perm == nullptr),
+                      "w4a16_gemm: FP8 weights take channelwise scales or groups of 128 rows, and no act_order");
   VAQ_CHECK_ARG(!w8 || size_k * size_n < (1ll << 32), "w4a16_gemm: problem too large for 8-bit weights");
   VAQ_CHECK_ARG(force_path >= 0 && force_path <= 2, "w4a16_gemm: force_path = %d", force_path);
   if (size_m == 0) return VAQ_OK;
@@ -161,7 +164,7 @@ extern "C" int vaq_w4a16_gemm_tuned(const void* a, int64_t lda, const int32_t* b
   }
   if (decode && decode_impl_for(size_m, size_n, lda, sub, w8) == 0)
     return w4a16_decode2_launch(a, lda, b, scales, zeros, perm, bias, c, c_tmp, c_tmp_bytes, counters, counter_ints, (int)size_m,
-                                (int)size_n, (int)size_k, sub, channelwise, w8, dtype, s);
+                                (int)size_n, (int)size_k, sub, channelwise, wt, dtype, s);
   if (decode) {
     VAQ_CHECK_SUPPORTED(sub == 1 && !w8, "w4a16_gemm: group_size = %d / 8-bit weights with an A of 2 GiB or more are not built",
                         group_size);
@@ -180,7 +183,7 @@ extern "C" int vaq_w4a16_gemm_tuned(const void* a, int64_t lda, const int32_t* b
     lda_eff = size_k;
   }
   return w4a16_prefill_launch(a_eff, lda_eff, b, scales, zeros, bias, c, c_tmp, c_tmp_bytes, counters, counter_ints, (int)size_m,
-                              (int)size_n, (int)size_k, sub, channelwise, w8, dtype, s);
+                              (int)size_n, (int)size_k, sub, channelwise, wt, dtype, s);
 }
 
 // ----------------------------------------------------------------------------- the GEMM on library-owned scratch

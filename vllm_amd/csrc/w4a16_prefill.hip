@@ -105,8 +105,9 @@ int w4a16_prefill_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* co
 
 int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
                          const void* bias, void* c, float* c_tmp, int64_t c_tmp_bytes, int32_t* counters,
-                         int64_t counter_ints, int M, int N, int K, int sub, bool channelwise, bool w8, int dtype,
+                         int64_t counter_ints, int M, int N, int K, int sub, bool channelwise, int wt, int dtype,
                          hipStream_t s) {
+  const bool w8 = wt != 0;      // 8-bit weights of either kind: two 1 KiB blocks per tile
   PrefillParams p;
   p.a = (const uint16_t*)a;
   p.lda = lda;
@@ -143,7 +144,8 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
   const int tile_other = pl.tile == 20 ? 10 : pl.tile;      // the alternating-phase variant exists for 4-bit codes, groups of 128
-  if (w8) rc = prefill_launch_w8(p, sub, tile_other, bf16, s);
+  if (wt == 2) rc = prefill_launch_f8(p, tile_other, bf16, s);
+  else if (w8) rc = prefill_launch_w8(p, sub, tile_other, bf16, s);
   else if (sub > 1) rc = prefill_launch_sub(p, sub, tile_other, bf16, zp, s);
   else if (bf16) rc = zp ? dispatch_tile<true, true>(p, pl.tile, s) : dispatch_tile<true, false>(p, pl.tile, s);
   else rc = zp ? dispatch_tile<false, true>(p, pl.tile, s) : dispatch_tile<false, false>(p, pl.tile, s);

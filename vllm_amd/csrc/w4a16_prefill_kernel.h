@@ -96,6 +96,30 @@ static __device__ inline v4u dequant_scaled8(uint32_t hi, uint32_t lo, float s, 
   return scale_bytes<BF16>(((hi & 0x0f0f0f0fu) << 4) | (lo & 0x0f0f0f0fu), (hi & 0xf0f0f0f0u) | ((lo >> 4) & 0x0f0f0f0fu), s, neg_zs);
 }
 
+// FP8 e4m3 weights: eight bytes of 8 consecutive k (words wa: 0..3, wb: 4..7) -> 8 scaled 16-bit weights.  The packed
+// conversion is exact (its scale operand only contributes a power of two: 1.0), the product with the scale is exact in
+// fp32 (4 x 8..11 significant bits) and rounded once to the 16-bit type: the bits of `fp8.to(dtype) * scale`.
+template <bool BF16>
+static __device__ inline uint32_t fp8_pair_scaled(uint32_t w, bool hi, float s) {
+  typedef float v2f __attribute__((ext_vector_type(2)));
+  const v2f f = hi ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(w, 1.0f, true) : __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(w, 1.0f, false);
+  return pack2<BF16>(f[0] * s, f[1] * s);
+}
+template <bool BF16>
+static __device__ inline v4u dequant_fp8(uint32_t wa, uint32_t wb, float s) {
+  v4u r;
+  r.x = fp8_pair_scaled<BF16>(wa, false, s);
+  r.y = fp8_pair_scaled<BF16>(wa, true, s);
+  r.z = fp8_pair_scaled<BF16>(wb, false, s);
+  r.w = fp8_pair_scaled<BF16>(wb, true, s);
+  return r;
+}
+// Register t (0..3) of dequant_fp8's result.
+template <bool BF16>
+static __device__ inline uint32_t dequant_fp8_part(uint32_t wa, uint32_t wb, float s, int t) {
+  return fp8_pair_scaled<BF16>((t >> 1) ? wb : wa, (t & 1) != 0, s);
+}
+
 // Register t (0..3) of scale_bytes' result: elements 2t and 2t+1.
 template <bool BF16>
 static __device__ inline uint32_t scale_bytes_part(uint32_t tb, uint32_t ub, float s, float neg_zs, int t) {
@@ -320,9 +344,12 @@ __global__ __launch_bounds__(256) void w4a16_prefill_kernel(const PrefillParams 
 //  * the MFMAs take the weight fragment as A operand, so four consecutive accumulator registers are four consecutive
 //    output columns of one row: 8 bytes per lane into the epilogue's LDS staging (16-byte global stores from there);
 //  * weight words of group g+1 are requested one K step before they are needed (two register sets, by group parity).
-template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP, int SUBG, bool W8 = false, bool PP = false>
+template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP, int SUBG, int WT = 0, bool PP = false>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(const PrefillParams p) {
   using T = F16Traits<BF16>;
+  constexpr bool W8 = WT != 0;      // two 1 KiB blocks per tile: nibble planes of 8-bit codes (WT = 1) or FP8 e4m3 bytes (WT = 2)
+  constexpr bool F8 = WT == 2;
+  static_assert(!F8 || SUBG == 1, "FP8 weights: channelwise scales or groups of 128 rows");
   static_assert(!PP || (!W8 && SUBG == 1 && (BM / (8 * WAVES_M * WAVES_N)) % 2 == 0 && WAVES_M * WAVES_N == 8),
                 "alternating phases: 8 wavefronts, groups of 128 rows, an even number of DMA instructions per step");
   static_assert(!W8 || !HAS_ZP, "8-bit codes: symmetric");
@@ -424,7 +451,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
 #pragma unroll
       for (int sj = 0; sj < SUBG; ++sj) {
         const float sv = T::to_float(snxt_raw[i][sj]);
-        uint32_t zc = W8 ? 128u : 8u;
+        uint32_t zc = F8 ? 0u : (W8 ? 128u : 8u);
         if constexpr (HAS_ZP) zc = (znxt_raw[i][sj] >> ((r & 7) * 4)) & 0xFu;    // column n = 16 * tile + r
         scur[i][sj] = sv;
         if constexpr (HP) {
@@ -446,7 +473,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
       const int sj = (j * SUBG) >> 2;
       zv = -((float)((zcur[i] >> (8 * sj)) & 0xffu) * sv);
     } else {
-      zv = -(W8 ? 128.f : 8.f) * sv;
+      zv = -(F8 ? 0.f : (W8 ? 128.f : 8.f)) * sv;
     }
   };
   // Prologue only: dequantise half 0 of the current group into weight stage 0.
@@ -461,7 +488,8 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
       sub_vals(i, which, sv, zv);
       const int c0 = (row & 1) * 8 + o + which * 4, sw = (row >> 1) & 15;
       v4u dv;
-      if constexpr (W8) dv = dequant_scaled8<BF16>(wsel, which ? wcur_lo[i].y : wcur_lo[i].x, sv, zv);
+      if constexpr (F8) dv = dequant_fp8<BF16>(which ? wcur[i].z : wcur[i].x, which ? wcur[i].w : wcur[i].y, sv);      // block 0: words of j = 0, 1
+      else if constexpr (W8) dv = dequant_scaled8<BF16>(wsel, which ? wcur_lo[i].y : wcur_lo[i].x, sv, zv);
       else if constexpr (HP) dv = dequant_scaled_h(wsel, s2cur[i], nzb2cur[i]);
       else dv = dequant_scaled<BF16>(wsel, sv, zv);
       *reinterpret_cast<v4u*>(Bb + (row >> 1) * 256 + ((c0 ^ sw) * 16)) = dv;
@@ -549,7 +577,13 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
             const uint32_t wsel = half ? (which ? wcur[i].w : wcur[i].z) : (which ? wcur[i].y : wcur[i].x);
             float sv, zv;
             sub_vals(i, half * 2 + which, sv, zv);
-            if constexpr (W8) {
+            if constexpr (F8) {
+              // piece j = 2 * half + which: block `half` of the tile, words 2 * which and 2 * which + 1
+              const uint32_t wa = half ? (which ? wcur_lo[i].z : wcur_lo[i].x) : (which ? wcur[i].z : wcur[i].x);
+              const uint32_t wb = half ? (which ? wcur_lo[i].w : wcur_lo[i].y) : (which ? wcur[i].w : wcur[i].y);
+              if constexpr (SUB == 4) dq[slot][t] = dequant_fp8_part<BF16>(wa, wb, sv, t);
+              else dq[slot] = dequant_fp8<BF16>(wa, wb, sv);
+            } else if constexpr (W8) {
               const uint32_t wlo = half ? (which ? wcur_lo[i].w : wcur_lo[i].z) : (which ? wcur_lo[i].y : wcur_lo[i].x);
               if constexpr (SUB == 4) dq[slot][t] = dequant_part8<BF16>(wsel, wlo, sv, zv, t);
               else dq[slot] = dequant_scaled8<BF16>(wsel, wlo, sv, zv);
@@ -898,10 +932,10 @@ static int launch_prefill(const PrefillParams& p, hipStream_t s) {
   return VAQ_OK;
 }
 
-template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP, int SUBG, bool W8 = false, bool PP = false>
+template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N, bool HAS_ZP, int SUBG, int WT = 0, bool PP = false>
 static int launch_prefill2(const PrefillParams& p, hipStream_t s) {
   const size_t lds = (size_t)(3 * BM + 2 * BN) * 128;
-  auto kern = w4a16_prefill2_kernel<BF16, BM, BN, WAVES_M, WAVES_N, HAS_ZP, SUBG, W8, PP>;
+  auto kern = w4a16_prefill2_kernel<BF16, BM, BN, WAVES_M, WAVES_N, HAS_ZP, SUBG, WT, PP>;
   static size_t reserved[VAQ_MAX_DEVICES];
   if (const int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "w4a16_gemm(prefill)"); rc != VAQ_OK) return rc;
   const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
@@ -915,5 +949,7 @@ int prefill_launch_sub(const PrefillParams& p, int sub, int tile, bool bf16, boo
 // 8-bit codes; defined in w4a16_prefill_w8.hip for the direct-to-LDS tile ids 10, 12, 14, 15 (sub = 1, 2 or 4 groups per
 // 128 rows).
 int prefill_launch_w8(const PrefillParams& p, int sub, int tile, bool bf16, hipStream_t s);
+// FP8 e4m3 weights (bytes), channelwise scales or groups of 128 rows; defined in w4a16_prefill_f8.hip (tile ids 10, 12, 14, 15)
+int prefill_launch_f8(const PrefillParams& p, int tile, bool bf16, hipStream_t s);
 
 }  // namespace vaq

@@ -27,6 +27,10 @@
 //          order above, the next block the low nibbles, so the 4-bit kernels' dequantisation applies to each plane.
 //  MARLIN  16 x 64 tiles of 256 words; words th*8 + warp*2 + {0, 1} hold, one byte each, rows 16*kt + 2*(th%4) +
 //          {0, 8, 1, 9} of column 64*nt + 16*warp + th/4 (word 0) and that column + 8 (word 1).
+//  NATIVE_BYTES (FP8 e4m3 weights, whose codes are not linear in their bits, so the nibble planes are of no use): per
+//          tile two 1 KiB blocks; block h (0 / 1) gives lane L = 16*o + r the 16 bytes of rows 128*kt + 32*j + 8*o + e,
+//          j = 2h (bytes 0..7, e = byte index) and j = 2h + 1 (bytes 8..15), column 16*nt + r: every 8 bytes are the A
+//          operand of one v_mfma_f32_16x16x32 after four packed FP8 -> 16-bit conversions.
 //
 // With `perm` (act_order sort indices) output row k takes input row perm[k].
 #include "vaq_common.h"
@@ -159,6 +163,31 @@ __global__ __launch_bounds__(256) void repack_native8_kernel(const uint32_t* __r
   }
 }
 
+// 8-bit codes kept as bytes (NATIVE_BYTES): one thread per output word (four consecutive rows of one column).
+__global__ __launch_bounds__(256) void repack_native8_bytes_kernel(const uint32_t* __restrict__ qw,
+                                                                    const int32_t* __restrict__ perm,
+                                                                    uint32_t* __restrict__ out, int64_t size_k,
+                                                                    int64_t size_n) {
+  const int64_t total = size_k * size_n / 4;
+  const int64_t k_tiles = size_k / 128;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int q = idx & 3;
+    const int lane = (idx >> 2) & 63;
+    const int h = (idx >> 8) & 1;
+    const int64_t tile = idx >> 9;
+    const int64_t nt = tile / k_tiles, kt = tile - nt * k_tiles;
+    const int o = lane >> 4, r = lane & 15;
+    const int j = 2 * h + (q >> 1);
+    const int64_t k0 = kt * 128 + j * 32 + o * 8 + (q & 1) * 4;
+    const int64_t n = nt * 16 + r;
+    uint32_t res = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) res |= fetch_code8(qw, perm, k0 + e, n, size_n) << (8 * e);
+    out[idx] = res;
+  }
+}
+
 // 8-bit codes, reference (Marlin) order: one thread per output word.
 __global__ __launch_bounds__(256) void repack_marlin8_kernel(const uint32_t* __restrict__ qw,
                                                               const int32_t* __restrict__ perm,
@@ -194,8 +223,11 @@ static int repack_common(const int32_t* qweight, const int32_t* perm, int32_t* o
                 (long long)size_k);
   VAQ_CHECK_ARG(size_n > 0 && size_n % 64 == 0, "w4a16_repack: size_n = %lld is not divisible by tile_n_size = 64",
                 (long long)size_n);
-  VAQ_CHECK_ARG(layout == VAQ_LAYOUT_MARLIN || layout == VAQ_LAYOUT_NATIVE, "w4a16_repack: unknown layout %d", layout);
-  VAQ_CHECK_ARG(layout != VAQ_LAYOUT_NATIVE || size_k % 128 == 0,
+  VAQ_CHECK_ARG(layout == VAQ_LAYOUT_MARLIN || layout == VAQ_LAYOUT_NATIVE || layout == VAQ_LAYOUT_NATIVE_BYTES,
+                "w4a16_repack: unknown layout %d", layout);
+  VAQ_CHECK_ARG(layout != VAQ_LAYOUT_NATIVE_BYTES || (num_bits == 8 && !awq),
+                "w4a16_repack: the byte layout is for 8-bit GPTQ-packed weights");
+  VAQ_CHECK_ARG(layout == VAQ_LAYOUT_MARLIN || size_k % 128 == 0,
                 "w4a16_repack: native layout needs size_k %% 128 == 0, got size_k = %lld", (long long)size_k);
   VAQ_CHECK_ARG(qweight && out, "w4a16_repack: null pointer");
   const int64_t total = size_k * size_n / (32 / num_bits);
@@ -209,6 +241,7 @@ static int repack_common(const int32_t* qweight, const int32_t* perm, int32_t* o
   const dim3 grid((unsigned)blocks), block(threads);
   if (num_bits == 8) {
     if (layout == VAQ_LAYOUT_NATIVE) hipLaunchKernelGGL(repack_native8_kernel, grid, block, 0, s, qw, perm, o, size_k, size_n);
+    else if (layout == VAQ_LAYOUT_NATIVE_BYTES) hipLaunchKernelGGL(repack_native8_bytes_kernel, grid, block, 0, s, qw, perm, o, size_k, size_n);
     else hipLaunchKernelGGL(repack_marlin8_kernel, grid, block, 0, s, qw, perm, o, size_k, size_n);
   } else if (layout == VAQ_LAYOUT_NATIVE) {
     if (awq)

@@ -3,6 +3,7 @@
 non-Marlin branches) and ``ptpc_fp8.py`` (PTPCFp8LinearMethod :82-137: per-channel weights, per-token activations)."""
 from __future__ import annotations
 
+import os
 from typing import Any, Optional
 
 import torch
@@ -12,6 +13,7 @@ from vllm_amd import _custom_ops as ops
 from vllm_amd.parameter import ModelWeightParameter, PerTensorScaleParameter
 from .base_config import LinearMethodBase, QuantizationConfig, QuantizeMethodBase
 from .input_quant_fp8 import GroupShape
+from .utils.marlin_utils_fp8 import apply_fp8_marlin_linear, prepare_fp8_layer_for_marlin
 from .utils.w8a8_utils import Fp8LinearOp
 
 ACTIVATION_SCHEMES = ["static", "dynamic"]
@@ -71,6 +73,9 @@ class Fp8LinearMethod(LinearMethodBase):
         self.quant_config = quant_config
         self.out_dtype = torch.get_default_dtype()
         self.block_quant = False
+        # Weight-only FP8 on the W4A16 GEMM: the reference takes this route on GPUs without FP8 matrix hardware or when
+        # VLLM_TEST_FORCE_FP8_MARLIN is set (fp8.py:353-363).  gfx950 has FP8 MFMA: only when forced.
+        self.use_marlin = os.environ.get("VLLM_TEST_FORCE_FP8_MARLIN", "0").lower() in ("1", "true")
         self.act_q_static = self.quant_config.activation_scheme == "static"
         # per-token activation scales whenever they are dynamic: the fused GEMM takes them at no extra cost
         self.act_q_group_shape = GroupShape.PER_TENSOR if self.act_q_static else GroupShape.PER_TOKEN
@@ -118,7 +123,9 @@ class Fp8LinearMethod(LinearMethodBase):
                 # A module that is already fused on disk brings ONE scale: it sits in entry 0 and the last entry still
                 # holds its initial value.  Its weight is quantised with that single scale already and stays as it is.
                 unfused_in_checkpoint = bool(weight_scale[-1] > torch.finfo(torch.float8_e4m3fn).min)
-                if unfused_in_checkpoint:
+                if unfused_in_checkpoint and self.use_marlin:
+                    max_w_scale = weight_scale      # the weight-only path keeps one scale per shard (expanded per channel below)
+                elif unfused_in_checkpoint:
                     # one scale per shard: requantise every shard to the largest one
                     start = 0
                     deq = torch.zeros_like(weight, dtype=torch.float32)
@@ -136,8 +143,15 @@ class Fp8LinearMethod(LinearMethodBase):
         layer.weight_scale = Parameter(weight_scale.data.reshape(-1)[:1].reshape(()) if weight_scale.numel() == 1
                                        else weight_scale.data, requires_grad=False)
         layer.input_scale = Parameter(input_scale, requires_grad=False) if input_scale is not None else None
+        if self.use_marlin:
+            prepare_fp8_layer_for_marlin(layer, size_k_first=True)
+            layer.input_scale = None          # activations are not quantised on this path
 
     def apply(self, layer: torch.nn.Module, x: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+        if self.use_marlin:
+            return apply_fp8_marlin_linear(input=x, weight=layer.weight, weight_scale=layer.weight_scale,
+                                           workspace=layer.workspace, size_n=layer.output_size_per_partition,
+                                           size_k=layer.input_size_per_partition, bias=bias)
         return self.fp8_linear.apply(input=x, weight=layer.weight, weight_scale=layer.weight_scale,
                                      out_dtype=self.out_dtype if x.dtype not in (torch.float16, torch.bfloat16) else x.dtype,
                                      input_scale=layer.input_scale, bias=bias)
