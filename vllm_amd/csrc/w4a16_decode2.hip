@@ -23,9 +23,10 @@ static int round_gs(int x, int sub, bool w8) {
 
 // Groups per slab are limited by LDS (128 KiB of activations, 256 bytes per group and staged row): 512 / rows.
 // G, gslab, gs and slab_max below count weight tiles: one per 128 rows of K, two (nibble planes) for 8-bit codes.
-static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8) {
+// `nt_mult`: copies of every n-tile's stream that run side by side (rows split over workgroups, see the kernel).
+static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8, int nt_mult = 1) {
   const int TPG = w8 ? 2 : 1;
-  const int G = K / 128 * TPG, NT = N / 16;
+  const int G = K / 128 * TPG, NT = N / 16 * nt_mult;
   const int MB = (M + 15) / 16;
   Decode2Config c;
   c.mr = M == 1 ? 1 : (M <= 4 ? 4 : 16);
@@ -136,6 +137,23 @@ static int dispatch_mr2(const Decode2Params& p, const Decode2Config& c, bool bf1
   }
 }
 
+// Rows split over workgroups (one m-block each, see the kernel) instead of several m-blocks per workgroup: 4-bit codes
+// in groups of 128 rows / channelwise, no act_order, and only where a single m-block needs no split of K.
+// (development switch exp[2]: 1 forces it off, 2 on wherever it is built)
+static bool use_row_split(int M, int N, int K, int sub, int wt, bool has_perm) {
+  if (M <= 16 || sub != 1 || wt != 0 || has_perm || tuning().exp[2] == 1) return false;
+  const Decode2Config c = pick_decode2_config(16, N, K, sub, false, (M + 15) / 16);
+  if (c.sk != 1) return false;
+  if (tuning().exp[2] == 2) return true;
+  // One round of full workgroups.  Measured: 4096 x 4096 at M = 32 / 64: 8.5 / 10.5 -> 6.6 / 9.2 us, 4096 x 6144: 8.8 / 11.4
+  // -> 8.7 / 10.6 us; with three m-blocks the grids of those layers spill into a second round (15 us) or leave ten
+  // wavefronts per workgroup (9.9 -> 11.7 us).  A 28672-wide layer would need streams of 32 tiles (measured 20.4 -> 21.7 us).
+  const long wgs = (long)((N / 16 + c.wn - 1) / c.wn) * ((M + 15) / 16);
+  return wgs <= num_cus_current_device() && c.wks * c.wn >= 12;
+}
+
+int decode2_launch_msp(const Decode2Params& p, int gs, int rc, bool bf16, bool zp, hipStream_t s);      // w4a16_decode2_msp.hip
+
 int w4a16_decode2_workspace(int M, int N, int K, int sub, bool w8, size_t* c_tmp_bytes, size_t* counter_ints) {
   const Decode2Config c = pick_decode2_config(M, N, K, sub, w8);
   const int MB = (M + 15) / 16;
@@ -169,7 +187,8 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
   p.z_stride = channelwise ? 0 : N / 8;
   p.k_mask = 0x000f000fu;
   p.k_ex = dtype == VAQ_BF16 ? 0x43004300u : 0x64006400u;
-  const Decode2Config cfg = pick_decode2_config(M, N, K, sub, w8);
+  const bool row_split = use_row_split(M, N, K, sub, wt, perm != nullptr);
+  const Decode2Config cfg = row_split ? pick_decode2_config(16, N, K, sub, w8, (M + 15) / 16) : pick_decode2_config(M, N, K, sub, w8);
   p.SK = cfg.sk;
   p.WKS = cfg.wks;
   p.WN = cfg.wn;
@@ -189,7 +208,8 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
   }
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
-  if (wt == 2) rc = decode2_launch_f8(p, cfg.gs, MB, cfg.mr, bf16, s);
+  if (row_split) rc = decode2_launch_msp(p, cfg.gs, cfg.rc, bf16, zp, s);
+  else if (wt == 2) rc = decode2_launch_f8(p, cfg.gs, MB, cfg.mr, bf16, s);
   else if (w8 && sub > 1) rc = decode2_launch_w8sub(p, sub, cfg.gs, MB, cfg.mr, bf16, s);
   else if (w8) rc = decode2_launch_w8(p, cfg.gs, MB, cfg.mr, bf16, s);
   else if (sub == 2) rc = decode2_launch_sub2(p, cfg.gs, MB, cfg.mr, bf16, zp, s);

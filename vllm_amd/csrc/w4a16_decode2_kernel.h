@@ -70,9 +70,19 @@ static inline uint32_t d2_sat32(uint64_t bytes) { return bytes > 0xffffffffull ?
 
 constexpr int D2_WAVES = 16;
 
-template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, int WT = 0, int RC = 0>
+template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, int WT = 0, int RC = 0, bool MSP = false>
 __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Decode2Params p) {
   using T = F16Traits<BF16>;
+  static_assert(!MSP || (MB == 1 && MR == 16), "rows split over workgroups: one full m-block each");
+  // MSP: more than 16 rows handled as independent m-blocks, one per blockIdx.z -- every workgroup is the single-m-block
+  // kernel on rows 16z .. 16z+15 (the weights are read once per m-block; the workgroups of one n-tile run side by side
+  // and the later ones find the tiles in L2).  Against two m-blocks in one workgroup this halves the staged activations
+  // per workgroup: a K of 4096 fits LDS again and needs no split over workgroups.
+  const int mz = MSP ? (int)blockIdx.z : 0;
+  const int M_loc = MSP ? min(16, p.M - 16 * mz) : p.M;
+  const uint16_t* const a_loc = MSP ? p.a + (int64_t)mz * 16 * p.lda : p.a;
+  const uint32_t a_bytes_loc = MSP ? p.a_bytes - (uint32_t)mz * 32u * (uint32_t)p.lda : p.a_bytes;
+  uint16_t* const c_loc = MSP ? p.c + (int64_t)mz * 16 * p.N : p.c;
   static_assert(SUBG == 1 || SUBG == 2 || SUBG == 4, "quantisation groups per 128-row tile");
   constexpr bool W8 = WT == 1, F8 = WT == 2;           // 8-bit codes as two nibble planes / FP8 e4m3 bytes (see the head comment)
   constexpr int TPG = WT != 0 ? 2 : 1;                 // 1 KiB weight blocks per 128 rows of K
@@ -94,6 +104,11 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   //    most 8 wavefronts per compute unit, which are latency-bound with two slots (14336 x 4096 at M = 1: 9.2 -> 8.0 us
   //    with four slots; six slots 8.7 us; 16 wavefronts of two slots 10.3 us), and, with three slots, for 16 staged rows
   //    (4096 x 28672 at M = 16: 15.2 -> 14.8 us).
+  // Two or more m-blocks: the second MFMA of every pair would be the same for all n-tiles of a k-tile, and with 16
+  // MFMAs per tile the matrix core, not memory, sets the pace (4096 x 28672 at M = 32: the wavefronts of a compute unit
+  // finished 10 us apart).  The row sums S[m] of every staged 128-row tile are then computed once per workgroup, right
+  // after the fill, kept in LDS, and the correction is  P - (BIAS + z) * S  in fp32.
+  constexpr bool SPRE = MB >= 2 && WT == 0 && SUBG == 1;
   constexpr int LPT = 1 + SUBG * (HAS_ZP ? 2 : 1);              // vector-memory instructions per tile request
   constexpr int R_SHORT = (GS < 63 / LPT ? GS : 63 / LPT) & (WT != 0 ? ~1 : ~0);      // (8-bit weights: whole block pairs)
   constexpr bool SHORT = MR <= 4 && GS <= 8 && GS >= 2;
@@ -122,7 +137,8 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   const __amdgpu_buffer_rsrc_t rb = d2_rsrc32(p.b, p.b_bytes);
   const __amdgpu_buffer_rsrc_t rs = d2_rsrc32(p.scales, p.s_bytes);
   const __amdgpu_buffer_rsrc_t rz = d2_rsrc32(HAS_ZP ? (const void*)p.zeros : (const void*)p.scales, p.z_bytes);
-  const int vo_b = lane * 16, vo_s = o * 8, vo_z = (r16 >> 3) * 4;
+  // zero points: as an MFMA operand a lane needs the one of column r16, in the output layout those of columns 4o .. 4o+3
+  const int vo_b = lane * 16, vo_s = o * 8, vo_z = ((SPRE ? (o >> 1) : (r16 >> 3))) * 4;
   v4u wq[R];
   v2u sc[R][SUBG];
   uint32_t zq[R][SUBG];
@@ -163,7 +179,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
       // the next wavefront's slice (or of the next row) and writes there exactly what its owner writes.  The first
       // weight tile is requested before the activations, the others after them: the wait below then leaves R - 1 tiles
       // in flight.
-      const __amdgpu_buffer_rsrc_t ra = d2_rsrc32(p.a, p.a_bytes);
+      const __amdgpu_buffer_rsrc_t ra = d2_rsrc32(a_loc, a_bytes_loc);
       typedef __attribute__((address_space(3))) void* lds_ptr_t;
       issue_load(0, 0);
       const int own = (GS / TPG) * 16;                         // k-octets of this wavefront's slice
@@ -173,7 +189,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
           const int sl = c0 + lane;
           const int m2 = (int)__umulhi((uint32_t)sl, p.ko_magic), ko2 = sl - m2 * KO;
           const int k = k_slab0 + (ko2 ^ (m2 & (MR - 1))) * 8;
-          const bool ok = m2 < MR * MB && m2 < p.M && k < p.K;
+          const bool ok = m2 < MR * MB && m2 < M_loc && k < p.K;
           const uint32_t off = ok ? (uint32_t)(m2 * lda32 + k) * 2u : 0x80000000u;
           __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(lds + (size_t)c0 * 16), 16, (int)off, 0, 0, 0);
         }
@@ -188,11 +204,11 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
       // out-of-range offset of the buffer descriptor (which ends with the last valid element) and arrive as zeros; the
       // image is padded to a multiple of 1 KiB for the last instruction.  The weight tiles are requested after these
       // loads (loads retire in order as far as the wait counter is concerned) and stay in flight across the barrier.
-      const __amdgpu_buffer_rsrc_t ra = d2_rsrc32(p.a, p.a_bytes);
+      const __amdgpu_buffer_rsrc_t ra = d2_rsrc32(a_loc, a_bytes_loc);
       typedef __attribute__((address_space(3))) void* lds_ptr_t;
       for (int c0 = w * 64; c0 < chunks; c0 += NTHR) {
         const int k = k_slab0 + (ko ^ (m & (MR - 1))) * 8;
-        const bool ok = m < MR * MB && m < p.M && k < p.K;
+        const bool ok = m < MR * MB && m < M_loc && k < p.K;
         const uint32_t off = ok ? (uint32_t)(m * lda32 + k) * 2u : 0x80000000u;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(lds + (size_t)c0 * 16), 16, (int)off, 0, 0, 0);
         m += step_m;
@@ -220,8 +236,8 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
           kk[i] = ko;
           const int64_t k = (int64_t)k_slab0 + (int64_t)(ko ^ (m & (MR - 1))) * 8;
           v[i] = v4u{0u, 0u, 0u, 0u};
-          if (m < MR * MB && m < p.M && k < p.K) {
-            const uint16_t* row = p.a + (int64_t)m * p.lda;
+          if (m < MR * MB && m < M_loc && k < p.K) {
+            const uint16_t* row = a_loc + (int64_t)m * p.lda;
             const v4i p0 = *reinterpret_cast<const v4i*>(p.perm + k);
             const v4i p1 = *reinterpret_cast<const v4i*>(p.perm + k + 4);
             v[i].x = (uint32_t)row[p0.x] | ((uint32_t)row[p0.y] << 16);
@@ -243,6 +259,37 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
       }
       __syncthreads();
     }
+  }
+
+  // ---- 2. row sums of the staged tiles (two or more m-blocks) ----
+  constexpr bool RED_ALIAS = MB > 2;
+  // LDS behind the activation image (padded to 1 KiB): the reduction buffer of the K slices (see step 4; three and four
+  // m-blocks: on top of the activations), then the row sums.  With two m-blocks the buffer is compact -- the
+  // wavefronts of slice 0 write nothing, so it holds the tiles of the wavefronts WN .. WKS*WN - 1 only -- which is what
+  // lets 128 KiB of activations, the buffer and the sums fit the 160 KiB.
+  constexpr bool RED_COMPACT = MB == 2;
+  float* rowsum = nullptr;
+  if constexpr (SPRE) {
+    const size_t act_b = ((size_t)KO * MR * MB * 16 + 1023) & ~(size_t)1023;
+    const size_t red_b = WKS > 1 ? (size_t)(RED_COMPACT ? D2_WAVES - D2_WAVES / WKS : D2_WAVES) * MB * 1024 : 0;
+    rowsum = reinterpret_cast<float*>(lds + (RED_ALIAS ? (act_b > red_b ? act_b : red_b) : act_b + red_b));
+    constexpr uint32_t ONE2 = BF16 ? 0x3f803f80u : 0x3c003c00u;
+    const v4u ones = {ONE2, ONE2, ONE2, ONE2};
+    const int NW = WKS * WN;
+    for (int t = w; t < slab_groups; t += NW) {          // tile t of the slab: its 128 k of every staged row
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        v4f q = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          const v4u bop = *reinterpret_cast<const v4u*>(lds + (uint32_t)((r16 * KO + t * 16 + ((jj * 4 + o) ^ r16)) * 16) + (uint32_t)(mb * KO * MR * 16));
+          q = T::mfma16(ones, bop, q);
+        }
+        if (o == 0) rowsum[(t * MB + mb) * 16 + r16] = q[0];      // every register of column r16 holds the sum of row r16
+      }
+    }
+    // the LDS writes only: the weight tiles requested above stay in flight across this barrier
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   }
 
   // ---- 3. the K loop of this wavefront: GS tiles, fully unrolled ----
@@ -284,6 +331,18 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
       else zbits = NEG_BIAS_BITS | 8u;
       const uint32_t z2 = zbits | (zbits << 16);
       const v4u zop = {z2, z2, z2, z2};
+      // (row sums kept in LDS: the factor -(BIAS + z) of output column 4o + r, and the sums of this lane's row)
+      float zf[4], rs_m[MB];
+      if constexpr (SPRE) {
+        constexpr float BIASF = BF16 ? 128.0f : 1024.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if constexpr (HAS_ZP) zf[r] = -(BIASF + (float)((zqt[sj] >> ((((o & 1) * 4 + r)) * 4)) & 0xFu));
+          else zf[r] = -(BIASF + 8.0f);
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) rs_m[mb] = rowsum[((wks * GS + gi) * MB + mb) * 16 + r16];
+      }
 
       // Two accumulation chains per m-block -- the products with the codes in P, the bias / zero-point correction in Q --
       // issued alternately: an MFMA that accumulates on the previous one's result waits for it, and one chain of eight
@@ -330,9 +389,15 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
         for (int mb = 0; mb < MB; ++mb) {
           const v4u bop = *reinterpret_cast<const v4u*>(lds + abase[jj] + (uint32_t)(mb * KO * MR * 16) + (uint32_t)((gi / TPG) * 256));
           P[mb] = T::mfma16(aop, bop, P[mb]);
-          Q[mb] = T::mfma16(zop, bop, Q[mb]);
+          if constexpr (!SPRE) Q[mb] = T::mfma16(zop, bop, Q[mb]);
         }
       }
+      }
+      if constexpr (SPRE) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) Q[mb][r] = zf[r] * rs_m[mb];
       }
       float s[4];
       if constexpr (BF16) {
@@ -381,12 +446,15 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   // ---- 4. reduce the K slices of the workgroup ----
   // [16 waves][MB][64] partial tiles: behind the activations, or -- with three or four m-blocks, where both would not
   // fit -- on top of them once every wavefront is through its K loop
-  constexpr bool RED_ALIAS = MB > 2;
-  v4f* red = reinterpret_cast<v4f*>(RED_ALIAS ? lds : lds + (((size_t)KO * MR * MB * 16 + 1023) & ~(size_t)1023));
+  // (one m-block: the unused tile of wavefront 0 doubles as the padding that the last instruction of a private fill
+  // may write zeros into)
+  v4f* red = reinterpret_cast<v4f*>(RED_ALIAS ? lds : lds + (((size_t)KO * MR * MB * 16 + 1023) & ~(size_t)1023)) - (RED_COMPACT ? WN * MB * 64 : 0);
   if (WKS > 1) {
     if constexpr (RED_ALIAS) __syncthreads();
+    if (!RED_COMPACT || wks != 0) {
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) red[(w * MB + mb) * 64 + lane] = acc[mb];
+      for (int mb = 0; mb < MB; ++mb) red[(w * MB + mb) * 64 + lane] = acc[mb];
+    }
     __syncthreads();
     if (wks != 0) return;
     // the partial tiles of the other slices, added in slice order; with many slices, seven reads in flight at a time
@@ -455,7 +523,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
     v4f val = acc[mb];
     const bool write_out = true;
     const int m = mb * 16 + r16;
-    if (write_out && m < p.M) {
+    if (write_out && m < M_loc) {
       const int n = nt * 16 + o * 4;
       if (p.bias) {
         const v2u bb = *reinterpret_cast<const v2u*>(p.bias + n);
@@ -467,21 +535,23 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
       v2u outv;
       outv.x = (uint32_t)T::from_float(val[0]) | ((uint32_t)T::from_float(val[1]) << 16);
       outv.y = (uint32_t)T::from_float(val[2]) | ((uint32_t)T::from_float(val[3]) << 16);
-      *reinterpret_cast<v2u*>(p.c + (int64_t)m * p.N + n) = outv;
+      *reinterpret_cast<v2u*>(c_loc + (int64_t)m * p.N + n) = outv;
     }
   }
 }
 
-// LDS of a workgroup: activations of `groups` = WKS * (groups per wavefront) quantisation groups for MR x MB rows, 16
-// spare bytes, and the reduction buffer of the K slices (on top of the activations for MB > 2, see the kernel).
+// LDS of a workgroup: activations of `groups` = WKS * (groups per wavefront) quantisation groups for MR x MB rows, the
+// reduction buffer of the K slices (on top of the activations for MB > 2, see the kernel), and with two or more
+// m-blocks the row sums of the staged tiles.
 static inline size_t decode2_lds_bytes(int wks, int groups_per_wave, int mr, int mb) {
   const size_t act = ((size_t)wks * groups_per_wave * 256 * mr * mb + 1023) & ~(size_t)1023;     // padded to 1 KiB (see the fill)
-  const size_t red = wks > 1 ? (size_t)D2_WAVES * mb * 1024 : 0;
-  if (mb > 2) return act > red ? act : red;
-  return act + red;
+  const size_t red = wks > 1 ? (size_t)(mb == 2 ? D2_WAVES - D2_WAVES / wks : D2_WAVES) * mb * 1024 : 0;
+  const size_t sums = mb >= 2 ? (size_t)wks * groups_per_wave * mb * 64 : 0;      // row sums of the staged tiles (see SPRE)
+  if (mb > 2) return (act > red ? act : red) + sums;
+  return act + red + sums;
 }
 
-template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, int WT = 0, int RC = 0>
+template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, int WT = 0, int RC = 0, bool MSP = false>
 static int launch_decode2(const Decode2Params& p_in, hipStream_t s) {
   Decode2Params p = p_in;
   const int WN = p.WN;
@@ -502,11 +572,11 @@ static int launch_decode2(const Decode2Params& p_in, hipStream_t s) {
     }
   }
   const size_t lds = decode2_lds_bytes(p.WKS, GS / (WT != 0 ? 2 : 1), MR, MB);
-  auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP, MR, SUBG, WT, RC>;
+  auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP, MR, SUBG, WT, RC, MSP>;
   static size_t reserved[VAQ_MAX_DEVICES];
   if (const int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "w4a16_gemm(decode)"); rc != VAQ_OK) return rc;
   const int gx = (p.NT + WN - 1) / WN;
-  hipLaunchKernelGGL(kern, dim3(gx, p.SK), dim3(64, p.WKS * WN), lds, s, p);
+  hipLaunchKernelGGL(kern, dim3(gx, p.SK, MSP ? (p.M + 15) / 16 : 1), dim3(64, p.WKS * WN), lds, s, p);
   return VAQ_OK;
 }
 
