@@ -917,9 +917,12 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   // the largest tile shape that fills 70 % of the compute units (measured on the Llama shapes, M = 256 .. 4096: a
   // partly filled device of large tiles beats a full one of small tiles by 25-40 %); for 128 x 128 also when two
   // parts of a long K get it there (14336 x 4096 at M = 512, cold, 73 -> 62 us)
+  // ... and for 256 x 256 when two parts of a very long K do (14336 x 4096 at M = 1536 / 2048, cold: 139 / 145 -> 116 / 130 us;
+  // 4096 x 4096 at M = 2048 in two parts: 45 -> 66 us)
   const int parts128 = K / 64 >= 128 ? 2 : 1;
+  const int parts256 = K / 64 >= 192 ? 2 : 1;
   if (pl.cfg <= 0)
-    pl.cfg = tiles(256, 256) * 10 >= cus * 7 ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (tiles(128, 128) * parts128 * 10 >= cus * 7 ? 3 : 4));
+    pl.cfg = tiles(256, 256) * parts256 * 10 >= cus * 7 ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (tiles(128, 128) * parts128 * 10 >= cus * 7 ? 3 : 4));
   // the smallest tile with two k-slices per step: 5-8 % faster on a short K (half the barriers), no gain on a long one
   if (tuning().fp8_tile_cfg <= 0 && pl.cfg == 4 && K % 128 == 0 && K <= 8192) pl.cfg = 14;
   if (pl.cfg >= 10 && K % 128 != 0) pl.cfg %= 10;      // two k-slices per step need K % 128 == 0
@@ -1079,7 +1082,14 @@ static bool dispatch_stream(const Fp8MMParams& p, hipStream_t s) {
   // 31.8 / 38.0 -> 30.4 / 31.9 us, M = 1 unchanged or 3 % faster)
   const int cus = num_cus_current_device();
   const int rounds = (NT + cus - 1) / cus;
-  int gx = tuning().fp8_gx > 0 ? tuning().fp8_gx : (NT + rounds - 1) / rounds;
+  int gx = (NT + rounds - 1) / rounds;
+  // One m-block, measured with cold weights: on a layer of many rounds two workgroups per compute unit are ahead
+  // (4096 x 28672 at M = 1 / 4 / 16: 28.1 / 28.2 / 29.2 -> 25.7 / 26.1 / 27.8 us; at M = 32 30.5 -> 33.0 us), and with up to
+  // four rows a layer of one to two rounds runs one tile per workgroup (4096 x 6144 at M = 1 / 4: 9.3 / 9.4 -> 8.6 / 9.0 us;
+  // at M = 16 10.2 -> 10.9 us).
+  if (MB == 1 && NT >= 4 * cus) gx = 2 * cus;
+  else if (p.M <= 4 && NT > cus && NT <= 2 * cus) gx = NT;
+  if (tuning().fp8_gx > 0) gx = tuning().fp8_gx;
   if (gx > NT) gx = NT;
   if (MB == 1) {
     if (ks == 4) launch_stream<BF16_OUT, 4, 1>(p, wk, gx, s);
