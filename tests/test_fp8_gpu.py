@@ -246,9 +246,13 @@ def test_scaled_mm_small_m_every_route_exact(device, m):
     rows (three for K = 1664 .. 4096, four only up to two rounds of workgroups), with one and with several n-tiles per
     workgroup, the same kernel over two halves of K with a hand-over (16 < M <= 32 up to K = 16384),
     the tile kernel with K split over workgroups for a K beyond it (also at M <= 32) and without a split.
+    Up to 32 rows the streaming kernel exists in two forms -- weights fetched in the MFMA operand layout, or as whole
+    cache lines through wavefront-private LDS rings with 4, 8 or 16 K steps per wavefront -- and each case runs with the
+    automatic choice, with the LDS form switched off and with each of its step counts forced (per-call tuning override).
     Small-integer operands, power-of-two scales and an integer bias: the result must equal the integer GEMM, scaled and
     shifted, rounded once to bf16; the arrival counters of the splits must be back at zero."""
     import vllm_amd._custom_ops as ops
+    from vllm_amd import _tuning
     g = torch.Generator().manual_seed(m)
     for n, k in ((128, 1664), (256, 4096), (4096, 2048), (4112, 2048), (8208, 1664), (64, 1536), (128, 14336),
                  (4096, 8192 + 128), (48, 4224), (128, 28672), (4112, 14336 + 256), (64, 16384 + 128)):
@@ -257,10 +261,15 @@ def test_scaled_mm_small_m_every_route_exact(device, m):
         sa = torch.pow(2.0, -(torch.arange(m) % 2).float()).reshape(m, 1)
         sb = torch.pow(2.0, (torch.arange(n) % 3).float()).reshape(n, 1)
         bias = (torch.arange(n) % 5).float()
-        out = ops.cutlass_scaled_mm(a.to(torch.float8_e4m3fn).to(device), w.to(torch.float8_e4m3fn).to(device).t(),
-                                    sa.to(device), sb.to(device), torch.bfloat16, bias.to(torch.bfloat16).to(device))
         want = (sa * (sb.t() * (a @ w.t())) + bias).to(torch.bfloat16)
-        assert torch.equal(out.cpu().float(), want.float()), (m, n, k)
+        a_dev, w_dev = a.to(torch.float8_e4m3fn).to(device), w.to(torch.float8_e4m3fn).to(device).t()
+        for lds_form in ((0, 9, 1, 2, 3) if m <= 32 else (0,)):
+            switches = [0] * 15
+            switches[4] = lds_form
+            with _tuning.override(exp=switches):
+                out = ops.cutlass_scaled_mm(a_dev, w_dev, sa.to(device), sb.to(device), torch.bfloat16,
+                                            bias.to(torch.bfloat16).to(device))
+            assert torch.equal(out.cpu().float(), want.float()), (m, n, k, lds_form)
     assert all(bool((t == 0).all()) for t in ops._FP8_COUNTERS.values()), "arrival counters not restored to zero"
 
 

@@ -858,6 +858,161 @@ __global__ __launch_bounds__(512) void fp8_mm_stream_kernel(const Fp8MMParams p,
   }
 }
 
+// ----------------------------------------------------------------------------- stream kernel, weights through LDS
+// The stream kernel above fetches the weights in the MFMA operand layout: every load instruction takes 64-byte pieces
+// of 16 rows, half a cache line each.  Measured on bare reads of a 4096 x 28672 byte matrix with cold lines, that
+// pattern reaches 4.2-5.3 TB/s where instructions that read whole lines reach 5.3-5.9 TB/s.  Here every load
+// instruction is a direct-to-LDS load of 4 rows x 256 contiguous bytes into a ring that belongs to the wavefront alone
+// (no barrier: the wavefront waits on its own load counter), and the operands are read back from LDS, 16-byte chunks
+// XOR-swizzled by the row so that the 16 rows of an operand read hit 16 different bank groups.
+//  * blockDim = (64, WK).  Wavefront w owns K steps [w*KS, (w+1)*KS) of 128 bytes; its activations live in registers;
+//    the workgroup walks a contiguous range of 16-row n-tiles; per n-tile the wavefronts reduce through LDS as above.
+//  * A stage is two steps (16 rows x 256 bytes = 4 KiB, four load instructions); the ring holds NSR stages, and the
+//    stage NSR ahead -- of this n-tile or the next -- is requested as soon as a stage's operands have been read.
+template <bool BF16_OUT, int KS, int MB, int NSR>
+__global__ __launch_bounds__(512) void fp8_mm_stream2_kernel(const Fp8MMParams p, int WK) {
+  using T = F16Traits<BF16_OUT>;
+  constexpr int NS = KS / 2;                       // stages per n-tile
+  static_assert(KS % 2 == 0 && NS % NSR == 0, "whole stages, ring slots fixed at compile time");
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds8[];
+  const int lane = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(threadIdx.y);
+  const int q = lane >> 4, r16 = lane & 15;
+  const int kw = w * KS * 128;                     // first byte of K of this wavefront
+  const int kbase = kw + q * 32;
+  uint8_t* const ring = lds8 + (size_t)w * NSR * 4096;
+  v4f* const red = reinterpret_cast<v4f*>(lds8 + (size_t)WK * NSR * 4096);      // [2][WK][MB][64]
+
+  constexpr uint32_t OOB = 0x80000000u;
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.a), 0, (int)p.a_extent, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.b), 0, (int)p.b_extent, 0x00020000);
+  v8i breg[KS][MB];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int m = mb * 16 + r16;
+      const int k = kbase + s * 128;
+      const uint32_t base = (uint32_t)m * (uint32_t)p.lda + (uint32_t)k;
+      const uint32_t o_lo = (m < p.M && k < p.K) ? base : OOB, o_hi = (m < p.M && k + 16 < p.K) ? base + 16u : OOB;
+      const v4i lo = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ra, (int)o_lo, 0, 0));
+      const v4i hi = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ra, (int)o_hi, 0, 0));
+      breg[s][mb] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
+  }
+
+  const int NT = p.N / 16;
+  const int bx = blockIdx.x;
+  const int nt0 = bx * p.nt_base + (bx < p.nt_rem ? bx : p.nt_rem);
+  const int nt1 = nt0 + p.nt_base + (bx < p.nt_rem ? 1 : 0);
+
+  // Load instruction i of a stage fills LDS bytes [1024 i, 1024 i + 1024) = rows 4i .. 4i+3; lane l lands at row
+  // 4i + l/16, position l & 15, which holds chunk (l & 15) ^ row of the row's 256 bytes.
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  uint32_t voffb[4], kchunk[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = 4 * i + (lane >> 4);
+    kchunk[i] = (uint32_t)(((lane & 15) ^ row) * 16);
+    voffb[i] = (uint32_t)row * (uint32_t)p.ldb + kchunk[i];
+  }
+  // `live` = false requests nothing (offsets beyond the extent) but keeps the count of loads in flight the same
+  auto issue_stage = [&](int nt, int st, int slot, bool live) {
+    const int k0 = kw + st * 256;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t vo = (live && k0 + (int)kchunk[i] < p.K) ? voffb[i] : OOB;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(ring + slot * 4096 + i * 1024), 16, (int)vo,
+                                               (int)((uint32_t)(nt * 16) * (uint32_t)p.ldb + (uint32_t)k0), 0, 2);
+    }
+  };
+#pragma unroll
+  for (int st = 0; st < NSR; ++st) issue_stage(nt0, st, st, nt0 < nt1);
+
+  const bool reducer_wave = WK > 1 ? w < MB : true;
+  float sam_mb[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int m = mb * 16 + r16;
+    sam_mb[mb] = (reducer_wave && m < p.M) ? p.sa[p.sa_per_row ? m : 0] : 0.f;
+  }
+
+  int parity = 0;
+  for (int nt = nt0; nt < nt1; ++nt) {
+    v4f acc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb] = v4f{0.f, 0.f, 0.f, 0.f};
+    float sb_r[4] = {0.f, 0.f, 0.f, 0.f};
+    uint16_t bias_r[4] = {0, 0, 0, 0};
+    if (reducer_wave) {
+      const int n = nt * 16 + q * 4;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        sb_r[r] = p.sb[p.sb_per_col ? n + r : 0];
+        if (p.bias) bias_r[r] = p.bias[n + r];
+      }
+    }
+#pragma unroll
+    for (int st = 0; st < NS; ++st) {
+      constexpr int W_AFTER = (NSR - 1) * 4;      // load instructions requested after this stage's (any others in flight only make the wait stricter)
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(W_AFTER) : "memory");
+      const int slot = st % NSR;
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const int c0 = 8 * s2 + 2 * q;
+        const v4i lo = *reinterpret_cast<const v4i*>(ring + slot * 4096 + r16 * 256 + ((c0 ^ r16) << 4));
+        const v4i hi = *reinterpret_cast<const v4i*>(ring + slot * 4096 + r16 * 256 + (((c0 + 1) ^ r16) << 4));
+        const v8i aop = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[mb] = mfma_fp8_16(aop, breg[2 * st + s2][mb], acc[mb]);
+      }
+      // the slot is free once its operands are in registers: request the stage NSR ahead into it
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      if (st + NSR < NS) issue_stage(nt, st + NSR, slot, true);
+      else issue_stage(nt + 1, st + NSR - NS, slot, nt + 1 < nt1);
+    }
+
+    v4f tot = v4f{0.f, 0.f, 0.f, 0.f};
+    bool reducer = w < MB;
+    if (WK > 1) {
+      v4f* buf = red + (size_t)parity * WK * MB * 64;
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) buf[(w * MB + mb) * 64 + lane] = acc[mb];
+      // the partial tiles are written; the bare barrier leaves the next tile's weight requests in flight (a
+      // __syncthreads() would wait for every direct-to-LDS load)
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      if (reducer)
+        for (int ww = 0; ww < WK; ++ww) tot += buf[(ww * MB + w) * 64 + lane];
+      parity ^= 1;
+    } else {
+      reducer = true;
+    }
+    if (reducer) {
+      const int mb_lo = (WK > 1) ? w : 0, mb_hi = (WK > 1) ? w + 1 : MB;
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        if (mb < mb_lo || mb >= mb_hi) continue;
+        const v4f val = (WK > 1) ? tot : acc[mb];
+        const int m = mb * 16 + r16;
+        if (m < p.M) {
+#pragma clang fp contract(off)      // sa * (sb * acc), then + bias: two fp32 roundings, like the tile kernels
+          const int n = nt * 16 + q * 4;
+          float o[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            o[r] = sam_mb[mb] * (sb_r[r] * val[r]);
+            if (p.bias) o[r] += T::to_float(bias_r[r]);
+          }
+          v2u ov;
+          ov.x = (uint32_t)T::from_float(o[0]) | ((uint32_t)T::from_float(o[1]) << 16);
+          ov.y = (uint32_t)T::from_float(o[2]) | ((uint32_t)T::from_float(o[3]) << 16);
+          *reinterpret_cast<v2u*>(p.out + (int64_t)m * p.ldc + n) = ov;
+        }
+      }
+    }
+  }
+}
+
 // ----------------------------------------------------------------------------- host side
 
 // Overrides for tests and benchmarks come through tuning() (all zero = automatic): fp8_path 1 stream / 2 tile,
@@ -1068,6 +1223,62 @@ static bool dispatch_stream_split(const Fp8MMParams& p, int64_t c_tmp_bytes, int
   return true;
 }
 
+template <bool BF16_OUT, int KS, int MB, int NSR>
+static bool launch_stream2(const Fp8MMParams& p_in, int wk, int gx, hipStream_t s) {
+  Fp8MMParams p = p_in;
+  p.nt_base = (p.N / 16) / gx;
+  p.nt_rem = (p.N / 16) % gx;
+  p.a_extent = (uint32_t)((int64_t)(p.M - 1) * p.lda + p.K);
+  p.b_extent = (uint32_t)((int64_t)(p.N - 1) * p.ldb + p.K);
+  const size_t lds = (size_t)wk * NSR * 4096 + (wk > 1 ? (size_t)2 * wk * MB * 64 * sizeof(v4f) : 0);
+  auto kern = fp8_mm_stream2_kernel<BF16_OUT, KS, MB, NSR>;
+  static size_t reserved[VAQ_MAX_DEVICES];
+  if (reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "fp8_scaled_mm") != VAQ_OK) return false;      // (the kernel above then takes the problem)
+  hipLaunchKernelGGL(kern, dim3(gx), dim3(64, wk), lds, s, p, wk);
+  return true;
+}
+
+// Steps per wavefront of the stream kernel with the weights through LDS, 0 where the kernel above stays.  Measured with
+// cold weights against the kernel above (us, M = 1 / 4 / 16): 4096 x 6144 8.6 / 9.0 / 10.3 -> 7.7 / 7.8 / 8.6, 4096 x 4096
+// 6.0 / 6.2 / 7.1 -> 5.7 / 5.9 / 6.6, 4096 x 28672 25.8 / 26.1 / 27.8 -> 21.9 / 22.0 / 23.3, 14336 x 4096 13.8 / 14.8 / 18.0 ->
+// 12.0 / 12.4 / 15.3; two m-blocks (M = 32): 4096 x 6144 11.4 -> 10.5, 4096 x 28672 30.6 -> 26.5, 4096 x 4096 8.7 -> 8.9.
+// (development switch exp[4]: 1 / 2 / 3 force 8 / 4 / 16 steps, 9 switches the kernel off)
+static int stream2_steps_per_wave(const Fp8MMParams& p) {
+  const int sw = tuning().exp[4];
+  if (sw == 9 || p.M > 32 || p.K % 16 != 0 || !stream_offsets_fit(p)) return 0;
+  const int steps = (p.K + 127) / 128, MB = (p.M + 15) / 16;
+  int ks = 0;
+  if (sw >= 1 && sw <= 3) ks = sw == 1 ? 8 : (sw == 2 ? 4 : 16);
+  else if (MB == 1) ks = steps <= 64 ? 8 : (steps <= 128 ? 16 : 0);
+  else ks = (steps <= 32 && p.N / 16 > num_cus_current_device()) ? 4 : 0;
+  if (ks == 0 || (steps + ks - 1) / ks > 8 || (MB == 2 && ks == 16)) return 0;
+  return ks;
+}
+
+template <bool BF16_OUT>
+static bool dispatch_stream2(const Fp8MMParams& p, hipStream_t s) {
+  const int ks = stream2_steps_per_wave(p);
+  if (ks == 0) return false;
+  const int steps = (p.K + 127) / 128;
+  const int wk = (steps + ks - 1) / ks;
+  const int MB = (p.M + 15) / 16, NT = p.N / 16;
+  const int cus = num_cus_current_device();
+  const int rounds = (NT + cus - 1) / cus;
+  int gx = (NT + rounds - 1) / rounds;
+  // one m-block on a layer of many rounds: two workgroups per compute unit (4096 x 28672 at M = 1: 23.8 -> 21.9 us; three
+  // or more per unit 25.8 us and up)
+  if (MB == 1 && NT >= 4 * cus) gx = 2 * cus;
+  if (tuning().fp8_gx > 0) gx = tuning().fp8_gx;
+  if (gx > NT) gx = NT;
+  if (MB == 1) {
+    if (ks == 4) return launch_stream2<BF16_OUT, 4, 1, 2>(p, wk, gx, s);
+    if (ks == 8) return launch_stream2<BF16_OUT, 8, 1, 4>(p, wk, gx, s);
+    return launch_stream2<BF16_OUT, 16, 1, 4>(p, wk, gx, s);
+  }
+  if (ks == 4) return launch_stream2<BF16_OUT, 4, 2, 2>(p, wk, gx, s);
+  return launch_stream2<BF16_OUT, 8, 2, 4>(p, wk, gx, s);
+}
+
 template <bool BF16_OUT>
 static bool dispatch_stream(const Fp8MMParams& p, hipStream_t s) {
   const int steps = (p.K + 127) / 128;
@@ -1200,7 +1411,8 @@ extern "C" int vaq_fp8_scaled_mm_ws_tuned(const uint8_t* a, int64_t lda, const u
   const bool bf16 = out_dtype == VAQ_BF16;
   bool done = false;
   const bool want_stream = tuning().fp8_path != 2 && stream_steps_per_wave(size_m, size_n, size_k) != 0;
-  if (want_stream) done = bf16 ? dispatch_stream<true>(p, s) : dispatch_stream<false>(p, s);
+  if (tuning().fp8_path != 2) done = bf16 ? dispatch_stream2<true>(p, s) : dispatch_stream2<false>(p, s);
+  if (!done && want_stream) done = bf16 ? dispatch_stream<true>(p, s) : dispatch_stream<false>(p, s);
   if (!done && tuning().fp8_path != 2)
     done = bf16 ? dispatch_stream_split<true>(p, c_tmp_bytes, counter_ints, s)
                 : dispatch_stream_split<false>(p, c_tmp_bytes, counter_ints, s);
