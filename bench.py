@@ -293,13 +293,14 @@ def fused_norm_quant_section(dev):
 
 def variants_section(dev):
     """The other weight formats of the W4A16 GEMM -- groups of 64 / 32 rows, channelwise scales, 8-bit codes
-    (uint8b128) -- on gate_up_proj (4096 x 28672) at a decode size (cold weights, several copies cycling) and at
+    (uint8b128), FP8 e4m3 weights with 16-bit activations -- on gate_up_proj (4096 x 28672) at a decode size (cold weights, several copies cycling) and at
     M = 4096.  Bytes count weights, scales and zero points of the format."""
     from vllm_amd.scalar_type import scalar_types
     rows = []
     gen = torch.Generator(device=dev).manual_seed(7)
     k, n = 4096, 28672
-    for name, gs, bits in (("g128", 128, 4), ("g64", 64, 4), ("g32", 32, 4), ("channelwise", -1, 4), ("8bit_g128", 128, 8)):
+    for name, gs, bits in (("g128", 128, 4), ("g64", 64, 4), ("g32", 32, 4), ("channelwise", -1, 4), ("8bit_g128", 128, 8),
+                           ("fp8_weights_channelwise", -1, 8)):
         grp = 1 if gs == -1 else k // gs
         copies = 6
         layers = []
@@ -308,6 +309,10 @@ def variants_section(dev):
             if bits == 8:
                 l.w = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 16, 4 * n), dtype=torch.int32, device=dev, generator=gen)
                 l.wtype = scalar_types.uint8b128
+                if name.startswith("fp8"):
+                    # e4m3 bytes in the byte-native order: any byte but the two NaN codes (0x7f, 0xff -> clear bit 0)
+                    l.w &= ~0x01010101
+                    l.wtype = scalar_types.float8_e4m3fn
             l.s = (torch.randn(grp, n, device=dev, generator=gen).abs() * 0.01 + 1e-3).to(torch.bfloat16)
             layers.append(l)
         wbytes = k * n * bits // 8 + grp * n * 2
