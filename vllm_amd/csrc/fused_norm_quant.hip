@@ -17,7 +17,7 @@
 // per-tensor scale:  q = cvt(clamp(y * (1/scale), +-448)).
 //
 // HBM-bound: one workgroup per token; the row (and the residual sum) stays in registers between the three passes when
-// it has at most 256 x 8 x 8 = 16384 elements and is 16-byte aligned; other rows re-read global memory.
+// it has at most 512 x 8 x 8 = 32768 elements and is 16-byte aligned; other rows re-read global memory.
 #include "vaq_common.h"
 
 #include <type_traits>
@@ -27,7 +27,7 @@ namespace vaq {
 namespace {
 
 constexpr float NQ_FP8_MAX = 448.0f;
-constexpr int NQ_T = 256;
+constexpr int NQ_T = 512;
 // Chunks of 8 elements per thread that the row-in-registers path holds (template parameter NV): 2, 4 or 8, the smallest
 // that covers the row -- the register arrays are sized by it, and with them the number of rows a compute unit works on
 // at a time.
