@@ -87,11 +87,13 @@ def test_per_token_quant_strided_rows_and_padding(device):
     assert np.array_equal(_codes(q[:9]), _codes(q_ref)) and np.array_equal(s[:9].cpu().numpy(), s_ref.numpy())
 
 
-@pytest.mark.parametrize("hidden,tokens", [(8, 515), (1000, 601), (1024, 4096), (1032, 2051), (2048, 2050)])
+@pytest.mark.parametrize("hidden,tokens", [(8, 515), (1000, 601), (1024, 4096), (1032, 2051), (2048, 2050),
+                                           (4096, 2049), (5128, 2050), (8192, 2048), (2056, 4097)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_per_token_quant_many_short_rows_bit_exact(device, hidden, tokens, dtype):
-    """Large batches of short rows take the kernel that keeps one row per wavefront (no barrier); ragged row lengths,
-    a row count that does not fill the last workgroup, strided rows, scale_ub.  Scales and codes bit-exact."""
+    """Large batches of short rows take the kernel that keeps one row per wavefront (no barrier), longer rows in large
+    batches the one with a workgroup per row; ragged row lengths, a row count that does not fill the last workgroup,
+    strided rows, scale_ub.  Scales and codes bit-exact."""
     import vllm_amd._custom_ops as ops
     g = torch.Generator().manual_seed(hidden + tokens)
     big = (torch.randn(tokens, hidden + 16, generator=g) * 3).to(dtype)
