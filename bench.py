@@ -354,6 +354,36 @@ def variants_section(dev):
     return rows
 
 
+def host_overhead_section(dev):
+    """Host time per eager call of the ops (Python checks + ctypes + workspace query + launch), M = 1 on 4096 x 4096: what a
+    caller pays per GEMM outside a HIP graph.  The queue is kept short enough that the host, not the device, is timed."""
+    import vllm_amd._custom_ops as ops
+    gen = torch.Generator(device=dev).manual_seed(9)
+    k = n = 4096
+    layer = W4Layer(k, n, dev, gen)
+    a = torch.randn(1, k, device=dev, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(n, k, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+    wq, wsc = ops.scaled_fp8_quant(w, use_per_token_if_dynamic=True)
+    aq, sa = ops.scaled_fp8_quant(a, use_per_token_if_dynamic=True)
+    calls = (("gptq_marlin_gemm", lambda: layer(a)),
+             ("cutlass_scaled_mm", lambda: ops.cutlass_scaled_mm(aq, wq.t(), sa, wsc, torch.bfloat16)),
+             ("scaled_fp8_quant", lambda: ops.scaled_fp8_quant(a, use_per_token_if_dynamic=True)))
+    rows = []
+    for name, fn in calls:
+        for _ in range(50):
+            fn()
+        torch.cuda.synchronize()
+        n_calls = 1000
+        t0 = time.perf_counter()
+        for _ in range(n_calls):
+            fn()
+        t = (time.perf_counter() - t0) / n_calls
+        torch.cuda.synchronize()
+        rows.append(dict(kind="eager_host_time_per_call", op=name, us=t * 1e6))
+        log(f"[host overhead] {name:18s}: {t * 1e6:6.1f} us of host time per eager call")
+    return rows
+
+
 def vendor_ceiling_section(dev):
     """Practical ceilings on the same box and shapes: the vendor GEMM library through torch (bf16 `matmul`, row-wise
     scaled FP8 `_scaled_mm`) at M = 4096.  Context for the MFMA fractions above, not part of the product path."""
@@ -675,6 +705,7 @@ def main():
         for name, fn in (("prefill", prefill_section), ("fp8", fp8_section), ("fused_norm_quant", fused_norm_quant_section),
                          ("variants", variants_section),
                          ("vendor_ceiling", vendor_ceiling_section),
+                         ("host_overhead", host_overhead_section),
                          ("decode_step", decode_step_section)):
             if args.sections and name not in args.sections.split(","):
                 continue

@@ -26,16 +26,24 @@ GPTQ_MARLIN_MIN_THREAD_K = 128
 _LAYOUTS = {"marlin": _lib.VAQ_LAYOUT_MARLIN, "native": _lib.VAQ_LAYOUT_NATIVE, "native_bytes": _lib.VAQ_LAYOUT_NATIVE_BYTES}
 
 
-def _check(cond: bool, msg: str) -> None:
+def _check(cond: bool, msg) -> None:
+    """``msg`` is a string, or a callable that builds one: formatted messages cost more than the test they belong to, so
+    they are only built on failure."""
     if not cond:
-        raise RuntimeError(msg)
+        raise RuntimeError(msg() if callable(msg) else msg)
 
 
 def _ptr(t: torch.Tensor | None):
     return None if t is None else ctypes.c_void_p(t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(device: torch.device):
+    """The hipStream_t that torch currently launches on for ``device``."""
+    if _raw_stream is not None and device.index is not None:
+        return ctypes.c_void_p(_raw_stream(device.index))
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
@@ -57,22 +65,22 @@ def _is_gpu(t: torch.Tensor) -> bool:
 
 def _check_repack_args(b_q_weight, perm, size_k, size_n, num_bits) -> None:
     """Host checks of gptq_marlin_repack.cu:255-280, same order."""
-    _check(size_k % GPTQ_MARLIN_TILE == 0, f"size_k = {size_k} is not divisible by tile_k_size = {GPTQ_MARLIN_TILE}")
+    _check(size_k % GPTQ_MARLIN_TILE == 0, lambda: f"size_k = {size_k} is not divisible by tile_k_size = {GPTQ_MARLIN_TILE}")
     _check(size_n % GPTQ_MARLIN_MIN_THREAD_N == 0,
-           f"size_n = {size_n} is not divisible by tile_n_size = {GPTQ_MARLIN_MIN_THREAD_N}")
-    _check(num_bits in (4, 8), f"num_bits must be 4 or 8. Got = {num_bits}")
+           lambda: f"size_n = {size_n} is not divisible by tile_n_size = {GPTQ_MARLIN_MIN_THREAD_N}")
+    _check(num_bits in (4, 8), lambda: f"num_bits must be 4 or 8. Got = {num_bits}")
     pack_factor = 32 // num_bits
     _check(b_q_weight.dim() == 2 and size_k // pack_factor == b_q_weight.size(0),
-           f"Shape mismatch: b_q_weight.size(0) = {b_q_weight.size(0) if b_q_weight.dim() else None}, "
+           lambda: f"Shape mismatch: b_q_weight.size(0) = {b_q_weight.size(0) if b_q_weight.dim() else None}, "
            f"size_k = {size_k}, pack_factor = {pack_factor}")
-    _check(b_q_weight.size(1) == size_n, f"b_q_weight.size(1) = {b_q_weight.size(1)} is not size_n = {size_n}")
+    _check(b_q_weight.size(1) == size_n, lambda: f"b_q_weight.size(1) = {b_q_weight.size(1)} is not size_n = {size_n}")
     _check(_is_gpu(b_q_weight), "b_q_weight is not on GPU")
     _check(b_q_weight.is_contiguous(), "b_q_weight is not contiguous")
     _check(b_q_weight.dtype == torch.int32, "b_q_weight type is not kInt")
     _check(_is_gpu(perm), "perm is not on GPU")
     _check(perm.is_contiguous(), "perm is not contiguous")
     _check(perm.dtype == torch.int32, "perm type is not at::kInt")
-    _check(perm.numel() in (0, size_k), f"perm.numel() = {perm.numel()} must be 0 or size_k = {size_k}")
+    _check(perm.numel() in (0, size_k), lambda: f"perm.numel() = {perm.numel()} must be 0 or size_k = {size_k}")
 
 
 def _repack_impl(b_q_weight: torch.Tensor, perm: torch.Tensor, size_k: int, size_n: int, num_bits: int,
@@ -96,15 +104,15 @@ def _repack_fake(b_q_weight, perm, size_k, size_n, num_bits, layout=1):
 
 def _check_awq_repack_args(b_q_weight: torch.Tensor, size_k: int, size_n: int, num_bits: int) -> None:
     """Host checks of awq_marlin_repack.cu:208-232 in the same order."""
-    _check(size_k % GPTQ_MARLIN_TILE == 0, f"size_k = {size_k} is not divisible by tile_k_size = {GPTQ_MARLIN_TILE}")
+    _check(size_k % GPTQ_MARLIN_TILE == 0, lambda: f"size_k = {size_k} is not divisible by tile_k_size = {GPTQ_MARLIN_TILE}")
     _check(size_n % GPTQ_MARLIN_MIN_THREAD_N == 0,
-           f"size_n = {size_n} is not divisible by tile_n_size = {GPTQ_MARLIN_MIN_THREAD_N}")
-    _check(num_bits in (4, 8), f"num_bits must be 4 or 8. Got = {num_bits}")
+           lambda: f"size_n = {size_n} is not divisible by tile_n_size = {GPTQ_MARLIN_MIN_THREAD_N}")
+    _check(num_bits in (4, 8), lambda: f"num_bits must be 4 or 8. Got = {num_bits}")
     pack_factor = 32 // num_bits
     _check(b_q_weight.dim() == 2 and b_q_weight.size(0) == size_k,
-           f"b_q_weight.size(0) = {b_q_weight.size(0) if b_q_weight.dim() else None} is not size_k = {size_k}")
+           lambda: f"b_q_weight.size(0) = {b_q_weight.size(0) if b_q_weight.dim() else None} is not size_k = {size_k}")
     _check(size_n // pack_factor == b_q_weight.size(1),
-           f"Shape mismatch: b_q_weight.size(1) = {b_q_weight.size(1)}, size_n = {size_n}, pack_factor = {pack_factor}")
+           lambda: f"Shape mismatch: b_q_weight.size(1) = {b_q_weight.size(1)}, size_n = {size_n}, pack_factor = {pack_factor}")
     _check(_is_gpu(b_q_weight), "b_q_weight is not on GPU")
     _check(b_q_weight.is_contiguous(), "b_q_weight is not contiguous")
     _check(b_q_weight.dtype == torch.int32, "b_q_weight type is not kInt")
@@ -144,17 +152,17 @@ def _check_gemm_args(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, 
                      size_m, size_n, size_k, is_k_full, is_zp_float):
     """Host checks of gptq_marlin.cu:689-902 in the same order.  Returns (group_size, has_act_order, has_zp, wtype)."""
     b_q_type = ScalarType.from_id(b_q_type_id)
-    _check(b_q_type.size_bits in (4, 8), f"unsupported weight type {b_q_type}")
+    _check(b_q_type.size_bits in (4, 8), lambda: f"unsupported weight type {b_q_type}")
     pack_factor = 32 // b_q_type.size_bits
-    _check(a.dim() == 2 and a.size(0) == size_m, f"Shape mismatch: a.size(0) = {a.size(0)}, size_m = {size_m}")
-    _check(a.size(1) == size_k, f"Shape mismatch: a.size(1) = {a.size(1)}, size_k = {size_k}")
-    _check(size_k % GPTQ_MARLIN_TILE == 0, f"size_k = {size_k} is not divisible by tile_size = {GPTQ_MARLIN_TILE}")
+    _check(a.dim() == 2 and a.size(0) == size_m, lambda: f"Shape mismatch: a.size(0) = {a.size(0)}, size_m = {size_m}")
+    _check(a.size(1) == size_k, lambda: f"Shape mismatch: a.size(1) = {a.size(1)}, size_k = {size_k}")
+    _check(size_k % GPTQ_MARLIN_TILE == 0, lambda: f"size_k = {size_k} is not divisible by tile_size = {GPTQ_MARLIN_TILE}")
     _check(b_q_weight.dim() == 2 and size_k // GPTQ_MARLIN_TILE == b_q_weight.size(0),
-           f"Shape mismatch: b_q_weight.size(0) = {b_q_weight.size(0)}, size_k = {size_k}, tile_size = {GPTQ_MARLIN_TILE}")
+           lambda: f"Shape mismatch: b_q_weight.size(0) = {b_q_weight.size(0)}, size_k = {size_k}, tile_size = {GPTQ_MARLIN_TILE}")
     _check(b_q_weight.size(1) % GPTQ_MARLIN_TILE == 0,
-           f"b_q_weight.size(1) = {b_q_weight.size(1)} is not divisible by tile_size = {GPTQ_MARLIN_TILE}")
+           lambda: f"b_q_weight.size(1) = {b_q_weight.size(1)} is not divisible by tile_size = {GPTQ_MARLIN_TILE}")
     actual_size_n = (b_q_weight.size(1) // GPTQ_MARLIN_TILE) * pack_factor
-    _check(size_n == actual_size_n, f"size_n = {size_n}, actual_size_n = {actual_size_n}")
+    _check(size_n == actual_size_n, lambda: f"size_n = {size_n}, actual_size_n = {actual_size_n}")
     _check(_is_gpu(a), "A is not on GPU")
     _check(a.stride(1) == 1, "A.stride(1) is not 1")
     _check(a.stride(0) % 8 == 0, "A.stride(0) must divisible by 8")
@@ -166,10 +174,10 @@ def _check_gemm_args(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, 
     if c is not None:
         _check(_is_gpu(c), "c is not on GPU")
         _check(c.is_contiguous(), "c is not contiguous")
-        _check(c.size(0) == size_m, f"Shape mismatch: c.size(0) = {c.size(0)}, size_m = {size_m}")
-        _check(c.size(1) == size_n, f"Shape mismatch: c.size(1) = {c.size(1)}, size_n = {size_n}")
-    _check(b_scales.dim() == 2, f"b_scales rank = {b_scales.dim()} is not 2")
-    _check(b_scales.size(1) == size_n, f"b_scales dim 1 = {b_scales.size(1)} is not size_n = {size_n}")
+        _check(c.size(0) == size_m, lambda: f"Shape mismatch: c.size(0) = {c.size(0)}, size_m = {size_m}")
+        _check(c.size(1) == size_n, lambda: f"Shape mismatch: c.size(1) = {c.size(1)}, size_n = {size_n}")
+    _check(b_scales.dim() == 2, lambda: f"b_scales rank = {b_scales.dim()} is not 2")
+    _check(b_scales.size(1) == size_n, lambda: f"b_scales dim 1 = {b_scales.size(1)} is not size_n = {size_n}")
     num_groups = b_scales.size(0)
 
     has_act_order = False
@@ -179,17 +187,17 @@ def _check_gemm_args(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, 
         _check(_is_gpu(perm), "perm is not on GPU")
         _check(perm.is_contiguous(), "perm is not contiguous")
         _check((g_idx.size(-1) == 0 and perm.size(-1) == 0) or (g_idx.size(-1) == size_k and perm.size(-1) == size_k),
-               f"Unexpected g_idx.size(-1) = {g_idx.size(-1)} and perm.size(-1) = {perm.size(-1)}, where size_k = {size_k}")
+               lambda: f"Unexpected g_idx.size(-1) = {g_idx.size(-1)} and perm.size(-1) = {perm.size(-1)}, where size_k = {size_k}")
         has_act_order = g_idx.size(-1) > 0 and perm.size(-1) > 0
     if has_act_order:
         if is_k_full:
             _check(num_groups > 1, "For act_order, num_groups must be > 1")
-            _check(size_k % num_groups == 0, f"size_k = {size_k}, is not divisible by num_groups = {num_groups}")
+            _check(size_k % num_groups == 0, lambda: f"size_k = {size_k}, is not divisible by num_groups = {num_groups}")
             group_size = size_k // num_groups
         else:
             group_size = 0
     elif num_groups > 1:
-        _check(size_k % num_groups == 0, f"size_k = {size_k}, is not divisible by b_scales.size(0) = {b_scales.size(0)}")
+        _check(size_k % num_groups == 0, lambda: f"size_k = {size_k}, is not divisible by b_scales.size(0) = {b_scales.size(0)}")
         group_size = size_k // num_groups
     else:
         group_size = -1
@@ -206,27 +214,27 @@ def _check_gemm_args(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, 
         _check(b_zeros.is_contiguous(), "b_zeros is not contiguous")
     if has_zp:
         _check(b_q_type in (scalar_types.uint4, scalar_types.uint8),
-               f"b_q_type must be u4 or u8 when has_zp = True. Got = {b_q_type}")
+               lambda: f"b_q_type must be u4 or u8 when has_zp = True. Got = {b_q_type}")
     else:
         _check(b_q_type in (scalar_types.uint4b8, scalar_types.uint8b128, scalar_types.float8_e4m3fn),
-               "b_q_type must be uint4b8, uint8b128, float8_e4m3fn or float4_e2m1f when has_zp = False. "
+               lambda: "b_q_type must be uint4b8, uint8b128, float8_e4m3fn or float4_e2m1f when has_zp = False. "
                f"Got = {b_q_type}")
     if has_zp and is_zp_float:
         _check(a.dtype == torch.float16, "Computation type must be float16 (half) when using float zero points.")
     if has_zp:
-        _check(b_zeros.dim() == 2, f"b_zeros rank = {b_zeros.dim()} is not 2")
+        _check(b_zeros.dim() == 2, lambda: f"b_zeros rank = {b_zeros.dim()} is not 2")
         if is_zp_float:
-            _check(b_zeros.size(1) == size_n, f"b_zeros dim 1 = {b_zeros.size(1)} is not size_n = {size_n}")
-            _check(num_groups == b_zeros.size(0), f"b_zeros dim 0 = {b_zeros.size(0)} is not num_groups = {num_groups}")
+            _check(b_zeros.size(1) == size_n, lambda: f"b_zeros dim 1 = {b_zeros.size(1)} is not size_n = {size_n}")
+            _check(num_groups == b_zeros.size(0), lambda: f"b_zeros dim 0 = {b_zeros.size(0)} is not num_groups = {num_groups}")
         else:
-            _check(b_zeros.size(0) == num_groups, f"b_zeros dim 0 = {b_zeros.size(0)} is not num_groups = {num_groups}")
+            _check(b_zeros.size(0) == num_groups, lambda: f"b_zeros dim 0 = {b_zeros.size(0)} is not num_groups = {num_groups}")
             _check(b_zeros.size(1) == size_n // pack_factor,
-                   f"b_zeros dim 1 = {b_zeros.size(1)} is not size_n / pack_factor = {size_n // pack_factor}")
+                   lambda: f"b_zeros dim 1 = {b_zeros.size(1)} is not size_n / pack_factor = {size_n // pack_factor}")
     _check(size_n % GPTQ_MARLIN_MIN_THREAD_N == 0,
-           f"size_n = {size_n}, is not divisible by min_thread_n = {GPTQ_MARLIN_MIN_THREAD_N}")
+           lambda: f"size_n = {size_n}, is not divisible by min_thread_n = {GPTQ_MARLIN_MIN_THREAD_N}")
     _check(_is_gpu(workspace) and workspace.dtype == torch.int32, "workspace must be an int32 tensor on GPU")
     _check(a.dtype in (torch.float16, torch.bfloat16), "gpt_marlin_gemm only supports bfloat16 and float16")
-    _check(b_scales.dtype == a.dtype, f"b_scales dtype {b_scales.dtype} must equal the activation dtype {a.dtype}")
+    _check(b_scales.dtype == a.dtype, lambda: f"b_scales dtype {b_scales.dtype} must equal the activation dtype {a.dtype}")
 
     # what this build implements out of everything the reference accepts
     if b_q_type not in (scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8b128, scalar_types.float8_e4m3fn):
@@ -244,7 +252,7 @@ def _check_gemm_args(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, 
             raise NotImplementedError(f"gptq_marlin_gemm: group_size = {group_size} is not built for gfx950 "
                                       "(only -1, 32, 64, 128)")
     _check(size_k % GPTQ_MARLIN_MIN_THREAD_K == 0,
-           f"size_k = {size_k}, is not divisible by min_thread_k = {GPTQ_MARLIN_MIN_THREAD_K}")
+           lambda: f"size_k = {size_k}, is not divisible by min_thread_k = {GPTQ_MARLIN_MIN_THREAD_K}")
     if b_q_type == scalar_types.float8_e4m3fn:
         # weight-only FP8 (marlin_utils_fp8.py): channelwise scales or groups of 128 rows, no act_order
         if group_size not in (-1, 128) or has_act_order:
@@ -326,8 +334,8 @@ def _check_quant_io(result: torch.Tensor, input: torch.Tensor) -> tuple[int, int
     _check(_is_gpu(input) and _is_gpu(result), "input and result must be on GPU")
     _check(input.dim() >= 1 and input.stride(-1) == 1, "last dimension of input must be contiguous")
     _check(result.stride(-1) == 1, "last dimension of output must be contiguous")
-    _check(result.dtype == FP8_DTYPE, f"result must be {FP8_DTYPE}")
-    _check(input.dtype in (torch.float16, torch.bfloat16, torch.float32), f"unsupported input dtype {input.dtype}")
+    _check(result.dtype == FP8_DTYPE, lambda: f"result must be {FP8_DTYPE}")
+    _check(input.dtype in (torch.float16, torch.bfloat16, torch.float32), lambda: f"unsupported input dtype {input.dtype}")
     _check(input.dim() == 2 and result.dim() == 2, "input and result must be 2-D")
     hidden = input.size(-1)
     tokens = input.numel() // hidden if hidden else 0
@@ -381,7 +389,7 @@ def _check_scaled_mm_args(out, a, b, a_scales, b_scales, bias) -> None:
     """scaled_mm_entry.cu:179-193 plus the scale-shape rules of c3x/scaled_mm_helper.hpp:5-52."""
     _check(a.dim() == 2 and b.dim() == 2 and out.dim() == 2, "a, b and out must be 2-D")
     _check(out.size(0) == a.size(0) and a.size(1) == b.size(0) and b.size(1) == out.size(1),
-           f"shape mismatch: a {tuple(a.shape)}, b {tuple(b.shape)}, out {tuple(out.shape)}")
+           lambda: f"shape mismatch: a {tuple(a.shape)}, b {tuple(b.shape)}, out {tuple(out.shape)}")
     _check(a.stride(1) == 1 and out.stride(1) == 1, "a and out must be row-major")
     _check(b.stride(0) == 1, "b must be column-major")
     _check(out.stride(0) % 16 == 0 and b.stride(1) % 16 == 0, "out.stride(0) and b.stride(1) must be multiples of 16")
@@ -391,8 +399,8 @@ def _check_scaled_mm_args(out, a, b, a_scales, b_scales, bias) -> None:
     _check(all(_is_gpu(t) for t in (out, a, b, a_scales, b_scales)), "all tensors must be on GPU")
     _check(a_scales.dtype == torch.float32 and b_scales.dtype == torch.float32, "scales must be fp32")
     _check(a_scales.is_contiguous() and b_scales.is_contiguous(), "scales must be contiguous")
-    _check(a_scales.numel() in (1, a.size(0)), f"a_scales.numel() = {a_scales.numel()} must be 1 or M = {a.size(0)}")
-    _check(b_scales.numel() in (1, b.size(1)), f"b_scales.numel() = {b_scales.numel()} must be 1 or N = {b.size(1)}")
+    _check(a_scales.numel() in (1, a.size(0)), lambda: f"a_scales.numel() = {a_scales.numel()} must be 1 or M = {a.size(0)}")
+    _check(b_scales.numel() in (1, b.size(1)), lambda: f"b_scales.numel() = {b_scales.numel()} must be 1 or N = {b.size(1)}")
     _check(out.dtype in (torch.float16, torch.bfloat16), "out must be float16 or bfloat16")
     if a.dtype != FP8_DTYPE or b.dtype != FP8_DTYPE:
         raise NotImplementedError(f"cutlass_scaled_mm: only {FP8_DTYPE} x {FP8_DTYPE} is built for gfx950 "
@@ -489,7 +497,7 @@ def _rms_norm_static_common(who, result, input, residual, weight, scale, epsilon
     _check(_is_gpu(input) and _is_gpu(result) and _is_gpu(weight) and _is_gpu(scale), "tensors must be on GPU")
     if result.dtype != FP8_DTYPE:
         raise NotImplementedError(f"{who}: only {FP8_DTYPE} output is built for gfx950 (got {result.dtype})")
-    _check(input.dtype in (torch.float16, torch.bfloat16), f"{who}: input must be float16 or bfloat16")
+    _check(input.dtype in (torch.float16, torch.bfloat16), lambda: f"{who}: input must be float16 or bfloat16")
     _check(weight.dtype == input.dtype, "weight.dtype must equal input.dtype")
     _check(scale.dtype == torch.float32 and scale.numel() == 1, "scale must be a float32 scalar")
     _check(result.is_contiguous(), "out must be contiguous")
@@ -523,7 +531,7 @@ def _fused_add_rms_norm_static_impl(result, input, residual, weight, scale, epsi
 def _silu_and_mul_quant_impl(result: torch.Tensor, input: torch.Tensor, scale: torch.Tensor) -> None:
     """Host checks of activation_kernels.cu:560-568."""
     _check(_is_gpu(input) and _is_gpu(result) and _is_gpu(scale), "tensors must be on GPU")
-    _check(result.dtype == FP8_DTYPE, f"silu_and_mul_quant: out must be {FP8_DTYPE}")
+    _check(result.dtype == FP8_DTYPE, lambda: f"silu_and_mul_quant: out must be {FP8_DTYPE}")
     _check(input.dtype in (torch.float16, torch.bfloat16), "silu_and_mul_quant: input must be float16 or bfloat16")
     _check(input.size(-1) % 2 == 0, "silu_and_mul_quant: the last dimension of input must be even")
     _check(scale.dtype == torch.float32 and scale.numel() == 1, "scale must be a float32 scalar")
