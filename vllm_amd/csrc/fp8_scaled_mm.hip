@@ -640,21 +640,37 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
     if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     old = __builtin_amdgcn_readfirstlane(old);      // lane 0 holds it; a scalar keeps what depends on it scalar
     if (old != p.SK - 1) return;
+    // CH pieces of two splits in flight at a time (one piece after the other, every load waited for, the last arriver
+    // spent NV4 x SK memory round trips here); each element is still summed in split order, starting from zero
+    constexpr int CH = NV4 < 8 ? NV4 : 8;
 #pragma unroll
-    for (int i = 0; i < WMB; ++i)
+    for (int c0 = 0; c0 < NV4; c0 += CH) {
+      v4f sum[CH];
 #pragma unroll
-      for (int j = 0; j < WNB; ++j)
+      for (int c = 0; c < CH; ++c) sum[c] = v4f{0.f, 0.f, 0.f, 0.f};
+      for (int s0 = 0; s0 < p.SK; s0 += 2) {
+        const int s1 = s0 + 1 < p.SK ? s0 + 1 : s0;
+        v4u r0[CH], r1[CH];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          v4f sum = {0.f, 0.f, 0.f, 0.f};
-          for (int s2 = 0; s2 < p.SK; ++s2) {             // fixed order: deterministic
-            const v4u r = __builtin_amdgcn_raw_buffer_load_b128(
-                rt, lane * 16, (int)(s2 * split_stride + unit + ((i * WNB + j) * 4 + q) * 1024), SC1);
-            sum += __builtin_bit_cast(v4f, r);
-          }
+        for (int c = 0; c < CH; ++c)
+          r0[c] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s0 * split_stride + unit + (c0 + c) * 1024), SC1);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = sum[e];
+        for (int c = 0; c < CH; ++c)
+          r1[c] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s1 * split_stride + unit + (c0 + c) * 1024), SC1);
+#pragma unroll
+        for (int c = 0; c < CH; ++c) sum[c] += __builtin_bit_cast(v4f, r0[c]);
+        if (s0 + 1 < p.SK) {
+#pragma unroll
+          for (int c = 0; c < CH; ++c) sum[c] += __builtin_bit_cast(v4f, r1[c]);
         }
+      }
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const int pc = c0 + c, ij = pc / 4, q = pc % 4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[ij / WNB][ij % WNB][4 * q + e] = sum[c][e];
+      }
+    }
     if (lane == 0) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
@@ -1059,11 +1075,8 @@ struct Fp8TilePlan {
   int64_t tiles;
 };
 
-// Tile shape and K split of the multi-stage kernel.  K is split when the output tiles alone leave compute units idle:
-// as many workgroups as fit the device at once (one or two per compute unit), at most 8 splits, each at least 64 steps
-// (4096 bytes of K) long, 32 steps when the tiles leave three quarters of the device idle -- measured with cold weights:
-// 14336 x 4096 at M = 48 / 128 47.7 -> 34.7 / 35.5 us with 4 splits, 4096 x 4096 at M = 48 .. 128 24.4 -> 20.6 us with
-// 2; with more tiles the shorter parts lose (14336 x 4096 at M = 256: 4 splits 50.5 us, 2 splits 48.7 us).
+// Tile shape and K split of the multi-stage kernel.  K is split when the output tiles alone leave compute units idle,
+// at most 8 ways; the rules for large and small tiles are below, each measured with cold weights.
 static Fp8TilePlan plan_tile3(int M, int N, int K) {
   const int cus = num_cus_current_device();
   auto tiles = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
@@ -1091,14 +1104,30 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   pl.tiles = tiles(pl.bm, pl.bn);
   int sk = 1;
   const int steps = K / 64;
-  if (pl.tiles < cus) {
-    const int per_cu = pl.bm * pl.bn >= 128 * 256 ? 1 : 2;      // workgroups of this tile shape that share a compute unit
+  if (pl.tiles < cus && pl.bm * pl.bn >= 128 * 256) {
+    // large tiles, one workgroup per compute unit
     const int min_steps = pl.tiles * 4 <= cus ? 32 : 64;        // shorter parts only when the tiles leave 3/4 of the device idle
-    sk = (int)((per_cu * (int64_t)cus) / pl.tiles);
+    sk = (int)((int64_t)cus / pl.tiles);
     if (sk > 8) sk = 8;
     if (sk > steps / min_steps) sk = steps / min_steps;
     if (sk < 1) sk = 1;
     while (sk & (sk - 1)) --sk;       // a power of two (3 splits measured slower than 2)
+  } else if (pl.tiles < cus) {
+    // Small tiles (two workgroups share a compute unit), measured with cold weights on the Llama shapes, M = 48 .. 512:
+    // tiles that leave 3/4 of the device idle are split until there is about one workgroup per compute unit (parts of
+    // at least 16 steps: 4096 x 4096 at M = 128, 4 parts of 16 steps 15.7 us, 2 of 32 18.4 us, 8 of 8 22.7 us); fuller
+    // devices stay unsplit (the rotated K loop of the unsplit kernel is worth more there: 4096 x 6144 at M = 192,
+    // 20.8 against 31.0 us in 2 parts; 96 tiles in 2 parts: -3 % on 4096 x 6144, +6 % on 4096 x 4096) unless K is very
+    // long, where a part is halved while the halves stay 50 steps long and the workgroups fit the device at once
+    // (14336 x 4096 at M = 256: 62.6 / 45.8 / 44.3 us in 1 / 2 / 4 parts).
+    if (pl.tiles * 4 <= (int64_t)cus) {
+      sk = (int)((int64_t)cus / pl.tiles);
+      if (sk > 8) sk = 8;
+      if (sk > steps / 16) sk = steps / 16;
+      if (sk < 1) sk = 1;
+      while (sk & (sk - 1)) --sk;
+    }
+    while (sk < 8 && steps / sk >= 100 && pl.tiles * sk * 2 <= 2 * (int64_t)cus) sk *= 2;
   }
   if (tuning().fp8_split > 0) sk = tuning().fp8_split <= steps ? tuning().fp8_split : steps;
   while (sk > 1 && (uint64_t)sk * (uint64_t)pl.tiles * pl.bm * pl.bn * 4 >= (1ull << 32)) --sk;   // 32-bit buffer offsets

@@ -817,21 +817,37 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
     if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     old = __builtin_amdgcn_readfirstlane(old);      // lane 0 holds it; a scalar keeps what depends on it scalar
     if (old != p.SK - 1) return;
+    // CH pieces of two splits in flight at a time (one piece after the other, every load waited for, the last arriver
+    // spent NV4 x SK memory round trips here); each element is still summed in split order, starting from zero
+    constexpr int CH = NV4 < 8 ? NV4 : 8;
 #pragma unroll
-    for (int i = 0; i < WMB; ++i)
+    for (int c0 = 0; c0 < NV4; c0 += CH) {
+      v4f sum[CH];
 #pragma unroll
-      for (int j = 0; j < WNB; ++j)
+      for (int c = 0; c < CH; ++c) sum[c] = v4f{0.f, 0.f, 0.f, 0.f};
+      for (int s0 = 0; s0 < p.SK; s0 += 2) {
+        const int s1 = s0 + 1 < p.SK ? s0 + 1 : s0;
+        v4u r0[CH], r1[CH];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          v4f sum = {0.f, 0.f, 0.f, 0.f};
-          for (int s2 = 0; s2 < p.SK; ++s2) {             // fixed order: deterministic
-            const v4u r = __builtin_amdgcn_raw_buffer_load_b128(
-                rt, lane * 16, (int)(s2 * split_stride + unit + ((i * WNB + j) * 4 + q) * 1024), SC1);
-            sum += __builtin_bit_cast(v4f, r);
-          }
+        for (int c = 0; c < CH; ++c)
+          r0[c] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s0 * split_stride + unit + (c0 + c) * 1024), SC1);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = sum[e];
+        for (int c = 0; c < CH; ++c)
+          r1[c] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s1 * split_stride + unit + (c0 + c) * 1024), SC1);
+#pragma unroll
+        for (int c = 0; c < CH; ++c) sum[c] += __builtin_bit_cast(v4f, r0[c]);
+        if (s0 + 1 < p.SK) {
+#pragma unroll
+          for (int c = 0; c < CH; ++c) sum[c] += __builtin_bit_cast(v4f, r1[c]);
         }
+      }
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const int pc = c0 + c, ij = pc / 4, q = pc % 4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[ij / WNB][ij % WNB][4 * q + e] = sum[c][e];
+      }
+    }
     if (lane == 0) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
