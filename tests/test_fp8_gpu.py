@@ -395,7 +395,7 @@ def test_scaled_mm_into_a_view_of_a_wider_buffer(device, offset):
         assert bool((got[:, :offset] == 7).all()) and bool((got[:, offset + n:] == 7).all()), "wrote outside the view"
 
 
-@pytest.mark.parametrize("cfg", [1, 8, 3, 4, 7, 13, 23, 14, 24, 17])
+@pytest.mark.parametrize("cfg", [1, 8, 3, 4, 5, 7, 13, 23, 14, 24, 15, 17])
 def test_scaled_mm_every_tile_shape_exact(device, cfg):
     """Every shape of the multi-stage tile kernel, forced through a per-call tuning override (the automatic choice only reaches
     some of them at any one problem size), including the ones that take two k-slices per step: small-integer operands

@@ -1089,14 +1089,24 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   // 4096 x 4096 at M = 2048 in two parts: 45 -> 66 us)
   const int parts128 = K / 64 >= 128 ? 2 : 1;
   const int parts256 = K / 64 >= 192 ? 2 : 1;
+  // 128 x 128 also from half a device's worth of tiles on a long K (14336 x 4096 at M = 160 / 224: 42 -> 35 us), and
+  // wherever the 64 x 128 tiles (one workgroup per compute unit) would need a second round and these do not
+  // (4096 x 6144 at M = 384: 39 -> 27 us; 4096 x 4096 at M = 640: 38.5 -> 28 us)
+  const bool take128 = tiles(128, 128) * parts128 * 10 >= cus * (parts128 == 2 ? 5 : 7) ||
+                       (tiles(64, 128) > cus && tiles(128, 128) <= cus);
   if (pl.cfg <= 0)
-    pl.cfg = tiles(256, 256) * parts256 * 10 >= cus * 7 ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (tiles(128, 128) * parts128 * 10 >= cus * 7 ? 3 : 4));
+    pl.cfg = tiles(256, 256) * parts256 * 10 >= cus * 7 ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (take128 ? 3 : 4));
   // the smallest tile with two k-slices per step: 5-8 % faster on a short K (half the barriers), no gain on a long one
   if (tuning().fp8_tile_cfg <= 0 && pl.cfg == 4 && K % 128 == 0 && K <= 8192) pl.cfg = 14;
+  // 64 x 64 tiles while they fit the device in one round, on a short K: twice the workgroups with loads in flight
+  // (cold weights: 4096 x 6144 at M = 128 21.8 -> 15.0 us, 4096 x 4096 at M = 192 19.8 -> 13.8 us; 14336 x 4096 at
+  // M = 128 30.0 -> 34.0 us, and slower as soon as the tiles need a second round)
+  if (tuning().fp8_tile_cfg <= 0 && pl.cfg == 14 && tiles(64, 64) <= cus) pl.cfg = 15;
   if (pl.cfg >= 10 && K % 128 != 0) pl.cfg %= 10;      // two k-slices per step need K % 128 == 0
   switch (pl.cfg) {
     case 3: case 13: case 23: pl.bm = 128; pl.bn = 128; pl.nw = 4; break;
     case 4: case 14: case 24: pl.bm = 64; pl.bn = 128; pl.nw = 4; break;
+    case 5: case 15: pl.bm = 64; pl.bn = 64; pl.nw = 4; break;
     case 7: case 17: pl.bm = 128; pl.bn = 256; pl.nw = 8; break;
     case 2: pl.bm = 256; pl.bn = 256; pl.nw = 4; break;
     default: pl.bm = 256; pl.bn = 256; pl.nw = 8; break;
@@ -1158,7 +1168,6 @@ static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t c
       case 2: return launch_tile3<BF16_OUT, 256, 256, 2, 2, 5>(p, s);
       case 3: return launch_tile3<BF16_OUT, 128, 128, 2, 2, 5>(p, s);
       case 4: return launch_tile3<BF16_OUT, 64, 128, 2, 2, 5>(p, s);
-      case 5: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 4>(p, s);
       case 6: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 3>(p, s);
       case 7: return launch_tile3<BF16_OUT, 128, 256, 2, 4, 5>(p, s);
       // two k-slices per step (K % 128 == 0)
@@ -1166,6 +1175,8 @@ static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t c
       case 23: return launch_tile3<BF16_OUT, 128, 128, 2, 2, 2, 2>(p, s);
       case 14: return launch_tile3<BF16_OUT, 64, 128, 2, 2, 5, 2>(p, s);
       case 24: return launch_tile3<BF16_OUT, 64, 128, 2, 2, 3, 2>(p, s);
+      case 15: return launch_tile3<BF16_OUT, 64, 64, 2, 2, 5, 2>(p, s);
+      case 5: return launch_tile3<BF16_OUT, 64, 64, 2, 2, 5>(p, s);
       case 17: return launch_tile3<BF16_OUT, 128, 256, 2, 4, 3, 2>(p, s);
       default: break;
     }

@@ -45,7 +45,14 @@ static int pick_tile(int M, int N, int K, bool direct_ok) {
     if (tiles(128, 128) >= cus) return 12;
     // Few tiles: 64 x 128, or 128 x 64 once M fills more than one 64-row tile (the dequantisation of a weight tile is
     // then shared by twice as many rows: 7-15 % faster at M = 128 .. 768 on the narrow layers); K is split over
-    // workgroups when the tiles leave units idle.
+    // workgroups when the tiles leave units idle.  Measured on the Llama shapes, M = 80 .. 1280, cold weights:
+    //  * 128 x 128 where the 128 x 64 tiles fill the device or need a second round and these fill half of it (4096 x 6144 at
+    //    M = 384: 44.5 -> 33.7 us; 4096 x 4096 at M = 640: 44.3 -> 34.9 us), and on a long K from 3/8 of the device on
+    //    (14336 x 4096 at M = 320 .. 512: 79 .. 88 -> 61 .. 79 us);
+    //  * 64 x 128 where an odd number of 64-row blocks would leave the last 128-row tile half empty (4096 x 6144 at
+    //    M = 192: 28.2 -> 23.4 us; 4096 x 4096 at M = 320: 28.1 -> 23.5 us).
+    if ((tiles(128, 64) >= cus && tiles(128, 128) * 2 >= cus) || (K >= 8192 && tiles(128, 128) * 8 >= (int64_t)cus * 3)) return 12;
+    if (M > 64 && ((M + 63) / 64) % 2 == 1 && tiles(64, 128) <= cus) return 14;
     return M > 64 ? 15 : 14;
   }
   if (tiles(256, 256) >= cus) return 0;
