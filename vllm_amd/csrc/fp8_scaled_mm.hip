@@ -1087,6 +1087,9 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   // parts of a long K get it there (14336 x 4096 at M = 512, cold, 73 -> 62 us)
   // ... and for 256 x 256 when two parts of a very long K do (14336 x 4096 at M = 1536 / 2048, cold: 139 / 145 -> 116 / 130 us;
   // 4096 x 4096 at M = 2048 in two parts: 45 -> 66 us)
+  // (256 x 256 from 55 % of the compute units on, 50 % in two parts of a long K: 4096 x 6144 at M = 1408 .. 1792 70 ->
+  // 49 .. 55 us, 4096 x 4096 at M = 2304 / 2560 70 -> 54 us, 14336 x 4096 at M = 1024 / 1280 89 / 132 -> 79 / 105 us;
+  // at 47-50 % on a short K the smaller tiles win, 4096 x 4096 at M = 2048 45 against 53 us)
   const int parts128 = K / 64 >= 128 ? 2 : 1;
   const int parts256 = K / 64 >= 192 ? 2 : 1;
   // 128 x 128 also from half a device's worth of tiles on a long K (14336 x 4096 at M = 160 / 224: 42 -> 35 us), and
@@ -1095,7 +1098,7 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   const bool take128 = tiles(128, 128) * parts128 * 10 >= cus * (parts128 == 2 ? 5 : 7) ||
                        (tiles(64, 128) > cus && tiles(128, 128) <= cus);
   if (pl.cfg <= 0)
-    pl.cfg = tiles(256, 256) * parts256 * 10 >= cus * 7 ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (take128 ? 3 : 4));
+    pl.cfg = tiles(256, 256) * parts256 * 20 >= cus * (parts256 == 2 ? 10 : 11) ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (take128 ? 3 : 4));
   // the smallest tile with two k-slices per step: 5-8 % faster on a short K (half the barriers), no gain on a long one
   if (tuning().fp8_tile_cfg <= 0 && pl.cfg == 4 && K % 128 == 0 && K <= 8192) pl.cfg = 14;
   // 64 x 64 tiles while they fit the device in one round, on a short K: twice the workgroups with loads in flight
