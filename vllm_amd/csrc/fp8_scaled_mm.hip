@@ -1284,7 +1284,9 @@ static bool launch_stream2(const Fp8MMParams& p_in, int wk, int gx, hipStream_t 
 // Steps per wavefront of the stream kernel with the weights through LDS, 0 where the kernel above stays.  Measured with
 // cold weights against the kernel above (us, M = 1 / 4 / 16): 4096 x 6144 8.6 / 9.0 / 10.3 -> 7.7 / 7.8 / 8.6, 4096 x 4096
 // 6.0 / 6.2 / 7.1 -> 5.7 / 5.9 / 6.6, 4096 x 28672 25.8 / 26.1 / 27.8 -> 21.9 / 22.0 / 23.3, 14336 x 4096 13.8 / 14.8 / 18.0 ->
-// 12.0 / 12.4 / 15.3; two m-blocks (M = 32): 4096 x 6144 11.4 -> 10.5, 4096 x 28672 30.6 -> 26.5, 4096 x 4096 8.7 -> 8.9.
+// 12.0 / 12.4 / 15.3; two m-blocks (M = 32): 4096 x 6144 11.4 -> 10.5, 4096 x 28672 30.6 -> 26.5, 4096 x 4096 8.7 -> 8.9
+// with 4 steps per wavefront and 8.3 with 8 (M = 17 / 24: 7.5 / 8.2 -> 7.1 / 7.7), which layers of at most one n-tile per
+// compute unit therefore take.
 // (development switch exp[4]: 1 / 2 / 3 force 8 / 4 / 16 steps, 9 switches the kernel off)
 static int stream2_steps_per_wave(const Fp8MMParams& p) {
   const int sw = tuning().exp[4];
@@ -1293,7 +1295,7 @@ static int stream2_steps_per_wave(const Fp8MMParams& p) {
   int ks = 0;
   if (sw >= 1 && sw <= 3) ks = sw == 1 ? 8 : (sw == 2 ? 4 : 16);
   else if (MB == 1) ks = steps <= 64 ? 8 : (steps <= 128 ? 16 : 0);
-  else ks = (steps <= 32 && p.N / 16 > num_cus_current_device()) ? 4 : 0;
+  else ks = steps > 32 ? 0 : (p.N / 16 > num_cus_current_device() ? 4 : 8);
   if (ks == 0 || (steps + ks - 1) / ks > 8 || (MB == 2 && ks == 16)) return 0;
   return ks;
 }
