@@ -37,7 +37,9 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8, 
   // K slices wanted: about 16 wavefronts per compute unit, 8 when few rows are staged (measured: with little LDS to
   // fill, longer per-wavefront tile streams beat more wavefronts on layers with few n-tiles)
   // (also with 16 staged rows when there is at most one workgroup per compute unit: 4096 x 4096 at M = 16, 6.60 -> 6.34 us)
-  int want = (cus * ((c.mr <= 4 && NT <= 2 * cus) || NT * c.sk <= cus ? 8 : D2_WAVES)) / (NT * c.sk);
+  // (and with 16 staged rows on up to two (n-tile, K slab) pairs per compute unit: four K slices of 8 tiles with the
+  // three-slot ring below, 4096 x 6144 at M = 16 6.9 -> 6.5 us, 8192 x 6144 10.9 -> 9.5 us, 4096 x 8192 7.5 -> 7.0 us)
+  int want = (cus * ((NT * c.sk <= 2 * cus && MB == 1) || NT * c.sk <= cus ? 8 : D2_WAVES)) / (NT * c.sk);
   int wks = 1;
   while (wks * 2 <= want && wks < 16) wks *= 2;
   while (wks > 1 && wks > gslab) wks /= 2;
@@ -91,8 +93,8 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8, 
     if (slots < 1) slots = 1;
     const long per_cu = ((long)((NT + c.wn - 1) / c.wn) * c.sk + cus - 1) / cus;
     const long waves_cu = (per_cu < slots ? per_cu : slots) * wks * c.wn;
-    if (waves_cu <= 8) c.rc = 1;
-    else if (c.mr == 16 && gs >= 14) c.rc = 2;      // (7 tiles per wavefront, 14336 x 4096 at M = 16: three slots 11.5 us, two 11.2 us)
+    if (c.mr == 16 && (gs >= 8 || waves_cu <= 8)) c.rc = 2;      // (7 tiles per wavefront, 16 wavefronts, 14336 x 4096 at M = 16: three slots 11.5 us, two 11.2 us)
+    else if (waves_cu <= 8) c.rc = 1;
   }
   if (tn.exp[1] > 0) c.rc = tn.exp[1] - 1;      // (development switch: forced ring variant + 1)
   return c;
