@@ -150,8 +150,9 @@ static bool use_row_split(int M, int N, int K, int sub, int wt, bool has_perm) {
   // One round of full workgroups.  Measured: 4096 x 4096 at M = 32 / 64: 8.5 / 10.5 -> 6.6 / 9.2 us, 4096 x 6144: 8.8 / 11.4
   // -> 8.7 / 10.6 us; with three m-blocks the grids of those layers spill into a second round (15 us) or leave ten
   // wavefronts per workgroup (9.9 -> 11.7 us).  A 28672-wide layer would need streams of 32 tiles (measured 20.4 -> 21.7 us).
+  // (Two m-blocks also as eight wavefronts of 8-tile streams with the three-slot ring: 4096 x 4096 at M = 32 6.3 us.)
   const long wgs = (long)((N / 16 + c.wn - 1) / c.wn) * ((M + 15) / 16);
-  return wgs <= num_cus_current_device() && c.wks * c.wn >= 12;
+  return wgs <= num_cus_current_device() && c.wks * c.wn >= (M <= 32 ? 8 : 12);
 }
 
 int decode2_launch_msp(const Decode2Params& p, int gs, int rc, bool bf16, bool zp, hipStream_t s);      // w4a16_decode2_msp.hip
