@@ -44,8 +44,47 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8, 
   while (wks * 2 <= want && wks < 16) wks *= 2;
   while (wks > 1 && wks > gslab) wks /= 2;
   const VaqTuning& tn = tuning();
+  // Two m-blocks of a long K on a layer of at most one n-tile per compute unit: slabs of one 14-tile stream per
+  // wavefront with the four-slot ring (14336 x 4096 at M = 17 / 32: 13.8 / 14.7 -> 12.9 / 13.2 us; 11008 x 4096 14.1 -> 12.4 us;
+  // 16-tile streams, two slices of 7 or 8, and the same on 8192 x 8192 or a 28672-wide layer are slower).
+  // n-tiles per workgroup (at most 16 / wks).  A compute unit holds 16 of these wavefronts and as many workgroups as
+  // its LDS allows.  First the fewest rounds of workgroups per compute unit, then the fewest wavefronts on the busiest
+  // compute unit (i.e. spread over the device), then the smaller workgroup.
+  auto pick_wn = [&](int wks_, int gs_, int sk_, long* rounds_out) {
+    int best_wn = 1;
+    long best_rounds = -1, best_waves = -1;
+    const size_t lds_wg = decode2_lds_bytes(wks_, gs_ / TPG, c.mr, MB);
+    for (int wn = 1; wn <= D2_WAVES / wks_; ++wn) {
+      long slots = D2_WAVES / (wks_ * wn);
+      const long lds_slots = (long)((size_t)(160 * 1024) / lds_wg);
+      if (slots > lds_slots) slots = lds_slots;
+      if (slots < 1) slots = 1;
+      const long wgs = (long)((NT + wn - 1) / wn) * sk_;
+      const long per_cu = (wgs + cus - 1) / cus;
+      const long rounds = (per_cu + slots - 1) / slots;
+      const long waves = (per_cu < slots ? per_cu : slots) * wn * wks_;
+      if (best_rounds < 0 || rounds < best_rounds || (rounds == best_rounds && waves < best_waves)) {
+        best_rounds = rounds;
+        best_waves = waves;
+        best_wn = wn;
+      }
+    }
+    if (rounds_out) *rounds_out = best_rounds;
+    return best_wn;
+  };
+  bool long_k_two_blocks = MB == 2 && NT <= cus && G >= 80 && sub == 1 && !w8 && nt_mult == 1;
+  if (long_k_two_blocks) {
+    // ... and only as one round of workgroups of 7 to 10 wavefronts that fill 85 % of the device (measured slower with
+    // 4, 11 and 15 wavefronts: 14336 x 2048 10.3 -> 12.2 us, 16384 x 4096 14.2 -> 15.5 us, 24576 x 4096 18.9 -> 20.3 us)
+    const int sk_b = (G + 13) / 14;
+    long rounds_b = 0;
+    const int wn_b = pick_wn(1, 14, sk_b, &rounds_b);
+    const long wgs_b = (long)((NT + wn_b - 1) / wn_b) * sk_b;
+    long_k_two_blocks = rounds_b == 1 && wn_b >= 7 && wn_b <= 10 && wgs_b * 100 >= (long)cus * 85;
+  }
+  if (long_k_two_blocks) wks = 1;
   if (tn.decode2_wks > 0) wks = tn.decode2_wks;
-  int gs = round_gs((gslab + wks - 1) / wks, sub, w8);
+  int gs = long_k_two_blocks ? 14 : round_gs((gslab + wks - 1) / wks, sub, w8);
   if (tn.decode2_gs > 0) gs = tn.decode2_gs;
   while (wks * gs > slab_max && wks > 1) wks /= 2;     // respect the LDS limit
   if (gs > slab_max) {                                 // rounding up went past it: largest instantiated size below
@@ -60,27 +99,8 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8, 
   c.sk = (G + wks * gs - 1) / (wks * gs);
   c.gs = gs;
   c.wks = wks;
-  // n-tiles per workgroup (at most 16 / wks).  A compute unit holds 16 of these wavefronts and as many workgroups as
-  // its LDS allows.  First the fewest rounds of workgroups per compute unit, then the fewest wavefronts on the busiest
-  // compute unit (i.e. spread over the device), then the smaller workgroup.
-  int best_wn = 1;
-  long best_rounds = -1, best_waves = -1;
   const size_t lds_wg = decode2_lds_bytes(wks, gs / TPG, c.mr, MB);
-  for (int wn = 1; wn <= D2_WAVES / wks; ++wn) {
-    long slots = D2_WAVES / (wks * wn);
-    const long lds_slots = (long)((size_t)(160 * 1024) / lds_wg);
-    if (slots > lds_slots) slots = lds_slots;
-    if (slots < 1) slots = 1;
-    const long wgs = (long)((NT + wn - 1) / wn) * c.sk;
-    const long per_cu = (wgs + cus - 1) / cus;
-    const long rounds = (per_cu + slots - 1) / slots;
-    const long waves = (per_cu < slots ? per_cu : slots) * wn * wks;
-    if (best_rounds < 0 || rounds < best_rounds || (rounds == best_rounds && waves < best_waves)) {
-      best_rounds = rounds;
-      best_waves = waves;
-      best_wn = wn;
-    }
-  }
+  const int best_wn = pick_wn(wks, gs, c.sk, nullptr);
   c.wn = tn.decode2_wn > 0 ? tn.decode2_wn : best_wn;
   if (c.wn * wks > D2_WAVES) c.wn = D2_WAVES / wks;
   // ring variant of long streams (instances exist for 4-bit codes in groups of 128 rows / channelwise, up to two
@@ -93,7 +113,8 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8, 
     if (slots < 1) slots = 1;
     const long per_cu = ((long)((NT + c.wn - 1) / c.wn) * c.sk + cus - 1) / cus;
     const long waves_cu = (per_cu < slots ? per_cu : slots) * wks * c.wn;
-    if (c.mr == 16 && (gs >= 8 || waves_cu <= 8)) c.rc = 2;      // (7 tiles per wavefront, 16 wavefronts, 14336 x 4096 at M = 16: three slots 11.5 us, two 11.2 us)
+    if (long_k_two_blocks && wks == 1 && gs == 14) c.rc = 1;
+    else if (c.mr == 16 && (gs >= 8 || waves_cu <= 8)) c.rc = 2;      // (7 tiles per wavefront, 16 wavefronts, 14336 x 4096 at M = 16: three slots 11.5 us, two 11.2 us)
     else if (waves_cu <= 8) c.rc = 1;
   }
   if (tn.exp[1] > 0) c.rc = tn.exp[1] - 1;      // (development switch: forced ring variant + 1)
