@@ -285,19 +285,29 @@ def _gemm_impl(a: torch.Tensor, c_or_none: torch.Tensor | None, b_q_weight: torc
         # graph capture), arrival counters from the caller's `workspace`.  The library checks what it is handed against
         # what the kernel it picks needs and reports a workspace that is too small (gptq_marlin.cu:899-902).
         tune = _tuning.current_ref()
-        n_ctmp, n_atmp, n_cnt = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
-        q_args = (size_m, size_n, size_k, int(has_act_order), dev.index or 0, ctypes.byref(n_ctmp), ctypes.byref(n_atmp),
-                  ctypes.byref(n_cnt))
-        _lib.check(lib.vaq_w4a16_gemm_workspace(*q_args) if tune is None
-                   else lib.vaq_w4a16_gemm_workspace_tuned(*q_args, tune))
-        c_tmp = torch.empty((n_ctmp.value // 4,), dtype=torch.float32, device=dev) if n_ctmp.value else None
-        a_tmp = torch.empty((n_atmp.value // 2,), dtype=a.dtype, device=dev) if n_atmp.value else None
+        key = (size_m, size_n, size_k, has_act_order, dev.index or 0)
+        sizes = _W4_WORKSPACE_SIZES.get(key) if tune is None else None
+        if sizes is None:
+            n_ctmp, n_atmp, n_cnt = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+            q_args = (size_m, size_n, size_k, int(has_act_order), dev.index or 0, ctypes.byref(n_ctmp),
+                      ctypes.byref(n_atmp), ctypes.byref(n_cnt))
+            _lib.check(lib.vaq_w4a16_gemm_workspace(*q_args) if tune is None
+                       else lib.vaq_w4a16_gemm_workspace_tuned(*q_args, tune))
+            sizes = (n_ctmp.value, n_atmp.value)
+            if tune is None and len(_W4_WORKSPACE_SIZES) < 4096:
+                _W4_WORKSPACE_SIZES[key] = sizes      # (the library's answer depends on the shape and the device only)
+        ctmp_bytes, atmp_bytes = sizes
+        c_tmp = torch.empty((ctmp_bytes // 4,), dtype=torch.float32, device=dev) if ctmp_bytes else None
+        a_tmp = torch.empty((atmp_bytes // 2,), dtype=a.dtype, device=dev) if atmp_bytes else None
         g_args = (_ptr(a), a.stride(0), _ptr(b_q_weight), _ptr(b_scales), _ptr(b_zeros_or_none) if has_zp else None,
                   _ptr(perm_or_none) if has_act_order else None, _ptr(b_bias_or_none), _ptr(c), _ptr(c_tmp),
-                  n_ctmp.value, _ptr(a_tmp), _ptr(workspace), workspace.numel(), size_m, size_n, size_k, group_size,
+                  ctmp_bytes, _ptr(a_tmp), _ptr(workspace), workspace.numel(), size_m, size_n, size_k, group_size,
                   _dtype_tag(a.dtype), wtype, 0, _stream(dev))
         _lib.check(lib.vaq_w4a16_gemm(*g_args) if tune is None else lib.vaq_w4a16_gemm_tuned(*g_args, tune))
     return c
+
+
+_W4_WORKSPACE_SIZES: dict[tuple, tuple[int, int]] = {}
 
 
 def _gemm_fake(a, c_or_none, b_q_weight, b_bias_or_none, b_scales, global_scale, b_zeros_or_none, g_idx_or_none,
@@ -420,21 +430,29 @@ def _scaled_mm_impl(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor, a_scale
         # scratch for the K split of mid-sized M: partial tiles from the caching allocator (capture-safe), arrival
         # counters that are zero on entry and left zero, one array per (device, stream)
         tune = _tuning.current_ref()
-        n_ctmp, n_cnt = ctypes.c_size_t(), ctypes.c_size_t()
-        q_args = (a.size(0), b.size(1), a.size(1), ctypes.byref(n_ctmp), ctypes.byref(n_cnt))
-        _lib.check(lib.vaq_fp8_scaled_mm_workspace(*q_args) if tune is None
-                   else lib.vaq_fp8_scaled_mm_workspace_tuned(*q_args, tune))
+        key = (a.size(0), b.size(1), a.size(1), dev.index or 0)
+        sizes = _FP8_WORKSPACE_SIZES.get(key) if tune is None else None
+        if sizes is None:
+            n_ctmp, n_cnt = ctypes.c_size_t(), ctypes.c_size_t()
+            q_args = (a.size(0), b.size(1), a.size(1), ctypes.byref(n_ctmp), ctypes.byref(n_cnt))
+            _lib.check(lib.vaq_fp8_scaled_mm_workspace(*q_args) if tune is None
+                       else lib.vaq_fp8_scaled_mm_workspace_tuned(*q_args, tune))
+            sizes = (n_ctmp.value, n_cnt.value)
+            if tune is None and len(_FP8_WORKSPACE_SIZES) < 4096:
+                _FP8_WORKSPACE_SIZES[key] = sizes
+        ctmp_bytes, cnt_ints = sizes
         c_tmp = counters = None
-        if n_ctmp.value:
-            counters = _fp8_counters(dev, n_cnt.value)
-            c_tmp = torch.empty((n_ctmp.value // 4,), dtype=torch.float32, device=dev)
+        if ctmp_bytes:
+            counters = _fp8_counters(dev, cnt_ints)
+            c_tmp = torch.empty((ctmp_bytes // 4,), dtype=torch.float32, device=dev)
         args = (_ptr(a), a.stride(0), _ptr(b), b.stride(1), _ptr(a_scales), a_scales.numel(), _ptr(b_scales),
                 b_scales.numel(), _ptr(bias), _ptr(out), out.stride(0), _dtype_tag(out.dtype), a.size(0), b.size(1),
-                a.size(1), _ptr(c_tmp), n_ctmp.value if c_tmp is not None else 0, _ptr(counters),
+                a.size(1), _ptr(c_tmp), ctmp_bytes if c_tmp is not None else 0, _ptr(counters),
                 counters.numel() if counters is not None else 0, _stream(dev))
         _lib.check(lib.vaq_fp8_scaled_mm_ws(*args) if tune is None else lib.vaq_fp8_scaled_mm_ws_tuned(*args, tune))
 
 
+_FP8_WORKSPACE_SIZES: dict[tuple, tuple[int, int]] = {}
 _FP8_COUNTERS: dict[tuple[int, int], torch.Tensor] = {}
 _FP8_COUNTER_INTS = 16384
 
