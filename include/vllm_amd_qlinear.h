@@ -248,7 +248,10 @@ typedef struct VaqTuning {
   int fp8_gx;           /*   workgroups of the weight-streaming kernel                                               */
   int fp8_stream_split; /*   -1 = never run the weight-streaming kernel over two halves of K                         */
   int quant_wg_per_row; /* per-token FP8 quant: 1 = always one workgroup per row                                     */
-  int exp[15];          /* experiment switches of development builds; ignored by released kernels                    */
+  int exp[15];          /* further switches of the same kind, for A/B timing runs: [0] = 1 shared instead of private  */
+                        /*   activation fill, [1] = ring variant + 1, [2] rows over workgroups (1 off, 2 forced) of   */
+                        /*   the LDS-staged decode kernel; [4] FP8 streaming through LDS (1 / 2 / 3 = 8 / 4 / 16 steps */
+                        /*   per wavefront, 9 = off); the rest unused                                                  */
 } VaqTuning;
 
 /* The entry points of the same name without `_tuned`, with `tuning` (may be NULL) applied to this call. */
