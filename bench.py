@@ -524,6 +524,33 @@ def fp8_section(dev):
     return rows
 
 
+def medium_m_section(dev):
+    """The sizes between decode and prefill (M = 64 .. 1024: large decode batches, chunked prefill), cold weights (~600 MB of
+    distinct copies cycling): W4A16 (symmetric, groups of 128) and FP8 W8A8 per shape and M."""
+    import vllm_amd._custom_ops as ops
+    rows = []
+    gen = torch.Generator(device=dev).manual_seed(5)
+    for (k, n) in LLAMA_SHAPES:
+        layers = [W4Layer(k, n, dev, gen) for _ in range(max(2, int(600e6 // (k * n // 2))))]
+        wq, ws = ops.scaled_fp8_quant((torch.randn(n, k, device=dev, generator=gen) * 0.02).to(torch.bfloat16),
+                                      use_per_token_if_dynamic=True)
+        copies = [wq.clone().t() for _ in range(max(2, int(600e6 // (k * n))))]
+        for m in (64, 128, 256, 512, 1024):
+            a = torch.randn(m, k, device=dev, generator=gen).to(torch.bfloat16)
+            aq, sa = ops.scaled_fp8_quant(a, use_per_token_if_dynamic=True)
+            t4 = time_graph(lambda: [l(a) for l in layers], iters=5, warmup=2, inner=len(layers))
+            t8 = time_graph(lambda: [ops.cutlass_scaled_mm(aq, wc, sa, ws, torch.bfloat16, None) for wc in copies],
+                            iters=5, warmup=2, inner=len(copies))
+            fl = 2.0 * m * n * k
+            rows.append(dict(kind="medium_m", K=k, N=n, M=m, w4a16_us=t4 * 1e6, w4a16_TFLOPs=fl / t4 / 1e12,
+                             fp8_us=t8 * 1e6, fp8_TFLOPs=fl / t8 / 1e12, cold=True))
+            log(f"[medium M    ] K={k:5d} N={n:5d} M={m:4d}: W4A16 {t4 * 1e6:7.1f} us {fl / t4 / 1e12:6.0f} TFLOP/s | "
+                f"FP8 {t8 * 1e6:7.1f} us {fl / t8 / 1e12:6.0f} TFLOP/s")
+        del layers, copies, wq
+        torch.cuda.empty_cache()
+    return rows
+
+
 def roofline_mfma(extra):
     """The compute-bound kernels against the dense MFMA peaks, from the M = 4096 rows of the prefill and FP8 sections
     (HIP-graph timings of this run): per kernel the FLOPs of one launch, its average duration and the fraction of peak."""
@@ -706,6 +733,7 @@ def main():
                          ("variants", variants_section),
                          ("vendor_ceiling", vendor_ceiling_section),
                          ("host_overhead", host_overhead_section),
+                         ("medium_m", medium_m_section),
                          ("decode_step", decode_step_section)):
             if args.sections and name not in args.sections.split(","):
                 continue
