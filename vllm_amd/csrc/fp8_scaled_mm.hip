@@ -1127,16 +1127,19 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
     while (sk & (sk - 1)) --sk;       // a power of two (3 splits measured slower than 2)
   } else if (pl.tiles < cus) {
     // Small tiles (two workgroups share a compute unit), measured with cold weights on the Llama shapes, M = 48 .. 512:
-    // tiles that leave 3/4 of the device idle are split until there is about one workgroup per compute unit (parts of
+    // tiles that leave 2/3 of the device idle are split until there is about one workgroup per compute unit (parts of
     // at least 16 steps: 4096 x 4096 at M = 128, 4 parts of 16 steps 15.7 us, 2 of 32 18.4 us, 8 of 8 22.7 us); fuller
     // devices stay unsplit (the rotated K loop of the unsplit kernel is worth more there: 4096 x 6144 at M = 192,
     // 20.8 against 31.0 us in 2 parts; 96 tiles in 2 parts: -3 % on 4096 x 6144, +6 % on 4096 x 4096) unless K is very
     // long, where a part is halved while the halves stay 50 steps long and the workgroups fit the device at once
     // (14336 x 4096 at M = 256: 62.6 / 45.8 / 44.3 us in 1 / 2 / 4 parts).
-    if (pl.tiles * 4 <= (int64_t)cus) {
+    if (pl.tiles * 3 <= (int64_t)cus) {
       sk = (int)((int64_t)cus / pl.tiles);
       if (sk > 8) sk = 8;
-      if (sk > steps / 16) sk = steps / 16;
+      // (parts of at least 16 steps; 32 between 1/4 and 1/3 of the device: 5120 x 5120 at M = 64, 80 tiles in two parts
+      // of 40 steps, 22.8 -> 18.2 us; 2560 x 2560 at M = 128 in two parts of 20, 11.5 -> 12.3 us)
+      const int min_part = pl.tiles * 4 <= (int64_t)cus ? 16 : 32;
+      if (sk > steps / min_part) sk = steps / min_part;
       if (sk < 1) sk = 1;
       while (sk & (sk - 1)) --sk;
     }
