@@ -42,7 +42,8 @@ static int pick_tile(int M, int N, int K, bool direct_ok) {
     // measured: the 256x256 / 8-wavefront tile wins as soon as it fills ~55 % of the compute units, also when it
     // takes a split of a long K to get there (14336 x 4096 at M = 1024 / 2048: 4 % / 21 % faster than 128 x 128)
     // (from 55 % on: 4096 x 6144 at M = 1536, 144 tiles, 112 -> 85 us; at 50 %, 4096 x 4096 at M = 2048, 76 against 85 us)
-    if (tiles(256, 256) * splits_256(tiles(256, 256), K, cus) * 20 >= cus * 11) return 20;      // 256 x 256, alternating phases
+    // (not for a single tile row that M fills at most half: 8192 x 28672 at M = 128, 104 against 85 us with 128 x 128)
+    if (M > 128 && tiles(256, 256) * splits_256(tiles(256, 256), K, cus) * 20 >= cus * 11) return 20;      // 256 x 256, alternating phases
     if (tiles(128, 128) >= cus) return 12;
     // Few tiles: 64 x 128, or 128 x 64 once M fills more than one 64-row tile (the dequantisation of a weight tile is
     // then shared by twice as many rows: 7-15 % faster at M = 128 .. 768 on the narrow layers); K is split over
