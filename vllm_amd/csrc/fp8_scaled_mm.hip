@@ -1091,7 +1091,7 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   // 49 .. 55 us, 4096 x 4096 at M = 2304 / 2560 70 -> 54 us, 14336 x 4096 at M = 1024 / 1280 89 / 132 -> 79 / 105 us;
   // at 47-50 % on a short K the smaller tiles win, 4096 x 4096 at M = 2048 45 against 53 us)
   const int parts128 = K / 64 >= 128 ? 2 : 1;
-  const int parts256 = K / 64 >= 192 ? 2 : 1;
+  const int parts256 = K / 64 >= 160 ? 2 : 1;      // (11008 x 4096 at M = 2048 in two parts: 115 -> 98 us)
   // 128 x 128 also from half a device's worth of tiles on a long K (14336 x 4096 at M = 160 / 224: 42 -> 35 us), and
   // wherever the 64 x 128 tiles (one workgroup per compute unit) would need a second round and these do not
   // (4096 x 6144 at M = 384: 39 -> 27 us; 4096 x 4096 at M = 640: 38.5 -> 28 us)
