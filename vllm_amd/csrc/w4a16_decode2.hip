@@ -43,6 +43,12 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8, 
   int wks = 1;
   while (wks * 2 <= want && wks < 16) wks *= 2;
   while (wks > 1 && wks > gslab) wks /= 2;
+  // A single row: as many K slices as it takes to cover K with streams of at most 16 tiles, rather than a split over
+  // workgroups and its hand-over (28672 x 8192 at M = 1: 30.2 -> 24.5 us, 28672 x 4096 17.7 -> 14.8 us; from two rows on
+  // the split wins or ties) -- where those workgroups, one per n-tile, make full rounds (20480 x 5120, 320 n-tiles:
+  // 16.7 -> 19.4 us).
+  if (c.mr == 1 && (NT <= cus || NT % cus == 0 || (NT % cus) * 5 >= cus * 4))
+    while (wks < 16 && wks * 16 < gslab) wks *= 2;
   const VaqTuning& tn = tuning();
   // Two m-blocks of a long K on a layer of at most one n-tile per compute unit: slabs of one 14-tile stream per
   // wavefront with the four-slot ring (14336 x 4096 at M = 17 / 32: 13.8 / 14.7 -> 12.9 / 13.2 us; 11008 x 4096 14.1 -> 12.4 us;
