@@ -119,7 +119,7 @@ SMALL = [(128, 64), (512, 256), (1024, 192), (2048, 576), (14336 // 4, 128)]
 
 
 @pytest.mark.parametrize("k,n", SMALL)
-@pytest.mark.parametrize("m", [1, 4, 16, 17, 32])
+@pytest.mark.parametrize("m", [1, 3, 4, 5, 8, 16, 17, 32])
 @pytest.mark.parametrize("asym,act_order", [(False, False), (True, False), (False, True), (True, True)])
 def test_decode_gemm_small(device, decode_kernel, k, n, m, asym, act_order):
     if act_order and k == 128:

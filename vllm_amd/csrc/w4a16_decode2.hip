@@ -29,7 +29,7 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8, 
   const int G = K / 128 * TPG, NT = N / 16 * nt_mult;
   const int MB = (M + 15) / 16;
   Decode2Config c;
-  c.mr = M == 1 ? 1 : (M <= 4 ? 4 : 16);
+  c.mr = M == 1 ? 1 : (M <= 4 ? 4 : (M <= 8 && sub == 1 && !w8 ? 8 : 16));      // rows staged (8: 4-bit codes in groups of 128 rows only)
   const int slab_max = 512 / (c.mr * MB) * TPG;
   c.sk = (G + slab_max - 1) / slab_max;
   const int gslab = (G + c.sk - 1) / c.sk;            // groups per slab
@@ -120,7 +120,7 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8, 
     const long per_cu = ((long)((NT + c.wn - 1) / c.wn) * c.sk + cus - 1) / cus;
     const long waves_cu = (per_cu < slots ? per_cu : slots) * wks * c.wn;
     if (long_k_two_blocks && wks == 1 && gs == 14) c.rc = 1;
-    else if (c.mr == 16 && (gs >= 8 || waves_cu <= 8)) c.rc = 2;      // (7 tiles per wavefront, 16 wavefronts, 14336 x 4096 at M = 16: three slots 11.5 us, two 11.2 us)
+    else if (c.mr >= 8 && (gs >= 8 || waves_cu <= 8)) c.rc = 2;      // (7 tiles per wavefront, 16 wavefronts, 14336 x 4096 at M = 16: three slots 11.5 us, two 11.2 us)
     else if (waves_cu <= 8) c.rc = 1;
   }
   if (tn.exp[1] > 0) c.rc = tn.exp[1] - 1;      // (development switch: forced ring variant + 1)
@@ -162,6 +162,9 @@ static int dispatch_mr2(const Decode2Params& p, const Decode2Config& c, bool bf1
   switch (c.mr) {
     case 1: return dispatch_types2<MB, 1>(p, c.gs, c.rc, bf16, zp, s);
     case 4: return dispatch_types2<MB, 4>(p, c.gs, c.rc, bf16, zp, s);
+    case 8:
+      if constexpr (MB == 1) return dispatch_types2<MB, 8>(p, c.gs, c.rc, bf16, zp, s);
+      [[fallthrough]];
     default: return dispatch_types2<MB, 16>(p, c.gs, c.rc, bf16, zp, s);
   }
 }

@@ -115,7 +115,7 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   constexpr bool LATE = RC != 0 && !SHORT;
   constexpr int R_LATE = RC == 1 ? 4 : (RC == 2 ? 3 : 2);
   static_assert(!(WT != 0 && RC != 0), "8-bit weights take the block of a tile from the slot parity: even rings only");
-  constexpr int R = SHORT ? R_SHORT : (LATE ? (GS < R_LATE ? GS : R_LATE) : ((MR == 16 && MB == 1 && GS >= 7) ? 4 : (GS < 2 ? GS : 2)));
+  constexpr int R = SHORT ? R_SHORT : (LATE ? (GS < R_LATE ? GS : R_LATE) : ((MR >= 8 && MB == 1 && GS >= 7) ? 4 : (GS < 2 ? GS : 2)));
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
   const int lane = threadIdx.x;
