@@ -98,6 +98,16 @@ static PrefillPlan plan_prefill(int M, int N, int K, bool direct_ok) {
     const int min_groups = pl.tiles < cus ? 8 : 32;     // a device already full of tiles only splits a very long K
     if (sk > G / min_groups) sk = G / min_groups;
     if (sk < 1) sk = 1;
+    // A short K on few tiles (what the 8-group minimum leaves unsplit or nearly so): parts of at least 3 groups, up to
+    // one workgroup per compute unit.  Cold weights, M = 96 .. 512: 1536 x 1536 15.4 -> 10.4 .. 12.7 us, 2048 x 2048 at
+    // M = 128 / 256 13.7 / 14.1 -> 11.3 / 12.4 us, 2560 x 2560 15.8 / 16.2 / 20.7 -> 12.5 / 14.0 / 18.2 us, 1024 x 4096 at
+    // M = 128 11.6 -> 10.6 us (finer parts than these lose again: 1536 x 1536 at M = 256 in 6 parts 13.1 us).
+    if (pl.tiles * 2 < (int64_t)cus) {
+      int fine = (int)((int64_t)cus / pl.tiles);
+      if (fine > 8) fine = 8;
+      if (fine > G / 3) fine = G / 3;
+      if (fine > sk) sk = fine;
+    }
   }
   if (tuning().prefill_split > 0) sk = tuning().prefill_split <= G ? tuning().prefill_split : G;
   while (sk > 1 && (uint64_t)sk * (uint64_t)pl.tiles * pl.bm * pl.bn * 4 >= (1ull << 32)) --sk;   // 32-bit buffer offsets
