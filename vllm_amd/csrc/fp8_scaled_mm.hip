@@ -1144,6 +1144,18 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
       while (sk & (sk - 1)) --sk;
     }
     while (sk < 8 && steps / sk >= 100 && pl.tiles * sk * 2 <= 2 * (int64_t)cus) sk *= 2;
+    // between one and 1.75 workgroups per compute unit some units run two of them and set the pace: the parts that give
+    // one per unit instead, unless they get longer than 128 steps (13824 x 5120 at M = 65 .. 256, 80 tiles: 320 workgroups
+    // 41 .. 57 us, 240 workgroups 33 .. 42 us; 6656 x 6656 at M = 65, 208 tiles of 64 x 64: 20.8 -> 17.7 us unsplit;
+    // 17920 x 6656 at M = 512, 208 tiles: 97 us in two parts of 140 steps, 105 us unsplit)
+    const int64_t wgs = pl.tiles * sk;
+    if (sk > 1 && wgs > cus && wgs * 4 < (int64_t)cus * 7) {
+      const int fit = (int)((int64_t)cus / pl.tiles);
+      // (an unsplit K, which also saves the hand-over, from 75 % of the units on; fewer parts from 90 % on -- 14336 x 4096
+      // at M = 384, 96 tiles: 4 parts 52.0 us, 2 parts 54.8 us)
+      const int64_t filled = (int64_t)fit * pl.tiles;
+      if (fit >= 1 && steps / fit <= 128 && (fit == 1 ? filled * 4 >= (int64_t)cus * 3 : filled * 10 >= (int64_t)cus * 9)) sk = fit;
+    }
   }
   if (tuning().fp8_split > 0) sk = tuning().fp8_split <= steps ? tuning().fp8_split : steps;
   while (sk > 1 && (uint64_t)sk * (uint64_t)pl.tiles * pl.bm * pl.bn * 4 >= (1ull << 32)) --sk;   // 32-bit buffer offsets
