@@ -24,12 +24,12 @@ static int round_gs(int x, int sub, bool w8) {
 // Groups per slab are limited by LDS (128 KiB of activations, 256 bytes per group and staged row): 512 / rows.
 // G, gslab, gs and slab_max below count weight tiles: one per 128 rows of K, two (nibble planes) for 8-bit codes.
 // `nt_mult`: copies of every n-tile's stream that run side by side (rows split over workgroups, see the kernel).
-static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8, int nt_mult = 1) {
+static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8, int nt_mult = 1, bool allow8 = true) {
   const int TPG = w8 ? 2 : 1;
   const int G = K / 128 * TPG, NT = N / 16 * nt_mult;
   const int MB = (M + 15) / 16;
   Decode2Config c;
-  c.mr = M == 1 ? 1 : (M <= 4 ? 4 : (M <= 8 && sub == 1 && !w8 ? 8 : 16));      // rows staged (8: 4-bit codes in groups of 128 rows only)
+  c.mr = M == 1 ? 1 : (M <= 4 ? 4 : (M <= 8 && sub == 1 && !w8 && allow8 && tuning().exp[3] != 1 ? 8 : 16));      // rows staged (8: 4-bit codes in groups of 128 rows only)
   const int slab_max = 512 / (c.mr * MB) * TPG;
   c.sk = (G + slab_max - 1) / slab_max;
   const int gslab = (G + c.sk - 1) / c.sk;            // groups per slab
@@ -124,6 +124,14 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8, 
     else if (waves_cu <= 8) c.rc = 1;
   }
   if (tn.exp[1] > 0) c.rc = tn.exp[1] - 1;      // (development switch: forced ring variant + 1)
+  // 8 staged rows allow slabs twice as long, and a slab is a whole number of instantiated stream lengths: where that
+  // leaves a last slab of less than 60 % of the others the workgroups of the full slabs set the pace, and the plan for
+  // 16 staged rows (shorter, evener slabs) is taken instead (M = 8, cold: 10240 x 2560, slabs of 56 + 24 groups, 9.7 us
+  // against 7.5 us; 5120 x 27648, 32 + 8, 23.2 against 20.8 us; 17920 x 6656, 4 x 32 + 12, 20.0 against 16.9 us)
+  if (c.mr == 8 && c.sk > 1 && tn.decode2_gs <= 0 && tn.decode2_wks <= 0) {
+    const int slab = c.wks * c.gs, last = G - (c.sk - 1) * slab;
+    if (last * 10 < slab * 6) return pick_decode2_config(M, N, K, sub, w8, nt_mult, false);
+  }
   return c;
 }
 
