@@ -250,8 +250,9 @@ typedef struct VaqTuning {
   int quant_wg_per_row; /* per-token FP8 quant: 1 = always one workgroup per row                                     */
   int exp[15];          /* further switches of the same kind, for A/B timing runs: [0] = 1 shared instead of private  */
                         /*   activation fill, [1] = ring variant + 1, [2] rows over workgroups (1 off, 2 forced) of   */
-                        /*   the LDS-staged decode kernel, [3] = 1 sixteen staged rows for M = 5 .. 8; [4] FP8        */
-                        /*   streaming through LDS (1 / 2 / 3 = 8 / 4 / 16 steps per wavefront, 9 = off); rest unused  */
+                        /*   the LDS-staged decode kernel, [3] = 1 sixteen staged rows for M = 5 .. 8, [5] = 1 two K   */
+                        /*   slabs never merged into one; [4] FP8 streaming through LDS (1 / 2 / 3 = 8 / 4 / 16 steps   */
+                        /*   per wavefront, 9 = off); the rest unused                                                  */
 } VaqTuning;
 
 /* The entry points of the same name without `_tuned`, with `tuning` (may be NULL) applied to this call. */

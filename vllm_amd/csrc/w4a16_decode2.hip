@@ -11,6 +11,8 @@ struct Decode2Config {
   int rc;      // ring variant of long streams (see the kernel): 0 two slots refilled early, 1 / 2 four / three slots refilled late
 };
 
+static inline bool exp_off(const VaqTuning& tn, int i) { return tn.exp[i] != 1; }      // development switch i not set to "off"
+
 static int round_gs(int x, int sub, bool w8) {
   const int opts[] = {1, 2, 4, 7, 8, 14, 16};
   for (int o : opts) {
@@ -100,6 +102,18 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8, 
         gs = o;
         break;
       }
+  }
+  // Two slabs that twice the K slices would cover as one (at most 15 % of their tiles beyond K): one slab, no hand-over
+  // between workgroups.  Cold, M = 1 / 4 / 16: 3584 x 37888 (16 + 12 groups) 20.3 / 27.8 / 23.2 -> 17.7 / 17.7 / 19.6 us,
+  // 13824 x 5120 (64 + 44) 12.1 / 12.9 -> 11.0 / 11.9 us.
+  if (MB == 1 && sub == 1 && !w8 && !long_k_two_blocks && tn.decode2_gs <= 0 && tn.decode2_wks <= 0 && exp_off(tn, 5) &&
+      (G + wks * gs - 1) / (wks * gs) == 2 && wks * 2 <= 16) {
+    const int g2 = round_gs((G + 2 * wks - 1) / (2 * wks), sub, w8);
+    const int cover = 2 * wks * g2;
+    if (cover >= G && cover <= slab_max && (cover - G) * 100 <= G * 15) {
+      wks *= 2;
+      gs = g2;
+    }
   }
   // the slab is now wks*gs groups; recompute the number of slabs
   c.sk = (G + wks * gs - 1) / (wks * gs);
