@@ -257,7 +257,8 @@ def test_scaled_mm_small_m_every_route_exact(device, m):
     from vllm_amd import _tuning
     g = torch.Generator().manual_seed(m)
     for n, k in ((128, 1664), (256, 4096), (4096, 2048), (4112, 2048), (8208, 1664), (64, 1536), (128, 14336),
-                 (4096, 8192 + 128), (48, 4224), (128, 28672), (4112, 14336 + 256), (64, 16384 + 128)):
+                 (4096, 8192 + 128), (48, 4224), (272, 8192), (4112, 5120), (128, 28672), (4112, 14336 + 256),
+                 (64, 16384 + 128)):
         a = torch.randint(-2, 3, (m, k), generator=g).float()
         w = torch.randint(-1, 2, (n, k), generator=g).float()
         sa = torch.pow(2.0, -(torch.arange(m) % 2).float()).reshape(m, 1)

@@ -1310,7 +1310,9 @@ static int stream2_steps_per_wave(const Fp8MMParams& p) {
   int ks = 0;
   if (sw >= 1 && sw <= 3) ks = sw == 1 ? 8 : (sw == 2 ? 4 : 16);
   else if (MB == 1) ks = steps < 64 ? 8 : (steps <= 128 ? 16 : 0);      // (K = 8192: 8192 x 8192 at M = 1 16.9 us with 8 steps, 14.6 with 16)
-  else ks = steps > 32 ? 0 : (p.N / 16 > num_cus_current_device() ? 4 : 8);
+  // (two m-blocks of K = 4224 .. 8192 with 8 steps per wavefront, M = 24 / 32 against the kernel above: 5120 x 5120 13.9 / 14.7 ->
+  // 10.9 / 11.8 us, 6656 x 6656 16.8 / 18.0 -> 13.6 / 14.7 us, 5120 x 27648 38.2 / 39.2 -> 29.4 / 30.4 us, 8192 x 8192 20.9 / 22.3 -> 19.4 / 20.7 us)
+  else ks = steps > 64 ? 0 : (steps > 32 ? 8 : (p.N / 16 > num_cus_current_device() ? 4 : 8));
   if (ks == 0 || (steps + ks - 1) / ks > 8 || (MB == 2 && ks == 16)) return 0;
   return ks;
 }
