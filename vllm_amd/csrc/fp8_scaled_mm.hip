@@ -1097,8 +1097,26 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   // (4096 x 6144 at M = 384: 39 -> 27 us; 4096 x 4096 at M = 640: 38.5 -> 28 us)
   const bool take128 = tiles(128, 128) * parts128 * 10 >= cus * (parts128 == 2 ? 5 : 7) ||
                        (tiles(64, 128) > cus && tiles(128, 128) <= cus);
+  // ... and when the K parts that 256 x 256 tiles get, counted only down to 40 steps, bring them to 60 % of the compute units
+  // and M fills 80 % of their rows (cold: 18944 x 3584 at M = 640 .. 1024, 42 / 56 tiles in 4 parts, 94 .. 101 -> 76 .. 84 us;
+  // 8192 x 8192 at M = 640 / 768, 96 tiles in 2 parts, 84 / 81 -> 62 / 70 us; 14336 x 4096 at M = 640 / 768 79 -> 64 / 71 us;
+  // parts of 32 steps lose 5 %, 8192 x 8192 at M = 512; rows filled to 75 % lose 15 %, 13824 x 5120 at M = 384)
+  auto long_k_256 = [&]() {
+    const int64_t t = tiles(256, 256);
+    if (t >= cus || t < 1) return false;
+    // the parts these tiles would get below, of those only parts of at least 40 steps
+    const int min_steps = t * 4 <= cus ? 32 : 64;
+    int sk = (int)((int64_t)cus / t);
+    if (sk > 8) sk = 8;
+    if (sk > K / 64 / min_steps) sk = K / 64 / min_steps;
+    if (sk < 1) sk = 1;
+    while (sk & (sk - 1)) --sk;
+    while (sk > 1 && K / 64 / sk < 40) sk /= 2;
+    return t * sk * 10 >= (int64_t)cus * 6 && (int64_t)M * 5 >= (int64_t)((M + 255) / 256) * 256 * 4;
+  };
+  const bool take256 = tiles(256, 256) * parts256 * 20 >= cus * (parts256 == 2 ? 10 : 11) || long_k_256();
   if (pl.cfg <= 0)
-    pl.cfg = tiles(256, 256) * parts256 * 20 >= cus * (parts256 == 2 ? 10 : 11) ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (take128 ? 3 : 4));
+    pl.cfg = take256 ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (take128 ? 3 : 4));
   // the smallest tile with two k-slices per step: 5-8 % faster on a short K (half the barriers), no gain on a long one
   if (tuning().fp8_tile_cfg <= 0 && pl.cfg == 4 && K % 128 == 0 && K <= 8192) pl.cfg = 14;
   // 64 x 64 tiles while they fit the device in one round, on a short K: twice the workgroups with loads in flight
