@@ -44,6 +44,15 @@ static int pick_tile(int M, int N, int K, bool direct_ok) {
     // (from 55 % on: 4096 x 6144 at M = 1536, 144 tiles, 112 -> 85 us; at 50 %, 4096 x 4096 at M = 2048, 76 against 85 us)
     // (not for a single tile row that M fills at most half: 8192 x 28672 at M = 128, 104 against 85 us with 128 x 128)
     if (M > 128 && tiles(256, 256) * splits_256(tiles(256, 256), K, cus) * 20 >= cus * 11) return 20;      // 256 x 256, alternating phases
+    // An odd number of 64-row blocks on a short K: 64 x 128 tiles (the last 128-row tile would be half empty) where they
+    // come to 80-100 % of one or of two workgroups per compute unit (cold: 3584 x 18944 at M = 136 .. 192, 444 tiles, 60 ->
+    // 45 us; 2560 x 10240, 240 tiles, 30.8 -> 22.6 us; 4096 x 11008 at M = 288 / 320, 430 tiles, 67 -> 50 us; with 258 or
+    // 324 tiles they lose 15-20 %, and on K = 8192 as well)
+    // (three or five blocks; with seven or nine the half-empty tile is a tenth of the rows and these tiles lose 6-9 %)
+    if (M > 64 && M <= 320 && ((M + 63) / 64) % 2 == 1 && K <= 4096) {
+      const int64_t t = tiles(64, 128);
+      if ((t * 5 >= (int64_t)cus * 4 && t <= cus) || (t * 5 >= (int64_t)cus * 8 && t <= 2 * (int64_t)cus)) return 14;
+    }
     if (tiles(128, 128) >= cus) return 12;
     // Few tiles: 64 x 128, or 128 x 64 once M fills more than one 64-row tile (the dequantisation of a weight tile is
     // then shared by twice as many rows: 7-15 % faster at M = 128 .. 768 on the narrow layers); K is split over
