@@ -1169,10 +1169,11 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
     const int64_t wgs = pl.tiles * sk;
     if (sk > 1 && wgs > cus && wgs * 4 < (int64_t)cus * 7) {
       const int fit = (int)((int64_t)cus / pl.tiles);
-      // (an unsplit K, which also saves the hand-over, from 75 % of the units on; fewer parts from 90 % on -- 14336 x 4096
+      // (an unsplit K, which also saves the hand-over, from 60 % of the units on -- 6656 x 6656 at M = 136 / 192, 156 tiles:
+      // 41 / 45 -> 33 us, 7680 x 7680 47 / 51 -> 40 us; fewer parts from 90 % on -- 14336 x 4096
       // at M = 384, 96 tiles: 4 parts 52.0 us, 2 parts 54.8 us)
       const int64_t filled = (int64_t)fit * pl.tiles;
-      if (fit >= 1 && steps / fit <= 128 && (fit == 1 ? filled * 4 >= (int64_t)cus * 3 : filled * 10 >= (int64_t)cus * 9)) sk = fit;
+      if (fit >= 1 && steps / fit <= 128 && (fit == 1 ? filled * 5 >= (int64_t)cus * 3 : filled * 10 >= (int64_t)cus * 9)) sk = fit;
     }
   }
   if (tuning().fp8_split > 0) sk = tuning().fp8_split <= steps ? tuning().fp8_split : steps;
