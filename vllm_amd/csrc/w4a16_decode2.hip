@@ -115,6 +115,25 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8, 
       gs = g2;
     }
   }
+  // A last slab of less than 35 % of the others on a layer of at most two n-tiles per compute unit: the stream length
+  // (same K slices) that leaves the fewest tiles beyond K, a further slab counted as 3 %.  Cold, M = 1 / 4: 9216 x 4608
+  // (64 + 8 groups -> 3 x 28) 11.0 / 12.1 -> 8.9 / 9.3 us, 18944 x 3584 at M = 4 (64 + 64 + 20 -> 3 x 56) 13.5 -> 12.0 us; on
+  // a wide layer the further slab costs more than it brings (5120 x 27648, 32 + 8 -> 3 x 14: +3 .. +13 %).
+  if (MB == 1 && sub == 1 && !w8 && !long_k_two_blocks && tn.decode2_gs <= 0 && tn.decode2_wks <= 0 && exp_off(tn, 5) &&
+      NT <= 2 * cus) {
+    auto slabs = [&](int g) { return (G + wks * g - 1) / (wks * g); };
+    const int sk0 = slabs(gs), last = G - (sk0 - 1) * wks * gs;
+    if (sk0 >= 2 && last * 20 < wks * gs * 7) {
+      auto score = [&](int g) { return (double)(slabs(g) * wks * g - G) / G + 0.03 * slabs(g); };
+      int bg = gs;
+      double best = score(gs);
+      for (int g : {16, 14, 8, 7}) {
+        if (wks * g > slab_max || slabs(g) > 10) continue;
+        if (score(g) < best - 1e-9) { best = score(g); bg = g; }
+      }
+      gs = bg;
+    }
+  }
   // the slab is now wks*gs groups; recompute the number of slabs
   c.sk = (G + wks * gs - 1) / (wks * gs);
   c.gs = gs;
