@@ -134,6 +134,28 @@ static Decode2Config pick_decode2_config(int M, int N, int K, int sub, bool w8, 
       gs = bg;
     }
   }
+  // One slab whose streams reach 35 % and more beyond K (wavefronts without tiles) on a layer of at most 1.25 n-tiles per
+  // compute unit: two or three slabs of streams of 7 tiles and more (the K slices as planned or half of them) that fit K
+  // better.  Cold, M = 2 / 4 / 16: 5120 x 5120 (4 x 14 for 40 groups -> 3 slabs of 2 x 7) 7.9 / 7.9 / 8.6 -> 6.9 / 6.9 / 7.4 us,
+  // 10240 x 2560 (8 x 14 for 80 -> 3 slabs of 4 x 7) 8.0 / 8.0 -> 6.8 / 6.9 us, 9216 x 2304 8.0 -> 6.8 us; wider layers lose with
+  // it (2560 x 10240, 5120 x 15360: +20 .. +60 %), so do a single row (10240 x 4096: +18 %) and a K of 2560 (+11 .. +14 %);
+  // 10240 x 4096 at M = 2 / 4 is 3 % slower with it.
+  if (MB == 1 && sub == 1 && !w8 && !long_k_two_blocks && tn.decode2_gs <= 0 && tn.decode2_wks <= 0 && exp_off(tn, 5) &&
+      c.mr >= 4 && G >= 32 && NT * 4 <= cus * 5 && wks <= 8 && wks * gs >= G && (wks * gs - G) * 100 >= G * 35) {
+    auto slabs = [&](int w, int g) { return (G + w * g - 1) / (w * g); };
+    auto score = [&](int w, int g) { return (double)(slabs(w, g) * w * g - G) / G + 0.03 * slabs(w, g); };
+    int bw = wks, bg = gs;
+    double best = score(wks, gs);
+    for (int w : {wks, wks / 2}) {
+      if (w < 1) continue;
+      for (int g : {14, 8, 7}) {
+        if (w * g > slab_max || slabs(w, g) > 3) continue;
+        if (score(w, g) < best - 1e-9) { best = score(w, g); bw = w; bg = g; }
+      }
+    }
+    wks = bw;
+    gs = bg;
+  }
   // the slab is now wks*gs groups; recompute the number of slabs
   c.sk = (G + wks * gs - 1) / (wks * gs);
   c.gs = gs;
