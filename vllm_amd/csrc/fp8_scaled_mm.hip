@@ -1124,6 +1124,11 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   // M = 128 30.0 -> 34.0 us, and slower as soon as the tiles need a second round)
   if (tuning().fp8_tile_cfg <= 0 && pl.cfg == 14 && tiles(64, 64) <= cus) pl.cfg = 15;
   if (pl.cfg >= 10 && K % 128 != 0) pl.cfg %= 10;      // two k-slices per step need K % 128 == 0
+  int sk = 1;
+  const int steps = K / 64;
+  Fp8TilePlan saved = pl;
+  for (int pass = 0; pass < 2; ++pass) {
+  sk = 1;
   switch (pl.cfg) {
     case 3: case 13: case 23: pl.bm = 128; pl.bn = 128; pl.nw = 4; break;
     case 4: case 14: case 24: pl.bm = 64; pl.bn = 128; pl.nw = 4; break;
@@ -1133,8 +1138,6 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
     default: pl.bm = 256; pl.bn = 256; pl.nw = 8; break;
   }
   pl.tiles = tiles(pl.bm, pl.bn);
-  int sk = 1;
-  const int steps = K / 64;
   if (pl.tiles < cus && pl.bm * pl.bn >= 128 * 256) {
     // large tiles, one workgroup per compute unit
     const int min_steps = pl.tiles * 4 <= cus ? 32 : 64;        // shorter parts only when the tiles leave 3/4 of the device idle
@@ -1175,6 +1178,28 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
       const int64_t filled = (int64_t)fit * pl.tiles;
       if (fit >= 1 && steps / fit <= 128 && (fit == 1 ? filled * 5 >= (int64_t)cus * 3 : filled * 10 >= (int64_t)cus * 9)) sk = fit;
     }
+  }
+  // 64 x 128 tiles of a long K whose parts still run 64 steps and more: 128 x 128 tiles instead -- half the tiles, so twice
+  // the parts of half the length on the same number of workgroups (cold, M = 80 .. 128: 18944 x 3584 33.8 -> 31.7 us,
+  // 9216 x 4608 30.7 -> 25.9 us, 17920 x 6656 52.6 -> 42.2 us, 24576 x 6144 71.7 -> 61.1 us; M = 136 .. 256: 12288 x 3072
+  // 41 -> 32 us; with parts of 56 steps and less they lose 1-9 %: 14336 x 4096, 11008 x 4096, 10240 x 2560)
+  // -- where those are fewer tiles (M beyond one 64-row block) and come to at least 80 % of the workgroups, or of the compute
+  // units if the 64 x 128 tiles exceed them (13824 x 5120, 20480 x 5120: 240 against 160 workgroups, +3 .. +9 %)
+  if (pass == 0 && tuning().fp8_tile_cfg <= 0 && tuning().fp8_split <= 0 && pl.cfg == 4 && steps / sk >= 64 &&
+      tiles(128, 128) < pl.tiles) {
+    saved = pl;
+    saved.sk = sk;
+    pl.cfg = 3;
+    continue;
+  }
+  if (pass == 1) {
+    const int64_t w4 = saved.tiles * saved.sk < cus ? saved.tiles * saved.sk : cus;
+    if (pl.tiles * sk * 10 < w4 * 8) {      // too few workgroups: back to the 64 x 128 plan
+      pl = saved;
+      sk = saved.sk;
+    }
+  }
+  break;
   }
   if (tuning().fp8_split > 0) sk = tuning().fp8_split <= steps ? tuning().fp8_split : steps;
   while (sk > 1 && (uint64_t)sk * (uint64_t)pl.tiles * pl.bm * pl.bn * 4 >= (1ull << 32)) --sk;   // 32-bit buffer offsets
