@@ -64,6 +64,21 @@ static int pick_tile(int M, int N, int K, bool direct_ok) {
     //    M = 192: 28.2 -> 23.4 us; 4096 x 4096 at M = 320: 28.1 -> 23.5 us).
     if ((tiles(128, 64) >= cus && tiles(128, 128) * 2 >= cus) || (K >= 8192 && tiles(128, 128) * 8 >= (int64_t)cus * 3)) return 12;
     if (M > 64 && ((M + 63) / 64) % 2 == 1 && tiles(64, 128) <= cus) return 14;
+    if (M > 64 && tuning().exp[8] != 1) {
+      // 128 x 64 tiles whose K parts (two workgroups per compute unit, at most 8 parts of at least 8 groups) would still
+      // run 24 groups and more: 128 x 128 tiles, half as many, in twice the parts, where that is at least 80 % as many
+      // workgroups (cold: 28672 x 8192 at M = 80 .. 128 92 -> 81 us, 22016 x 4096 at M = 256 74 -> 67 us, 12288 x 3072 at
+      // M = 384 50.6 -> 46.5 us, 13824 x 5120, 18944 x 3584, 6656 x 6656, 7168 x 7168 at M = 256 -5 .. -7 %; 12288 x 3072 at
+      // M = 640 +4 %)
+      auto parts = [&](int64_t t) {
+        int sk = (int)((2 * (int64_t)cus) / t);
+        if (sk > 8) sk = 8;
+        if (sk > K / 128 / 8) sk = K / 128 / 8;
+        return sk < 1 ? 1 : sk;
+      };
+      const int64_t t15 = tiles(128, 64), t12 = tiles(128, 128);
+      if (t15 < cus && K / 128 / parts(t15) >= 24 && t12 * parts(t12) * 10 >= t15 * parts(t15) * 8) return 12;
+    }
     return M > 64 ? 15 : 14;
   }
   if (tiles(256, 256) >= cus) return 0;
