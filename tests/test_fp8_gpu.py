@@ -433,6 +433,31 @@ def test_scaled_mm_split_k_exact_and_deterministic(device):
         assert all(bool((t == 0).all()) for t in ops._FP8_COUNTERS.values()), "arrival counters not restored to zero"
 
 
+@pytest.mark.parametrize("k,n", [(13824, 5120), (6656, 6656), (18944, 3584), (9216, 4608), (5120, 5120)])
+def test_tile_plan_branches_other_model_shapes(device, k, n):
+    """Layer shapes of other models on which the tile planner takes branches that the Llama-3-8B shapes do not reach
+    (K parts rebalanced to one workgroup per compute unit, an unsplit K from 60 % fill on, 256 x 256 tiles in parts of
+    a long K, 128 x 128 instead of 64 x 128 tiles for long parts, two m-blocks of K up to 8192 through LDS rings):
+    per-token x per-channel with bias, sampled rows against the fp64 oracle, bit-identical run to run, arrival
+    counters back at zero."""
+    import vllm_amd._custom_ops as ops
+    w_q, sb = f.make_fp8_weight(n, k, seed=3)
+    w_dev = w_q.to(device).t()
+    g = torch.Generator().manual_seed(4)
+    bias = (torch.randn(n, generator=g) * 0.01).to(torch.bfloat16)
+    for m in (24, 32, 65, 96, 136, 192, 256, 384, 640, 896):
+        a = torch.randn(m, k, generator=g).to(torch.bfloat16)
+        a_q, sa = ops.scaled_fp8_quant(a.to(device), use_per_token_if_dynamic=True)
+        rows = np.concatenate([np.random.default_rng(m).choice(m, 14, replace=False), [0, m - 1]])
+        out = ops.cutlass_scaled_mm(a_q, w_dev, sa, sb.to(device), torch.bfloat16, bias.to(device))
+        ref = f.scaled_mm_ref(a_q[rows].cpu(), w_q.t(), sa[rows].cpu(), sb, torch.bfloat16, bias)
+        _check_mm(out[rows], ref, f"k={k} n={n} m={m}")
+        assert torch.isfinite(out.float()).all()
+        again = ops.cutlass_scaled_mm(a_q, w_dev, sa, sb.to(device), torch.bfloat16, bias.to(device))
+        assert torch.equal(out, again), f"k={k} n={n} m={m}: not deterministic run to run"
+    assert all(bool((t == 0).all()) for t in ops._FP8_COUNTERS.values())
+
+
 @pytest.mark.parametrize("k,n", LLAMA_SHAPES)
 def test_config4_llama_shapes(device, k, n):
     """BASELINE.json config 4: M in {1, 16, 256, 4096}, per-token x per-channel (+bias); activations quantised on the GPU

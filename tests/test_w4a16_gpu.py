@@ -439,6 +439,31 @@ def test_decode_three_and_four_m_blocks(device, k, n, m):
         assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
 
 
+# layer shapes of other models on which the planners take branches that the Llama-3-8B shapes do not reach: K slabs that
+# would come out uneven (9216 x 4608, 10240 x 2560), a ragged single slab on a narrow layer (5120 x 5120), a short K on
+# few tiles (1536 x 1536), an odd number of 64-row blocks on a wide short-K layer (2560 x 10240), long K parts on few
+# 128 x 64 tiles (12288 x 3072)
+OTHER_MODEL_SHAPES = [(9216, 4608), (10240, 2560), (5120, 5120), (1536, 1536), (2560, 10240), (12288, 3072)]
+
+
+@pytest.mark.parametrize("k,n", OTHER_MODEL_SHAPES)
+def test_planner_branches_other_model_shapes(device, k, n):
+    """Symmetric 4-bit, groups of 128, M across the decode and tile kernels; M <= 64 against the full fp64 oracle, larger M
+    on sampled rows.  Run to run the result must be bit-identical (the K splits sum in a fixed order) and the arrival
+    counters must be back at zero."""
+    case = o.make_w4a16_case(k, n, 128, seed=k + n)
+    layer = W4A16Layer(case, device)
+    w_ref = o.case_w_ref(case)
+    for m in (1, 2, 4, 8, 16, 32, 48, 96, 160, 256, 384, 640):
+        a = _acts(m, k, device, seed=m)
+        out = layer(a)
+        rows = np.arange(m) if m <= 64 else np.concatenate([np.random.default_rng(m).choice(m, 16, replace=False), [0, m - 1]])
+        check_gemm_close(out[rows], o.gemm_ref(a.cpu()[rows], w_ref), f"k={k} n={n} m={m}")
+        assert torch.isfinite(out).all() and bool((out.float().norm(dim=1) > 0).all())
+        assert torch.equal(out, layer(a)), f"k={k} n={n} m={m}: not deterministic run to run"
+    assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
+
+
 @pytest.mark.parametrize("k,n", LLAMA_SHAPES)
 @pytest.mark.parametrize("group_level", [False, True])
 def test_config3_prefill_llama_shapes_sampled(device, k, n, group_level):
