@@ -1115,8 +1115,12 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
     return t * sk * 10 >= (int64_t)cus * 6 && (int64_t)M * 5 >= (int64_t)((M + 255) / 256) * 256 * 4;
   };
   const bool take256 = tiles(256, 256) * parts256 * 20 >= cus * (parts256 == 2 ? 10 : 11) || long_k_256();
+  // (not when M fills less than 70 % of the 256-row tiles and the 128 x 256 tiles fit the device in one round: 3584 x 18944
+  // at M = 288 / 320, 222 tiles, 47.4 -> 41.3 us; on 4096 x 28672, 336 tiles, the 256 x 256 tiles stay ahead, 53 against 75 us)
+  const bool rows_poorly_filled = (int64_t)M * 10 < (int64_t)((M + 255) / 256) * 256 * 7 && tiles(128, 256) <= cus &&
+                                  tiles(128, 256) * 10 >= cus * 7 && tuning().exp[9] != 1;
   if (pl.cfg <= 0)
-    pl.cfg = take256 ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (take128 ? 3 : 4));
+    pl.cfg = take256 && !rows_poorly_filled ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (take128 ? 3 : 4));
   // the smallest tile with two k-slices per step: 5-8 % faster on a short K (half the barriers), no gain on a long one
   if (tuning().fp8_tile_cfg <= 0 && pl.cfg == 4 && K % 128 == 0 && K <= 8192) pl.cfg = 14;
   // 64 x 64 tiles while they fit the device in one round, on a short K: twice the workgroups with loads in flight

@@ -43,7 +43,12 @@ static int pick_tile(int M, int N, int K, bool direct_ok) {
     // takes a split of a long K to get there (14336 x 4096 at M = 1024 / 2048: 4 % / 21 % faster than 128 x 128)
     // (from 55 % on: 4096 x 6144 at M = 1536, 144 tiles, 112 -> 85 us; at 50 %, 4096 x 4096 at M = 2048, 76 against 85 us)
     // (not for a single tile row that M fills at most half: 8192 x 28672 at M = 128, 104 against 85 us with 128 x 128)
-    if (M > 128 && tiles(256, 256) * splits_256(tiles(256, 256), K, cus) * 20 >= cus * 11) return 20;      // 256 x 256, alternating phases
+    // (... nor when M fills less than 70 % of the 256-row tiles and the 128 x 128 tiles fit the device in one round of two
+    // workgroups per compute unit: 3584 x 18944 at M = 288 / 320, 444 tiles, 78 -> 63 us; on 4096 x 28672, 672 tiles, the
+    // 256 x 256 tiles stay ahead, 90 against 108 us)
+    const bool rows_poorly_filled = (int64_t)M * 10 < (int64_t)((M + 255) / 256) * 256 * 7 && tiles(128, 128) <= 2 * (int64_t)cus &&
+                                    tuning().exp[9] != 1;
+    if (M > 128 && !rows_poorly_filled && tiles(256, 256) * splits_256(tiles(256, 256), K, cus) * 20 >= cus * 11) return 20;      // 256 x 256, alternating phases
     // An odd number of 64-row blocks on a short K: 64 x 128 tiles (the last 128-row tile would be half empty) where they
     // come to 80-100 % of one or of two workgroups per compute unit (cold: 3584 x 18944 at M = 136 .. 192, 444 tiles, 60 ->
     // 45 us; 2560 x 10240, 240 tiles, 30.8 -> 22.6 us; 4096 x 11008 at M = 288 / 320, 430 tiles, 67 -> 50 us; with 258 or
