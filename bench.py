@@ -211,8 +211,12 @@ def stream_ceiling_section(dev):
     once), best of a few wavefront counts and depths per size.  The sum over the 12 headline GEMMs is the practical
     ceiling the headline is also priced against."""
     import ctypes
-    from vllm_amd import _lib
-    lib = _lib.load()
+    from vllm_amd.build import BENCH_PROBE_PATH
+    if not BENCH_PROBE_PATH.exists():
+        raise RuntimeError(f"{BENCH_PROBE_PATH.name} is not built")
+    lib = ctypes.CDLL(str(BENCH_PROBE_PATH))
+    lib.vaq_stream_read_probe.restype = ctypes.c_int
+    lib.vaq_stream_read_probe.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
     rows = []
     sink = torch.zeros(4, dtype=torch.int32, device=dev)
     pool = torch.empty(640 << 20, dtype=torch.uint8, device=dev).random_()
@@ -228,8 +232,10 @@ def stream_ceiling_section(dev):
 
                 def fn():
                     for c in range(copies):
-                        _lib.check(lib.vaq_stream_read_probe(ctypes.c_void_p(pool.data_ptr() + c * (nbytes & ~1023)), nbytes, waves,
-                                                             depth, ctypes.c_void_p(sink.data_ptr()), stream()))
+                        rc = lib.vaq_stream_read_probe(ctypes.c_void_p(pool.data_ptr() + c * (nbytes & ~1023)), nbytes, waves,
+                                                       depth, ctypes.c_void_p(sink.data_ptr()), stream())
+                        if rc != 0:
+                            raise RuntimeError(f"vaq_stream_read_probe returned {rc}")
                 t = time_graph(fn, iters=5, warmup=2, inner=copies)
                 read = (nbytes // 1024 // waves) * waves * 1024
                 t_full = t * nbytes / read                                  # (the probe reads whole KiB per wavefront)
@@ -674,6 +680,39 @@ def cpu_baseline(budget_s: float = 15.0):
                        f"scaled matmul at M={m}, {k}x{n}: {fp8_mm_bytes(m, k, n, False) / f8_t / 1e9:.3f} GB/s")
 
 
+# --------------------------------------------------------------------------------------------- output
+
+MAX_LINE_BYTES = 4096
+
+
+def final_line(record: dict) -> str:
+    """The one JSON line for stdout: the headline record without the per-section tables, at most MAX_LINE_BYTES long so
+    that a reader who keeps only the tail of stdout still gets all of it.  Over the limit, the free-text fields are
+    shortened first and the compact matrix-core rows dropped last; the headline, `roofline` and `cpu_baseline` stay."""
+    rec = {k: v for k, v in record.items() if k != "extra"}
+    line = json.dumps(rec, separators=(",", ":"))
+    if len(line) > MAX_LINE_BYTES and isinstance(rec.get("cpu_baseline"), dict):
+        rec["cpu_baseline"] = dict(rec["cpu_baseline"], sample=str(rec["cpu_baseline"].get("sample", ""))[:200])
+        line = json.dumps(rec, separators=(",", ":"))
+    if len(line) > MAX_LINE_BYTES:
+        rec.pop("roofline_mfma", None)
+        line = json.dumps(rec, separators=(",", ":"))
+    assert len(line) <= MAX_LINE_BYTES and "\n" not in line
+    return line
+
+
+def write_extra(extra: dict, path: str | None = None) -> None:
+    """The per-section tables (per-shape decode, prefill, FP8, vendor library, ...) go to a side file, never to stdout."""
+    path = path or os.path.join(os.path.dirname(os.path.abspath(__file__)), "gpurun_out", "bench_extra.json")
+    try:
+        os.makedirs(os.path.dirname(path), exist_ok=True)
+        with open(path, "w") as f:
+            json.dump(extra, f, indent=1)
+        log(f"[extra] per-section tables written to {path}")
+    except OSError as e:
+        log(f"[extra] not written ({e})")
+
+
 # --------------------------------------------------------------------------------------------- main
 
 def main():
@@ -771,9 +810,9 @@ def main():
                      "practical_frac": None if practical is None else round(value / practical, 4)},
         "roofline_mfma": roofline_mfma(extra),
         "cpu_baseline": cpu,
-        "extra": extra,
     }
-    print(json.dumps(out))
+    write_extra(extra)
+    print(final_line(out))
 
 
 if __name__ == "__main__":

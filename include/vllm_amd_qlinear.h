@@ -24,6 +24,9 @@
 extern "C" {
 #endif
 
+/* The library is built with hidden visibility; only what this header declares is exported. */
+#pragma GCC visibility push(default)
+
 #define VAQ_OK 0
 #define VAQ_ERR_INVALID_ARG (-1)   /* shape / stride / alignment / enum check failed (TORCH_CHECK analogue)   */
 #define VAQ_ERR_UNSUPPORTED (-2)   /* valid request outside what is built (TORCH_CHECK_NOT_IMPLEMENTED analogue) */
@@ -225,63 +228,7 @@ int vaq_fp8_scaled_mm_ws(const uint8_t* a, int64_t lda, const uint8_t* b, int64_
                          int64_t size_m, int64_t size_n, int64_t size_k, float* c_tmp, int64_t c_tmp_bytes,
                          int32_t* counters, int64_t counter_ints, void* stream);
 
-/*
- * Kernel-variant overrides for tests and benchmarks.  No counterpart in the reference (its kernels take no such
- * argument); the drop-in surface never passes one.  A VaqTuning applies to the ONE call it is handed to, on the calling
- * thread only: the library keeps no tuning state between calls.  Every field: 0 = the automatic choice.
- */
-typedef struct VaqTuning {
-  int decode_impl;      /* W4A16 decode kernel: 1 LDS-staged activations, 2 register-resident activations          */
-  int decode2_gs;       /* LDS-staged kernel: weight tiles per wavefront                                             */
-  int decode2_wks;      /*   K slices per workgroup                                                                  */
-  int decode2_wn;       /*   n-tiles per workgroup                                                                   */
-  int decode_tg;        /* register-resident kernel: groups per wavefront                                            */
-  int decode_wk;        /*   wavefronts along K per workgroup                                                        */
-  int decode_gx;        /*   workgroups along N                                                                      */
-  int decode_depth;     /*   prefetch depth                                                                          */
-  int prefill_tile;     /* W4A16 tile kernel: tile id + 1                                                            */
-  int prefill_split;    /*   K split                                                                                 */
-  int fp8_path;         /* FP8 GEMM: 1 weight-streaming kernel, 2 tile kernel                                        */
-  int fp8_tile_impl;    /*   1 register-staged tile kernel                                                           */
-  int fp8_tile_cfg;     /*   multi-stage tile shape id, -1 = two-stage kernel                                        */
-  int fp8_split;        /*   K split of the tile kernel                                                              */
-  int fp8_gx;           /*   workgroups of the weight-streaming kernel                                               */
-  int fp8_stream_split; /*   -1 = never run the weight-streaming kernel over two halves of K                         */
-  int quant_wg_per_row; /* per-token FP8 quant: 1 = always one workgroup per row                                     */
-  int exp[15];          /* further switches of the same kind, for A/B timing runs: [0] = 1 shared instead of private  */
-                        /*   activation fill, [1] = ring variant + 1, [2] rows over workgroups (1 off, 2 forced) of   */
-                        /*   the LDS-staged decode kernel, [3] = 1 sixteen staged rows for M = 5 .. 8, [5] = 1 two K   */
-                        /*   slabs never merged into one; [4] FP8 streaming through LDS (1 / 2 / 3 = 8 / 4 / 16 steps   */
-                        /*   per wavefront, 9 = off); [8] = 1 W4A16 tile kernel: no 128 x 128 tiles for long K parts;   */
-                        /*   [9] = 1 both tile kernels: 256-row tiles also when M fills them poorly; the rest unused   */
-} VaqTuning;
-
-/* The entry points of the same name without `_tuned`, with `tuning` (may be NULL) applied to this call. */
-int vaq_w4a16_gemm_workspace_tuned(int64_t size_m, int64_t size_n, int64_t size_k, int has_perm, int device,
-                                   size_t* c_tmp_bytes, size_t* a_tmp_bytes, size_t* counter_ints,
-                                   const VaqTuning* tuning);
-int vaq_w4a16_gemm_tuned(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
-                         const int32_t* perm, const void* bias, void* c, float* c_tmp, int64_t c_tmp_bytes, void* a_tmp,
-                         int32_t* counters, int64_t counter_ints, int64_t size_m, int64_t size_n, int64_t size_k,
-                         int group_size, int dtype, int wtype, int force_path, void* stream, const VaqTuning* tuning);
-int vaq_fp8_scaled_mm_workspace_tuned(int64_t size_m, int64_t size_n, int64_t size_k, size_t* c_tmp_bytes,
-                                      size_t* counter_ints, const VaqTuning* tuning);
-int vaq_fp8_scaled_mm_ws_tuned(const uint8_t* a, int64_t lda, const uint8_t* b, int64_t ldb, const float* sa,
-                               int64_t sa_count, const float* sb, int64_t sb_count, const void* bias, void* out,
-                               int64_t ldc, int out_dtype, int64_t size_m, int64_t size_n, int64_t size_k, float* c_tmp,
-                               int64_t c_tmp_bytes, int32_t* counters, int64_t counter_ints, void* stream,
-                               const VaqTuning* tuning);
-int vaq_fp8_quant_per_token_tuned(const void* in, int in_dtype, int64_t in_row_stride, uint8_t* out,
-                                  int64_t out_row_stride, float* scales, const float* scale_ub, int64_t rows,
-                                  int64_t hidden, void* stream, const VaqTuning* tuning);
-
-/*
- * Measurement aid (no counterpart in the reference): a kernel that only reads `bytes` (rounded down to whole KiB per
- * wavefront) from `src`, `waves` wavefronts (a multiple of 4) with `depth` (2, 4 or 8) 16-byte loads per lane in flight.
- * The benchmark times it on cold buffers of each layer's size to report the practical ceiling of the memory-bound
- * kernels beside the nominal HBM peak.  `sink` is a device word that is practically never written.
- */
-int vaq_stream_read_probe(const void* src, int64_t bytes, int waves, int depth, void* sink, void* stream);
+#pragma GCC visibility pop
 
 #ifdef __cplusplus
 }

@@ -16,9 +16,26 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 # ------------------------------------------------------------------------------------------------ C ABI
 
 def _header_symbols():
-    text = open(os.path.join(ROOT, "include", "vllm_amd_qlinear.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(vaq_[a-z0-9_]+)\s*\(", text)))
+    """Declared by the drop-in header plus the library's own tuning header (tests and benchmarks only)."""
+    names = set()
+    for path in (("include", "vllm_amd_qlinear.h"), ("vllm_amd", "csrc", "vaq_tuning.h")):
+        text = open(os.path.join(ROOT, *path)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(vaq_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
+
+
+def test_library_exports_nothing_but_the_c_abi():
+    """Built with hidden visibility: the dynamic symbol table holds the declared entry points and no C++ internals."""
+    import subprocess
+    from vllm_amd import _lib
+    out = subprocess.run(["nm", "-D", "--defined-only", str(_lib.LIB_PATH)], capture_output=True, text=True, check=True).stdout
+    # only code: the data symbols that remain are the device-code registration objects the HIP toolchain emits itself
+    defined = sorted(l.split()[-1] for l in out.splitlines() if l.split() and l.split()[-2] in "Tt")
+    extra = [n for n in defined if n not in _header_symbols() and not n.startswith(("_init", "_fini"))]
+    assert not extra, f"symbols exported beyond the headers: {extra[:10]}"
+    drop_in = open(os.path.join(ROOT, "include", "vllm_amd_qlinear.h")).read()
+    assert "VaqTuning" not in drop_in and "_tuned" not in drop_in and "probe" not in drop_in
 
 
 def test_library_loads_and_exports_every_declared_symbol():

@@ -34,7 +34,6 @@ _SIGNATURES = {
                                c_int, c_void_p]),
     "vaq_w4a16_gemm_static": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                       c_int64, c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
-    "vaq_stream_read_probe": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p]),
     "vaq_permute_cols": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
     "vaq_fp8_quant_per_token": (c_int, [c_void_p, c_int, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
                                         c_int64, c_void_p]),

@@ -1,9 +1,10 @@
-// Measurement aid, not part of the quantized-linear path: a kernel that does nothing but read a buffer, every load of
+// Measurement aid, not part of the quantized-linear library (built into libvaq_bench_probe.so, which only the
+// benchmark loads): a kernel that does nothing but read a buffer, every load of
 // a wavefront in flight at once.  Launched inside the same kind of HIP graph as the decode GEMMs, on buffers of a
 // layer's size that have left the caches, its launch-to-launch time is the ceiling any kernel that has to read those
 // bytes can reach on this machine (launch gap + first-byte latency + streaming): the "practical peak" the benchmark
 // reports beside the nominal 8 TB/s.
-#include "vaq_common.h"
+#include "../vaq_common.h"
 
 namespace vaq {
 
@@ -27,18 +28,20 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const v4u* __restrict_
 
 }  // namespace vaq
 
-extern "C" int vaq_stream_read_probe(const void* src, int64_t bytes, int waves, int depth, void* sink, void* stream) {
+// Reads `bytes` (rounded down to whole KiB per wavefront) from `src` with `waves` wavefronts (a multiple of 4) and
+// `depth` (2, 4 or 8) 16-byte loads per lane in flight.  `sink` is a device word that is practically never written.
+// Returns 0, or -1 for arguments it does not take and -3 for a refused launch.
+extern "C" __attribute__((visibility("default"))) int vaq_stream_read_probe(const void* src, int64_t bytes, int waves, int depth, void* sink, void* stream) {
   using namespace vaq;
-  VAQ_CHECK_ARG(src && sink && ((uintptr_t)src % 16) == 0, "stream_read_probe: src must be a 16-byte aligned device pointer");
-  VAQ_CHECK_ARG(waves > 0 && waves % 4 == 0 && waves <= (1 << 20), "stream_read_probe: waves = %d must be a positive multiple of 4", waves);
-  VAQ_CHECK_ARG(depth == 2 || depth == 4 || depth == 8, "stream_read_probe: depth = %d (2, 4 or 8 loads in flight)", depth);
+  if (!(src && sink && ((uintptr_t)src % 16) == 0)) return -1;
+  if (!(waves > 0 && waves % 4 == 0 && waves <= (1 << 20))) return -1;
+  if (!(depth == 2 || depth == 4 || depth == 8)) return -1;
   const int64_t per = bytes / 1024 / waves;
-  VAQ_CHECK_ARG(per >= 1 && per < (1 << 30), "stream_read_probe: %lld bytes over %d wavefronts", (long long)bytes, waves);
+  if (!(per >= 1 && per < (1 << 30))) return -1;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid(waves / 4), block(256);
   if (depth == 2) hipLaunchKernelGGL(stream_read_kernel<2>, grid, block, 0, s, (const v4u*)src, (uint32_t*)sink, (int)per);
   else if (depth == 4) hipLaunchKernelGGL(stream_read_kernel<4>, grid, block, 0, s, (const v4u*)src, (uint32_t*)sink, (int)per);
   else hipLaunchKernelGGL(stream_read_kernel<8>, grid, block, 0, s, (const v4u*)src, (uint32_t*)sink, (int)per);
-  VAQ_CHECK_LAUNCH("stream_read_probe");
-  return VAQ_OK;
+  return hipGetLastError() == hipSuccess ? 0 : -3;
 }

@@ -7,6 +7,7 @@
 #include <stdio.h>
 
 #include "../../include/vllm_amd_qlinear.h"
+#include "vaq_tuning.h"
 
 namespace vaq {
 
