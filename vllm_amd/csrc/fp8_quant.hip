@@ -2,7 +2,8 @@
 //
 // Bit-exactness contract (codes AND scales) with the reference kernels:
 //   per token : amax = max|float(x)| ; s = max(min(amax, ub) / 448, 1/(448*512)) ; q = cvt(clamp(float(x) / s, +-448))
-//               -- a true IEEE fp32 division per element, not a reciprocal multiply;
+//               -- the correctly rounded fp32 quotient per element, not a reciprocal multiply (for 16-bit inputs without
+//               an upper bound on the scale it comes from div16_exact: three instructions, the same bits);
 //   per tensor: s = amax_all / 448 ; q = cvt(clamp(float(x) * (1 / s), +-448))   (reciprocal multiply);
 //   static    : q = cvt(clamp(float(x) * (1 / scale), +-448)).
 // cvt is the hardware v_cvt_pk_fp8_f32 (round-to-nearest-even; inputs are already clamped, NaN stays NaN).
@@ -134,20 +135,38 @@ __global__ __launch_bounds__(QT) void fp8_quant_kernel(const T* __restrict__ in,
     }
   }
 
+  // MODE 0 on 16-bit inputs whose quotients cannot leave the normal range (no upper bound that could shrink the scale
+  // below amax / 448, finite scale): the exact three-instruction division; the same for every thread of the row
+  bool fast = false;
+  float rcp = 0.f;
+  if constexpr (MODE == 0 && sizeof(T) == 2) {
+    fast = scale_ub == nullptr && scale_or_inv < __builtin_inff();
+    rcp = 1.0f / scale_or_inv;
+  }
   auto conv = [&](float v) -> float {
     if constexpr (MODE == 0) return clamp448(v / scale_or_inv);
     else return clamp448(v * scale_or_inv);
   };
+  auto conv_fast = [&](float v) -> float { return clamp448(div16_exact(v, scale_or_inv, rcp)); };
+  auto pack8 = [&](const float (&f)[8], auto&& cv) {
+    v2u o;
+    o.x = cvt2(cv(f[0]), cv(f[1])) | (cvt2(cv(f[2]), cv(f[3])) << 16);
+    o.y = cvt2(cv(f[4]), cv(f[5])) | (cvt2(cv(f[6]), cv(f[7])) << 16);
+    return o;
+  };
 
   if (vec_ok) {
+    if (fast) {
 #pragma unroll
-    for (int i = 0; i < QV; ++i) {
-      const int v = tid + i * QT;
-      if (v < nvec) {
-        v2u o;
-        o.x = cvt2(conv(cache[i].f[0]), conv(cache[i].f[1])) | (cvt2(conv(cache[i].f[2]), conv(cache[i].f[3])) << 16);
-        o.y = cvt2(conv(cache[i].f[4]), conv(cache[i].f[5])) | (cvt2(conv(cache[i].f[6]), conv(cache[i].f[7])) << 16);
-        *reinterpret_cast<v2u*>(y + (int64_t)v * 8) = o;
+      for (int i = 0; i < QV; ++i) {
+        const int v = tid + i * QT;
+        if (v < nvec) *reinterpret_cast<v2u*>(y + (int64_t)v * 8) = pack8(cache[i].f, conv_fast);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < QV; ++i) {
+        const int v = tid + i * QT;
+        if (v < nvec) *reinterpret_cast<v2u*>(y + (int64_t)v * 8) = pack8(cache[i].f, conv);
       }
     }
   } else {
@@ -190,18 +209,26 @@ __global__ __launch_bounds__(QTW) void fp8_quant_row_per_wave_kernel(const T* __
   float s = scale_ub ? fminf(amax, *scale_ub) : amax;
   s = fmaxf(s / FP8_MAX, 1.0f / (FP8_MAX * 512.0f));
   if (lane == 0) scales[row] = s;
-#pragma unroll
-  for (int i = 0; i < NV; ++i) {
+  const bool fast = scale_ub == nullptr && s < __builtin_inff();      // see fp8_quant_kernel
+  const float rcp = 1.0f / s;
+  auto store8 = [&](int i, auto&& cv) {
     const int v = lane + i * 64;
     if (v < nvec) {
       float q[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) q[e] = clamp448(cache[i].f[e] / s);
+      for (int e = 0; e < 8; ++e) q[e] = clamp448(cv(cache[i].f[e]));
       v2u o;
       o.x = cvt2(q[0], q[1]) | (cvt2(q[2], q[3]) << 16);
       o.y = cvt2(q[4], q[5]) | (cvt2(q[6], q[7]) << 16);
       *reinterpret_cast<v2u*>(y + (int64_t)v * 8) = o;
     }
+  };
+  if (fast) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) store8(i, [&](float v) { return div16_exact(v, s, rcp); });
+  } else {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) store8(i, [&](float v) { return v / s; });
   }
 }
 
@@ -283,8 +310,9 @@ extern "C" int vaq_fp8_quant_per_token_tuned(const void* in, int in_dtype, int64
   // Measured: a row per wavefront is 1.1-1.6x faster for short rows in large batches; with few rows a whole workgroup
   // per row has the shorter latency, and from 4096 elements on the 64 registers of row data per lane cost more than the
   // barriers saved.
-  const bool many_short_rows = hidden <= 1024 ? rows >= 512 : (hidden <= 2048 && rows >= 2048);
-  if (tuning().quant_wg_per_row == 0 && many_short_rows &&
+  const bool many_short_rows = hidden <= 1024 ? rows >= 1024 : (hidden <= 2048 && rows >= 2048);
+  const int force = tuning().quant_wg_per_row;      // 1: a workgroup per row, 2: a wavefront per row where it can run
+  if ((force == 2 || (force == 0 && many_short_rows)) &&
       row_per_wave_ok(in, in_dtype, in_row_stride, out, out_row_stride, hidden)) {
     if (in_dtype == VAQ_BF16)
       launch_row_per_wave<bf16_t>(in, in_row_stride, out, out_row_stride, scales, scale_ub, rows, hidden, (hipStream_t)stream);

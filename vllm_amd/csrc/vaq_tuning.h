@@ -36,7 +36,7 @@ typedef struct VaqTuning {
   int fp8_split;        /*   K split of the tile kernel                                                              */
   int fp8_gx;           /*   workgroups of the weight-streaming kernel                                               */
   int fp8_stream_split; /*   -1 = never run the weight-streaming kernel over two halves of K                         */
-  int quant_wg_per_row; /* per-token FP8 quant: 1 = always one workgroup per row                                     */
+  int quant_wg_per_row; /* per-token FP8 quant: 1 = one workgroup per row, 2 = one wavefront per row (where it can)    */
   int exp[15];          /* further switches of the same kind, for A/B timing runs: [0] = 1 shared instead of private  */
                         /*   activation fill, [1] = ring variant + 1, [2] rows over workgroups (1 off, 2 forced) of   */
                         /*   the LDS-staged decode kernel, [3] = 1 sixteen staged rows for M = 5 .. 8, [5] = 1 two K   */
