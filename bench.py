@@ -248,6 +248,42 @@ def stream_ceiling_section(dev):
     return rows
 
 
+def mix_probe(dev, iters=3000):
+    """The matrix core under the instruction mixes of candidate GEMM main loops (`vaq_mfma_mix_probe` of the bench-only
+    probe library: MFMAs of either shape with LDS fragment reads and VALU work between them, operands that vary).  Not a
+    measurement of the product: it prices design alternatives (weights dequantised into LDS or in registers, one or two
+    wavefronts per SIMD, 32x32 or 16x16 MFMAs) and gives the ceiling a real main loop can be read against.  Each
+    configuration runs twice; the second launch is timed by its own 100 MHz counter and by events."""
+    import ctypes
+    from vllm_amd.build import BENCH_PROBE_PATH
+    lib = ctypes.CDLL(str(BENCH_PROBE_PATH))
+    lib.vaq_mfma_mix_probe_name.restype = ctypes.c_char_p
+    lib.vaq_mfma_mix_probe_flops.restype = ctypes.c_double
+    lib.vaq_mfma_mix_probe.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    ticks = torch.zeros(2048, dtype=torch.int64, device=dev)
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    rows = []
+    for i in range(lib.vaq_mfma_mix_probe_count()):
+        name = lib.vaq_mfma_mix_probe_name(i).decode()
+        flops = lib.vaq_mfma_mix_probe_flops(i, iters)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for rep in range(2):
+            ticks.zero_()
+            e0.record()
+            rc = lib.vaq_mfma_mix_probe(i, iters, ctypes.c_void_p(ticks.data_ptr()), ctypes.c_void_p(sink.data_ptr()), stream)
+            e1.record()
+            if rc != 0:
+                raise RuntimeError(f"vaq_mfma_mix_probe({i}) returned {rc}")
+            torch.cuda.synchronize()
+        t = ticks[ticks > 0].double()
+        loop_us = float(t.mean()) / 100.0
+        ev_us = e0.elapsed_time(e1) * 1e3
+        rows.append(dict(config=name, loop_us=loop_us, event_us=ev_us, PFLOPs_loop=flops / loop_us / 1e9, PFLOPs_event=flops / ev_us / 1e9))
+        log(f"[mix probe] {flops / ev_us / 1e9:5.2f} PFLOP/s by events ({flops / loop_us / 1e9:5.2f} by the in-kernel counter)  {name}")
+    return rows
+
+
 def prefill_section(dev):
     """BASELINE.json config 3: asymmetric uint4 + act_order, both readings of its act_order wording.  `rows`: g_idx from a
     random permutation of the K rows (the reference's generator): activations are reordered on every call.  `groups`:
@@ -725,6 +761,8 @@ def main():
     ap.add_argument("--mfma-pass", action="store_true",
                     help="for `rocprofv3 --pmc`: three eager passes of [vendor bf16 GEMM 4096^3, W4A16 and FP8 GEMMs at M = 4096], no timing")
     ap.add_argument("--sections", default="", help="comma-separated subset of the extra sections to run (default: all)")
+    ap.add_argument("--mix-probe", action="store_true",
+                    help="run the matrix-core instruction-mix probe (bench-only library) and print its table; no product timing")
     ap.add_argument("--counter-pass", action="store_true",
                     help="for `rocprofv3 --pmc`: three eager passes of [256 MiB device copy, the 12 headline GEMMs], no timing")
     args = ap.parse_args()
@@ -740,6 +778,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.mix_probe:
+        print(json.dumps(mix_probe(dev), indent=1))
+        return
     if args.counter_pass:
         counter_pass(dev)
         return

@@ -197,15 +197,45 @@ def test_prefill_every_tile_shape(device, asym, dtype):
         a = _acts(m, k, device, dtype, seed=m)
         ref = o.gemm_ref(a.cpu(), o.case_w_ref(case))
         first = None
-        for tile in (10, 20, 11, 12, 13, 14, 15, 0, 1, 2):
+        for tile in (10, 20, 11, 12, 13, 14, 15, 30, 0, 1, 2):
             for split in ((1, 0, 2, 3) if tile >= 10 else (0,)):      # 0: the automatic split, 1: none
                 with _tuning.override(prefill_tile=tile + 1, prefill_split=split):
                     out = layer(a)
                 check_gemm_close(out, ref, f"tile {tile} split {split} k={k} n={n} m={m}")
-                if tile >= 10 and split == 1:
+                # (tile 30 dequantises in registers and pairs other k-octets in an MFMA: same products, another order)
+                if 10 <= tile < 30 and split == 1:
                     if first is None:
                         first = out
                     assert torch.equal(out, first), f"tile {tile} differs from tile 10 (k={k} n={n} m={m})"
+        assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("asym", [False, True])
+def test_prefill_register_dequant_tile(device, dtype, asym):
+    """The 256 x 256 tile whose weights are dequantised in registers (tile id 30), forced: one-hot activations return
+    rn16((q - z) * s) bit for bit (every k-octet lands in the MFMA slot its activation chunk is read for, every column in
+    its lane after the lane swap), ragged M and N (columns past N, rows past M, a last tile of one 64-column strip),
+    one to many K steps, channelwise scales, and K split over workgroups."""
+    from vllm_amd import _tuning
+    for k, n, g in ((128, 64, 128), (256, 320, 128), (1024, 576, 128), (512, 256, -1), (2560, 832, 128)):
+        case = o.make_w4a16_case(k, n, g, asym=asym, dtype=dtype, seed=k + n)
+        layer = W4A16Layer(case, device, dtype)
+        w = o.case_w_ref(case)
+        for m in (65, 256, 300):
+            rows = [(37 * i + 32 * (i % 4) + m) % k for i in range(m)]
+            a = torch.zeros(m, k, dtype=dtype)
+            for i, r in enumerate(rows):
+                a[i, r] = 1
+            with _tuning.override(prefill_tile=31, prefill_split=1):
+                assert torch.equal(layer(a.to(device)).cpu(), w[rows]), f"one-hot k={k} n={n} m={m}"
+            a = _acts(m, k, device, dtype, seed=m)
+            ref = o.gemm_ref(a.cpu(), w)
+            for split in (1, 0, 2, 5):
+                with _tuning.override(prefill_tile=31, prefill_split=split):
+                    out = layer(a)
+                    check_gemm_close(out, ref, f"tile 30 split {split} k={k} n={n} m={m}")
+                    assert torch.equal(out, layer(a)), "not deterministic run to run"
         assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
 
 

@@ -6,12 +6,16 @@ namespace vaq {
 
 // ----------------------------------------------------------------------------- host side
 
-// tile ids: 0..2 = register-staged kernel (256x256, 128x128, 64x128); 10.. = direct-to-LDS kernel (BM x BN)
+// tile ids: 0..2 = register-staged kernel (256x256, 128x128, 64x128); 10.. = direct-to-LDS kernel (BM x BN);
+// 30 = 256 x 256 with the weights dequantised in registers (w4a16_prefill3_kernel.h)
+int prefill_launch_reg(const PrefillParams& p, bool bf16, bool zp, hipStream_t s);      // w4a16_prefill3.hip
+
 template <bool BF16, bool HAS_ZP>
 static int dispatch_tile(const PrefillParams& p, int tile, hipStream_t s) {
   switch (tile) {
     case 10: return launch_prefill2<BF16, 256, 256, 2, 4, HAS_ZP, 1>(p, s);   // 8 wavefronts, 128 x 64 each
     case 20: return launch_prefill2<BF16, 256, 256, 2, 4, HAS_ZP, 1, false, true>(p, s);   // the same, alternating phases
+    case 30: return prefill_launch_reg(p, BF16, HAS_ZP, s);                                // 4 wavefronts, 256 x 64 each
     case 11: return launch_prefill2<BF16, 256, 256, 2, 2, HAS_ZP, 1>(p, s);   // 4 wavefronts, 128 x 128 each
     case 12: return launch_prefill2<BF16, 128, 128, 2, 2, HAS_ZP, 1>(p, s);   // 4 wavefronts, 64 x 64 each
     case 13: return launch_prefill2<BF16, 128, 256, 2, 4, HAS_ZP, 1>(p, s);   // 8 wavefronts, 64 x 64 each
@@ -105,7 +109,7 @@ static PrefillPlan plan_prefill(int M, int N, int K, bool direct_ok) {
   pl.tile = pick_tile(M, N, K, direct_ok);
   switch (pl.tile) {
     case 10: case 20: pl.bm = 256; pl.bn = 256; pl.nw = 8; break;
-    case 11: pl.bm = 256; pl.bn = 256; pl.nw = 4; break;
+    case 11: case 30: pl.bm = 256; pl.bn = 256; pl.nw = 4; break;
     case 12: pl.bm = 128; pl.bn = 128; pl.nw = 4; break;
     case 13: pl.bm = 128; pl.bn = 256; pl.nw = 8; break;
     case 14: pl.bm = 64; pl.bn = 128; pl.nw = 4; break;
@@ -119,7 +123,7 @@ static PrefillPlan plan_prefill(int M, int N, int K, bool direct_ok) {
   const int cus = num_cus_current_device();
   const int G = K / 128;
   int sk = 1;
-  if (pl.bm == 256 && pl.bn == 256 && pl.nw == 8) {
+  if (pl.bm == 256 && pl.bn == 256 && (pl.nw == 8 || pl.tile == 30)) {
     sk = splits_256(pl.tiles, K, cus);
   } else if (pl.tiles < 2 * (int64_t)cus) {
     sk = (int)((2 * (int64_t)cus) / pl.tiles);
@@ -191,7 +195,8 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
   p.SK = pl.sk;
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
-  const int tile_other = pl.tile == 20 ? 10 : pl.tile;      // the alternating-phase variant exists for 4-bit codes, groups of 128
+  // the alternating-phase and the register-dequantising variants exist for 4-bit codes in groups of 128 rows / channelwise
+  const int tile_other = (pl.tile == 20 || pl.tile == 30) ? 10 : pl.tile;
   if (wt == 2) rc = prefill_launch_f8(p, tile_other, bf16, s);
   else if (w8) rc = prefill_launch_w8(p, sub, tile_other, bf16, s);
   else if (sub > 1) rc = prefill_launch_sub(p, sub, tile_other, bf16, zp, s);

@@ -332,6 +332,158 @@ __global__ __launch_bounds__(256) void w4a16_prefill_kernel(const PrefillParams 
   }
 }
 
+// The tail of a tile kernel: (split K) hand the partial tile over and let the last arriver sum, then bias, rounding and
+// the stores.  `acc[i][j]` = 32 x 32 block (i along m, j along n) of this wavefront's TM x TN part of the tile at
+// (m0 + wm * TM, n0 + wn * TN), in the layout of an MFMA whose A operand held the weights: lane = column m, four
+// consecutive registers = four consecutive n.  `t` = tile number, `total` = tiles of the problem, `split` = this
+// workgroup's K part; `lds8` = at least NW * 32 * (TN * 2 + 16) bytes of LDS that every wavefront is done with.
+template <bool BF16, int WMB, int WNB, int NW, int TM, int TN>
+static __device__ inline void tile_epilogue(const PrefillParams& p, v16f (&acc)[WMB][WNB], uint8_t* lds8, int t, int total,
+                                            int split, int wave, int lane, int m0, int n0, int wm, int wn) {
+  using T = F16Traits<BF16>;
+  // ---- split K: hand the partial tile over; the last of the SK workgroups to arrive sums them in split order ----
+  if (p.SK > 1) {
+    // 16-byte buffer stores / loads with the sc1 cache-policy bit (device scope: written through to, and read from,
+    // memory that all XCDs share -- each XCD has its own L2).  One unit of NV4 KiB per (tile, wavefront).
+    constexpr int NV4 = WMB * WNB * 4;                     // 16-byte pieces per lane
+    constexpr int SC1 = 16;
+    const uint32_t unit = (uint32_t)((t * NW + wave) * NV4) * 1024u;           // bytes
+    const uint32_t split_stride = (uint32_t)total * (uint32_t)(NW * NV4) * 1024u;
+    const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(p.c_tmp, 0, (int)(split_stride * (uint32_t)p.SK), 0x00020000);
+#pragma unroll
+    for (int i = 0; i < WMB; ++i)
+#pragma unroll
+      for (int j = 0; j < WNB; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), rt, lane * 16,
+                                                 (int)(split * split_stride + unit + ((i * WNB + j) * 4 + q) * 1024), SC1);
+        }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // partial tile acknowledged before the counter moves
+    int32_t* ctr = p.counters + (int64_t)t * NW + wave;
+    int old = 0;
+    if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    old = __builtin_amdgcn_readfirstlane(old);      // lane 0 holds it; a scalar keeps what depends on it scalar
+    if (old != p.SK - 1) return;
+    // CH pieces of two splits in flight at a time (one piece after the other, every load waited for, the last arriver
+    // spent NV4 x SK memory round trips here); each element is still summed in split order, starting from zero
+    constexpr int CH = NV4 < 8 ? NV4 : 8;
+#pragma unroll
+    for (int c0 = 0; c0 < NV4; c0 += CH) {
+      v4f sum[CH];
+#pragma unroll
+      for (int c = 0; c < CH; ++c) sum[c] = v4f{0.f, 0.f, 0.f, 0.f};
+      for (int s0 = 0; s0 < p.SK; s0 += 2) {
+        const int s1 = s0 + 1 < p.SK ? s0 + 1 : s0;
+        v4u r0[CH], r1[CH];
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+          r0[c] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s0 * split_stride + unit + (c0 + c) * 1024), SC1);
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+          r1[c] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s1 * split_stride + unit + (c0 + c) * 1024), SC1);
+#pragma unroll
+        for (int c = 0; c < CH; ++c) sum[c] += __builtin_bit_cast(v4f, r0[c]);
+        if (s0 + 1 < p.SK) {
+#pragma unroll
+          for (int c = 0; c < CH; ++c) sum[c] += __builtin_bit_cast(v4f, r1[c]);
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const int pc = c0 + c, ij = pc / 4, q = pc % 4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[ij / WNB][ij % WNB][4 * q + e] = sum[c][e];
+      }
+    }
+    if (lane == 0) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+
+  // ---- epilogue: four consecutive accumulator registers = four consecutive n of one row.  The 16-bit results cross a
+  // wavefront-private piece of LDS (32 rows of TN * 2 + 16 bytes, the operand stages being free by now) and leave as
+  // 16-byte stores, 4-16 lanes to a row: stored directly, every instruction touches 32 rows with 16 bytes each, and
+  // the write requests of a device whose tiles all finish together took 10-17 us per tile. ----
+  if (((uintptr_t)p.c & 15) == 0) {
+    constexpr int PITCH = TN * 2 + 16;
+    constexpr int CPR = TN / 8;                // 16-byte chunks per row
+    static_assert((32 * CPR) % 64 == 0, "whole store instructions");
+    uint8_t* wave_lds = lds8 + wave * (32 * PITCH);
+    v2u bv[WNB][4];
+#pragma unroll
+    for (int j = 0; j < WNB; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + wn * TN + j * 32 + 8 * q + 4 * (lane >> 5);
+        bv[j][q] = v2u{0u, 0u};
+        if (p.bias && n < p.N) bv[j][q] = *reinterpret_cast<const v2u*>(p.bias + n);
+      }
+#pragma unroll
+    for (int i = 0; i < WMB; ++i) {
+#pragma unroll
+      for (int j = 0; j < WNB; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          float ov[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) ov[e] = acc[i][j][4 * q + e];
+          if (p.bias) {
+            ov[0] += T::to_float((uint16_t)(bv[j][q].x & 0xffffu));
+            ov[1] += T::to_float((uint16_t)(bv[j][q].x >> 16));
+            ov[2] += T::to_float((uint16_t)(bv[j][q].y & 0xffffu));
+            ov[3] += T::to_float((uint16_t)(bv[j][q].y >> 16));
+          }
+          v2u pk;
+          pk.x = pack2<BF16>(ov[0], ov[1]);
+          pk.y = pack2<BF16>(ov[2], ov[3]);
+          *reinterpret_cast<v2u*>(wave_lds + (lane & 31) * PITCH + (j * 32 + 8 * q + 4 * (lane >> 5)) * 2) = pk;
+        }
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_wave_barrier();         // lanes exchange data through LDS; its operations run in program order
+#pragma unroll
+      for (int it = 0; it < 32 * CPR / 64; ++it) {
+        const int idx = it * 64 + lane;
+        const int row = idx / CPR, ch = idx % CPR;
+        const v4u v = *reinterpret_cast<const v4u*>(wave_lds + row * PITCH + ch * 16);
+        const int m = m0 + wm * TM + i * 32 + row;
+        const int n = n0 + wn * TN + ch * 8;
+        if (m < p.M && n < p.N) *reinterpret_cast<v4u*>(p.c + (int64_t)m * p.N + n) = v;
+      }
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_wave_barrier();
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < WMB; ++i) {
+    const int m = m0 + wm * TM + i * 32 + (lane & 31);
+    if (m >= p.M) continue;
+    uint16_t* orow = p.c + (int64_t)m * p.N;
+#pragma unroll
+    for (int j = 0; j < WNB; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + wn * TN + j * 32 + 8 * q + 4 * (lane >> 5);
+        if (n >= p.N) continue;
+        float ov[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ov[e] = acc[i][j][4 * q + e];
+        if (p.bias) {
+          const v2u bb = *reinterpret_cast<const v2u*>(p.bias + n);
+          ov[0] += T::to_float((uint16_t)(bb.x & 0xffffu));
+          ov[1] += T::to_float((uint16_t)(bb.x >> 16));
+          ov[2] += T::to_float((uint16_t)(bb.y & 0xffffu));
+          ov[3] += T::to_float((uint16_t)(bb.y >> 16));
+        }
+        v2u pk;
+        pk.x = pack2<BF16>(ov[0], ov[1]);
+        pk.y = pack2<BF16>(ov[2], ov[3]);
+        *reinterpret_cast<v2u*>(orow + n) = pk;
+      }
+    }
+  }
+}
+
 // ----------------------------------------------------------------------------- direct-to-LDS variant
 // Same arithmetic, different plumbing:
 //  * the activation tile goes global -> LDS with `buffer_load_dwordx4 ... lds` (no registers, no VALU);
@@ -792,148 +944,8 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
   // every wavefront is done with the operand stages: the epilogue reuses them
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
-  // ---- split K: hand the partial tile over; the last of the SK workgroups to arrive sums them in split order ----
-  if (p.SK > 1) {
-    // 16-byte buffer stores / loads with the sc1 cache-policy bit (device scope: written through to, and read from,
-    // memory that all XCDs share -- each XCD has its own L2).  One unit of NV4 KiB per (tile, wavefront).
-    constexpr int NV4 = WMB * WNB * 4;                     // 16-byte pieces per lane
-    constexpr int SC1 = 16;
-    const uint32_t unit = (uint32_t)((t * NW + wave) * NV4) * 1024u;           // bytes
-    const uint32_t split_stride = (uint32_t)total * (uint32_t)(NW * NV4) * 1024u;
-    const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(p.c_tmp, 0, (int)(split_stride * (uint32_t)p.SK), 0x00020000);
-#pragma unroll
-    for (int i = 0; i < WMB; ++i)
-#pragma unroll
-      for (int j = 0; j < WNB; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), rt, lane * 16,
-                                                 (int)(split * split_stride + unit + ((i * WNB + j) * 4 + q) * 1024), SC1);
-        }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // partial tile acknowledged before the counter moves
-    int32_t* ctr = p.counters + (int64_t)t * NW + wave;
-    int old = 0;
-    if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    old = __builtin_amdgcn_readfirstlane(old);      // lane 0 holds it; a scalar keeps what depends on it scalar
-    if (old != p.SK - 1) return;
-    // CH pieces of two splits in flight at a time (one piece after the other, every load waited for, the last arriver
-    // spent NV4 x SK memory round trips here); each element is still summed in split order, starting from zero
-    constexpr int CH = NV4 < 8 ? NV4 : 8;
-#pragma unroll
-    for (int c0 = 0; c0 < NV4; c0 += CH) {
-      v4f sum[CH];
-#pragma unroll
-      for (int c = 0; c < CH; ++c) sum[c] = v4f{0.f, 0.f, 0.f, 0.f};
-      for (int s0 = 0; s0 < p.SK; s0 += 2) {
-        const int s1 = s0 + 1 < p.SK ? s0 + 1 : s0;
-        v4u r0[CH], r1[CH];
-#pragma unroll
-        for (int c = 0; c < CH; ++c)
-          r0[c] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s0 * split_stride + unit + (c0 + c) * 1024), SC1);
-#pragma unroll
-        for (int c = 0; c < CH; ++c)
-          r1[c] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s1 * split_stride + unit + (c0 + c) * 1024), SC1);
-#pragma unroll
-        for (int c = 0; c < CH; ++c) sum[c] += __builtin_bit_cast(v4f, r0[c]);
-        if (s0 + 1 < p.SK) {
-#pragma unroll
-          for (int c = 0; c < CH; ++c) sum[c] += __builtin_bit_cast(v4f, r1[c]);
-        }
-      }
-#pragma unroll
-      for (int c = 0; c < CH; ++c) {
-        const int pc = c0 + c, ij = pc / 4, q = pc % 4;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[ij / WNB][ij % WNB][4 * q + e] = sum[c][e];
-      }
-    }
-    if (lane == 0) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-
-  // ---- epilogue: four consecutive accumulator registers = four consecutive n of one row.  The 16-bit results cross a
-  // wavefront-private piece of LDS (32 rows of TN * 2 + 16 bytes, the operand stages being free by now) and leave as
-  // 16-byte stores, 4-16 lanes to a row: stored directly, every instruction touches 32 rows with 16 bytes each, and
-  // the write requests of a device whose tiles all finish together took 10-17 us per tile. ----
-  if (((uintptr_t)p.c & 15) == 0) {
-    constexpr int PITCH = TN * 2 + 16;
-    constexpr int CPR = TN / 8;                // 16-byte chunks per row
-    static_assert((3 * BM + 2 * BN) * 128 >= NW * 32 * PITCH, "operand stages too small for the epilogue staging");
-    static_assert((32 * CPR) % 64 == 0, "whole store instructions");
-    uint8_t* wave_lds = lds8 + wave * (32 * PITCH);
-    v2u bv[WNB][4];
-#pragma unroll
-    for (int j = 0; j < WNB; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = n0 + wn * TN + j * 32 + 8 * q + 4 * (lane >> 5);
-        bv[j][q] = v2u{0u, 0u};
-        if (p.bias && n < p.N) bv[j][q] = *reinterpret_cast<const v2u*>(p.bias + n);
-      }
-#pragma unroll
-    for (int i = 0; i < WMB; ++i) {
-#pragma unroll
-      for (int j = 0; j < WNB; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          float ov[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) ov[e] = acc[i][j][4 * q + e];
-          if (p.bias) {
-            ov[0] += T::to_float((uint16_t)(bv[j][q].x & 0xffffu));
-            ov[1] += T::to_float((uint16_t)(bv[j][q].x >> 16));
-            ov[2] += T::to_float((uint16_t)(bv[j][q].y & 0xffffu));
-            ov[3] += T::to_float((uint16_t)(bv[j][q].y >> 16));
-          }
-          v2u pk;
-          pk.x = pack2<BF16>(ov[0], ov[1]);
-          pk.y = pack2<BF16>(ov[2], ov[3]);
-          *reinterpret_cast<v2u*>(wave_lds + (lane & 31) * PITCH + (j * 32 + 8 * q + 4 * (lane >> 5)) * 2) = pk;
-        }
-      asm volatile("" ::: "memory");
-      __builtin_amdgcn_wave_barrier();         // lanes exchange data through LDS; its operations run in program order
-#pragma unroll
-      for (int it = 0; it < 32 * CPR / 64; ++it) {
-        const int idx = it * 64 + lane;
-        const int row = idx / CPR, ch = idx % CPR;
-        const v4u v = *reinterpret_cast<const v4u*>(wave_lds + row * PITCH + ch * 16);
-        const int m = m0 + wm * TM + i * 32 + row;
-        const int n = n0 + wn * TN + ch * 8;
-        if (m < p.M && n < p.N) *reinterpret_cast<v4u*>(p.c + (int64_t)m * p.N + n) = v;
-      }
-      asm volatile("" ::: "memory");
-      __builtin_amdgcn_wave_barrier();
-    }
-    return;
-  }
-#pragma unroll
-  for (int i = 0; i < WMB; ++i) {
-    const int m = m0 + wm * TM + i * 32 + (lane & 31);
-    if (m >= p.M) continue;
-    uint16_t* orow = p.c + (int64_t)m * p.N;
-#pragma unroll
-    for (int j = 0; j < WNB; ++j) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = n0 + wn * TN + j * 32 + 8 * q + 4 * (lane >> 5);
-        if (n >= p.N) continue;
-        float ov[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) ov[e] = acc[i][j][4 * q + e];
-        if (p.bias) {
-          const v2u bb = *reinterpret_cast<const v2u*>(p.bias + n);
-          ov[0] += T::to_float((uint16_t)(bb.x & 0xffffu));
-          ov[1] += T::to_float((uint16_t)(bb.x >> 16));
-          ov[2] += T::to_float((uint16_t)(bb.y & 0xffffu));
-          ov[3] += T::to_float((uint16_t)(bb.y >> 16));
-        }
-        v2u pk;
-        pk.x = pack2<BF16>(ov[0], ov[1]);
-        pk.y = pack2<BF16>(ov[2], ov[3]);
-        *reinterpret_cast<v2u*>(orow + n) = pk;
-      }
-    }
-  }
+  static_assert((3 * BM + 2 * BN) * 128 >= NW * 32 * (TN * 2 + 16), "operand stages too small for the epilogue staging");
+  tile_epilogue<BF16, WMB, WNB, NW, TM, TN>(p, acc, lds8, t, total, split, wave, lane, m0, n0, wm, wn);
 }
 
 template <bool BF16, int WMB, int WNB, bool HAS_ZP, int SUBG>
