@@ -544,7 +544,9 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
 // reduction buffer of the K slices (on top of the activations for MB > 2, see the kernel), and with two or more
 // m-blocks the row sums of the staged tiles.
 static inline size_t decode2_lds_bytes(int wks, int groups_per_wave, int mr, int mb) {
-  const size_t act = ((size_t)wks * groups_per_wave * 256 * mr * mb + 1023) & ~(size_t)1023;     // padded to 1 KiB (see the fill)
+  // padded to 1 KiB (see the fill).  With one K slice per workgroup nothing else follows the image, and the last
+  // instruction of the private fill may write (zeros) up to 63 slots past it: one more KiB.
+  const size_t act = (((size_t)wks * groups_per_wave * 256 * mr * mb + 1023) & ~(size_t)1023) + (wks == 1 ? 1024 : 0);
   const size_t red = wks > 1 ? (size_t)(mb == 2 ? D2_WAVES - D2_WAVES / wks : D2_WAVES) * mb * 1024 : 0;
   const size_t sums = mb >= 2 ? (size_t)wks * groups_per_wave * mb * 64 : 0;      // row sums of the staged tiles (see SPRE)
   if (mb > 2) return (act > red ? act : red) + sums;
@@ -572,6 +574,13 @@ static int launch_decode2(const Decode2Params& p_in, hipStream_t s) {
     }
   }
   const size_t lds = decode2_lds_bytes(p.WKS, GS / (WT != 0 ? 2 : 1), MR, MB);
+  if (p.PRIV != 0) {
+    // the private fill writes whole 64-slot instructions: the last one (last row, last K slice) must end inside the
+    // allocation, whatever the planner chose; otherwise the shared fill, which stays inside the padded image, is taken
+    const int own = GS / (WT != 0 ? 2 : 1) * 16, ko = p.WKS * own;
+    const size_t last_c0 = (size_t)(MR * MB - 1) * ko + (size_t)(p.WKS - 1) * own + (size_t)((own - 1) / 64) * 64;
+    if ((last_c0 + 64) * 16 > lds) p.PRIV = 0;
+  }
   auto kern = w4a16_decode2_kernel<BF16, GS, MB, HAS_ZP, MR, SUBG, WT, RC, MSP>;
   static size_t reserved[VAQ_MAX_DEVICES];
   if (const int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "w4a16_gemm(decode)"); rc != VAQ_OK) return rc;

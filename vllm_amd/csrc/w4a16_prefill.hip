@@ -38,7 +38,7 @@ static int splits_256(int64_t tiles256, int K, int cus) {
   return sk < 1 ? 1 : (sk > 8 ? 8 : sk);
 }
 
-static int pick_tile(int M, int N, int K, bool direct_ok) {
+static int pick_tile(int M, int N, int K, bool direct_ok, bool reg_ok) {
   if (tuning().prefill_tile > 0) return tuning().prefill_tile - 1;
   const int cus = num_cus_current_device();
   auto tiles = [&](int bm, int bn) { return (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
@@ -52,7 +52,14 @@ static int pick_tile(int M, int N, int K, bool direct_ok) {
     // 256 x 256 tiles stay ahead, 90 against 108 us)
     const bool rows_poorly_filled = (int64_t)M * 10 < (int64_t)((M + 255) / 256) * 256 * 7 && tiles(128, 128) <= 2 * (int64_t)cus &&
                                     tuning().exp[9] != 1;
-    if (M > 128 && !rows_poorly_filled && tiles(256, 256) * splits_256(tiles(256, 256), K, cus) * 20 >= cus * 11) return 20;      // 256 x 256, alternating phases
+    if (M > 128 && !rows_poorly_filled && tiles(256, 256) * splits_256(tiles(256, 256), K, cus) * 20 >= cus * 11) {
+      // 256 x 256.  With at least one tile per compute unit and K unsplit, the kernel that dequantises in registers (four
+      // wavefronts of 256 x 64) is 1-4 % ahead at M = 4096 on the four Llama-3-8B layers (206 / 123 / 807 / 400 -> 205 / 121 /
+      // 792 / 384 us); with fewer tiles or a split K the 8-wavefront kernel with alternating phases is (its second
+      // wavefront per SIMD covers the waits of the first: 14336 x 4096 at M = 512, 95.8 against 102.5 us).  `reg_ok`: 4-bit
+      // codes in groups of 128 rows or channelwise -- what the register kernel is built for.
+      return (reg_ok && tiles(256, 256) >= cus) ? 30 : 20;
+    }
     // An odd number of 64-row blocks on a short K: 64 x 128 tiles (the last 128-row tile would be half empty) where they
     // come to 80-100 % of one or of two workgroups per compute unit (cold: 3584 x 18944 at M = 136 .. 192, 444 tiles, 60 ->
     // 45 us; 2560 x 10240, 240 tiles, 30.8 -> 22.6 us; 4096 x 11008 at M = 288 / 320, 430 tiles, 67 -> 50 us; with 258 or
@@ -104,9 +111,9 @@ struct PrefillPlan {
 // compute units idle: as many splits as bring the workgroup count to about two per compute unit, at most 8, every
 // split at least 8 groups (16 K steps) long, 32 groups when the tiles already fill the device -- measured on the Llama
 // shapes for M = 48 .. 512.
-static PrefillPlan plan_prefill(int M, int N, int K, bool direct_ok) {
+static PrefillPlan plan_prefill(int M, int N, int K, bool direct_ok, bool reg_ok = false) {
   PrefillPlan pl;
-  pl.tile = pick_tile(M, N, K, direct_ok);
+  pl.tile = pick_tile(M, N, K, direct_ok, reg_ok);
   switch (pl.tile) {
     case 10: case 20: pl.bm = 256; pl.bn = 256; pl.nw = 8; break;
     case 11: case 30: pl.bm = 256; pl.bn = 256; pl.nw = 4; break;
@@ -180,7 +187,7 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
     set_error("w4a16_gemm(prefill): 8-bit weights with an A of 4 GiB or more are not built");
     return VAQ_ERR_UNSUPPORTED;
   }
-  PrefillPlan pl = plan_prefill(M, N, K, direct_ok);
+  PrefillPlan pl = plan_prefill(M, N, K, direct_ok, !w8 && sub == 1);
   // A caller that passes no scratch at all gets the unsplit kernel (same result, no K split); scratch that is there but
   // too small is the caller's mistake and is reported, not worked around.
   if (pl.sk > 1 && c_tmp == nullptr && counters == nullptr) pl.sk = 1;
