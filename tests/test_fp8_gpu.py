@@ -396,7 +396,7 @@ def test_scaled_mm_into_a_view_of_a_wider_buffer(device, offset):
         assert bool((got[:, :offset] == 7).all()) and bool((got[:, offset + n:] == 7).all()), "wrote outside the view"
 
 
-@pytest.mark.parametrize("cfg", [1, 8, 3, 4, 5, 7, 13, 23, 14, 24, 15, 17])
+@pytest.mark.parametrize("cfg", [1, 8, 2, 10, 11, 3, 4, 5, 7, 13, 23, 14, 24, 15, 17])
 def test_scaled_mm_every_tile_shape_exact(device, cfg):
     """Every shape of the multi-stage tile kernel, forced through a per-call tuning override (the automatic choice only reaches
     some of them at any one problem size), including the ones that take two k-slices per step: small-integer operands
@@ -405,7 +405,8 @@ def test_scaled_mm_every_tile_shape_exact(device, cfg):
     from vllm_amd import _tuning
     g = torch.Generator().manual_seed(cfg)
     for m, n, k, split in ((300, 384, 1024, 0), (64, 256, 8192 + 128, 2), (513, 512, 640, 0), (257, 272, 384, 0),
-                           (100, 128, 448, 0), (520, 256, 64 * 13, 3)):
+                           (100, 128, 448, 0), (520, 256, 64 * 13, 3), (70, 320, 128, 0), (258, 256, 256, 0),
+                           (256, 512, 128 * 11, 3), (33, 64, 128 * 7, 5)):
         a = torch.randint(-2, 3, (m, k), generator=g).float()
         w = torch.randint(-1, 2, (n, k), generator=g).float()
         with _tuning.override(fp8_tile_cfg=cfg, fp8_split=split):

@@ -180,6 +180,77 @@ __device__ inline void tile_epilogue_lds(const Fp8MMParams& p, v16f (&acc)[WMB][
   }
 }
 
+// The tail of the multi-stage tile kernels: (split K) hand the partial tile over and let the last arriver sum, then the
+// scaled epilogue.  `t` = tile number, `total` = tiles of the problem, `split` = this workgroup's K part; `lds8` = at
+// least NW * 32 * (WNB * 64 + 16) bytes of LDS that every wavefront of the workgroup is done with.
+template <bool BF16_OUT, int WMB, int WNB, int NW>
+__device__ inline void fp8_tile_tail(const Fp8MMParams& p, v16f (&acc)[WMB][WNB], uint8_t* lds8, int t, int total, int split,
+                                     int wave, int lane, int m0, int n0, int wm, int wn) {
+  // ---- split K: hand the partial tile over; the last of the SK workgroups to arrive sums them in split order.
+  // 16-byte buffer stores / loads with the sc1 cache-policy bit (device scope: each XCD has its own L2), one unit of
+  // NV4 KiB per (tile, wavefront), one arrival counter per unit. ----
+  if (p.SK > 1) {
+    constexpr int NV4 = WMB * WNB * 4;
+    constexpr int SC1 = 16;
+    const uint32_t unit = (uint32_t)((t * NW + wave) * NV4) * 1024u;
+    const uint32_t split_stride = (uint32_t)total * (uint32_t)(NW * NV4) * 1024u;
+    const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(p.c_tmp, 0, (int)(split_stride * (uint32_t)p.SK), 0x00020000);
+#pragma unroll
+    for (int i = 0; i < WMB; ++i)
+#pragma unroll
+      for (int j = 0; j < WNB; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), rt, lane * 16,
+                                                 (int)(split * split_stride + unit + ((i * WNB + j) * 4 + q) * 1024), SC1);
+        }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // partial tile acknowledged before the counter moves
+    int32_t* ctr = p.counters + (int64_t)t * NW + wave;
+    int old = 0;
+    if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    old = __builtin_amdgcn_readfirstlane(old);      // lane 0 holds it; a scalar keeps what depends on it scalar
+    if (old != p.SK - 1) return;
+    // CH pieces of two splits in flight at a time (one piece after the other, every load waited for, the last arriver
+    // spent NV4 x SK memory round trips here); each element is still summed in split order, starting from zero
+    constexpr int CH = NV4 < 8 ? NV4 : 8;
+#pragma unroll
+    for (int c0 = 0; c0 < NV4; c0 += CH) {
+      v4f sum[CH];
+#pragma unroll
+      for (int c = 0; c < CH; ++c) sum[c] = v4f{0.f, 0.f, 0.f, 0.f};
+      for (int s0 = 0; s0 < p.SK; s0 += 2) {
+        const int s1 = s0 + 1 < p.SK ? s0 + 1 : s0;
+        v4u r0[CH], r1[CH];
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+          r0[c] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s0 * split_stride + unit + (c0 + c) * 1024), SC1);
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+          r1[c] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s1 * split_stride + unit + (c0 + c) * 1024), SC1);
+#pragma unroll
+        for (int c = 0; c < CH; ++c) sum[c] += __builtin_bit_cast(v4f, r0[c]);
+        if (s0 + 1 < p.SK) {
+#pragma unroll
+          for (int c = 0; c < CH; ++c) sum[c] += __builtin_bit_cast(v4f, r1[c]);
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const int pc = c0 + c, ij = pc / 4, q = pc % 4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[ij / WNB][ij % WNB][4 * q + e] = sum[c][e];
+      }
+    }
+    if (lane == 0) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+
+  if (((uintptr_t)p.out & 15) == 0)
+    tile_epilogue_lds<BF16_OUT, WMB, WNB>(p, acc, m0, n0, wm, wn, lane, lds8 + wave * (32 * (WNB * 64 + 16)));
+  else
+    tile_epilogue<BF16_OUT, WMB, WNB>(p, acc, m0, n0, wm, wn, lane);
+}
+
 // ----------------------------------------------------------------------------- tile kernel
 template <bool BF16_OUT, int WMB, int WNB>
 __global__ __launch_bounds__(256) void fp8_mm_tile_kernel(const Fp8MMParams p) {
@@ -615,70 +686,8 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
     }
   }
 
-  // ---- split K: hand the partial tile over; the last of the SK workgroups to arrive sums them in split order.
-  // 16-byte buffer stores / loads with the sc1 cache-policy bit (device scope: each XCD has its own L2), one unit of
-  // NV4 KiB per (tile, wavefront), one arrival counter per unit. ----
-  if (p.SK > 1) {
-    constexpr int NV4 = WMB * WNB * 4;
-    constexpr int SC1 = 16;
-    const uint32_t unit = (uint32_t)((t * NW + wave) * NV4) * 1024u;
-    const uint32_t split_stride = (uint32_t)total * (uint32_t)(NW * NV4) * 1024u;
-    const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(p.c_tmp, 0, (int)(split_stride * (uint32_t)p.SK), 0x00020000);
-#pragma unroll
-    for (int i = 0; i < WMB; ++i)
-#pragma unroll
-      for (int j = 0; j < WNB; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), rt, lane * 16,
-                                                 (int)(split * split_stride + unit + ((i * WNB + j) * 4 + q) * 1024), SC1);
-        }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // partial tile acknowledged before the counter moves
-    int32_t* ctr = p.counters + (int64_t)t * NW + wave;
-    int old = 0;
-    if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    old = __builtin_amdgcn_readfirstlane(old);      // lane 0 holds it; a scalar keeps what depends on it scalar
-    if (old != p.SK - 1) return;
-    // CH pieces of two splits in flight at a time (one piece after the other, every load waited for, the last arriver
-    // spent NV4 x SK memory round trips here); each element is still summed in split order, starting from zero
-    constexpr int CH = NV4 < 8 ? NV4 : 8;
-#pragma unroll
-    for (int c0 = 0; c0 < NV4; c0 += CH) {
-      v4f sum[CH];
-#pragma unroll
-      for (int c = 0; c < CH; ++c) sum[c] = v4f{0.f, 0.f, 0.f, 0.f};
-      for (int s0 = 0; s0 < p.SK; s0 += 2) {
-        const int s1 = s0 + 1 < p.SK ? s0 + 1 : s0;
-        v4u r0[CH], r1[CH];
-#pragma unroll
-        for (int c = 0; c < CH; ++c)
-          r0[c] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s0 * split_stride + unit + (c0 + c) * 1024), SC1);
-#pragma unroll
-        for (int c = 0; c < CH; ++c)
-          r1[c] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s1 * split_stride + unit + (c0 + c) * 1024), SC1);
-#pragma unroll
-        for (int c = 0; c < CH; ++c) sum[c] += __builtin_bit_cast(v4f, r0[c]);
-        if (s0 + 1 < p.SK) {
-#pragma unroll
-          for (int c = 0; c < CH; ++c) sum[c] += __builtin_bit_cast(v4f, r1[c]);
-        }
-      }
-#pragma unroll
-      for (int c = 0; c < CH; ++c) {
-        const int pc = c0 + c, ij = pc / 4, q = pc % 4;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[ij / WNB][ij % WNB][4 * q + e] = sum[c][e];
-      }
-    }
-    if (lane == 0) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-
   static_assert(NST * STAGE >= NW * 32 * (WNB * 64 + 16), "operand ring too small for the epilogue staging");
-  if (((uintptr_t)p.out & 15) == 0)
-    tile_epilogue_lds<BF16_OUT, WMB, WNB>(p, acc, m0, n0, wm, wn, lane, lds8 + wave * (32 * (WNB * 64 + 16)));
-  else
-    tile_epilogue<BF16_OUT, WMB, WNB>(p, acc, m0, n0, wm, wn, lane);
+  fp8_tile_tail<BF16_OUT, WMB, WNB, NW>(p, acc, lds8, t, total, split, wave, lane, m0, n0, wm, wn);
 }
 
 // ----------------------------------------------------------------------------- stream kernel (M <= 32, narrow layers M <= 64)
@@ -1121,6 +1130,13 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
                                   tiles(128, 256) * 10 >= cus * 7 && tuning().exp[9] != 1;
   if (pl.cfg <= 0)
     pl.cfg = take256 && !rows_poorly_filled ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (take128 ? 3 : 4));
+  // 256 x 384 tiles (wavefronts of 128 x 96) where the 256 x 256 tiles leave the last round of workgroups badly filled and
+  // these do not: 4096 x 6144 at M = 4096 is 384 tiles = 1.5 rounds, or 256 = one round (101.4 -> 92.3 us).  Per tile they
+  // are slower (4096 x 4096 at M = 4096: 62.8 against 72.7 us), so only for a gain of a fifth in the fill of the rounds.
+  if (tuning().fp8_tile_cfg <= 0 && pl.cfg == 1 && N % 384 == 0 && K / 64 < 160) {
+    auto fill = [&](int64_t t) { return (double)t / (double)(((t + cus - 1) / cus) * cus); };
+    if (tiles(256, 256) > cus && fill(tiles(256, 384)) >= 1.2 * fill(tiles(256, 256))) pl.cfg = 10;
+  }
   // the smallest tile with two k-slices per step: 5-8 % faster on a short K (half the barriers), no gain on a long one
   if (tuning().fp8_tile_cfg <= 0 && pl.cfg == 4 && K % 128 == 0 && K <= 8192) pl.cfg = 14;
   // 64 x 64 tiles while they fit the device in one round, on a short K: twice the workgroups with loads in flight
@@ -1139,6 +1155,7 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
     case 5: case 15: pl.bm = 64; pl.bn = 64; pl.nw = 4; break;
     case 7: case 17: pl.bm = 128; pl.bn = 256; pl.nw = 8; break;
     case 2: pl.bm = 256; pl.bn = 256; pl.nw = 4; break;
+    case 10: case 11: pl.bm = 256; pl.bn = 384; pl.nw = 8; break;
     default: pl.bm = 256; pl.bn = 256; pl.nw = 8; break;
   }
   pl.tiles = tiles(pl.bm, pl.bn);
@@ -1232,6 +1249,8 @@ static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t c
       case 1: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 5, 1, 1>(p, s);   // alternating phases (see the kernel)
       case 8: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 5>(p, s);
       case 2: return launch_tile3<BF16_OUT, 256, 256, 2, 2, 5>(p, s);
+      case 10: return launch_tile3<BF16_OUT, 256, 384, 2, 4, 4, 1, 1>(p, s);   // 8 wavefronts of 128 x 96, alternating phases
+      case 11: return launch_tile3<BF16_OUT, 256, 384, 2, 4, 4>(p, s);
       case 3: return launch_tile3<BF16_OUT, 128, 128, 2, 2, 5>(p, s);
       case 4: return launch_tile3<BF16_OUT, 64, 128, 2, 2, 5>(p, s);
       case 6: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 3>(p, s);
