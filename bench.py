@@ -595,16 +595,26 @@ def medium_m_section(dev):
 
 def roofline_mfma(extra):
     """The compute-bound kernels against the dense MFMA peaks, from the M = 4096 rows of the prefill and FP8 sections
-    (HIP-graph timings of this run): per kernel the FLOPs of one launch, its average duration and the fraction of peak."""
+    (HIP-graph timings of this run): per kernel the FLOPs of one launch, its average duration, the fraction of peak and,
+    where the vendor section ran, the vendor library's plain GEMM of the same shape and precision beside it."""
+    vendor = {(r["kind"], r["K"], r["N"]): r["us"] for r in extra.get("vendor_ceiling", []) if r.get("M") == 4096}
     out = []
     for r in extra.get("prefill", []):
         if r["M"] == 4096 and r["kind"].endswith("groups"):
-            out.append(dict(kernel="vaq::w4a16_prefill2_kernel", K=r["K"], N=r["N"], M=r["M"], flops_per_launch=2.0 * r["M"] * r["N"] * r["K"],
-                            avg_ns=round(r["us"] * 1e3), peak_TFLOPs=BF16_PEAK_TFLOPS, frac=round(r["mfma_frac"], 4)))
+            row = dict(kernel="vaq::w4a16_prefill3_kernel", K=r["K"], N=r["N"], M=r["M"], flops_per_launch=2.0 * r["M"] * r["N"] * r["K"],
+                       avg_ns=round(r["us"] * 1e3), peak_TFLOPs=BF16_PEAK_TFLOPS, frac=round(r["mfma_frac"], 4))
+            v = vendor.get(("vendor_bf16_matmul", r["K"], r["N"]))
+            if v:
+                row["vendor_bf16_gemm_ns"] = round(v * 1e3)
+            out.append(row)
     for r in extra.get("fp8", []):
         if r["M"] == 4096:
-            out.append(dict(kernel="vaq::fp8_mm_tile3_kernel", K=r["K"], N=r["N"], M=r["M"], flops_per_launch=2.0 * r["M"] * r["N"] * r["K"],
-                            avg_ns=round(r["us"] * 1e3), peak_TFLOPs=FP8_PEAK_TFLOPS, frac=round(r["mfma_frac"], 4)))
+            row = dict(kernel="vaq::fp8_mm_tile3_kernel", K=r["K"], N=r["N"], M=r["M"], flops_per_launch=2.0 * r["M"] * r["N"] * r["K"],
+                       avg_ns=round(r["us"] * 1e3), peak_TFLOPs=FP8_PEAK_TFLOPS, frac=round(r["mfma_frac"], 4))
+            v = vendor.get(("vendor_fp8_scaled_mm_rowwise", r["K"], r["N"]))
+            if v:
+                row["vendor_fp8_gemm_ns"] = round(v * 1e3)
+            out.append(row)
     return out or None
 
 

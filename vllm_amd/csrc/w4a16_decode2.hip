@@ -289,9 +289,9 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
   p.WKS = cfg.wks;
   p.WN = cfg.wn;
   // private activation fill (see the kernel): measured ahead only on short streams with few staged rows (4096 x 4096 at
-  // M = 1 / 4: 4.53 / 4.83 -> 4.38 / 4.52 us; 14336 x 4096 at M = 4: 9.1 -> 9.3 us)
+  // M = 1 / 4: 4.53 / 4.83 -> 4.38 / 4.52 us; 14336 x 4096 at M = 4: 9.1 -> 9.3 us; with 16 staged rows, where every
+  // wavefront would fetch 16 rows of its own slice: 4096 x 4096 at M = 16 5.39 -> 5.47 us, 14336 x 4096 11.08 -> 11.07 us)
   p.PRIV = (cfg.wn == 1 && perm == nullptr && cfg.mr <= 4 && cfg.gs <= 8 && tuning().exp[0] != 1) ? 1 : 0;
-  if (tuning().exp[0] == 2 && cfg.wn == 1 && perm == nullptr) p.PRIV = 1;      // (development switch: private fill wherever it can run)
   const int MB = (M + 15) / 16;
   if (cfg.sk > 1) {
     VAQ_CHECK_ARG(c_tmp != nullptr && counters != nullptr, "w4a16_gemm: split-K needs c_tmp and counters");
