@@ -417,6 +417,35 @@ def test_scaled_mm_every_tile_shape_exact(device, cfg):
         assert bool((t == 0).all()), "arrival counters not restored to zero"
 
 
+def test_scaled_mm_tiles_of_last_round_split_exact(device):
+    """More 256 x 256 tiles than compute units with a last round of workgroups at most half full (17 x 16 tiles on 256
+    units): the tiles of that round run in K parts, the others whole -- the library says so through the scratch it asks
+    for.  Small-integer operands make every partial sum exact: the result must equal the integer GEMM on every tile,
+    twice in a row, and the arrival counters return to zero."""
+    import ctypes
+    import vllm_amd._custom_ops as ops
+    from vllm_amd import _lib
+    m, n, k = 17 * 256, 4096, 2048
+    lib = _lib.load()
+    cus = lib.vaq_num_cus(torch.device(device).index or 0)
+    tiles = (m // 256) * (n // 256)
+    if not (tiles > cus and 0 < tiles % cus <= cus // 2):
+        pytest.skip(f"{tiles} tiles on {cus} compute units leave no half-empty last round")
+    sizes = [ctypes.c_size_t() for _ in range(2)]
+    _lib.check(lib.vaq_fp8_scaled_mm_workspace(m, n, k, *map(ctypes.byref, sizes)))
+    rest, parts = tiles % cus, min(cus // (tiles % cus), 4, k // 64 // 16)
+    assert sizes[0].value == rest * parts * 256 * 256 * 4, "the plan does not split exactly the tiles of the last round"
+    g = torch.Generator().manual_seed(2)
+    a = torch.randint(-2, 3, (m, k), generator=g).float()
+    w = torch.randint(-1, 2, (n, k), generator=g).float()
+    args = (a.to(torch.float8_e4m3fn).to(device), w.to(torch.float8_e4m3fn).to(device).t(),
+            torch.ones(m, 1, device=device), torch.ones(n, 1, device=device), torch.float16)
+    ref = (a.to(device) @ w.to(device).t()).cpu()
+    for rep in range(2):
+        assert torch.equal(ops.cutlass_scaled_mm(*args).cpu().float(), ref), f"run {rep}"
+    assert all(bool((t == 0).all()) for t in ops._FP8_COUNTERS.values()), "arrival counters not restored to zero"
+
+
 def test_scaled_mm_split_k_exact_and_deterministic(device):
     """Few output tiles and a long K: the tile kernel splits K over workgroups (fp32 partial tiles through the op's
     scratch, arrival counters left zero).  Small-integer operands make every partial sum exact, so the split result

@@ -239,6 +239,47 @@ def test_prefill_register_dequant_tile(device, dtype, asym):
         assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
 
 
+@pytest.mark.parametrize("asym", [False, True])
+def test_prefill_tiles_of_last_round_split(device, asym):
+    """More 256 x 256 tiles than compute units with a last round of workgroups at most half full (17 x 16 tiles on 256
+    units): the tiles of that round run in K parts, the others whole.  The library says so through the scratch it asks
+    for; one-hot activations come back exact from every tile, split or whole; against the same kernel with every tile
+    whole the result is equal on the whole tiles' rows and one rounding apart elsewhere; counters return to zero."""
+    from vllm_amd import _lib, _tuning
+    import ctypes
+    k, n, m = 2048, 4096, 17 * 256
+    lib = _lib.load()
+    cus = lib.vaq_num_cus(torch.device(device).index or 0)
+    tiles = (m // 256) * (n // 256)
+    if not (tiles > cus and 0 < tiles % cus <= cus // 2):
+        pytest.skip(f"{tiles} tiles on {cus} compute units leave no half-empty last round")
+    sizes = [ctypes.c_size_t() for _ in range(3)]
+    _lib.check(lib.vaq_w4a16_gemm_workspace(m, n, k, 0, 0, *map(ctypes.byref, sizes)))
+    rest, parts = tiles % cus, min(cus // (tiles % cus), 4, k // 128 // 8)
+    assert sizes[0].value == rest * parts * 256 * 256 * 4, "the plan does not split exactly the tiles of the last round"
+    case = o.make_w4a16_case(k, n, 128, asym=asym, seed=5)
+    layer = W4A16Layer(case, device)
+    w = o.case_w_ref(case)
+    rows = [(37 * i + 32 * (i % 4)) % k for i in range(m)]
+    a = torch.zeros(m, k, dtype=torch.bfloat16)
+    a[torch.arange(m), torch.tensor(rows)] = 1
+    assert torch.equal(layer(a.to(device)).cpu(), w[rows]), "one-hot rows through split and whole tiles"
+    a = _acts(m, k, device, seed=3)
+    out = layer(a)
+    assert torch.equal(out, layer(a)), "not deterministic run to run"
+    check_gemm_close(out[-512:], o.gemm_ref(a[-512:].cpu(), w), "rows of split and of whole tiles against the oracle")
+    for tile in (20, 30):      # the same tile kernel with and without the split
+        with _tuning.override(prefill_tile=tile + 1):
+            out = layer(a)
+        with _tuning.override(prefill_tile=tile + 1, exp=[0] * 10 + [1]):
+            whole = layer(a)
+        check_gemm_close(out, whole.double().cpu(), f"tile {tile}: tiles of the last round split against whole tiles")
+        same = (out == whole).all(dim=1)
+        assert int(same.sum()) >= m - 256 * ((rest + n // 256 - 1) // (n // 256) + 4), "whole tiles changed as well"
+        assert not bool(same.all()), "no tile was split"
+    assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
+
+
 @pytest.mark.parametrize("group_size", [-1, 32, 64])
 @pytest.mark.parametrize("k,n", [(128, 64), (1024, 192), (2048, 576), (14336 // 4, 128)])
 @pytest.mark.parametrize("m", [1, 4, 16, 17, 32, 33, 200, 257])

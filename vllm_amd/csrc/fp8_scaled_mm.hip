@@ -15,6 +15,7 @@
 // of which 32 bytes a lane supplies yields the exact dot product; both kernels give lane (row, q) the bytes
 // k0 + 32*q .. k0 + 32*q + 31 of its row.
 #include "vaq_common.h"
+#include "tile_handover.h"
 
 #include <type_traits>
 
@@ -36,6 +37,7 @@ struct Fp8MMParams {
   float* c_tmp = nullptr;        // fp32 partial tiles when K is split over workgroups (SK > 1)
   int32_t* counters = nullptr;   // arrival counters, zero on entry, left zero
   int SK = 1;
+  int tail_first = 0;            // 0: every tile in SK parts; > 0: only the tiles from this position on (see tile_slot)
   int rotate_k = 0;              // multi-stage tile kernel: tile rows start their K loop at different places (see the kernel)
   uint32_t a_extent = 0, b_extent = 0;   // stream kernel: bytes up to the end of the last row of a / b (below 2 GiB)
   int nt_base = 0, nt_rem = 0;   // stream kernel: n-tiles per workgroup = nt_base, one more for the first nt_rem (N/16 split on the host)
@@ -180,70 +182,13 @@ __device__ inline void tile_epilogue_lds(const Fp8MMParams& p, v16f (&acc)[WMB][
   }
 }
 
-// The tail of the multi-stage tile kernels: (split K) hand the partial tile over and let the last arriver sum, then the
-// scaled epilogue.  `t` = tile number, `total` = tiles of the problem, `split` = this workgroup's K part; `lds8` = at
-// least NW * 32 * (WNB * 64 + 16) bytes of LDS that every wavefront of the workgroup is done with.
+// The tail of the multi-stage tile kernels: (split K) hand the partial tile over and let one wavefront sum
+// (tile_handover.h), then the scaled epilogue.  `sl` = the workgroup's (tile, K part); `lds8` = at least
+// NW * 32 * (WNB * 64 + 16) bytes of LDS that every wavefront of the workgroup is done with.
 template <bool BF16_OUT, int WMB, int WNB, int NW>
-__device__ inline void fp8_tile_tail(const Fp8MMParams& p, v16f (&acc)[WMB][WNB], uint8_t* lds8, int t, int total, int split,
+__device__ inline void fp8_tile_tail(const Fp8MMParams& p, v16f (&acc)[WMB][WNB], uint8_t* lds8, const TileSlot& sl,
                                      int wave, int lane, int m0, int n0, int wm, int wn) {
-  // ---- split K: hand the partial tile over; the last of the SK workgroups to arrive sums them in split order.
-  // 16-byte buffer stores / loads with the sc1 cache-policy bit (device scope: each XCD has its own L2), one unit of
-  // NV4 KiB per (tile, wavefront), one arrival counter per unit. ----
-  if (p.SK > 1) {
-    constexpr int NV4 = WMB * WNB * 4;
-    constexpr int SC1 = 16;
-    const uint32_t unit = (uint32_t)((t * NW + wave) * NV4) * 1024u;
-    const uint32_t split_stride = (uint32_t)total * (uint32_t)(NW * NV4) * 1024u;
-    const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(p.c_tmp, 0, (int)(split_stride * (uint32_t)p.SK), 0x00020000);
-#pragma unroll
-    for (int i = 0; i < WMB; ++i)
-#pragma unroll
-      for (int j = 0; j < WNB; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), rt, lane * 16,
-                                                 (int)(split * split_stride + unit + ((i * WNB + j) * 4 + q) * 1024), SC1);
-        }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // partial tile acknowledged before the counter moves
-    int32_t* ctr = p.counters + (int64_t)t * NW + wave;
-    int old = 0;
-    if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    old = __builtin_amdgcn_readfirstlane(old);      // lane 0 holds it; a scalar keeps what depends on it scalar
-    if (old != p.SK - 1) return;
-    // CH pieces of two splits in flight at a time (one piece after the other, every load waited for, the last arriver
-    // spent NV4 x SK memory round trips here); each element is still summed in split order, starting from zero
-    constexpr int CH = NV4 < 8 ? NV4 : 8;
-#pragma unroll
-    for (int c0 = 0; c0 < NV4; c0 += CH) {
-      v4f sum[CH];
-#pragma unroll
-      for (int c = 0; c < CH; ++c) sum[c] = v4f{0.f, 0.f, 0.f, 0.f};
-      for (int s0 = 0; s0 < p.SK; s0 += 2) {
-        const int s1 = s0 + 1 < p.SK ? s0 + 1 : s0;
-        v4u r0[CH], r1[CH];
-#pragma unroll
-        for (int c = 0; c < CH; ++c)
-          r0[c] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s0 * split_stride + unit + (c0 + c) * 1024), SC1);
-#pragma unroll
-        for (int c = 0; c < CH; ++c)
-          r1[c] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s1 * split_stride + unit + (c0 + c) * 1024), SC1);
-#pragma unroll
-        for (int c = 0; c < CH; ++c) sum[c] += __builtin_bit_cast(v4f, r0[c]);
-        if (s0 + 1 < p.SK) {
-#pragma unroll
-          for (int c = 0; c < CH; ++c) sum[c] += __builtin_bit_cast(v4f, r1[c]);
-        }
-      }
-#pragma unroll
-      for (int c = 0; c < CH; ++c) {
-        const int pc = c0 + c, ij = pc / 4, q = pc % 4;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[ij / WNB][ij % WNB][4 * q + e] = sum[c][e];
-      }
-    }
-    if (lane == 0) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
+  if (sl.nsplit > 1 && !handover_finish<WMB, WNB, NW>(p.c_tmp, p.counters, acc, sl, wave, lane)) return;
 
   if (((uintptr_t)p.out & 15) == 0)
     tile_epilogue_lds<BF16_OUT, WMB, WNB>(p, acc, m0, n0, wm, wn, lane, lds8 + wave * (32 * (WNB * 64 + 16)));
@@ -492,8 +437,8 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
 
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   const int total = tiles_m * tiles_n;
-  int t = blockIdx.x;
-  if (total % 8 == 0) t = (t & 7) * (total / 8) + (t >> 3);          // one contiguous range of tile ids per XCD
+  const TileSlot sl = tile_slot(total, p.SK, p.tail_first);          // one contiguous range of tile positions per XCD
+  const int t = sl.pos;
   constexpr int GM = 4;                                              // band height in tiles (2 .. 16 measured: 4 is 1-2 % ahead of 8)
   const int band = t / (GM * tiles_n);
   const int first_m = band * GM;
@@ -512,10 +457,9 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
   const uint32_t voff_b = (uint32_t)lrow * (uint32_t)p.ldb + (uint32_t)(c16 & 3) * 16u;
 
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
-  // K may be split over blockIdx.y: this workgroup covers the steps [s_lo, s_hi)
+  // K may be split over workgroups: this one covers the steps [s_lo, s_hi)
   const int all_steps = p.K / (64 * KS);
-  const int split = blockIdx.y;
-  const int s_lo = (int)(((int64_t)all_steps * split) / p.SK), s_hi = (int)(((int64_t)all_steps * (split + 1)) / p.SK);
+  const int s_lo = (int)(((int64_t)all_steps * sl.split) / sl.nsplit), s_hi = (int)(((int64_t)all_steps * (sl.split + 1)) / sl.nsplit);
   const int steps = s_hi - s_lo;
   // Few tile rows (M at most 4 tiles high) on a device that the tiles do not fill: the tiles of one column would read
   // the same weight rows at the same time, which leaves only (ring depth x 64 KS) bytes per weight row in flight --
@@ -687,7 +631,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
   }
 
   static_assert(NST * STAGE >= NW * 32 * (WNB * 64 + 16), "operand ring too small for the epilogue staging");
-  fp8_tile_tail<BF16_OUT, WMB, WNB, NW>(p, acc, lds8, t, total, split, wave, lane, m0, n0, wm, wn);
+  fp8_tile_tail<BF16_OUT, WMB, WNB, NW>(p, acc, lds8, sl, wave, lane, m0, n0, wm, wn);
 }
 
 // ----------------------------------------------------------------------------- stream kernel (M <= 32, narrow layers M <= 64)
@@ -1075,13 +1019,19 @@ static int launch_tile3(const Fp8MMParams& p, hipStream_t s) {
   static size_t reserved[VAQ_MAX_DEVICES];
   if (const int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "fp8_scaled_mm"); rc != VAQ_OK) return rc;
   const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
-  hipLaunchKernelGGL(kern, dim3(tiles, p.SK), dim3(WAVES_M * WAVES_N * 64), lds, s, p);
+  const dim3 grid = p.tail_first > 0 ? dim3(p.tail_first + (tiles - p.tail_first) * p.SK) : dim3(tiles, p.SK);
+  hipLaunchKernelGGL(kern, grid, dim3(WAVES_M * WAVES_N * 64), lds, s, p);
   return VAQ_OK;
 }
 
 struct Fp8TilePlan {
   int cfg, sk, bm, bn, nw;
   int64_t tiles;
+  int64_t tail_first = 0;      // > 0: only the tiles from this position on are split (tile_handover.h)
+  // scratch of the K split: partial tiles and arrival counters of the tiles that are split
+  int64_t split_tiles() const { return sk > 1 ? tiles - tail_first : 0; }
+  int64_t tmp_bytes() const { return (int64_t)sk * split_tiles() * bm * bn * 4; }
+  int64_t counter_ints() const { return split_tiles() * nw; }
 };
 
 // Tile shape and K split of the multi-stage kernel.  K is split when the output tiles alone leave compute units idle,
@@ -1222,9 +1172,27 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   }
   break;
   }
+  // 256 x 256 tiles (one workgroup per compute unit) whose count ends in a round of workgroups that is at most half full:
+  // the tiles of that round are split over K so that their parts fill it, the others stay whole.  Parts of at least 16
+  // steps.  (The gain is less than the rounds saved: a half-empty round runs faster per workgroup than a full one -- the
+  // device is power-limited -- and the parts' hand-over costs 10-15 us.)
+  pl.tail_first = 0;
+  if (sk == 1 && pl.bm == 256 && pl.bn == 256 && pl.nw == 8 && pl.tiles > cus && tuning().exp[10] != 1 && tuning().fp8_split <= 0) {
+    const int64_t rest = pl.tiles % cus;
+    if (rest > 0 && rest * 2 <= cus && steps >= 32 && (steps >= 128 || rest * 8 <= cus || tuning().exp[10] == 2)) {
+      int parts = (int)(cus / rest);
+      if (parts > 4) parts = 4;
+      if (parts > steps / 16) parts = steps / 16;
+      if (parts >= 2) {
+        sk = parts;
+        pl.tail_first = pl.tiles - rest;
+      }
+    }
+  }
   if (tuning().fp8_split > 0) sk = tuning().fp8_split <= steps ? tuning().fp8_split : steps;
-  while (sk > 1 && (uint64_t)sk * (uint64_t)pl.tiles * pl.bm * pl.bn * 4 >= (1ull << 32)) --sk;   // 32-bit buffer offsets
+  while (sk > 1 && (uint64_t)sk * (uint64_t)(pl.tiles - pl.tail_first) * pl.bm * pl.bn * 4 >= (1ull << 32)) --sk;   // 32-bit buffer offsets
   pl.sk = sk;
+  if (sk == 1) pl.tail_first = 0;
   return pl;
 }
 
@@ -1236,10 +1204,12 @@ static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t c
   if (direct_ok && tuning().fp8_tile_impl == 0 && tuning().fp8_tile_cfg >= 0) {
     Fp8TilePlan pl = plan_tile3(p.M, p.N, p.K);
     // without (enough) scratch from the caller the unsplit kernel still gives the result
-    if (pl.sk > 1 && (p.c_tmp == nullptr || p.counters == nullptr || counter_ints < pl.tiles * pl.nw ||
-                      c_tmp_bytes < (int64_t)pl.sk * pl.tiles * pl.bm * pl.bn * 4))
+    if (pl.sk > 1 && (p.c_tmp == nullptr || p.counters == nullptr || counter_ints < pl.counter_ints() ||
+                      c_tmp_bytes < pl.tmp_bytes()))
       pl.sk = 1;
+    if (pl.sk == 1) pl.tail_first = 0;
     p.SK = pl.sk;
+    p.tail_first = (int)pl.tail_first;
     {
       const int64_t tiles_m = (p.M + pl.bm - 1) / pl.bm;
       // (with K split over workgroups the rotation gains nothing on cold weights and costs 20-30 % on cached ones)
@@ -1473,10 +1443,8 @@ extern "C" int vaq_fp8_scaled_mm_workspace_tuned(int64_t size_m, int64_t size_n,
   }
   if (size_k % 64 != 0 || tuning().fp8_tile_impl != 0 || tuning().fp8_tile_cfg < 0) return VAQ_OK;
   const Fp8TilePlan pl = plan_tile3((int)size_m, (int)size_n, (int)size_k);
-  if (pl.sk > 1) {
-    *c_tmp_bytes = (size_t)pl.sk * (size_t)pl.tiles * pl.bm * pl.bn * sizeof(float);
-    *counter_ints = (size_t)pl.tiles * pl.nw;
-  }
+  *c_tmp_bytes = (size_t)pl.tmp_bytes();
+  *counter_ints = (size_t)pl.counter_ints();
   return VAQ_OK;
 }
 

@@ -42,7 +42,8 @@ typedef struct VaqTuning {
                         /*   the LDS-staged decode kernel, [3] = 1 sixteen staged rows for M = 5 .. 8, [5] = 1 two K   */
                         /*   slabs never merged into one; [4] FP8 streaming through LDS (1 / 2 / 3 = 8 / 4 / 16 steps   */
                         /*   per wavefront, 9 = off); [8] = 1 W4A16 tile kernel: no 128 x 128 tiles for long K parts;   */
-                        /*   [9] = 1 both tile kernels: 256-row tiles also when M fills them poorly; the rest unused   */
+                        /*   [9] = 1 both tile kernels: 256-row tiles also when M fills them poorly; [10] = 1 both tile     */
+                        /*   kernels: never split only the tiles of a half-empty last round; the rest unused          */
 } VaqTuning;
 
 /* The entry points of the same name without `_tuned`, with `tuning` (may be NULL) applied to this call. */

@@ -230,7 +230,12 @@ extern "C" int vaq_w4a16_gemm_static(const void* a, int64_t lda, const int32_t* 
                                      int64_t size_n, int64_t size_k, int group_size, int dtype, int wtype, void* stream) {
   using namespace vaq;
   size_t c_tmp_bytes = 0, a_tmp_bytes = 0, counter_ints = 0;
-  int rc = vaq_w4a16_gemm_workspace(size_m, size_n, size_k, perm != nullptr, 0, &c_tmp_bytes, &a_tmp_bytes, &counter_ints);
+  // The tile kernel's option of splitting the tiles of a half-empty last round over K is left out here: it is worth
+  // tens of MB of partial tiles at thousands of rows, and whole tiles give the same result.
+  VaqTuning whole_tiles = {};
+  whole_tiles.exp[10] = 1;
+  int rc = vaq_w4a16_gemm_workspace_tuned(size_m, size_n, size_k, perm != nullptr, 0, &c_tmp_bytes, &a_tmp_bytes, &counter_ints,
+                                          &whole_tiles);
   if (rc != VAQ_OK) return rc;
   const size_t c_tmp_span = (c_tmp_bytes + 255) & ~(size_t)255;
   VAQ_CHECK_ARG(counter_ints <= STATIC_COUNTER_INTS && c_tmp_span + a_tmp_bytes <= STATIC_DATA_BYTES,
@@ -245,7 +250,8 @@ extern "C" int vaq_w4a16_gemm_static(const void* a, int64_t lda, const int32_t* 
   }
   int32_t* counters = reinterpret_cast<int32_t*>(base);
   unsigned char* data = base ? base + STATIC_COUNTER_INTS * 4 : nullptr;
-  return vaq_w4a16_gemm(a, lda, b, scales, zeros, perm, bias, c, c_tmp_bytes ? reinterpret_cast<float*>(data) : nullptr,
-                        (int64_t)c_tmp_bytes, a_tmp_bytes ? data + c_tmp_span : nullptr, counters,
-                        (int64_t)STATIC_COUNTER_INTS, size_m, size_n, size_k, group_size, dtype, wtype, 0, stream);
+  return vaq_w4a16_gemm_tuned(a, lda, b, scales, zeros, perm, bias, c, c_tmp_bytes ? reinterpret_cast<float*>(data) : nullptr,
+                              (int64_t)c_tmp_bytes, a_tmp_bytes ? data + c_tmp_span : nullptr, counters,
+                              (int64_t)STATIC_COUNTER_INTS, size_m, size_n, size_k, group_size, dtype, wtype, 0, stream,
+                              &whole_tiles);
 }

@@ -105,6 +105,11 @@ static int pick_tile(int M, int N, int K, bool direct_ok, bool reg_ok) {
 struct PrefillPlan {
   int tile, sk, bm, bn, nw;
   int64_t tiles;
+  int64_t tail_first;      // > 0: only the tiles from this position on are split (tile_handover.h)
+  // scratch of the K split: partial tiles and arrival counters of the tiles that are split
+  int64_t split_tiles() const { return sk > 1 ? tiles - tail_first : 0; }
+  int64_t tmp_bytes() const { return (int64_t)sk * split_tiles() * bm * bn * 4; }
+  int64_t counter_ints() const { return split_tiles() * nw; }
 };
 
 // Tile shape and K split for a problem.  K is split (direct-to-LDS tiles only) when the output tiles alone leave
@@ -125,6 +130,7 @@ static PrefillPlan plan_prefill(int M, int N, int K, bool direct_ok, bool reg_ok
   }
   pl.sk = 1;
   pl.tiles = 0;
+  pl.tail_first = 0;
   if (pl.bm == 0) return pl;
   pl.tiles = (int64_t)((M + pl.bm - 1) / pl.bm) * ((N + pl.bn - 1) / pl.bn);
   const int cus = num_cus_current_device();
@@ -149,16 +155,41 @@ static PrefillPlan plan_prefill(int M, int N, int K, bool direct_ok, bool reg_ok
       if (fine > sk) sk = fine;
     }
   }
+  // 256 x 256 tiles (one workgroup per compute unit) whose count ends in a round of workgroups that is at most half full:
+  // the tiles of that round are split over K so that their parts fill it, the others stay whole (4096 x 6144 at M = 4096:
+  // 384 tiles = 256 whole + 128 in two parts each, 205 -> 189 us; M = 3072, 256 + 32 in four parts, 196 -> 156 us;
+  // 14336 x 4096 at M = 5120: 662 -> 509 us; 4096 x 28672 at M = 2560, 1024 + 96 in two parts: 542 -> 516 us).  The gain is
+  // less than the rounds saved: a half-empty round runs faster per workgroup than a full one (the device is
+  // power-limited), and the parts' hand-over costs 15 us.  Parts of at least 8 groups.
+  if (sk == 1 && pl.bm == 256 && pl.bn == 256 && pl.tiles > cus && tuning().exp[10] != 1 && tuning().prefill_split <= 0) {
+    const int64_t rest = pl.tiles % cus;
+    if (rest > 0 && rest * 2 <= cus && G >= 16) {
+      int parts = (int)(cus / rest);
+      if (parts > 4) parts = 4;
+      if (parts > G / 8) parts = G / 8;
+      if (parts >= 2) {
+        sk = parts;
+        pl.tail_first = pl.tiles - rest;
+        // (the parts run on the 8-wavefront kernel: short K ranges suit the register-dequantising one badly -- 4096 x 6144
+        // at M = 4096: 205 -> 189 us against 207 -> 210 us; 4096 x 4096 at M = 4352: 195 -> 154 against 206 -> 176 us)
+        if (pl.tile == 30 && tuning().prefill_tile <= 0) {
+          pl.tile = 20;
+          pl.nw = 8;
+        }
+      }
+    }
+  }
   if (tuning().prefill_split > 0) sk = tuning().prefill_split <= G ? tuning().prefill_split : G;
-  while (sk > 1 && (uint64_t)sk * (uint64_t)pl.tiles * pl.bm * pl.bn * 4 >= (1ull << 32)) --sk;   // 32-bit buffer offsets
+  while (sk > 1 && (uint64_t)sk * (uint64_t)(pl.tiles - pl.tail_first) * pl.bm * pl.bn * 4 >= (1ull << 32)) --sk;   // 32-bit buffer offsets
   pl.sk = sk;
+  if (sk == 1) pl.tail_first = 0;
   return pl;
 }
 
 int w4a16_prefill_workspace(int M, int N, int K, size_t* c_tmp_bytes, size_t* counter_ints) {
   const PrefillPlan pl = plan_prefill(M, N, K, true);
-  *c_tmp_bytes = pl.sk > 1 ? (size_t)pl.sk * (size_t)pl.tiles * pl.bm * pl.bn * sizeof(float) : 0;
-  *counter_ints = pl.sk > 1 ? (size_t)pl.tiles * pl.nw : 0;
+  *c_tmp_bytes = (size_t)pl.tmp_bytes();
+  *counter_ints = (size_t)pl.counter_ints();
   return VAQ_OK;
 }
 
@@ -191,8 +222,12 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
   // A caller that passes no scratch at all gets the unsplit kernel (same result, no K split); scratch that is there but
   // too small is the caller's mistake and is reported, not worked around.
   if (pl.sk > 1 && c_tmp == nullptr && counters == nullptr) pl.sk = 1;
+  // Splitting only the tiles of a half-empty last round is an optimisation that whole tiles replace at no other cost than
+  // time: scratch that does not hold it (the library-owned scratch of the no-allocation entry point, say) switches it off.
+  if (pl.sk > 1 && pl.tail_first > 0 && (c_tmp_bytes < pl.tmp_bytes() || counter_ints < pl.counter_ints())) pl.sk = 1;
+  if (pl.sk == 1) pl.tail_first = 0;
   if (pl.sk > 1) {
-    const int64_t need_tmp = (int64_t)pl.sk * pl.tiles * pl.bm * pl.bn * 4, need_cnt = pl.tiles * pl.nw;
+    const int64_t need_tmp = pl.tmp_bytes(), need_cnt = pl.counter_ints();
     VAQ_CHECK_ARG(c_tmp != nullptr && counters != nullptr, "w4a16_gemm: split-K needs both c_tmp and counters");
     VAQ_CHECK_ARG(counter_ints >= need_cnt, "w4a16_gemm: workspace.numel = %lld is below min_workspace_size = %lld",
                   (long long)counter_ints, (long long)need_cnt);
@@ -200,6 +235,7 @@ int w4a16_prefill_launch(const void* a, int64_t lda, const int32_t* b, const voi
                   (long long)c_tmp_bytes, (long long)need_tmp);
   }
   p.SK = pl.sk;
+  p.tail_first = (int)pl.tail_first;
   const bool bf16 = dtype == VAQ_BF16, zp = zeros != nullptr;
   int rc;
   // the alternating-phase and the register-dequantising variants exist for 4-bit codes in groups of 128 rows / channelwise

@@ -42,8 +42,8 @@ __global__ __launch_bounds__(256) void w4a16_prefill3_kernel(const PrefillParams
 
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   const int total = tiles_m * tiles_n;
-  int t = blockIdx.x;
-  if (total % 8 == 0) t = (t & 7) * (total / 8) + (t >> 3);          // one contiguous range of tile ids per XCD
+  const TileSlot sl = tile_slot(total, p.SK, p.tail_first);          // one contiguous range of tile positions per XCD
+  const int t = sl.pos;
   constexpr int GM = 4;                                              // bands of 4 tile rows (see the LDS-staged kernel)
   const int band = t / (GM * tiles_n);
   const int first_m = band * GM;
@@ -148,9 +148,8 @@ __global__ __launch_bounds__(256) void w4a16_prefill3_kernel(const PrefillParams
     coff[sl] = (uint32_t)(((lane & 31) >> 1) * 256 + ((((lane & 1) * 8 + chunk) ^ ((lane >> 1) & 15)) * 16));
   }
 
-  // K may be split over blockIdx.y: this workgroup covers the groups [g_lo, g_hi)
-  const int split = blockIdx.y;
-  const int g_lo = (int)(((int64_t)p.G * split) / p.SK), g_hi = (int)(((int64_t)p.G * (split + 1)) / p.SK);
+  // K may be split over workgroups: this one covers the groups [g_lo, g_hi)
+  const int g_lo = (int)(((int64_t)p.G * sl.split) / sl.nsplit), g_hi = (int)(((int64_t)p.G * (sl.split + 1)) / sl.nsplit);
   const int s_lo = 2 * g_lo, s_last = 2 * g_hi - 1;      // K steps of 64
 
   v4u af[WMB];        // B operands (activations) of the current slice, refilled in place
@@ -242,7 +241,7 @@ __global__ __launch_bounds__(256) void w4a16_prefill3_kernel(const PrefillParams
   // epilogue reuses the LDS
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
   static_assert(NST * A_ST >= NW * 32 * (TN * 2 + 16), "stages too small for the epilogue staging");
-  tile_epilogue<BF16, WMB, WNB, NW, TM, TN>(p, acc, lds8, t, total, split, wave, lane, m0, n0, 0, wave);
+  tile_epilogue<BF16, WMB, WNB, NW, TM, TN>(p, acc, lds8, sl, wave, lane, m0, n0, 0, wave);
 }
 
 template <bool BF16, bool HAS_ZP>
@@ -252,7 +251,8 @@ static int launch_prefill3(const PrefillParams& p, hipStream_t s) {
   static size_t reserved[VAQ_MAX_DEVICES];
   if (const int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "w4a16_gemm(prefill)"); rc != VAQ_OK) return rc;
   const int tiles = ((p.M + 255) / 256) * ((p.N + 255) / 256);
-  hipLaunchKernelGGL(kern, dim3(tiles, p.SK), dim3(256), lds, s, p);
+  const dim3 grid = p.tail_first > 0 ? dim3(p.tail_first + (tiles - p.tail_first) * p.SK) : dim3(tiles, p.SK);
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, p);
   return VAQ_OK;
 }
 

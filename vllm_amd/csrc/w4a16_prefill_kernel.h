@@ -18,6 +18,7 @@
 //    lane's 16 bytes (rows 32j .. 32j+31 of the tile) takes the values of sub-group j*SUBG/4.
 #pragma once
 #include "vaq_common.h"
+#include "tile_handover.h"
 
 #include <type_traits>
 
@@ -34,6 +35,7 @@ struct PrefillParams {
   float* c_tmp;        // fp32 partial tiles when K is split over workgroups (SK > 1)
   int32_t* counters;   // arrival counters, zero on entry, left zero
   int M, N, K, G, NT, SK;
+  int tail_first;      // 0: every tile in SK parts; > 0: only the tiles from this position on (see tile_slot)
   int s_stride, z_stride;   // elements between consecutive rows of scales (N) / zeros (N/8); 0 for channelwise scales
 };
 
@@ -332,73 +334,16 @@ __global__ __launch_bounds__(256) void w4a16_prefill_kernel(const PrefillParams 
   }
 }
 
-// The tail of a tile kernel: (split K) hand the partial tile over and let the last arriver sum, then bias, rounding and
-// the stores.  `acc[i][j]` = 32 x 32 block (i along m, j along n) of this wavefront's TM x TN part of the tile at
-// (m0 + wm * TM, n0 + wn * TN), in the layout of an MFMA whose A operand held the weights: lane = column m, four
-// consecutive registers = four consecutive n.  `t` = tile number, `total` = tiles of the problem, `split` = this
-// workgroup's K part; `lds8` = at least NW * 32 * (TN * 2 + 16) bytes of LDS that every wavefront is done with.
+// The tail of a tile kernel: (split K) hand the partial tile over and let one wavefront sum (tile_handover.h), then bias,
+// rounding and the stores.  `acc[i][j]` = 32 x 32 block (i along m, j along n) of this wavefront's TM x TN part of the
+// tile at (m0 + wm * TM, n0 + wn * TN), in the layout of an MFMA whose A operand held the weights: lane = column m, four
+// consecutive registers = four consecutive n.  `sl` = the workgroup's (tile, K part); `lds8` = at least
+// NW * 32 * (TN * 2 + 16) bytes of LDS that every wavefront is done with.
 template <bool BF16, int WMB, int WNB, int NW, int TM, int TN>
-static __device__ inline void tile_epilogue(const PrefillParams& p, v16f (&acc)[WMB][WNB], uint8_t* lds8, int t, int total,
-                                            int split, int wave, int lane, int m0, int n0, int wm, int wn) {
+static __device__ inline void tile_epilogue(const PrefillParams& p, v16f (&acc)[WMB][WNB], uint8_t* lds8, const TileSlot& sl,
+                                            int wave, int lane, int m0, int n0, int wm, int wn) {
   using T = F16Traits<BF16>;
-  // ---- split K: hand the partial tile over; the last of the SK workgroups to arrive sums them in split order ----
-  if (p.SK > 1) {
-    // 16-byte buffer stores / loads with the sc1 cache-policy bit (device scope: written through to, and read from,
-    // memory that all XCDs share -- each XCD has its own L2).  One unit of NV4 KiB per (tile, wavefront).
-    constexpr int NV4 = WMB * WNB * 4;                     // 16-byte pieces per lane
-    constexpr int SC1 = 16;
-    const uint32_t unit = (uint32_t)((t * NW + wave) * NV4) * 1024u;           // bytes
-    const uint32_t split_stride = (uint32_t)total * (uint32_t)(NW * NV4) * 1024u;
-    const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(p.c_tmp, 0, (int)(split_stride * (uint32_t)p.SK), 0x00020000);
-#pragma unroll
-    for (int i = 0; i < WMB; ++i)
-#pragma unroll
-      for (int j = 0; j < WNB; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), rt, lane * 16,
-                                                 (int)(split * split_stride + unit + ((i * WNB + j) * 4 + q) * 1024), SC1);
-        }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // partial tile acknowledged before the counter moves
-    int32_t* ctr = p.counters + (int64_t)t * NW + wave;
-    int old = 0;
-    if (lane == 0) old = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    old = __builtin_amdgcn_readfirstlane(old);      // lane 0 holds it; a scalar keeps what depends on it scalar
-    if (old != p.SK - 1) return;
-    // CH pieces of two splits in flight at a time (one piece after the other, every load waited for, the last arriver
-    // spent NV4 x SK memory round trips here); each element is still summed in split order, starting from zero
-    constexpr int CH = NV4 < 8 ? NV4 : 8;
-#pragma unroll
-    for (int c0 = 0; c0 < NV4; c0 += CH) {
-      v4f sum[CH];
-#pragma unroll
-      for (int c = 0; c < CH; ++c) sum[c] = v4f{0.f, 0.f, 0.f, 0.f};
-      for (int s0 = 0; s0 < p.SK; s0 += 2) {
-        const int s1 = s0 + 1 < p.SK ? s0 + 1 : s0;
-        v4u r0[CH], r1[CH];
-#pragma unroll
-        for (int c = 0; c < CH; ++c)
-          r0[c] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s0 * split_stride + unit + (c0 + c) * 1024), SC1);
-#pragma unroll
-        for (int c = 0; c < CH; ++c)
-          r1[c] = __builtin_amdgcn_raw_buffer_load_b128(rt, lane * 16, (int)(s1 * split_stride + unit + (c0 + c) * 1024), SC1);
-#pragma unroll
-        for (int c = 0; c < CH; ++c) sum[c] += __builtin_bit_cast(v4f, r0[c]);
-        if (s0 + 1 < p.SK) {
-#pragma unroll
-          for (int c = 0; c < CH; ++c) sum[c] += __builtin_bit_cast(v4f, r1[c]);
-        }
-      }
-#pragma unroll
-      for (int c = 0; c < CH; ++c) {
-        const int pc = c0 + c, ij = pc / 4, q = pc % 4;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[ij / WNB][ij % WNB][4 * q + e] = sum[c][e];
-      }
-    }
-    if (lane == 0) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
+  if (sl.nsplit > 1 && !handover_finish<WMB, WNB, NW>(p.c_tmp, p.counters, acc, sl, wave, lane)) return;
 
   // ---- epilogue: four consecutive accumulator registers = four consecutive n of one row.  The 16-bit results cross a
   // wavefront-private piece of LDS (32 rows of TN * 2 + 16 bytes, the operand stages being free by now) and leave as
@@ -524,8 +469,8 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
 
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   const int total = tiles_m * tiles_n;
-  int t = blockIdx.x;
-  if (total % 8 == 0) t = (t & 7) * (total / 8) + (t >> 3);          // one contiguous range of tile ids per XCD
+  const TileSlot sl = tile_slot(total, p.SK, p.tail_first);          // one contiguous range of tile positions per XCD
+  const int t = sl.pos;
   constexpr int GM = 4;                                              // tiles are handed out in bands of 4 tile rows (2 .. 16
                                                                      // measured: 1-3 % ahead of 8 on the large shapes), so
   const int band = t / (GM * tiles_n);                               // that the tiles resident on one XCD share
@@ -765,9 +710,8 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
   using TT = std::true_type;
   using FF = std::false_type;
 
-  // K may be split over blockIdx.y: this workgroup covers the groups [g_lo, g_hi)
-  const int split = blockIdx.y;
-  const int g_lo = (int)(((int64_t)p.G * split) / p.SK), g_hi = (int)(((int64_t)p.G * (split + 1)) / p.SK);
+  // K may be split over workgroups: this one covers the groups [g_lo, g_hi)
+  const int g_lo = (int)(((int64_t)p.G * sl.split) / sl.nsplit), g_hi = (int)(((int64_t)p.G * (sl.split + 1)) / sl.nsplit);
 
   // ---- prologue: activation tiles of the first two steps, weights of the first step (group g_lo, half 0) ----
   issue_a(2 * g_lo, 0);
@@ -945,7 +889,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void w4a16_prefill2_kernel(
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
   static_assert((3 * BM + 2 * BN) * 128 >= NW * 32 * (TN * 2 + 16), "operand stages too small for the epilogue staging");
-  tile_epilogue<BF16, WMB, WNB, NW, TM, TN>(p, acc, lds8, t, total, split, wave, lane, m0, n0, wm, wn);
+  tile_epilogue<BF16, WMB, WNB, NW, TM, TN>(p, acc, lds8, sl, wave, lane, m0, n0, wm, wn);
 }
 
 template <bool BF16, int WMB, int WNB, bool HAS_ZP, int SUBG>
@@ -967,7 +911,8 @@ static int launch_prefill2(const PrefillParams& p, hipStream_t s) {
   static size_t reserved[VAQ_MAX_DEVICES];
   if (const int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "w4a16_gemm(prefill)"); rc != VAQ_OK) return rc;
   const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
-  hipLaunchKernelGGL(kern, dim3(tiles, p.SK), dim3(WAVES_M * WAVES_N * 64), lds, s, p);
+  const dim3 grid = p.tail_first > 0 ? dim3(p.tail_first + (tiles - p.tail_first) * p.SK) : dim3(tiles, p.SK);
+  hipLaunchKernelGGL(kern, grid, dim3(WAVES_M * WAVES_N * 64), lds, s, p);
   return VAQ_OK;
 }
 
