@@ -354,13 +354,39 @@ def test_fused_rms_norm_static_quant(device, tokens, hidden, dtype, add_residual
     _assert_codes_close(out, q_ref, 1e-3)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("hidden", [64, 1024, 4096, 17])
+def test_fused_rms_norm_quant_keeps_the_sign_of_zero(device, dtype, hidden):
+    """Zeros in a row: (-0) * rms * w is -0 and its FP8 code is 0x80, (+0) gives 0x00 -- on the dynamic and the static
+    kernel, rows per wavefront and per workgroup, vector and element-by-element paths.  (A 16-bit product that the
+    compiler forms as a fused multiply-add with a +0 addend would turn -0 into +0.)"""
+    import vllm_amd._custom_ops as ops
+    tokens = 2050 if hidden <= 1024 else 3
+    g = torch.Generator().manual_seed(hidden)
+    x = torch.randn(tokens, hidden, generator=g).to(dtype)
+    x[:, 1::4] = -0.0
+    x[:, 2::4] = 0.0
+    w = (torch.rand(hidden, generator=g) + 0.5).to(dtype)
+    want = torch.zeros(hidden, dtype=torch.uint8)
+    want[1::4] = 0x80
+    zeros = torch.zeros(hidden, dtype=torch.bool)
+    zeros[1::4] = True
+    zeros[2::4] = True
+    q, _ = ops.rms_norm_dynamic_per_token_quant(x.to(device), w.to(device), 1e-5, torch.float8_e4m3fn)
+    assert torch.equal(q.cpu().view(torch.uint8)[:, zeros], want[zeros].expand(tokens, -1)), "dynamic per token"
+    out = torch.empty(tokens, hidden, dtype=torch.float8_e4m3fn, device=device)
+    ops.rms_norm_static_fp8_quant(out, x.to(device), w.to(device), torch.tensor([0.05], device=device), 1e-6)
+    assert torch.equal(out.cpu().view(torch.uint8)[:, zeros], want[zeros].expand(tokens, -1)), "static scale"
+
+
 @pytest.mark.parametrize("tokens", [1, 17, 86, 1234, 3045])
 @pytest.mark.parametrize("hidden", [16, 48, 128, 1562, 4096, 28672])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_silu_and_mul_quant(device, tokens, hidden, dtype):
     """Twin of the reference's test_silu_and_mul (tests/kernels/test_fused_quant_activation.py:33-68, same size grid
-    plus Llama-3-8B's 2*14336).  Codes equal to the oracle's except where the device's expf and the CPU's exp differ in
-    the last bit and that moves a value over a rounding boundary (<= 0.2 %, one code step)."""
+    plus Llama-3-8B's 2*14336).  Codes equal to the oracle's except where the device's exponential and reciprocal and
+    the CPU's exp and division differ in the last bits and that moves a value over a rounding boundary (<= 0.2 %, one
+    code step)."""
     import vllm_amd._custom_ops as ops
     g = torch.Generator().manual_seed(tokens + hidden)
     scale = torch.randn(1, generator=g).abs() + 0.05
@@ -374,6 +400,22 @@ def test_silu_and_mul_quant(device, tokens, hidden, dtype):
         out3 = torch.empty(2, 43, hidden // 2, dtype=torch.float8_e4m3fn, device=device)
         ops.silu_and_mul_quant(out3, x3.to(device), scale.to(device))
         assert torch.equal(out3.reshape(tokens, -1).view(torch.uint8), out.view(torch.uint8))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_silu_and_mul_quant_saturation(device, dtype):
+    """Gate values where the exponential overflows or underflows, signed zeros and +inf: the codes of the oracle, on both
+    the 8-element and the element-by-element path of the kernel."""
+    import vllm_amd._custom_ops as ops
+    gate = torch.tensor([-1e4, -200.0, -100.0, -89.0, -88.0, -87.0, -30.0, -20.0, -0.0, 0.0, 20.0, 30.0, 88.0, 100.0,
+                         1e4, float("inf"), 2.0, -2.0, 1.0, -1.0, 0.5, -0.5, 3.0, -3.0])
+    for d in (24, 21):      # d % 8 == 0: vector path; otherwise scalar path
+        x = torch.cat([gate[:d], torch.full((d,), 1.5)]).to(dtype).reshape(1, 2 * d).repeat(3, 1)
+        out = torch.empty(3, d, dtype=torch.float8_e4m3fn, device=device)
+        scale = torch.tensor([0.25])
+        ops.silu_and_mul_quant(out, x.to(device), scale.to(device))
+        ref = f.ref_silu_and_mul_quant(x, scale)
+        assert torch.equal(out.cpu().view(torch.uint8), ref.view(torch.uint8)), (dtype, d)
 
 
 @pytest.mark.parametrize("offset", [0, 4, 8])

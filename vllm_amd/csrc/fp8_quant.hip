@@ -19,7 +19,7 @@ namespace vaq {
 constexpr float FP8_MAX = 448.0f;
 // (measured: 512 threads with 4 vectors each against 256 x 8: 2.95 -> 2.68 us at 16 rows of 4096, 3.65 -> 3.3 us at 256
 // rows, 41.5 -> 39.5 us at 4096 rows of 14336, unchanged at 4096 x 4096; 1024 x 2 and 128 x 16 are slower)
-constexpr int QT = 512;         // threads per workgroup of the row-per-workgroup kernel
+constexpr int QT = 512;         // threads per workgroup of the row-per-workgroup kernel (its TPB: QT or QT / 2)
 constexpr int QV = 4;           // cached 8-element vectors per thread
 constexpr int QTW = 256;        // threads per workgroup of the row-per-wavefront kernel (four rows)
 
@@ -65,6 +65,7 @@ struct Vec8 {
   }
 };
 
+template <int TPB>
 __device__ inline float block_max(float v, float* smem) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
@@ -73,7 +74,7 @@ __device__ inline float block_max(float v, float* smem) {
   __syncthreads();
   float r = smem[0];
 #pragma unroll
-  for (int i = 1; i < QT / 64; ++i) r = fmaxf(r, smem[i]);
+  for (int i = 1; i < TPB / 64; ++i) r = fmaxf(r, smem[i]);
   __syncthreads();
   return r;
 }
@@ -81,19 +82,19 @@ __device__ inline float block_max(float v, float* smem) {
 // MODE 0: dynamic per token (divide by row scale, scale written per row)
 // MODE 1: per tensor with a given scale (multiply by reciprocal) -- static, and pass 2 of dynamic per tensor
 // MODE 2: absmax only: atomic max of rowmax/448 into *scale (pass 1 of dynamic per tensor)
-template <typename T, int MODE>
-__global__ __launch_bounds__(QT) void fp8_quant_kernel(const T* __restrict__ in, int64_t in_stride,
+template <typename T, int MODE, int TPB>
+__global__ __launch_bounds__(TPB) void fp8_quant_kernel(const T* __restrict__ in, int64_t in_stride,
                                                         uint8_t* __restrict__ out, int64_t out_stride,
                                                         float* __restrict__ scales, const float* __restrict__ scale_ub,
                                                         int hidden) {
-  __shared__ float smem[QT / 64];
+  __shared__ float smem[TPB / 64];
   const int64_t row = blockIdx.x;
   const T* x = in + row * in_stride;
   uint8_t* y = out + row * out_stride;
   const int tid = threadIdx.x;
 
   const bool vec_ok = (hidden % 8 == 0) && (((uintptr_t)x % 16) == 0) && (((uintptr_t)y % 8) == 0) &&
-                      (hidden <= QT * QV * 8);
+                      (hidden <= TPB * QV * 8);
   Vec8<T> cache[QV];
   const int nvec = hidden / 8;
 
@@ -103,7 +104,7 @@ __global__ __launch_bounds__(QT) void fp8_quant_kernel(const T* __restrict__ in,
     if (vec_ok) {
 #pragma unroll
       for (int i = 0; i < QV; ++i) {
-        const int v = tid + i * QT;
+        const int v = tid + i * TPB;
         if (v < nvec) {
           cache[i].load(x + (int64_t)v * 8);
 #pragma unroll
@@ -111,9 +112,9 @@ __global__ __launch_bounds__(QT) void fp8_quant_kernel(const T* __restrict__ in,
         }
       }
     } else {
-      for (int e = tid; e < hidden; e += QT) amax = fmaxf(amax, fabsf(load_as_float<T>(x + e)));
+      for (int e = tid; e < hidden; e += TPB) amax = fmaxf(amax, fabsf(load_as_float<T>(x + e)));
     }
-    amax = block_max(amax, smem);
+    amax = block_max<TPB>(amax, smem);
     if constexpr (MODE == 2) {
       // non-negative floats order like their bit patterns
       if (tid == 0) atomicMax(reinterpret_cast<int*>(scales), __float_as_int(amax / FP8_MAX));
@@ -129,7 +130,7 @@ __global__ __launch_bounds__(QT) void fp8_quant_kernel(const T* __restrict__ in,
     if (vec_ok) {
 #pragma unroll
       for (int i = 0; i < QV; ++i) {
-        const int v = tid + i * QT;
+        const int v = tid + i * TPB;
         if (v < nvec) cache[i].load(x + (int64_t)v * 8);
       }
     }
@@ -159,18 +160,18 @@ __global__ __launch_bounds__(QT) void fp8_quant_kernel(const T* __restrict__ in,
     if (fast) {
 #pragma unroll
       for (int i = 0; i < QV; ++i) {
-        const int v = tid + i * QT;
+        const int v = tid + i * TPB;
         if (v < nvec) *reinterpret_cast<v2u*>(y + (int64_t)v * 8) = pack8(cache[i].f, conv_fast);
       }
     } else {
 #pragma unroll
       for (int i = 0; i < QV; ++i) {
-        const int v = tid + i * QT;
+        const int v = tid + i * TPB;
         if (v < nvec) *reinterpret_cast<v2u*>(y + (int64_t)v * 8) = pack8(cache[i].f, conv);
       }
     }
   } else {
-    for (int e = tid; e < hidden; e += QT) y[e] = cvt1(conv(load_as_float<T>(x + e)));
+    for (int e = tid; e < hidden; e += TPB) y[e] = cvt1(conv(load_as_float<T>(x + e)));
   }
 }
 
@@ -257,21 +258,25 @@ static void launch_row_per_wave(const void* in, int64_t in_stride, uint8_t* out,
                        scales, ub, (int)hidden, rows);
 }
 
-template <int MODE>
-static int launch_quant(const void* in, int in_dtype, int64_t in_stride, uint8_t* out, int64_t out_stride,
-                        float* scales, const float* ub, int64_t rows, int64_t hidden, hipStream_t s) {
-  const dim3 grid((unsigned)rows), block(QT);
+// Many rows of at most 5120 elements run on workgroups of 256 threads: twice the workgroups per compute unit, each a
+// dependent chain of load, reduction and store of its own, and half the wavefronts in every barrier (4096 rows of 3072 /
+// 4096 / 5120: 10.5 / 12.4 / 14.2 -> 8.3 / 11.0 / 13.4 us, 8192 x 4096 20.9 -> 17.8 us; rows of 8192: 18.6 against 19.3 us
+// with 512 threads; a few hundred rows of 4096: 3.0 against 3.2 us).
+template <int MODE, int TPB>
+static int launch_quant_tpb(const void* in, int in_dtype, int64_t in_stride, uint8_t* out, int64_t out_stride,
+                            float* scales, const float* ub, int64_t rows, int64_t hidden, hipStream_t s) {
+  const dim3 grid((unsigned)rows), block(TPB);
   switch (in_dtype) {
     case VAQ_BF16:
-      hipLaunchKernelGGL((fp8_quant_kernel<bf16_t, MODE>), grid, block, 0, s, (const bf16_t*)in, in_stride, out,
+      hipLaunchKernelGGL((fp8_quant_kernel<bf16_t, MODE, TPB>), grid, block, 0, s, (const bf16_t*)in, in_stride, out,
                          out_stride, scales, ub, (int)hidden);
       break;
     case VAQ_F16:
-      hipLaunchKernelGGL((fp8_quant_kernel<f16_t, MODE>), grid, block, 0, s, (const f16_t*)in, in_stride, out,
+      hipLaunchKernelGGL((fp8_quant_kernel<f16_t, MODE, TPB>), grid, block, 0, s, (const f16_t*)in, in_stride, out,
                          out_stride, scales, ub, (int)hidden);
       break;
     case VAQ_F32:
-      hipLaunchKernelGGL((fp8_quant_kernel<float, MODE>), grid, block, 0, s, (const float*)in, in_stride, out,
+      hipLaunchKernelGGL((fp8_quant_kernel<float, MODE, TPB>), grid, block, 0, s, (const float*)in, in_stride, out,
                          out_stride, scales, ub, (int)hidden);
       break;
     default:
@@ -279,6 +284,14 @@ static int launch_quant(const void* in, int in_dtype, int64_t in_stride, uint8_t
       return VAQ_ERR_INVALID_ARG;
   }
   return VAQ_OK;
+}
+
+template <int MODE>
+static int launch_quant(const void* in, int in_dtype, int64_t in_stride, uint8_t* out, int64_t out_stride,
+                        float* scales, const float* ub, int64_t rows, int64_t hidden, hipStream_t s) {
+  if (rows >= 1024 && hidden <= 5120)
+    return launch_quant_tpb<MODE, QT / 2>(in, in_dtype, in_stride, out, out_stride, scales, ub, rows, hidden, s);
+  return launch_quant_tpb<MODE, QT>(in, in_dtype, in_stride, out, out_stride, scales, ub, rows, hidden, s);
 }
 
 static int check_quant(const char* who, const void* in, int64_t in_stride, const uint8_t* out, int64_t out_stride,

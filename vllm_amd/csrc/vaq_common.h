@@ -86,6 +86,9 @@ inline int reserve_dynamic_lds(const void* kern, size_t lds, size_t (&reserved)[
 // finite s (callers take the general division otherwise); signed zeros keep their sign.
 // The two fused operations are written as instructions: merged into one expression a compiler may rewrite
 // -(q*s - x) as (-q)*s + x, which loses the sign of a zero residual (x = -0 must give -0, the code 0x80).
+// None of the operands may come straight out of a transcendental instruction (v_rcp_f32, v_exp_f32, v_rsq_f32 ...):
+// the wait state that such a result needs before its first use is inserted by the compiler for its own instructions
+// only, not in front of inline assembly.  The callers form r by the IEEE division, which ends in v_div_fixup_f32.
 __device__ inline float div16_exact(float x, float s, float r) {
   float q, e, o;
   asm("v_mul_f32 %0, %1, %2" : "=v"(q) : "v"(x), "v"(r));
