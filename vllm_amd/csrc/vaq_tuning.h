@@ -43,7 +43,8 @@ typedef struct VaqTuning {
                         /*   slabs never merged into one; [4] FP8 streaming through LDS (1 / 2 / 3 = 8 / 4 / 16 steps   */
                         /*   per wavefront, 9 = off); [8] = 1 W4A16 tile kernel: no 128 x 128 tiles for long K parts;   */
                         /*   [9] = 1 both tile kernels: 256-row tiles also when M fills them poorly; [10] = 1 both tile     */
-                        /*   kernels: never split only the tiles of a half-empty last round; the rest unused          */
+                        /*   kernels: never split only the tiles of a half-empty last round; [11] = 1 W4A16 tile kernel:  */
+                        /*   no 128 x 256 tiles; the rest unused                                                      */
 } VaqTuning;
 
 /* The entry points of the same name without `_tuned`, with `tuning` (may be NULL) applied to this call. */

@@ -31,10 +31,13 @@ static int dispatch_tile(const PrefillParams& p, int tile, hipStream_t s) {
 }
 
 // Splits of K for the 256 x 256 tile (one workgroup per compute unit): as many as bring the workgroup count to one per
-// compute unit, every split at least 28 groups (3584 rows) long.
+// compute unit, every split at least 28 groups (3584 rows) long -- 16 groups on a K of up to 4096, so that it can run in
+// two parts (72 .. 127 tiles: 4096 x 6144 at M = 768 / 1024 73.8 / 75.2 -> 62.8 / 68.8 us, 4096 x 4096 at M = 1280 / 1536
+// 73.9 / 76.1 -> 64.7 / 68.8 us, against the 128 x 128 tiles that ran there).
 static int splits_256(int64_t tiles256, int K, int cus) {
+  const int G = K / 128, min_groups = G <= 32 ? 16 : 28;
   int sk = (int)(cus / (tiles256 > 0 ? tiles256 : 1));
-  if (sk > K / 128 / 28) sk = K / 128 / 28;
+  if (sk > G / min_groups) sk = G / min_groups;
   return sk < 1 ? 1 : (sk > 8 ? 8 : sk);
 }
 
@@ -52,6 +55,11 @@ static int pick_tile(int M, int N, int K, bool direct_ok, bool reg_ok) {
     // 256 x 256 tiles stay ahead, 90 against 108 us)
     const bool rows_poorly_filled = (int64_t)M * 10 < (int64_t)((M + 255) / 256) * 256 * 7 && tiles(128, 128) <= 2 * (int64_t)cus &&
                                     tuning().exp[9] != 1;
+    // 128 x 256 tiles (8 wavefronts of 64 x 64) where they fill 85-100 % of the compute units in one round on a short K:
+    // no K split and so no hand-over (4096 x 4096 at M = 1792 / 2048: 75.3 / 82.0 us for 256 x 256 tiles in two parts,
+    // 73.6 / 78.5 us for these; 4096 x 6144 at M = 1280: 79.9 against 76.2 us; on K = 14336 they lose, 232 against 200 us)
+    // (built for 4-bit codes in groups of 128 rows / channelwise, like the register-dequantising kernel: `reg_ok`)
+    if (reg_ok && M > 128 && K <= 4096 && tiles(128, 256) <= cus && tiles(128, 256) * 20 >= (int64_t)cus * 17 && tuning().exp[11] != 1) return 13;
     if (M > 128 && !rows_poorly_filled && tiles(256, 256) * splits_256(tiles(256, 256), K, cus) * 20 >= cus * 11) {
       // 256 x 256.  With at least one tile per compute unit and K unsplit, the kernel that dequantises in registers (four
       // wavefronts of 256 x 64) is 1-4 % ahead at M = 4096 on the four Llama-3-8B layers (206 / 123 / 807 / 400 -> 205 / 121 /
@@ -154,6 +162,8 @@ static PrefillPlan plan_prefill(int M, int N, int K, bool direct_ok, bool reg_ok
       if (fine > G / 3) fine = G / 3;
       if (fine > sk) sk = fine;
     }
+    // 128 x 256 tiles that fill a round of workgroups on their own (what the automatic choice takes them for) stay whole
+    if (pl.tile == 13 && pl.tiles <= cus && pl.tiles * 20 >= (int64_t)cus * 17) sk = 1;
   }
   // 256 x 256 tiles (one workgroup per compute unit) whose count ends in a round of workgroups that is at most half full:
   // the tiles of that round are split over K so that their parts fill it, the others stay whole (4096 x 6144 at M = 4096:
