@@ -457,18 +457,19 @@ def test_scaled_mm_every_tile_shape_exact(device, cfg):
         assert bool((t == 0).all()), "arrival counters not restored to zero"
 
 
-def test_scaled_mm_tiles_of_last_round_split_exact(device):
+@pytest.mark.parametrize("m,n,k", [(17 * 256, 4096, 2048), (21 * 256 - 5, 3328, 2048)])
+def test_scaled_mm_tiles_of_last_round_split_exact(device, m, n, k):
     """More 256 x 256 tiles than compute units with a last round of workgroups at most half full (17 x 16 tiles on 256
-    units): the tiles of that round run in K parts, the others whole -- the library says so through the scratch it asks
+    units; 21 x 13 with a ragged last tile row, whose 17 left-over tiles are no multiple of the 8 XCDs): the tiles of
+    that round run in K parts, the others whole -- the library says so through the scratch it asks
     for.  Small-integer operands make every partial sum exact: the result must equal the integer GEMM on every tile,
     twice in a row, and the arrival counters return to zero."""
     import ctypes
     import vllm_amd._custom_ops as ops
     from vllm_amd import _lib
-    m, n, k = 17 * 256, 4096, 2048
     lib = _lib.load()
     cus = lib.vaq_num_cus(torch.device(device).index or 0)
-    tiles = (m // 256) * (n // 256)
+    tiles = ((m + 255) // 256) * (n // 256)
     if not (tiles > cus and 0 < tiles % cus <= cus // 2):
         pytest.skip(f"{tiles} tiles on {cus} compute units leave no half-empty last round")
     sizes = [ctypes.c_size_t() for _ in range(2)]

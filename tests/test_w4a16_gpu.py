@@ -239,18 +239,19 @@ def test_prefill_register_dequant_tile(device, dtype, asym):
         assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
 
 
+@pytest.mark.parametrize("k,n,m", [(2048, 4096, 17 * 256), (2048, 3328, 21 * 256 - 5)])
 @pytest.mark.parametrize("asym", [False, True])
-def test_prefill_tiles_of_last_round_split(device, asym):
+def test_prefill_tiles_of_last_round_split(device, asym, k, n, m):
     """More 256 x 256 tiles than compute units with a last round of workgroups at most half full (17 x 16 tiles on 256
-    units): the tiles of that round run in K parts, the others whole.  The library says so through the scratch it asks
+    units; 21 x 13 with a ragged last tile row, whose 17 left-over tiles are no multiple of the 8 XCDs): the tiles of
+    that round run in K parts, the others whole.  The library says so through the scratch it asks
     for; one-hot activations come back exact from every tile, split or whole; against the same kernel with every tile
     whole the result is equal on the whole tiles' rows and one rounding apart elsewhere; counters return to zero."""
     from vllm_amd import _lib, _tuning
     import ctypes
-    k, n, m = 2048, 4096, 17 * 256
     lib = _lib.load()
     cus = lib.vaq_num_cus(torch.device(device).index or 0)
-    tiles = (m // 256) * (n // 256)
+    tiles = ((m + 255) // 256) * (n // 256)
     if not (tiles > cus and 0 < tiles % cus <= cus // 2):
         pytest.skip(f"{tiles} tiles on {cus} compute units leave no half-empty last round")
     sizes = [ctypes.c_size_t() for _ in range(3)]
@@ -276,6 +277,7 @@ def test_prefill_tiles_of_last_round_split(device, asym):
         check_gemm_close(out, whole.double().cpu(), f"tile {tile}: tiles of the last round split against whole tiles")
         same = (out == whole).all(dim=1)
         assert int(same.sum()) >= m - 256 * ((rest + n // 256 - 1) // (n // 256) + 4), "whole tiles changed as well"
+        assert bool(same[:256].all()), "the first tile row is whole in both runs"
         assert not bool(same.all()), "no tile was split"
     assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
 

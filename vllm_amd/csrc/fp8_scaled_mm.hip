@@ -1078,8 +1078,10 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   // at M = 288 / 320, 222 tiles, 47.4 -> 41.3 us; on 4096 x 28672, 336 tiles, the 256 x 256 tiles stay ahead, 53 against 75 us)
   const bool rows_poorly_filled = (int64_t)M * 10 < (int64_t)((M + 255) / 256) * 256 * 7 && tiles(128, 256) <= cus &&
                                   tiles(128, 256) * 10 >= cus * 7 && tuning().exp[9] != 1;
+  // (128 x 256 from 55 % of the compute units on: 4096 x 6144 at M = 768, 144 tiles, 40.5 -> 36.1 us; 4096 x 4096 at M = 1280,
+  // 160 tiles, 41.2 -> 36.3 us; at 50 %, 4096 x 4096 at M = 1024, the 128 x 128 tiles win, 29.1 against 35.3 us)
   if (pl.cfg <= 0)
-    pl.cfg = take256 && !rows_poorly_filled ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (take128 ? 3 : 4));
+    pl.cfg = take256 && !rows_poorly_filled ? 1 : (tiles(128, 256) * 20 >= cus * 11 ? 7 : (take128 ? 3 : 4));
   // 256 x 384 tiles (wavefronts of 128 x 96) where the 256 x 256 tiles leave the last round of workgroups badly filled and
   // these do not: 4096 x 6144 at M = 4096 is 384 tiles = 1.5 rounds, or 256 = one round (101.4 -> 92.3 us).  Per tile they
   // are slower (4096 x 4096 at M = 4096: 62.8 against 72.7 us), so only for a gain of a fifth in the fill of the rounds.
