@@ -456,6 +456,40 @@ def vendor_ceiling_section(dev):
     return rows
 
 
+def vendor_small_m_section(dev):
+    """The same two vendor GEMMs beside this library's at M = 16 / 256 / 1024 with cold weights (distinct copies cycle
+    through the graph, as in the decode section): where the weight bytes and the launch matter more than the matrix
+    core.  The W4A16 GEMM stands beside the vendor's bf16 GEMM, which reads four times its weight bytes."""
+    import vllm_amd._custom_ops as ops
+    rows = []
+    gen = torch.Generator(device=dev).manual_seed(5)
+    for (k, n) in LLAMA_SHAPES:
+        n8 = max(2, int(600e6 // (k * n)))
+        w8 = [(torch.randn(n, k, device=dev, generator=gen) * 0.05).to(torch.float8_e4m3fn) for _ in range(n8)]
+        n16 = max(2, n8 // 2)
+        w16 = [(torch.randn(n, k, device=dev, generator=gen) * 0.05).to(torch.bfloat16) for _ in range(n16)]
+        layers = [W4Layer(k, n, dev, gen, asym=True) for _ in range(max(2, int(600e6 // (k * n // 2))))]
+        sb = torch.rand(n, 1, device=dev, generator=gen) + 0.5
+        for m in (16, 256, 1024):
+            a8 = torch.randn(m, k, device=dev, generator=gen).to(torch.float8_e4m3fn)
+            a16 = torch.randn(m, k, device=dev, generator=gen).to(torch.bfloat16)
+            sa = torch.rand(m, 1, device=dev, generator=gen) + 0.5
+            t = {}
+            t["fp8"] = time_graph(lambda: [ops.cutlass_scaled_mm(a8, w.t(), sa, sb, torch.bfloat16) for w in w8], iters=5, warmup=2, inner=n8)
+            try:
+                t["vendor_fp8"] = time_graph(lambda: [torch._scaled_mm(a8, w.t(), scale_a=sa, scale_b=sb.t(), out_dtype=torch.bfloat16)
+                                                      for w in w8], iters=5, warmup=2, inner=n8)
+            except Exception:   # not every torch build exposes row-wise FP8 scaling
+                t["vendor_fp8"] = float("nan")
+            t["w4a16"] = time_graph(lambda: [l(a16) for l in layers], iters=5, warmup=2, inner=len(layers))
+            t["vendor_bf16"] = time_graph(lambda: [torch.matmul(a16, w.t()) for w in w16], iters=5, warmup=2, inner=n16)
+            rows.append(dict(kind="vendor_small_m", K=k, N=n, M=m, cold=True, **{f"{name}_us": v * 1e6 for name, v in t.items()}))
+            log(f"[vendor small M] K={k:5d} N={n:5d} M={m:4d}: FP8 {t['fp8'] * 1e6:6.1f} us (vendor {t['vendor_fp8'] * 1e6:6.1f}) | "
+                f"W4A16 {t['w4a16'] * 1e6:6.1f} us (vendor bf16 {t['vendor_bf16'] * 1e6:6.1f})")
+        del w8, w16, layers
+    return rows
+
+
 def operand_toggle_section(dev):
     """The M = 4096 GEMMs on 4096 x 4096 with random operands and with operands that do not toggle (all activations 1.0,
     all weight codes / bytes equal): the same instruction stream on the same addresses, so the difference is what the
@@ -862,6 +896,7 @@ def main():
         for name, fn in (("prefill", prefill_section), ("fp8", fp8_section), ("fused_norm_quant", fused_norm_quant_section),
                          ("variants", variants_section),
                          ("vendor_ceiling", vendor_ceiling_section),
+                         ("vendor_small_m", vendor_small_m_section),
                          ("operand_toggle", operand_toggle_section),
                          ("host_overhead", host_overhead_section),
                          ("medium_m", medium_m_section),
