@@ -525,6 +525,19 @@ def operand_toggle_section(dev):
                 continue
             rows.append(dict(kind=name, operands="constant" if const else "random", K=k, N=n, M=m, us=t * 1e6, TFLOPs=fl / t / 1e12))
             log(f"[operand toggle] {name:11s} {'constant' if const else 'random  '} operands: {t * 1e6:7.1f} us  {fl / t / 1e12:7.1f} TFLOP/s")
+    # The other face of the same limit: one workgroup per 256 x 256 tile, K unsplit, on a quarter, half and all of the
+    # compute units (M = 1024 / 2048 / 4096).  Every workgroup does the same work; what changes is how many run at once.
+    from vllm_amd import _tuning
+    layer = W4Layer(k, n, dev, gen, asym=True)
+    for mm in (1024, 2048, 4096):
+        a = torch.randn(mm, k, device=dev, generator=gen).to(torch.bfloat16)
+
+        def whole_tiles():
+            with _tuning.override(prefill_tile=21, prefill_split=1):
+                layer(a)
+        t = time_graph(lambda: [whole_tiles() for _ in range(2)], iters=8, warmup=3, inner=2)
+        rows.append(dict(kind="w4a16_whole_tiles", workgroups=(mm // 256) * (n // 256), K=k, N=n, M=mm, us=t * 1e6))
+        log(f"[operand toggle] w4a16, one workgroup per 256 x 256 tile, K unsplit: {(mm // 256) * (n // 256):3d} workgroups {t * 1e6:7.1f} us")
     return rows
 
 
