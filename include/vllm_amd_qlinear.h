@@ -111,6 +111,9 @@ int vaq_w4a16_gemm_workspace(int64_t size_m, int64_t size_n, int64_t size_k, int
  * is internal; `force_path` = 0 auto, 1 decode, 2 prefill (tests / benchmarks).
  * Scratch: `c_tmp` holds at least `c_tmp_bytes` bytes and `counters` at least `counter_ints` zeroed ints; a call whose
  * kernel needs more than it was given returns VAQ_ERR_INVALID_ARG (sizes: vaq_w4a16_gemm_workspace) and launches nothing.
+ * One use of `c_tmp` is optional: at thousands of rows, 256 x 256 tiles that end in a round of workgroups at most half
+ * full run the tiles of that round in K parts when `c_tmp` holds their partial tiles, and whole (same result, slower)
+ * when it does not -- the workspace query reports the size with that use included.
  */
 int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
                    const int32_t* perm, const void* bias, void* c, float* c_tmp, int64_t c_tmp_bytes, void* a_tmp,
@@ -124,7 +127,8 @@ int vaq_w4a16_gemm(const void* a, int64_t lda, const int32_t* b, const void* sca
  * vaq_w4a16_gemm with force_path 0; the partial tiles, permuted activations and arrival counters live in one
  * file-scope device array of VAQ_STATIC_SCRATCH_COUNTER_INTS ints + VAQ_STATIC_SCRATCH_DATA_BYTES bytes per GPU, which
  * a GPU holds from the library's first use on it until the process ends.  The call allocates and frees nothing.
- * A problem whose scratch (vaq_w4a16_gemm_workspace) exceeds that returns VAQ_ERR_INVALID_ARG and launches nothing.
+ * A problem whose scratch (vaq_w4a16_gemm_workspace, without the optional use of c_tmp described above, which this
+ * entry point never makes) exceeds that returns VAQ_ERR_INVALID_ARG and launches nothing.
  * Every call on a GPU uses that GPU's one array: calls that may overlap in time on one GPU (different streams or
  * threads) race on it and must be serialised by the caller.  The first call on a GPU looks the array's address up
  * (hipGetSymbolAddress); make it outside any graph capture.
