@@ -688,7 +688,11 @@ def roofline_mfma(extra):
     out = []
     for r in extra.get("prefill", []):
         if r["M"] == 4096 and r["kind"].endswith("groups"):
-            row = dict(kernel="vaq::w4a16_prefill3_kernel", K=r["K"], N=r["N"], M=r["M"], flops_per_launch=2.0 * r["M"] * r["N"] * r["K"],
+            # whole 256 x 256 tiles run on the register-dequantising kernel; a count that ends in a round of workgroups at
+            # most half full runs on the 8-wavefront kernel, the tiles of that round in K parts
+            tiles, cus = -(-r["M"] // 256) * -(-r["N"] // 256), torch.cuda.get_device_properties(0).multi_processor_count
+            name = "vaq::w4a16_prefill2_kernel" if 0 < tiles % cus <= cus // 2 and tiles > cus else "vaq::w4a16_prefill3_kernel"
+            row = dict(kernel=name, K=r["K"], N=r["N"], M=r["M"], flops_per_launch=2.0 * r["M"] * r["N"] * r["K"],
                        avg_ns=round(r["us"] * 1e3), peak_TFLOPs=BF16_PEAK_TFLOPS, frac=round(r["mfma_frac"], 4))
             v = vendor.get(("vendor_bf16_matmul", r["K"], r["N"]))
             if v:
