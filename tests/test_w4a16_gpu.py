@@ -240,13 +240,14 @@ def test_prefill_register_dequant_tile(device, dtype, asym):
 
 
 @pytest.mark.parametrize("k,n,m", [(2048, 4096, 17 * 256), (2048, 3328, 21 * 256 - 5)])
-@pytest.mark.parametrize("asym", [False, True])
-def test_prefill_tiles_of_last_round_split(device, asym, k, n, m):
+@pytest.mark.parametrize("asym,group_size", [(False, 128), (True, 128), (True, 32)])
+def test_prefill_tiles_of_last_round_split(device, asym, group_size, k, n, m):
     """More 256 x 256 tiles than compute units with a last round of workgroups at most half full (17 x 16 tiles on 256
     units; 21 x 13 with a ragged last tile row, whose 17 left-over tiles are no multiple of the 8 XCDs): the tiles of
     that round run in K parts, the others whole.  The library says so through the scratch it asks
     for; one-hot activations come back exact from every tile, split or whole; against the same kernel with every tile
-    whole the result is equal on the whole tiles' rows and one rounding apart elsewhere; counters return to zero."""
+    whole the result is equal on the whole tiles' rows and one rounding apart elsewhere; counters return to zero.
+    Groups of 32 rows take the same plan on the instances for groups below 128 rows."""
     from vllm_amd import _lib, _tuning
     import ctypes
     lib = _lib.load()
@@ -258,7 +259,7 @@ def test_prefill_tiles_of_last_round_split(device, asym, k, n, m):
     _lib.check(lib.vaq_w4a16_gemm_workspace(m, n, k, 0, 0, *map(ctypes.byref, sizes)))
     rest, parts = tiles % cus, min(cus // (tiles % cus), 4, k // 128 // 8)
     assert sizes[0].value == rest * parts * 256 * 256 * 4, "the plan does not split exactly the tiles of the last round"
-    case = o.make_w4a16_case(k, n, 128, asym=asym, seed=5)
+    case = o.make_w4a16_case(k, n, group_size, asym=asym, seed=5)
     layer = W4A16Layer(case, device)
     w = o.case_w_ref(case)
     rows = [(37 * i + 32 * (i % 4)) % k for i in range(m)]
@@ -269,7 +270,7 @@ def test_prefill_tiles_of_last_round_split(device, asym, k, n, m):
     out = layer(a)
     assert torch.equal(out, layer(a)), "not deterministic run to run"
     check_gemm_close(out[-512:], o.gemm_ref(a[-512:].cpu(), w), "rows of split and of whole tiles against the oracle")
-    for tile in (20, 30):      # the same tile kernel with and without the split
+    for tile in ((20, 30) if group_size == 128 else (10,)):      # the same tile kernel with and without the split
         with _tuning.override(prefill_tile=tile + 1):
             out = layer(a)
         with _tuning.override(prefill_tile=tile + 1, exp=[0] * 10 + [1]):
