@@ -86,7 +86,9 @@ static int pick_tile(int M, int N, int K, bool direct_ok, bool reg_ok) {
     //    (14336 x 4096 at M = 320 .. 512: 79 .. 88 -> 61 .. 79 us);
     //  * 64 x 128 where an odd number of 64-row blocks would leave the last 128-row tile half empty (4096 x 6144 at
     //    M = 192: 28.2 -> 23.4 us; 4096 x 4096 at M = 320: 28.1 -> 23.5 us).
-    if ((tiles(128, 64) >= cus && tiles(128, 128) * 2 >= cus) || (K >= 8192 && tiles(128, 128) * 8 >= (int64_t)cus * 3)) return 12;
+    // (M beyond one 64-row block: with 64 rows or fewer the 128-row tiles are half empty -- 4096 x 28672 at M = 64, 224 tiles
+    // of either size: 48.1 us against 36.6 us for 64 x 128 tiles in two K parts)
+    if (M > 64 && ((tiles(128, 64) >= cus && tiles(128, 128) * 2 >= cus) || (K >= 8192 && tiles(128, 128) * 8 >= (int64_t)cus * 3))) return 12;
     if (M > 64 && ((M + 63) / 64) % 2 == 1 && tiles(64, 128) <= cus) return 14;
     if (M > 64 && tuning().exp[8] != 1) {
       // 128 x 64 tiles whose K parts (two workgroups per compute unit, at most 8 parts of at least 8 groups) would still
