@@ -487,6 +487,21 @@ def test_scaled_mm_tiles_of_last_round_split_exact(device, m, n, k):
     assert all(bool((t == 0).all()) for t in ops._FP8_COUNTERS.values()), "arrival counters not restored to zero"
 
 
+@pytest.mark.parametrize("m,n,k", [(320, 4096, 2048), (512, 4096, 4096), (1000, 2048, 2048 + 64), (200, 4096, 4096 + 192),
+                                   (1024, 6144, 4096), (72, 6656, 1024)])
+def test_scaled_mm_rotated_k_loop_exact(device, m, n, k):
+    """Unsplit tiles that fit one round of workgroups over small weights: every tile row starts its K loop at a
+    different step and wraps around (2 to 16 tile rows here, step counts that the number of tile rows does not divide).
+    Small-integer operands that differ from step to step make the sum exact: a step read twice or not at all changes it."""
+    import vllm_amd._custom_ops as ops
+    g = torch.Generator().manual_seed(m + k)
+    a = torch.randint(-2, 3, (m, k), generator=g).float()
+    w = torch.randint(-1, 2, (n, k), generator=g).float()
+    out = ops.cutlass_scaled_mm(a.to(torch.float8_e4m3fn).to(device), w.to(torch.float8_e4m3fn).to(device).t(),
+                                torch.ones(m, 1, device=device), torch.ones(n, 1, device=device), torch.float16)
+    assert torch.equal(out.cpu().float(), a @ w.t())
+
+
 def test_scaled_mm_split_k_exact_and_deterministic(device):
     """Few output tiles and a long K: the tile kernel splits K over workgroups (fp32 partial tiles through the op's
     scratch, arrival counters left zero).  Small-integer operands make every partial sum exact, so the split result

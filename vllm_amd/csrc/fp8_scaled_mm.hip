@@ -1071,17 +1071,22 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
     if (sk < 1) sk = 1;
     while (sk & (sk - 1)) --sk;
     while (sk > 1 && K / 64 / sk < 40) sk /= 2;
-    return t * sk * 10 >= (int64_t)cus * 6 && (int64_t)M * 5 >= (int64_t)((M + 255) / 256) * 256 * 4;
+    // (rows filled to 80 %; to 70 % from three tile rows on, where the poorly filled row is a third of the tiles or less:
+    // 14336 x 4096 at M = 544 .. 608, cold, 74 .. 76 -> 61 .. 62 us)
+    const int64_t rows256 = (M + 255) / 256;
+    const bool filled = (int64_t)M * 5 >= rows256 * 256 * 4 || (rows256 >= 3 && (int64_t)M * 10 >= rows256 * 256 * 7);
+    return t * sk * 10 >= (int64_t)cus * 6 && filled;
   };
   const bool take256 = tiles(256, 256) * parts256 * 20 >= cus * (parts256 == 2 ? 10 : 11) || long_k_256();
   // (not when M fills less than 70 % of the 256-row tiles and the 128 x 256 tiles fit the device in one round: 3584 x 18944
   // at M = 288 / 320, 222 tiles, 47.4 -> 41.3 us; on 4096 x 28672, 336 tiles, the 256 x 256 tiles stay ahead, 53 against 75 us)
   const bool rows_poorly_filled = (int64_t)M * 10 < (int64_t)((M + 255) / 256) * 256 * 7 && tiles(128, 256) <= cus &&
                                   tiles(128, 256) * 10 >= cus * 7 && tuning().exp[9] != 1;
-  // (128 x 256 from 55 % of the compute units on: 4096 x 6144 at M = 768, 144 tiles, 40.5 -> 36.1 us; 4096 x 4096 at M = 1280,
-  // 160 tiles, 41.2 -> 36.3 us; at 50 %, 4096 x 4096 at M = 1024, the 128 x 128 tiles win, 29.1 against 35.3 us)
+  // (128 x 256 from 70 % of the compute units on.  Between 55 and 70 % they win on weights that are already cached -- 4096 x
+  // 6144 at M = 768, 144 tiles, 40.5 -> 36.1 us -- and lose on cold ones, 36.1 against 42.5 us for the 128 x 128 tiles: a
+  // layer's weights are cold when its turn comes, so the cold figure decides.)
   if (pl.cfg <= 0)
-    pl.cfg = take256 && !rows_poorly_filled ? 1 : (tiles(128, 256) * 20 >= cus * 11 ? 7 : (take128 ? 3 : 4));
+    pl.cfg = take256 && !rows_poorly_filled ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (take128 ? 3 : 4));
   // 256 x 384 tiles (wavefronts of 128 x 96) where the 256 x 256 tiles leave the last round of workgroups badly filled and
   // these do not: 4096 x 6144 at M = 4096 is 384 tiles = 1.5 rounds, or 256 = one round (101.4 -> 92.3 us).  Per tile they
   // are slower (4096 x 4096 at M = 4096: 62.8 against 72.7 us), so only for a gain of a fifth in the fill of the rounds.
@@ -1214,8 +1219,15 @@ static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t c
     p.tail_first = (int)pl.tail_first;
     {
       const int64_t tiles_m = (p.M + pl.bm - 1) / pl.bm;
-      // (with K split over workgroups the rotation gains nothing on cold weights and costs 20-30 % on cached ones)
-      p.rotate_k = pl.sk == 1 && tiles_m > 1 && tiles_m <= 4 && pl.tiles * 5 < (int64_t)num_cus_current_device() * 4;
+      const int64_t cus = num_cus_current_device();
+      // (with K split over workgroups the rotation gains nothing on cold weights and costs 20-30 % on cached ones.)
+      // Up to 4 tile rows on a device that the tiles leave a fifth empty; any number of tile rows in one round of workgroups
+      // when the weights are small enough (32 MiB: 4 MiB per L2) that the part another tile row has just read is still in
+      // the L2 -- cold, 4096 x 4096 at M = 256 .. 512: 16.2 / 23.5 -> 12.7 / 18.8 us, 4096 x 6144 at M = 1024 41.4 -> 36.4 us,
+      // 2048 x 2048 at M = 1024 13.9 -> 11.2 us; larger weights lose (6656 x 6656 at M = 72: 17.3 -> 24.1 us; 4096 x 28672
+      // at M = 192 .. 384: +7 %), and so do tiles that need a second round (4096 x 6144 at M = 768: 35.9 -> 41.6 us).
+      p.rotate_k = pl.sk == 1 && tiles_m > 1 &&
+                   ((tiles_m <= 4 && pl.tiles * 5 < cus * 4) || (pl.tiles <= cus && (int64_t)p.K * p.N <= ((int64_t)32 << 20)));
     }
     switch (pl.cfg) {
       case 1: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 5, 1, 1>(p, s);   // alternating phases (see the kernel)
