@@ -436,7 +436,7 @@ def test_scaled_mm_into_a_view_of_a_wider_buffer(device, offset):
         assert bool((got[:, :offset] == 7).all()) and bool((got[:, offset + n:] == 7).all()), "wrote outside the view"
 
 
-@pytest.mark.parametrize("cfg", [1, 8, 2, 10, 11, 3, 4, 5, 7, 13, 23, 14, 24, 15, 17])
+@pytest.mark.parametrize("cfg", [1, 8, 2, 10, 11, 3, 4, 5, 7, 9, 13, 23, 14, 24, 15, 17])
 def test_scaled_mm_every_tile_shape_exact(device, cfg):
     """Every shape of the multi-stage tile kernel, forced through a per-call tuning override (the automatic choice only reaches
     some of them at any one problem size), including the ones that take two k-slices per step: small-integer operands
@@ -519,11 +519,12 @@ def test_scaled_mm_split_k_exact_and_deterministic(device):
         assert all(bool((t == 0).all()) for t in ops._FP8_COUNTERS.values()), "arrival counters not restored to zero"
 
 
-@pytest.mark.parametrize("k,n", [(13824, 5120), (6656, 6656), (18944, 3584), (9216, 4608), (5120, 5120)])
+@pytest.mark.parametrize("k,n", [(13824, 5120), (6656, 6656), (18944, 3584), (9216, 4608), (5120, 5120), (1024, 18944)])
 def test_tile_plan_branches_other_model_shapes(device, k, n):
     """Layer shapes of other models on which the tile planner takes branches that the Llama-3-8B shapes do not reach
     (K parts rebalanced to one workgroup per compute unit, an unsplit K from 60 % fill on, 256 x 256 tiles in parts of
-    a long K, 128 x 128 instead of 64 x 128 tiles for long parts, two m-blocks of K up to 8192 through LDS rings):
+    a long K, 128 x 128 instead of 64 x 128 tiles for long parts, two m-blocks of K up to 8192 through LDS rings,
+    256 x 128 tiles for one tile row of a wide layer):
     per-token x per-channel with bias, sampled rows against the fp64 oracle, bit-identical run to run, arrival
     counters back at zero."""
     import vllm_amd._custom_ops as ops

@@ -1087,6 +1087,13 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   // layer's weights are cold when its turn comes, so the cold figure decides.)
   if (pl.cfg <= 0)
     pl.cfg = take256 && !rows_poorly_filled ? 1 : (tiles(128, 256) * 10 >= cus * 7 ? 7 : (take128 ? 3 : 4));
+  // One tile row of 129 .. 256 rows on a wide layer: 256 x 128 tiles (8 wavefronts of 64 x 64) from 55 % of the compute units
+  // up to one round -- as many tiles as 128 x 256 ones, but every weight row is read by one workgroup only (cold:
+  // 4096 x 28672 at M = 224 / 256 49.7 / 51.9 -> 45.0 / 47.0 us, 3584 x 18944 at M = 136 .. 256 37.5 .. 46.3 -> 31.2 .. 39.1 us,
+  // 8192 x 28672 at M = 256 97.9 -> 85.7 us; at 42-44 % of the units, 5120 x 13824 and 4096 x 14336, the 128 x 128 tiles
+  // stay ahead by 6-10 %)
+  if (tuning().fp8_tile_cfg <= 0 && M > 128 && M <= 256 && tiles(256, 128) <= cus && tiles(256, 128) * 20 >= (int64_t)cus * 11)
+    pl.cfg = 9;
   // 256 x 384 tiles (wavefronts of 128 x 96) where the 256 x 256 tiles leave the last round of workgroups badly filled and
   // these do not: 4096 x 6144 at M = 4096 is 384 tiles = 1.5 rounds, or 256 = one round (101.4 -> 92.3 us).  Per tile they
   // are slower (4096 x 4096 at M = 4096: 62.8 against 72.7 us), so only for a gain of a fifth in the fill of the rounds.
@@ -1111,6 +1118,7 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
     case 4: case 14: case 24: pl.bm = 64; pl.bn = 128; pl.nw = 4; break;
     case 5: case 15: pl.bm = 64; pl.bn = 64; pl.nw = 4; break;
     case 7: case 17: pl.bm = 128; pl.bn = 256; pl.nw = 8; break;
+    case 9: pl.bm = 256; pl.bn = 128; pl.nw = 8; break;
     case 2: pl.bm = 256; pl.bn = 256; pl.nw = 4; break;
     case 10: case 11: pl.bm = 256; pl.bn = 384; pl.nw = 8; break;
     default: pl.bm = 256; pl.bn = 256; pl.nw = 8; break;
@@ -1247,6 +1255,7 @@ static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t c
       case 15: return launch_tile3<BF16_OUT, 64, 64, 2, 2, 5, 2>(p, s);
       case 5: return launch_tile3<BF16_OUT, 64, 64, 2, 2, 5>(p, s);
       case 17: return launch_tile3<BF16_OUT, 128, 256, 2, 4, 3, 2>(p, s);
+      case 9: return launch_tile3<BF16_OUT, 256, 128, 4, 2, 5>(p, s);
       default: break;
     }
   }
