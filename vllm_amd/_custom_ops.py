@@ -11,6 +11,7 @@ not on a GPU are rejected.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 
 import torch
@@ -34,7 +35,9 @@ def _check(cond: bool, msg) -> None:
 
 
 def _ptr(t: torch.Tensor | None):
-    return None if t is None else ctypes.c_void_p(t.data_ptr())
+    """Address of a tensor's first element for a ``void*`` parameter (a plain int: the declared argument types convert
+    it, and building a ``c_void_p`` object per pointer cost more than the conversion)."""
+    return None if t is None else t.data_ptr()
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -43,8 +46,8 @@ _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 def _stream(device: torch.device):
     """The hipStream_t that torch currently launches on for ``device``."""
     if _raw_stream is not None and device.index is not None:
-        return ctypes.c_void_p(_raw_stream(device.index))
-    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+        return _raw_stream(device.index)
+    return torch.cuda.current_stream(device).cuda_stream
 
 
 def _dtype_tag(dt: torch.dtype) -> int:
@@ -59,6 +62,18 @@ def _dtype_tag(dt: torch.dtype) -> int:
 
 def _is_gpu(t: torch.Tensor) -> bool:
     return t.device.type == "cuda"
+
+
+_NO_GUARD = contextlib.nullcontext()
+
+
+def _on(device: torch.device):
+    """Context in which ``device`` is the current one for the library call.  Nothing is switched, and nothing is paid,
+    when it already is (the usual case: ``torch.cuda.device`` costs 3-4 us of host time per call either way)."""
+    idx = device.index
+    if idx is None or idx == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(idx)
 
 
 # ============================================================================ repack
@@ -88,7 +103,7 @@ def _repack_impl(b_q_weight: torch.Tensor, perm: torch.Tensor, size_k: int, size
     _check_repack_args(b_q_weight, perm, size_k, size_n, num_bits)
     lib = _lib.load()
     pack_factor = 32 // num_bits
-    with torch.cuda.device(b_q_weight.device):
+    with _on(b_q_weight.device):
         out = torch.empty((size_k // GPTQ_MARLIN_TILE, size_n * GPTQ_MARLIN_TILE // pack_factor),
                           dtype=torch.int32, device=b_q_weight.device)
         _lib.check(lib.vaq_w4a16_repack(_ptr(b_q_weight), _ptr(perm) if perm.numel() else None, _ptr(out), size_k,
@@ -125,7 +140,7 @@ def _awq_repack_impl(b_q_weight: torch.Tensor, size_k: int, size_n: int, num_bit
     _check_awq_repack_args(b_q_weight, size_k, size_n, num_bits)
     lib = _lib.load()
     pack_factor = 32 // num_bits
-    with torch.cuda.device(b_q_weight.device):
+    with _on(b_q_weight.device):
         out = torch.empty((size_k // GPTQ_MARLIN_TILE, size_n * GPTQ_MARLIN_TILE // pack_factor),
                           dtype=torch.int32, device=b_q_weight.device)
         _lib.check(lib.vaq_w4a16_repack_awq(_ptr(b_q_weight), _ptr(out), size_k, size_n, num_bits, layout,
@@ -150,94 +165,146 @@ def _opt(t: torch.Tensor | None) -> torch.Tensor | None:
 
 def _check_gemm_args(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, g_idx, perm, workspace, b_q_type_id,
                      size_m, size_n, size_k, is_k_full, is_zp_float):
-    """Host checks of gptq_marlin.cu:689-902 in the same order.  Returns (group_size, has_act_order, has_zp, wtype)."""
-    b_q_type = ScalarType.from_id(b_q_type_id)
-    _check(b_q_type.size_bits in (4, 8), lambda: f"unsupported weight type {b_q_type}")
-    pack_factor = 32 // b_q_type.size_bits
-    _check(a.dim() == 2 and a.size(0) == size_m, lambda: f"Shape mismatch: a.size(0) = {a.size(0)}, size_m = {size_m}")
-    _check(a.size(1) == size_k, lambda: f"Shape mismatch: a.size(1) = {a.size(1)}, size_k = {size_k}")
-    _check(size_k % GPTQ_MARLIN_TILE == 0, lambda: f"size_k = {size_k} is not divisible by tile_size = {GPTQ_MARLIN_TILE}")
-    _check(b_q_weight.dim() == 2 and size_k // GPTQ_MARLIN_TILE == b_q_weight.size(0),
-           lambda: f"Shape mismatch: b_q_weight.size(0) = {b_q_weight.size(0)}, size_k = {size_k}, tile_size = {GPTQ_MARLIN_TILE}")
-    _check(b_q_weight.size(1) % GPTQ_MARLIN_TILE == 0,
-           lambda: f"b_q_weight.size(1) = {b_q_weight.size(1)} is not divisible by tile_size = {GPTQ_MARLIN_TILE}")
-    actual_size_n = (b_q_weight.size(1) // GPTQ_MARLIN_TILE) * pack_factor
-    _check(size_n == actual_size_n, lambda: f"size_n = {size_n}, actual_size_n = {actual_size_n}")
-    _check(_is_gpu(a), "A is not on GPU")
-    _check(a.stride(1) == 1, "A.stride(1) is not 1")
-    _check(a.stride(0) % 8 == 0, "A.stride(0) must divisible by 8")
-    _check(a.data_ptr() % 16 == 0, "A must aligned to 16 bytes")
-    _check(_is_gpu(b_q_weight), "b_q_weight is not on GPU")
-    _check(b_q_weight.is_contiguous(), "b_q_weight is not contiguous")
-    _check(_is_gpu(b_scales), "b_scales is not on GPU")
-    _check(b_scales.is_contiguous(), "b_scales is not contiguous")
+    """Host checks of gptq_marlin.cu:689-902 in the same order.  Returns (group_size, has_act_order, has_zp, wtype).
+    Written as plain tests (no helper call, no message built unless a test fails): the op is called once per layer and
+    decode step, and these checks were a third of its host time."""
+    b_q_type = _SCALAR_TYPE_BY_ID.get(b_q_type_id)      # the named types as the objects of `scalar_types`: compared by identity below
+    if b_q_type is None:
+        b_q_type = ScalarType.from_id(b_q_type_id)
+    bits = b_q_type.size_bits
+    if bits != 4 and bits != 8:
+        raise RuntimeError(f"unsupported weight type {b_q_type}")
+    pack_factor = 32 // bits
+    a_shape, w_shape, s_shape = a.shape, b_q_weight.shape, b_scales.shape
+    if len(a_shape) != 2 or a_shape[0] != size_m:
+        raise RuntimeError(f"Shape mismatch: a.size(0) = {a.size(0)}, size_m = {size_m}")
+    if a_shape[1] != size_k:
+        raise RuntimeError(f"Shape mismatch: a.size(1) = {a.size(1)}, size_k = {size_k}")
+    if size_k % GPTQ_MARLIN_TILE != 0:
+        raise RuntimeError(f"size_k = {size_k} is not divisible by tile_size = {GPTQ_MARLIN_TILE}")
+    if len(w_shape) != 2 or size_k // GPTQ_MARLIN_TILE != w_shape[0]:
+        raise RuntimeError(f"Shape mismatch: b_q_weight.size(0) = {b_q_weight.size(0)}, size_k = {size_k}, "
+                           f"tile_size = {GPTQ_MARLIN_TILE}")
+    if w_shape[1] % GPTQ_MARLIN_TILE != 0:
+        raise RuntimeError(f"b_q_weight.size(1) = {b_q_weight.size(1)} is not divisible by tile_size = {GPTQ_MARLIN_TILE}")
+    actual_size_n = (w_shape[1] // GPTQ_MARLIN_TILE) * pack_factor
+    if size_n != actual_size_n:
+        raise RuntimeError(f"size_n = {size_n}, actual_size_n = {actual_size_n}")
+    if not a.is_cuda:
+        raise RuntimeError("A is not on GPU")
+    a_stride = a.stride()
+    if a_stride[1] != 1:
+        raise RuntimeError("A.stride(1) is not 1")
+    if a_stride[0] % 8 != 0:
+        raise RuntimeError("A.stride(0) must divisible by 8")
+    if a.data_ptr() % 16 != 0:
+        raise RuntimeError("A must aligned to 16 bytes")
+    if not b_q_weight.is_cuda:
+        raise RuntimeError("b_q_weight is not on GPU")
+    if not b_q_weight.is_contiguous():
+        raise RuntimeError("b_q_weight is not contiguous")
+    if not b_scales.is_cuda:
+        raise RuntimeError("b_scales is not on GPU")
+    if not b_scales.is_contiguous():
+        raise RuntimeError("b_scales is not contiguous")
     if c is not None:
-        _check(_is_gpu(c), "c is not on GPU")
-        _check(c.is_contiguous(), "c is not contiguous")
-        _check(c.size(0) == size_m, lambda: f"Shape mismatch: c.size(0) = {c.size(0)}, size_m = {size_m}")
-        _check(c.size(1) == size_n, lambda: f"Shape mismatch: c.size(1) = {c.size(1)}, size_n = {size_n}")
-    _check(b_scales.dim() == 2, lambda: f"b_scales rank = {b_scales.dim()} is not 2")
-    _check(b_scales.size(1) == size_n, lambda: f"b_scales dim 1 = {b_scales.size(1)} is not size_n = {size_n}")
-    num_groups = b_scales.size(0)
+        if not c.is_cuda:
+            raise RuntimeError("c is not on GPU")
+        if not c.is_contiguous():
+            raise RuntimeError("c is not contiguous")
+        if c.size(0) != size_m:
+            raise RuntimeError(f"Shape mismatch: c.size(0) = {c.size(0)}, size_m = {size_m}")
+        if c.size(1) != size_n:
+            raise RuntimeError(f"Shape mismatch: c.size(1) = {c.size(1)}, size_n = {size_n}")
+    if len(s_shape) != 2:
+        raise RuntimeError(f"b_scales rank = {b_scales.dim()} is not 2")
+    if s_shape[1] != size_n:
+        raise RuntimeError(f"b_scales dim 1 = {b_scales.size(1)} is not size_n = {size_n}")
+    num_groups = s_shape[0]
 
     has_act_order = False
     if g_idx is not None and perm is not None:
-        _check(_is_gpu(g_idx), "g_idx is not on GPU")
-        _check(g_idx.is_contiguous(), "g_idx is not contiguous")
-        _check(_is_gpu(perm), "perm is not on GPU")
-        _check(perm.is_contiguous(), "perm is not contiguous")
-        _check((g_idx.size(-1) == 0 and perm.size(-1) == 0) or (g_idx.size(-1) == size_k and perm.size(-1) == size_k),
-               lambda: f"Unexpected g_idx.size(-1) = {g_idx.size(-1)} and perm.size(-1) = {perm.size(-1)}, where size_k = {size_k}")
-        has_act_order = g_idx.size(-1) > 0 and perm.size(-1) > 0
+        if not g_idx.is_cuda:
+            raise RuntimeError("g_idx is not on GPU")
+        if not g_idx.is_contiguous():
+            raise RuntimeError("g_idx is not contiguous")
+        if not perm.is_cuda:
+            raise RuntimeError("perm is not on GPU")
+        if not perm.is_contiguous():
+            raise RuntimeError("perm is not contiguous")
+        n_g, n_p = g_idx.size(-1), perm.size(-1)
+        if not ((n_g == 0 and n_p == 0) or (n_g == size_k and n_p == size_k)):
+            raise RuntimeError(f"Unexpected g_idx.size(-1) = {n_g} and perm.size(-1) = {n_p}, where size_k = {size_k}")
+        has_act_order = n_g > 0 and n_p > 0
     if has_act_order:
         if is_k_full:
-            _check(num_groups > 1, "For act_order, num_groups must be > 1")
-            _check(size_k % num_groups == 0, lambda: f"size_k = {size_k}, is not divisible by num_groups = {num_groups}")
+            if num_groups <= 1:
+                raise RuntimeError("For act_order, num_groups must be > 1")
+            if size_k % num_groups != 0:
+                raise RuntimeError(f"size_k = {size_k}, is not divisible by num_groups = {num_groups}")
             group_size = size_k // num_groups
         else:
             group_size = 0
     elif num_groups > 1:
-        _check(size_k % num_groups == 0, lambda: f"size_k = {size_k}, is not divisible by b_scales.size(0) = {b_scales.size(0)}")
+        if size_k % num_groups != 0:
+            raise RuntimeError(f"size_k = {size_k}, is not divisible by b_scales.size(0) = {b_scales.size(0)}")
         group_size = size_k // num_groups
     else:
         group_size = -1
 
-    _check(global_scale is None, "global_scale can only be used for nvfp4 format.")
+    if global_scale is not None:
+        raise RuntimeError("global_scale can only be used for nvfp4 format.")
     if b_bias is not None:
-        _check(_is_gpu(b_bias), "b_bias is not on GPU")
-        _check(b_bias.is_contiguous(), "b_bias is not contiguous")
-        _check(b_bias.size(0) == size_n, "b_bias.size(0) != size_n")
-        _check(b_bias.stride(0) == 1, "b_bias.stride(0) != 1")
+        if not b_bias.is_cuda:
+            raise RuntimeError("b_bias is not on GPU")
+        if not b_bias.is_contiguous():
+            raise RuntimeError("b_bias is not contiguous")
+        if b_bias.size(0) != size_n:
+            raise RuntimeError("b_bias.size(0) != size_n")
+        if b_bias.stride(0) != 1:
+            raise RuntimeError("b_bias.stride(0) != 1")
     has_zp = b_zeros is not None and b_zeros.size(-1) > 0
     if b_zeros is not None:
-        _check(_is_gpu(b_zeros), "b_zeros is not on GPU")
-        _check(b_zeros.is_contiguous(), "b_zeros is not contiguous")
+        if not b_zeros.is_cuda:
+            raise RuntimeError("b_zeros is not on GPU")
+        if not b_zeros.is_contiguous():
+            raise RuntimeError("b_zeros is not contiguous")
     if has_zp:
-        _check(b_q_type in (scalar_types.uint4, scalar_types.uint8),
-               lambda: f"b_q_type must be u4 or u8 when has_zp = True. Got = {b_q_type}")
-    else:
-        _check(b_q_type in (scalar_types.uint4b8, scalar_types.uint8b128, scalar_types.float8_e4m3fn),
-               lambda: "b_q_type must be uint4b8, uint8b128, float8_e4m3fn or float4_e2m1f when has_zp = False. "
-               f"Got = {b_q_type}")
-    if has_zp and is_zp_float:
-        _check(a.dtype == torch.float16, "Computation type must be float16 (half) when using float zero points.")
+        if b_q_type is not scalar_types.uint4 and b_q_type is not scalar_types.uint8:
+            raise RuntimeError(f"b_q_type must be u4 or u8 when has_zp = True. Got = {b_q_type}")
+    elif (b_q_type is not scalar_types.uint4b8 and b_q_type is not scalar_types.uint8b128
+          and b_q_type is not scalar_types.float8_e4m3fn):
+        raise RuntimeError("b_q_type must be uint4b8, uint8b128, float8_e4m3fn or float4_e2m1f when has_zp = False. "
+                           f"Got = {b_q_type}")
+    if has_zp and is_zp_float and a.dtype != torch.float16:
+        raise RuntimeError("Computation type must be float16 (half) when using float zero points.")
     if has_zp:
-        _check(b_zeros.dim() == 2, lambda: f"b_zeros rank = {b_zeros.dim()} is not 2")
+        z_shape = b_zeros.shape
+        if len(z_shape) != 2:
+            raise RuntimeError(f"b_zeros rank = {b_zeros.dim()} is not 2")
         if is_zp_float:
-            _check(b_zeros.size(1) == size_n, lambda: f"b_zeros dim 1 = {b_zeros.size(1)} is not size_n = {size_n}")
-            _check(num_groups == b_zeros.size(0), lambda: f"b_zeros dim 0 = {b_zeros.size(0)} is not num_groups = {num_groups}")
+            if z_shape[1] != size_n:
+                raise RuntimeError(f"b_zeros dim 1 = {b_zeros.size(1)} is not size_n = {size_n}")
+            if num_groups != z_shape[0]:
+                raise RuntimeError(f"b_zeros dim 0 = {b_zeros.size(0)} is not num_groups = {num_groups}")
         else:
-            _check(b_zeros.size(0) == num_groups, lambda: f"b_zeros dim 0 = {b_zeros.size(0)} is not num_groups = {num_groups}")
-            _check(b_zeros.size(1) == size_n // pack_factor,
-                   lambda: f"b_zeros dim 1 = {b_zeros.size(1)} is not size_n / pack_factor = {size_n // pack_factor}")
-    _check(size_n % GPTQ_MARLIN_MIN_THREAD_N == 0,
-           lambda: f"size_n = {size_n}, is not divisible by min_thread_n = {GPTQ_MARLIN_MIN_THREAD_N}")
-    _check(_is_gpu(workspace) and workspace.dtype == torch.int32, "workspace must be an int32 tensor on GPU")
-    _check(a.dtype in (torch.float16, torch.bfloat16), "gpt_marlin_gemm only supports bfloat16 and float16")
-    _check(b_scales.dtype == a.dtype, lambda: f"b_scales dtype {b_scales.dtype} must equal the activation dtype {a.dtype}")
+            if z_shape[0] != num_groups:
+                raise RuntimeError(f"b_zeros dim 0 = {b_zeros.size(0)} is not num_groups = {num_groups}")
+            if z_shape[1] != size_n // pack_factor:
+                raise RuntimeError(f"b_zeros dim 1 = {b_zeros.size(1)} is not size_n / pack_factor = {size_n // pack_factor}")
+    if size_n % GPTQ_MARLIN_MIN_THREAD_N != 0:
+        raise RuntimeError(f"size_n = {size_n}, is not divisible by min_thread_n = {GPTQ_MARLIN_MIN_THREAD_N}")
+    if not workspace.is_cuda or workspace.dtype != torch.int32:
+        raise RuntimeError("workspace must be an int32 tensor on GPU")
+    a_dtype = a.dtype
+    if a_dtype != torch.float16 and a_dtype != torch.bfloat16:
+        raise RuntimeError("gpt_marlin_gemm only supports bfloat16 and float16")
+    if b_scales.dtype != a_dtype:
+        raise RuntimeError(f"b_scales dtype {b_scales.dtype} must equal the activation dtype {a.dtype}")
 
     # what this build implements out of everything the reference accepts
-    if b_q_type not in (scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8b128, scalar_types.float8_e4m3fn):
+    if (b_q_type is not scalar_types.uint4b8 and b_q_type is not scalar_types.uint4 and b_q_type is not scalar_types.uint8b128
+            and b_q_type is not scalar_types.float8_e4m3fn):
         raise NotImplementedError(f"gptq_marlin_gemm: weight type {b_q_type} is not built for gfx950 "
                                   "(uint4b8 / uint4 / uint8b128 / float8_e4m3fn)")
     if is_zp_float:
@@ -251,18 +318,23 @@ def _check_gemm_args(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, 
         else:
             raise NotImplementedError(f"gptq_marlin_gemm: group_size = {group_size} is not built for gfx950 "
                                       "(only -1, 32, 64, 128)")
-    _check(size_k % GPTQ_MARLIN_MIN_THREAD_K == 0,
-           lambda: f"size_k = {size_k}, is not divisible by min_thread_k = {GPTQ_MARLIN_MIN_THREAD_K}")
-    if b_q_type == scalar_types.float8_e4m3fn:
+    if size_k % GPTQ_MARLIN_MIN_THREAD_K != 0:
+        raise RuntimeError(f"size_k = {size_k}, is not divisible by min_thread_k = {GPTQ_MARLIN_MIN_THREAD_K}")
+    if b_q_type is scalar_types.float8_e4m3fn:
         # weight-only FP8 (marlin_utils_fp8.py): channelwise scales or groups of 128 rows, no act_order
         if group_size not in (-1, 128) or has_act_order:
             raise NotImplementedError("gptq_marlin_gemm: float8_e4m3fn weights take group_size -1 or 128 and no act_order")
         wtype = _lib.VAQ_WTYPE_FE4M3
-    elif b_q_type == scalar_types.uint8b128:
+    elif b_q_type is scalar_types.uint8b128:
         wtype = _lib.VAQ_WTYPE_U8B128
     else:
         wtype = _lib.VAQ_WTYPE_U4 if has_zp else _lib.VAQ_WTYPE_U4B8
     return group_size, has_act_order, has_zp, wtype
+
+
+_SCALAR_TYPE_BY_ID: dict[int, ScalarType] = {
+    t.id: t for t in (scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8, scalar_types.uint8b128,
+                      scalar_types.float8_e4m3fn)}
 
 
 def _gemm_impl(a: torch.Tensor, c_or_none: torch.Tensor | None, b_q_weight: torch.Tensor,
@@ -277,7 +349,7 @@ def _gemm_impl(a: torch.Tensor, c_or_none: torch.Tensor | None, b_q_weight: torc
         workspace, b_q_type, size_m, size_n, size_k, is_k_full, is_zp_float)
     lib = _lib.load()
     dev = a.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         c = c_or_none if c_or_none is not None else torch.empty((size_m, size_n), dtype=a.dtype, device=dev)
         if size_m == 0:
             return c
@@ -326,7 +398,7 @@ def _permute_cols_impl(A: torch.Tensor, perm: torch.Tensor) -> torch.Tensor:
            "perm must be a contiguous int32 tensor of A.size(1) entries")
     _check(A.size(1) % 8 == 0, "A columns must be a multiple of 8")
     lib = _lib.load()
-    with torch.cuda.device(A.device):
+    with _on(A.device):
         out = torch.empty((A.size(0), A.size(1)), dtype=A.dtype, device=A.device)
         _lib.check(lib.vaq_permute_cols(_ptr(A), A.stride(0), _ptr(perm), _ptr(out), A.size(0), A.size(1),
                                         _stream(A.device)))
@@ -341,15 +413,24 @@ def _permute_cols_fake(A, perm):
 
 def _check_quant_io(result: torch.Tensor, input: torch.Tensor) -> tuple[int, int]:
     """common.cu:139-142 / :217-220 checks; returns (num_tokens, hidden)."""
-    _check(_is_gpu(input) and _is_gpu(result), "input and result must be on GPU")
-    _check(input.dim() >= 1 and input.stride(-1) == 1, "last dimension of input must be contiguous")
-    _check(result.stride(-1) == 1, "last dimension of output must be contiguous")
-    _check(result.dtype == FP8_DTYPE, lambda: f"result must be {FP8_DTYPE}")
-    _check(input.dtype in (torch.float16, torch.bfloat16, torch.float32), lambda: f"unsupported input dtype {input.dtype}")
-    _check(input.dim() == 2 and result.dim() == 2, "input and result must be 2-D")
-    hidden = input.size(-1)
-    tokens = input.numel() // hidden if hidden else 0
-    _check(result.size(-1) == hidden and result.size(0) >= tokens, "result shape does not cover input")
+    if not (input.is_cuda and result.is_cuda):
+        raise RuntimeError("input and result must be on GPU")
+    if input.dim() < 1 or input.stride(-1) != 1:
+        raise RuntimeError("last dimension of input must be contiguous")
+    if result.stride(-1) != 1:
+        raise RuntimeError("last dimension of output must be contiguous")
+    if result.dtype != FP8_DTYPE:
+        raise RuntimeError(f"result must be {FP8_DTYPE}")
+    dt = input.dtype
+    if dt != torch.bfloat16 and dt != torch.float16 and dt != torch.float32:
+        raise RuntimeError(f"unsupported input dtype {input.dtype}")
+    in_shape, r_shape = input.shape, result.shape
+    if len(in_shape) != 2 or len(r_shape) != 2:
+        raise RuntimeError("input and result must be 2-D")
+    hidden = in_shape[1]
+    tokens = in_shape[0] if hidden else 0
+    if r_shape[1] != hidden or r_shape[0] < tokens:
+        raise RuntimeError("result shape does not cover input")
     return tokens, hidden
 
 
@@ -359,7 +440,7 @@ def _static_quant_impl(result: torch.Tensor, input: torch.Tensor, scale: torch.T
     if tokens == 0:
         return
     lib = _lib.load()
-    with torch.cuda.device(input.device):
+    with _on(input.device):
         _lib.check(lib.vaq_fp8_quant_static(_ptr(input), _dtype_tag(input.dtype), input.stride(0), _ptr(result),
                                             result.stride(0), _ptr(scale), tokens, hidden, _stream(input.device)))
 
@@ -370,7 +451,7 @@ def _dynamic_quant_impl(result: torch.Tensor, input: torch.Tensor, scale: torch.
     if tokens == 0:
         return
     lib = _lib.load()
-    with torch.cuda.device(input.device):
+    with _on(input.device):
         _lib.check(lib.vaq_fp8_quant_dynamic(_ptr(input), _dtype_tag(input.dtype), input.stride(0), _ptr(result),
                                              result.stride(0), _ptr(scale), tokens, hidden, _stream(input.device)))
 
@@ -386,7 +467,7 @@ def _per_token_quant_impl(result: torch.Tensor, input: torch.Tensor, scale: torc
     if tokens == 0:
         return
     lib = _lib.load()
-    with torch.cuda.device(input.device):
+    with _on(input.device):
         args = (_ptr(input), _dtype_tag(input.dtype), input.stride(0), _ptr(result), result.stride(0), _ptr(scale),
                 _ptr(scale_ub), tokens, hidden, _stream(input.device))
         tune = _tuning.current_ref()
@@ -396,27 +477,48 @@ def _per_token_quant_impl(result: torch.Tensor, input: torch.Tensor, scale: torc
 # ============================================================================ FP8 scaled GEMM
 
 def _check_scaled_mm_args(out, a, b, a_scales, b_scales, bias) -> None:
-    """scaled_mm_entry.cu:179-193 plus the scale-shape rules of c3x/scaled_mm_helper.hpp:5-52."""
-    _check(a.dim() == 2 and b.dim() == 2 and out.dim() == 2, "a, b and out must be 2-D")
-    _check(out.size(0) == a.size(0) and a.size(1) == b.size(0) and b.size(1) == out.size(1),
-           lambda: f"shape mismatch: a {tuple(a.shape)}, b {tuple(b.shape)}, out {tuple(out.shape)}")
-    _check(a.stride(1) == 1 and out.stride(1) == 1, "a and out must be row-major")
-    _check(b.stride(0) == 1, "b must be column-major")
-    _check(out.stride(0) % 16 == 0 and b.stride(1) % 16 == 0, "out.stride(0) and b.stride(1) must be multiples of 16")
+    """scaled_mm_entry.cu:179-193 plus the scale-shape rules of c3x/scaled_mm_helper.hpp:5-52 (plain tests, messages
+    built on failure only: see ``_check_gemm_args``)."""
+    a_shape, b_shape, o_shape = a.shape, b.shape, out.shape
+    if len(a_shape) != 2 or len(b_shape) != 2 or len(o_shape) != 2:
+        raise RuntimeError("a, b and out must be 2-D")
+    m, k = a_shape
+    n = b_shape[1]
+    if o_shape[0] != m or k != b_shape[0] or n != o_shape[1]:
+        raise RuntimeError(f"shape mismatch: a {tuple(a.shape)}, b {tuple(b.shape)}, out {tuple(out.shape)}")
+    a_stride, b_stride, o_stride = a.stride(), b.stride(), out.stride()
+    if a_stride[1] != 1 or o_stride[1] != 1:
+        raise RuntimeError("a and out must be row-major")
+    if b_stride[0] != 1:
+        raise RuntimeError("b must be column-major")
+    if o_stride[0] % 16 != 0 or b_stride[1] % 16 != 0:
+        raise RuntimeError("out.stride(0) and b.stride(1) must be multiples of 16")
+    o_dtype = out.dtype
     if bias is not None:
-        _check(bias.numel() == b.size(1) and bias.is_contiguous() and bias.dim() == 1, "bias must be contiguous [N]")
-        _check(bias.dtype == out.dtype, "bias dtype must equal the output dtype")
-    _check(all(_is_gpu(t) for t in (out, a, b, a_scales, b_scales)), "all tensors must be on GPU")
-    _check(a_scales.dtype == torch.float32 and b_scales.dtype == torch.float32, "scales must be fp32")
-    _check(a_scales.is_contiguous() and b_scales.is_contiguous(), "scales must be contiguous")
-    _check(a_scales.numel() in (1, a.size(0)), lambda: f"a_scales.numel() = {a_scales.numel()} must be 1 or M = {a.size(0)}")
-    _check(b_scales.numel() in (1, b.size(1)), lambda: f"b_scales.numel() = {b_scales.numel()} must be 1 or N = {b.size(1)}")
-    _check(out.dtype in (torch.float16, torch.bfloat16), "out must be float16 or bfloat16")
+        if bias.numel() != n or not bias.is_contiguous() or bias.dim() != 1:
+            raise RuntimeError("bias must be contiguous [N]")
+        if bias.dtype != o_dtype:
+            raise RuntimeError("bias dtype must equal the output dtype")
+    if not (out.is_cuda and a.is_cuda and b.is_cuda and a_scales.is_cuda and b_scales.is_cuda):
+        raise RuntimeError("all tensors must be on GPU")
+    if a_scales.dtype != torch.float32 or b_scales.dtype != torch.float32:
+        raise RuntimeError("scales must be fp32")
+    if not (a_scales.is_contiguous() and b_scales.is_contiguous()):
+        raise RuntimeError("scales must be contiguous")
+    na, nb = a_scales.numel(), b_scales.numel()
+    if na != 1 and na != m:
+        raise RuntimeError(f"a_scales.numel() = {na} must be 1 or M = {m}")
+    if nb != 1 and nb != n:
+        raise RuntimeError(f"b_scales.numel() = {nb} must be 1 or N = {n}")
+    if o_dtype != torch.float16 and o_dtype != torch.bfloat16:
+        raise RuntimeError("out must be float16 or bfloat16")
     if a.dtype != FP8_DTYPE or b.dtype != FP8_DTYPE:
         raise NotImplementedError(f"cutlass_scaled_mm: only {FP8_DTYPE} x {FP8_DTYPE} is built for gfx950 "
                                   f"(got {a.dtype} x {b.dtype})")
-    _check(a.stride(0) % 16 == 0, "a.stride(0) must be a multiple of 16")
-    _check(b.size(0) % 16 == 0 and b.size(1) % 16 == 0, "K and N must be multiples of 16")
+    if a_stride[0] % 16 != 0:
+        raise RuntimeError("a.stride(0) must be a multiple of 16")
+    if k % 16 != 0 or n % 16 != 0:
+        raise RuntimeError("K and N must be multiples of 16")
 
 
 def _scaled_mm_impl(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor, a_scales: torch.Tensor,
@@ -426,7 +528,7 @@ def _scaled_mm_impl(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor, a_scale
         return
     lib = _lib.load()
     dev = a.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         # scratch for the K split of mid-sized M: partial tiles from the caching allocator (capture-safe), arrival
         # counters that are zero on entry and left zero, one array per (device, stream)
         tune = _tuning.current_ref()
@@ -504,7 +606,7 @@ def _rms_norm_quant_impl(result: torch.Tensor, input: torch.Tensor, weight: torc
     if tokens == 0:
         return
     lib = _lib.load()
-    with torch.cuda.device(input.device):
+    with _on(input.device):
         _lib.check(lib.vaq_rms_norm_dynamic_per_token_fp8_quant(
             _ptr(result), _ptr(scale), _ptr(input), inp2.stride(0), _ptr(weight), _ptr(scale_ub), float(epsilon),
             _ptr(residual), _dtype_tag(input.dtype), tokens, hidden, _stream(input.device)))
@@ -532,7 +634,7 @@ def _rms_norm_static_common(who, result, input, residual, weight, scale, epsilon
     if tokens == 0:
         return
     lib = _lib.load()
-    with torch.cuda.device(input.device):
+    with _on(input.device):
         _lib.check(lib.vaq_rms_norm_static_fp8_quant(
             _ptr(result), _ptr(input), inp2.stride(0), _ptr(weight), _ptr(scale), float(epsilon), _ptr(residual),
             _dtype_tag(input.dtype), tokens, hidden, _stream(input.device)))
@@ -560,7 +662,7 @@ def _silu_and_mul_quant_impl(result: torch.Tensor, input: torch.Tensor, scale: t
     if tokens == 0:
         return
     lib = _lib.load()
-    with torch.cuda.device(input.device):
+    with _on(input.device):
         _lib.check(lib.vaq_silu_and_mul_fp8_quant(_ptr(result), _ptr(input), _ptr(scale), _dtype_tag(input.dtype), tokens,
                                                   d, _stream(input.device)))
 

@@ -6,6 +6,7 @@ bias(32) | finite_values_only(1) | nan_repr(8).
 """
 from __future__ import annotations
 
+import functools
 import struct
 from dataclasses import dataclass
 from enum import Enum
@@ -30,8 +31,8 @@ class ScalarType:
     nan_repr: NanRepr = NanRepr.IEEE_754
 
     # ------------------------------------------------------------------ id
-    @property
-    def id(self) -> int:
+    @functools.cached_property
+    def id(self) -> int:      # (computed once per object: the GEMM op takes it on every call)
         val, off = 0, 0
         for name, width in _FIELDS:
             v = getattr(self, name)
