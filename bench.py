@@ -286,6 +286,48 @@ def mix_probe(dev, iters=3000):
     return rows
 
 
+def weight_walk_probe(dev):
+    """Cold read rate of a GEMM tile kernel's weight access pattern, without the GEMM (`vaq_weight_walk_probe` of the
+    bench-only probe library): workgroups that own 64 .. 256 rows of a 4096 x 28672-byte weight matrix (the FP8 gate_up
+    layer) and take 64 .. 512 bytes of each row per step, against long contiguous runs.  Copies of the matrix cycle
+    through 700 MB, so every launch reads from HBM; launch to launch in a HIP graph like the GEMMs."""
+    import ctypes
+    from vllm_amd.build import BENCH_PROBE_PATH
+    lib = ctypes.CDLL(str(BENCH_PROBE_PATH))
+    lib.vaq_weight_walk_probe_name.restype = ctypes.c_char_p
+    lib.vaq_weight_walk_probe.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    rows_total, rowbytes, copies = 28672, 4096, 6
+    pool = torch.empty(copies * rows_total * rowbytes, dtype=torch.uint8, device=dev).random_()
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    out = []
+    for i in range(lib.vaq_weight_walk_probe_count()):
+        name = lib.vaq_weight_walk_probe_name(i).decode()
+
+        def fn():
+            st = torch.cuda.current_stream(dev).cuda_stream
+            for c in range(copies):
+                rc = lib.vaq_weight_walk_probe(i, pool.data_ptr() + c * rows_total * rowbytes, rows_total, rowbytes,
+                                               sink.data_ptr(), st)
+                if rc != 0:
+                    raise RuntimeError(f"vaq_weight_walk_probe({i}) returned {rc}")
+        t = time_graph(fn, iters=5, warmup=2, inner=copies)
+        out.append(dict(config=name, us=t * 1e6, GBps=rows_total * rowbytes / t / 1e9))
+        log(f"[weight walk] {t * 1e6:6.1f} us = {rows_total * rowbytes / t / 1e9:5.0f} GB/s  {name}")
+    # the GEMM beside it: the same bytes as FP8 weights at M = 256, cold
+    import vllm_amd._custom_ops as ops
+    gen = torch.Generator(device=dev).manual_seed(5)
+    w = [pool[c * rows_total * rowbytes:(c + 1) * rows_total * rowbytes].view(torch.float8_e4m3fn).view(rows_total, rowbytes).t()
+         for c in range(copies)]
+    for m in (16, 256):
+        a = torch.randn(m, rowbytes, device=dev, generator=gen).to(torch.float8_e4m3fn)
+        sa = torch.rand(m, 1, device=dev, generator=gen) + 0.5
+        sb = torch.rand(rows_total, 1, device=dev, generator=gen) + 0.5
+        t = time_graph(lambda: [ops.cutlass_scaled_mm(a, wc, sa, sb, torch.bfloat16) for wc in w], iters=5, warmup=2, inner=copies)
+        out.append(dict(config=f"FP8 GEMM M={m}", us=t * 1e6, GBps=rows_total * rowbytes / t / 1e9))
+        log(f"[weight walk] {t * 1e6:6.1f} us = {rows_total * rowbytes / t / 1e9:5.0f} GB/s  the FP8 GEMM on the same bytes at M = {m}")
+    return out
+
+
 def prefill_section(dev):
     """BASELINE.json config 3: asymmetric uint4 + act_order, both readings of its act_order wording.  `rows`: g_idx from a
     random permutation of the K rows (the reference's generator): activations are reordered on every call.  `groups`:
@@ -862,6 +904,8 @@ def main():
     ap.add_argument("--mfma-pass", action="store_true",
                     help="for `rocprofv3 --pmc`: three eager passes of [vendor bf16 GEMM 4096^3, W4A16 and FP8 GEMMs at M = 4096], no timing")
     ap.add_argument("--sections", default="", help="comma-separated subset of the extra sections to run (default: all)")
+    ap.add_argument("--weight-walk-probe", action="store_true",
+                    help="run the weight access pattern probe (bench-only library) and print its table; no product timing")
     ap.add_argument("--mix-probe", action="store_true",
                     help="run the matrix-core instruction-mix probe (bench-only library) and print its table; no product timing")
     ap.add_argument("--counter-pass", action="store_true",
@@ -879,6 +923,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.weight_walk_probe:
+        print(json.dumps(weight_walk_probe(dev), indent=1))
+        return
     if args.mix_probe:
         print(json.dumps(mix_probe(dev), indent=1))
         return
