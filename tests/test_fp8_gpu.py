@@ -488,10 +488,11 @@ def test_scaled_mm_tiles_of_last_round_split_exact(device, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(320, 4096, 2048), (512, 4096, 4096), (1000, 2048, 2048 + 64), (200, 4096, 4096 + 192),
-                                   (1024, 6144, 4096), (72, 6656, 1024)])
+                                   (1024, 6144, 4096), (72, 6656, 1024), (200, 28672, 1024 + 64), (100, 32768, 512 + 64)])
 def test_scaled_mm_rotated_k_loop_exact(device, m, n, k):
     """Unsplit tiles that fit one round of workgroups over small weights: every tile row starts its K loop at a
-    different step and wraps around (2 to 16 tile rows here, step counts that the number of tile rows does not divide).
+    different step and wraps around (2 to 16 tile rows here, step counts that the number of tile rows does not divide);
+    a single tile row on a wide layer: every tile column does (the last two cases).
     Small-integer operands that differ from step to step make the sum exact: a step read twice or not at all changes it."""
     import vllm_amd._custom_ops as ops
     g = torch.Generator().manual_seed(m + k)

@@ -38,7 +38,7 @@ struct Fp8MMParams {
   int32_t* counters = nullptr;   // arrival counters, zero on entry, left zero
   int SK = 1;
   int tail_first = 0;            // 0: every tile in SK parts; > 0: only the tiles from this position on (see tile_slot)
-  int rotate_k = 0;              // multi-stage tile kernel: tile rows start their K loop at different places (see the kernel)
+  int rotate_k = 0;              // multi-stage tile kernel: 1 tile rows, 2 tile columns start their K loop at different places (see the kernel)
   uint32_t a_extent = 0, b_extent = 0;   // stream kernel: bytes up to the end of the last row of a / b (below 2 GiB)
   int nt_base = 0, nt_rem = 0;   // stream kernel: n-tiles per workgroup = nt_base, one more for the first nt_rem (N/16 split on the host)
 };
@@ -466,7 +466,11 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
   // with cold weights the kernel then runs at a fraction of the memory bandwidth.  Tile row tm starts its K loop
   // tm / tiles_m of the way into its range and wraps around: the rows are read at tiles_m places at once, and the later
   // readers find them in the L2 (4096 x 4096 at M = 256, cold: 24.4 -> 18.3 us).
-  const int rot = p.rotate_k ? (tm * steps) / tiles_m : 0;
+  // rotate_k = 2, one or two tile rows on a wide layer: every workgroup reads the same activation rows, and with K a power
+  // of two all of them ask the same few L2 channels for the same lines at the same time.  Tile column tn starts tn / tiles_n
+  // of the way into K instead (4096 x 28672 at M = 72 .. 256, cold: 33.9 .. 45.4 -> 31.1 .. 43.6 us; no change on K = 3584 or
+  // 5120; with 16 tile rows it costs 3-9 %: the tiles of one column then no longer read their weights together).
+  const int rot = p.rotate_k == 1 ? (tm * steps) / tiles_m : (p.rotate_k == 2 ? (tn * steps) / tiles_n : 0);
   auto issue_loads = [&](int step_in, int stage) {
     int step = step_in - s_lo + rot;
     if (step >= steps) step -= steps;
@@ -1149,6 +1153,11 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
       if (sk > steps / min_part) sk = steps / min_part;
       if (sk < 1) sk = 1;
       while (sk & (sk - 1)) --sk;
+      // (two tile rows and more of a short K stay whole: their tile rows start at different K steps, which parts of 16
+      // steps and a hand-over do not beat -- 2048 x 2048 at M = 72 .. 128, 64 tiles: 9.7 .. 10.6 us in two parts, 7.5 .. 8.6 us
+      // whole, 3072 x 1024 at M = 128 11.8 against 11.0 us; from 56 steps on the parts are ahead, 3584 x 2048 at M = 128: 11.9
+      // against 12.8 us, 4096 x 2048: 12.4 against 13.1 us)
+      if (M > pl.bm && steps < 56) sk = 1;
     }
     while (sk < 8 && steps / sk >= 100 && pl.tiles * sk * 2 <= 2 * (int64_t)cus) sk *= 2;
     // between one and 1.75 workgroups per compute unit some units run two of them and set the pace: the parts that give
@@ -1236,6 +1245,16 @@ static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t c
       // at M = 192 .. 384: +7 %), and so do tiles that need a second round (4096 x 6144 at M = 768: 35.9 -> 41.6 us).
       p.rotate_k = pl.sk == 1 && tiles_m > 1 &&
                    ((tiles_m <= 4 && pl.tiles * 5 < cus * 4) || (pl.tiles <= cus && (int64_t)p.K * p.N <= ((int64_t)32 << 20)));
+      // A last tile row filled to a third at most.  Two tile rows: nobody rotates (the nearly empty row finishes early
+      // whatever it reads, and rotated it reads for nothing what the full row does not read with it; cold: 4096 x 4096 at
+      // M = 66 .. 84 13.3 -> 11.1 .. 11.8 us, 4096 x 6144 13.7 -> 11.6 .. 12.5 us).  64 x 64 tiles: the same with three and
+      // four rows (4096 x 4096 at M = 132 .. 144 13.2 -> 11.2 .. 11.9 us, at M = 196 .. 208 13.1 -> 11.5 .. 12.1 us; from a fill
+      // of 24 rows on the rotation is level or ahead).  Larger tiles with three rows and more keep the rotation (64 x 128:
+      // 4096 x 6144 at M = 132 19.5 against 21.2 us, 4096 x 4096 at M = 264 18.2 against 21.1 us).
+      if (p.rotate_k == 1 && ((int64_t)p.M - (tiles_m - 1) * pl.bm) * 3 <= pl.bm && (tiles_m == 2 || pl.bn == 64)) p.rotate_k = 0;
+      // one or two tile rows on a wide layer: by tile column instead (see the kernel)
+      if (p.rotate_k == 0 && pl.sk == 1 && tiles_m <= 2 && pl.tiles * 5 >= cus * 2) p.rotate_k = 2;
+      if (tuning().exp[12] == 1) p.rotate_k = 0;      // (development switch: every tile starts at the first K step)
     }
     switch (pl.cfg) {
       case 1: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 5, 1, 1>(p, s);   // alternating phases (see the kernel)
