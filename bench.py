@@ -245,6 +245,16 @@ def stream_ceiling_section(dev):
                          waves=best[1], depth=best[2]))
         log(f"[read ceiling] {nbytes / 1e6:6.2f} MB (K={k} N={n}): {best[0] * 1e6:6.2f} us launch to launch = {nbytes / best[0] / 1e9:5.0f} GB/s "
             f"({best[1]} wavefronts, {best[2]} loads in flight)")
+    # for scale: what the same kernel reaches when one launch reads the whole pool (more than twice the memory-side cache)
+    big = pool.numel() & ~((1 << 23) - 1)
+
+    def fn_big():
+        rc = lib.vaq_stream_read_probe(ctypes.c_void_p(pool.data_ptr()), big, 8192, 8, ctypes.c_void_p(sink.data_ptr()), stream())
+        if rc != 0:
+            raise RuntimeError(f"vaq_stream_read_probe returned {rc}")
+    t_big = time_graph(fn_big, iters=5, warmup=2, inner=1)
+    log(f"[read ceiling] {big / 1e6:6.1f} MB in one launch: {t_big * 1e6:6.1f} us = {big / t_big / 1e9:5.0f} GB/s (8192 wavefronts, 8 loads in flight): "
+        "what the layers' sizes leave unreached")
     return rows
 
 
