@@ -513,6 +513,31 @@ def test_decode_three_and_four_m_blocks(device, k, n, m):
         assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
 
 
+@pytest.mark.parametrize("k,n,m", [(4096, 4096, 128), (4096, 4096, 121), (4096, 6144, 80), (4096, 6144, 70), (2048, 2048, 256),
+                                   (2048, 2048, 250), (4096, 2048, 128), (4096, 2048, 200), (1024, 1024, 96), (4096, 4096, 96)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_rows_over_workgroups_beyond_four_m_blocks(device, k, n, m, dtype):
+    """65 .. 256 rows on a narrow layer: where workgroups of 16 rows each make one round, the decode kernel takes the rows
+    as five to sixteen m-blocks with workgroups of their own (a ragged last block among them); elsewhere -- the last
+    case, 258 workgroups -- and with act_order the tile kernel does.  Same answer either way: symmetric and with zero
+    points against the fp64 oracle, one-hot rows bit for bit, no scratch used, deterministic."""
+    for asym, act_order in ((False, False), (True, False), (True, True)):
+        case = o.make_w4a16_case(k, n, 128, asym=asym, act_order=act_order, dtype=dtype, seed=k + n + m)
+        layer = W4A16Layer(case, device, dtype)
+        w_ref = o.case_w_ref(case)
+        a = _acts(m, k, device, dtype=dtype, seed=m)
+        out = layer(a)
+        assert out.shape == (m, n) and out.dtype == dtype
+        check_gemm_close(out, o.gemm_ref(a.cpu(), w_ref), f"k={k} n={n} m={m} asym={asym} act_order={act_order}")
+        assert torch.equal(out, layer(a)), "not deterministic run to run"
+        assert bool((layer.workspace == 0).all()), "workspace counters not restored to zero"
+        rows = [(37 * i + 5) % k for i in range(m)]
+        hot = torch.zeros(m, k, dtype=dtype)
+        for i, r in enumerate(rows):
+            hot[i, r] = 1
+        assert torch.equal(layer(hot.to(device)).cpu(), w_ref[rows]), "one-hot rows must return the dequantised weights exactly"
+
+
 # layer shapes of other models on which the planners take branches that the Llama-3-8B shapes do not reach: K slabs that
 # would come out uneven (9216 x 4608, 10240 x 2560), a ragged single slab on a narrow layer (5120 x 5120), a short K on
 # few tiles (1536 x 1536), an odd number of 64-row blocks on a wide short-K layer (2560 x 10240), long K parts on few

@@ -233,19 +233,49 @@ static int dispatch_mr2(const Decode2Params& p, const Decode2Config& c, bool bf1
 }
 
 // Rows split over workgroups (one m-block each, see the kernel) instead of several m-blocks per workgroup: 4-bit codes
-// in groups of 128 rows / channelwise, no act_order, and only where a single m-block needs no split of K.
+// in groups of 128 rows / channelwise, no act_order, and only where a single m-block needs no split of K.  On success
+// `out` is the configuration of the one-m-block kernel that every workgroup runs.
 // (development switch exp[2]: 1 forces it off, 2 on wherever it is built)
-static bool use_row_split(int M, int N, int K, int sub, int wt, bool has_perm) {
+static bool row_split_config(int M, int N, int K, int sub, int wt, bool has_perm, Decode2Config* out) {
   if (M <= 16 || sub != 1 || wt != 0 || has_perm || tuning().exp[2] == 1) return false;
-  const Decode2Config c = pick_decode2_config(16, N, K, sub, false, (M + 15) / 16);
+  const int MB = (M + 15) / 16, NT = N / 16;
+  Decode2Config c = pick_decode2_config(16, N, K, sub, false, MB);
   if (c.sk != 1) return false;
+  *out = c;
   if (tuning().exp[2] == 2) return true;
-  // One round of full workgroups.  Measured: 4096 x 4096 at M = 32 / 64: 8.5 / 10.5 -> 6.6 / 9.2 us, 4096 x 6144: 8.8 / 11.4
-  // -> 8.7 / 10.6 us; with three m-blocks the grids of those layers spill into a second round (15 us) or leave ten
-  // wavefronts per workgroup (9.9 -> 11.7 us).  A 28672-wide layer would need streams of 32 tiles (measured 20.4 -> 21.7 us).
-  // (Two m-blocks also as eight wavefronts of 8-tile streams with the three-slot ring: 4096 x 4096 at M = 32 6.3 us.)
-  const long wgs = (long)((N / 16 + c.wn - 1) / c.wn) * ((M + 15) / 16);
-  return wgs <= num_cus_current_device() && c.wks * c.wn >= (M <= 32 ? 8 : 12);
+  const long cus = num_cus_current_device();
+  if (M <= DECODE2_MAX_M) {
+    // Against two to four m-blocks in one workgroup: one round of full workgroups.  Measured: 4096 x 4096 at M = 32 / 64:
+    // 8.5 / 10.5 -> 6.6 / 9.2 us, 4096 x 6144: 8.8 / 11.4 -> 8.7 / 10.6 us; with three m-blocks the grids of those layers spill
+    // into a second round (15 us) or leave ten wavefronts per workgroup (9.9 -> 11.7 us).  A 28672-wide layer would need
+    // streams of 32 tiles (measured 20.4 -> 21.7 us).
+    // (Two m-blocks also as eight wavefronts of 8-tile streams with the three-slot ring: 4096 x 4096 at M = 32 6.3 us.)
+    const long wgs = (long)((NT + c.wn - 1) / c.wn) * MB;
+    return wgs <= cus && c.wks * c.wn >= (M <= 32 ? 8 : 12);
+  }
+  // Five to sixteen m-blocks, against the tile kernel (whose K step is a latency chain of half a microsecond at these
+  // sizes): the fewest n-tiles per workgroup whose grid -- counted exactly -- is one round of workgroups with at least 12
+  // wavefronts on a compute unit.  Cold: 4096 x 4096 at M = 128 16.2 -> 13.4 us, 4096 x 6144 at M = 80 18.8 -> 13.5 us,
+  // 4096 x 2048 at M = 128 / 256 14.8 / 16.0 -> 8.8 / 13.2 us, 2048 x 2048 at M = 128 / 256 11.5 / 12.5 -> 6.3 / 8.3 us; grids
+  // of a second round lose (4096 x 4096 at M = 96 with 258 workgroups: 16.1 -> 22.3 us), ten wavefronts too (M = 80: 20.2 us).
+  const long lds_slots = (long)((size_t)(160 * 1024) / decode2_lds_bytes(c.wks, c.gs, c.mr, 1));
+  for (int wn = 1; wn * c.wks <= D2_WAVES; ++wn) {
+    long slots = D2_WAVES / (c.wks * wn);
+    if (slots > lds_slots) slots = lds_slots;
+    if (slots < 1) slots = 1;
+    const long wgs = (long)((NT + wn - 1) / wn) * MB;
+    const long per_cu = (wgs + cus - 1) / cus;
+    if (per_cu <= slots && per_cu * c.wks * wn >= 12) {
+      out->wn = wn;
+      return true;
+    }
+  }
+  return false;
+}
+
+bool w4a16_decode2_takes_rows(int M, int N, int K, int sub, int wt, bool has_perm) {
+  Decode2Config c;
+  return M > DECODE2_MAX_M && M <= DECODE2_MAX_M_ROWS && row_split_config(M, N, K, sub, wt, has_perm, &c);
 }
 
 int decode2_launch_msp(const Decode2Params& p, int gs, int rc, bool bf16, bool zp, hipStream_t s);      // w4a16_decode2_msp.hip
@@ -283,8 +313,12 @@ int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const voi
   p.z_stride = channelwise ? 0 : N / 8;
   p.k_mask = 0x000f000fu;
   p.k_ex = dtype == VAQ_BF16 ? 0x43004300u : 0x64006400u;
-  const bool row_split = use_row_split(M, N, K, sub, wt, perm != nullptr);
-  const Decode2Config cfg = row_split ? pick_decode2_config(16, N, K, sub, w8, (M + 15) / 16) : pick_decode2_config(M, N, K, sub, w8);
+  Decode2Config cfg;
+  const bool row_split = row_split_config(M, N, K, sub, wt, perm != nullptr, &cfg);
+  if (!row_split) {
+    VAQ_CHECK_ARG(M <= DECODE2_MAX_M, "w4a16_gemm(decode): %d rows without the split of the rows over workgroups", M);
+    cfg = pick_decode2_config(M, N, K, sub, w8);
+  }
   p.SK = cfg.sk;
   p.WKS = cfg.wks;
   p.WN = cfg.wn;

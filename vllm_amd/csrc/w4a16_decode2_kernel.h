@@ -69,6 +69,8 @@ static __device__ inline __amdgpu_buffer_rsrc_t d2_rsrc32(const void* base, uint
 static inline uint32_t d2_sat32(uint64_t bytes) { return bytes > 0xffffffffull ? 0xffffffffu : (uint32_t)bytes; }
 
 constexpr int D2_WAVES = 16;
+constexpr int DECODE2_MAX_M = 64;           // rows of one workgroup: up to four m-blocks of 16
+constexpr int DECODE2_MAX_M_ROWS = 256;     // rows when every m-block has workgroups of its own (see MSP)
 
 template <bool BF16, int GS, int MB, bool HAS_ZP, int MR, int SUBG, int WT = 0, int RC = 0, bool MSP = false>
 __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Decode2Params p) {

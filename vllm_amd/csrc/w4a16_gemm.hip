@@ -11,6 +11,7 @@ int w4a16_decode_launch(const void* a, int64_t lda, const int32_t* b, const void
                         int32_t* counters, int64_t counter_ints, int M, int N, int K, bool channelwise, int dtype,
                         hipStream_t s);
 int w4a16_decode2_workspace(int M, int N, int K, int sub, bool w8, size_t* c_tmp_bytes, size_t* counter_ints);
+bool w4a16_decode2_takes_rows(int M, int N, int K, int sub, int wt, bool has_perm);
 int w4a16_decode2_launch(const void* a, int64_t lda, const int32_t* b, const void* scales, const int32_t* zeros,
                          const int32_t* perm, const void* bias, void* c, float* c_tmp, int64_t c_tmp_bytes,
                          int32_t* counters, int64_t counter_ints, int M, int N, int K, int sub, bool channelwise,
@@ -161,6 +162,11 @@ extern "C" int vaq_w4a16_gemm_tuned(const void* a, int64_t lda, const int32_t* b
     decode = true;
   } else if (force_path == 2) {
     decode = false;
+  } else if (!decode && !two_blocks_only && size_m <= 256 && size_n < (1 << 24) && size_k < (1 << 24) &&
+             w4a16_decode2_takes_rows((int)size_m, (int)size_n, (int)size_k, sub, wt, perm != nullptr)) {
+    // more rows than one workgroup of the decode kernel takes, on a layer narrow enough that workgroups of 16 rows each
+    // make one round: ahead of the tile kernel there (see row_split_config in w4a16_decode2.hip); needs no scratch
+    decode = true;
   }
   if (decode && decode_impl_for(size_m, size_n, lda, sub, w8) == 0)
     return w4a16_decode2_launch(a, lda, b, scales, zeros, perm, bias, c, c_tmp, c_tmp_bytes, counters, counter_ints, (int)size_m,
