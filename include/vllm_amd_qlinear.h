@@ -106,9 +106,10 @@ int vaq_w4a16_gemm_workspace(int64_t size_m, int64_t size_n, int64_t size_k, int
  *   c        [M, N] activation dtype, contiguous
  *   group_size  128, 64, 32, or -1 / K for channelwise scales (the reference's MARLIN_SUPPORTED_GROUP_SIZES,
  *               marlin_utils.py:24), for every wtype; anything else returns VAQ_ERR_UNSUPPORTED
- * M == 0 is a no-op.  Kernel choice (decode: M <= 32, up to 64 for 4-bit codes in groups of 128 rows or channelwise,
- * MFMA GEMV with in-register dequant; prefill: LDS-staged MFMA)
- * is internal; `force_path` = 0 auto, 1 decode, 2 prefill (tests / benchmarks).
+ * M == 0 is a no-op.  Kernel choice (decode: M <= 32, up to 64 for 4-bit codes in groups of 128 rows or channelwise --
+ * up to 256 on layers narrow enough that workgroups of 16 rows each make one round -- MFMA GEMV with in-register
+ * dequant; prefill: tile kernels, weights dequantised through LDS or in registers)
+ * is internal; `force_path` = 0 auto, 1 decode (M <= 64 at most), 2 prefill (tests / benchmarks).
  * Scratch: `c_tmp` holds at least `c_tmp_bytes` bytes and `counters` at least `counter_ints` zeroed ints; a call whose
  * kernel needs more than it was given returns VAQ_ERR_INVALID_ARG (sizes: vaq_w4a16_gemm_workspace) and launches nothing.
  * One use of `c_tmp` is optional: at thousands of rows, 256 x 256 tiles that end in a round of workgroups at most half
