@@ -503,6 +503,28 @@ def test_scaled_mm_rotated_k_loop_exact(device, m, n, k):
     assert torch.equal(out.cpu().float(), a @ w.t())
 
 
+@pytest.mark.parametrize("m,n,k", [(64, 4096, 4096), (50, 6144, 4096), (33, 8192, 4096), (100, 4096, 2048), (192, 4096, 1024),
+                                   (384, 6144, 512), (130, 2048, 2048), (70, 5120, 5120), (190, 2048, 6656)])
+def test_scaled_mm_tile_row_past_m_exact(device, m, n, k):
+    """Up to three tile rows with compute units to spare: one more row of workgroups runs past M beside them (it reads the
+    same weights, its activation rows do not exist, it stores nothing).  Small-integer operands: the result must equal
+    the integer GEMM, rows next to the output (a taller buffer, M rows of it handed in) must stay untouched, and two
+    runs must agree."""
+    import vllm_amd._custom_ops as ops
+    g = torch.Generator().manual_seed(m * 7 + k)
+    a = torch.randint(-2, 3, (m, k), generator=g).float()
+    w = torch.randint(-1, 2, (n, k), generator=g).float()
+    a_dev = torch.zeros(m + 200, k, dtype=torch.float8_e4m3fn, device=device)      # rows past M exist in memory and are not zero
+    a_dev[m:] = torch.ones(200, k).to(torch.float8_e4m3fn).to(device)
+    a_dev[:m] = a.to(torch.float8_e4m3fn).to(device)
+    args = (a_dev[:m], w.to(torch.float8_e4m3fn).to(device).t(), torch.ones(m, 1, device=device), torch.ones(n, 1, device=device),
+            torch.float16)
+    out = ops.cutlass_scaled_mm(*args)
+    assert out.shape == (m, n)
+    assert torch.equal(out.cpu().float(), a @ w.t())
+    assert torch.equal(out, ops.cutlass_scaled_mm(*args))
+
+
 def test_scaled_mm_split_k_exact_and_deterministic(device):
     """Few output tiles and a long K: the tile kernel splits K over workgroups (fp32 partial tiles through the op's
     scratch, arrival counters left zero).  Small-integer operands make every partial sum exact, so the split result

@@ -39,6 +39,7 @@ struct Fp8MMParams {
   int SK = 1;
   int tail_first = 0;            // 0: every tile in SK parts; > 0: only the tiles from this position on (see tile_slot)
   int rotate_k = 0;              // multi-stage tile kernel: 1 tile rows, 2 tile columns start their K loop at different places (see the kernel)
+  int m_tiles_extra = 0;         // multi-stage tile kernel: tile rows past M (see dispatch_tile: they read the weights with the real ones and store nothing)
   uint32_t a_extent = 0, b_extent = 0;   // stream kernel: bytes up to the end of the last row of a / b (below 2 GiB)
   int nt_base = 0, nt_rem = 0;   // stream kernel: n-tiles per workgroup = nt_base, one more for the first nt_rem (N/16 split on the host)
 };
@@ -435,7 +436,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
-  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  const int tiles_m = (p.M + BM - 1) / BM + p.m_tiles_extra, tiles_n = (p.N + BN - 1) / BN;
   const int total = tiles_m * tiles_n;
   const TileSlot sl = tile_slot(total, p.SK, p.tail_first);          // one contiguous range of tile positions per XCD
   const int t = sl.pos;
@@ -635,6 +636,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void fp8_mm_tile3_kernel(co
   }
 
   static_assert(NST * STAGE >= NW * 32 * (WNB * 64 + 16), "operand ring too small for the epilogue staging");
+  if (m0 >= p.M) return;      // a tile row past M (m_tiles_extra): nothing to hand over or store
   fp8_tile_tail<BF16_OUT, WMB, WNB, NW>(p, acc, lds8, sl, wave, lane, m0, n0, wm, wn);
 }
 
@@ -1022,7 +1024,7 @@ static int launch_tile3(const Fp8MMParams& p, hipStream_t s) {
   auto kern = fp8_mm_tile3_kernel<BF16_OUT, BM, BN, WAVES_M, WAVES_N, NST, KS, PP>;
   static size_t reserved[VAQ_MAX_DEVICES];
   if (const int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "fp8_scaled_mm"); rc != VAQ_OK) return rc;
-  const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  const int tiles = ((p.M + BM - 1) / BM + p.m_tiles_extra) * ((p.N + BN - 1) / BN);
   const dim3 grid = p.tail_first > 0 ? dim3(p.tail_first + (tiles - p.tail_first) * p.SK) : dim3(tiles, p.SK);
   hipLaunchKernelGGL(kern, grid, dim3(WAVES_M * WAVES_N * 64), lds, s, p);
   return VAQ_OK;
@@ -1173,6 +1175,14 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
       const int64_t filled = (int64_t)fit * pl.tiles;
       if (fit >= 1 && steps / fit <= 128 && (fit == 1 ? filled * 5 >= (int64_t)cus * 3 : filled * 10 >= (int64_t)cus * 9)) sk = fit;
     }
+    // Up to three tile rows of K <= 6656 with compute units left for one more row of workgroups stay whole: that row
+    // then runs past M beside them (see m_tiles_extra in dispatch_tile), which parts and their hand-over do not beat:
+    // 5120 x 5120 at M = 40 .. 128 14.2 .. 18.4 -> 13.2 us, 6656 x 6656 at M = 40 / 64 17.7 / 20.7 -> 16.0 / 16.7 us, 4096 x 2048 at
+    // M = 192 12.6 -> 10.6 us; on K = 7168 and 8192 the parts stay ahead, 8192 x 3584 at M = 64 15.7 against 17.8 us.
+    {
+      const int64_t rows = (M + pl.bm - 1) / pl.bm;
+      if (K <= 6656 && rows <= 3 && pl.tiles + pl.tiles / rows <= (int64_t)cus && tuning().exp[13] != 1) sk = 1;
+    }
   }
   // 64 x 128 tiles of a long K whose parts still run 64 steps and more: 128 x 128 tiles instead -- half the tiles, so twice
   // the parts of half the length on the same number of workgroups (cold, M = 80 .. 128: 18944 x 3584 33.8 -> 31.7 us,
@@ -1255,6 +1265,20 @@ static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t c
       // one or two tile rows on a wide layer: by tile column instead (see the kernel)
       if (p.rotate_k == 0 && pl.sk == 1 && tiles_m <= 2 && pl.tiles * 5 >= cus * 2) p.rotate_k = 2;
       if (tuning().exp[12] == 1) p.rotate_k = 0;      // (development switch: every tile starts at the first K step)
+      // A tile row past M.  With at most three tile rows and compute units to spare, one more row of workgroups runs
+      // beside the real ones: its activation rows lie past M (the loads return zeros, nothing is stored), its weight
+      // loads are the real tiles' own.  Every weight line is then asked for by two workgroups on two compute units,
+      // whichever gets there first, and arrives earlier for the other: what one compute unit has in flight is what bounds
+      // a tile's operand stream at these sizes (deeper rings do not help, a second requester does).  Cold, 64 x 64 tiles:
+      // 4096 x 4096 at M = 64 .. 192 13.2 .. 16.4 -> 10.8 .. 11.1 us, 5120 x 5120 at M = 64 / 128 17.0 / 17.4 -> 13.2 / 13.3 us,
+      // 2048 x 2048 at M = 128 8.6 -> 7.3 us; 128 x 128 tiles: 4096 x 6144 at M = 384 25.8 -> 23.5 us, 8192 x 8192 at M = 384
+      // 46.7 -> 41.7 us.  The real rows then start together (rotated they lose the gain); from four tile rows on the
+      // rotation alone is level or ahead (3072 x 3072 at M = 384 14.8 against 16.0 us) and stays.
+      p.m_tiles_extra = 0;
+      if (pl.sk == 1 && pl.tail_first == 0 && tiles_m <= 3 && pl.tiles + pl.tiles / tiles_m <= cus && tuning().exp[13] != 1) {
+        p.m_tiles_extra = 1;
+        p.rotate_k = 0;
+      }
     }
     switch (pl.cfg) {
       case 1: return launch_tile3<BF16_OUT, 256, 256, 2, 4, 5, 1, 1>(p, s);   // alternating phases (see the kernel)
@@ -1323,6 +1347,15 @@ static int stream_steps_per_wave(int64_t M, int64_t N, int64_t K) {
   // 35.9 / 38.7 us: four m-blocks only up to two rounds of workgroups.
   if (M > 32) {
     const bool fits = steps <= 8 * 4 && steps >= 13;
+    // ... unless the 64 x 64 tiles with one more tile row past M fit the device (see m_tiles_extra in dispatch_tile) and the
+    // weights are large enough: that plan takes the same time for 33 as for 64 rows, this kernel's time grows with the
+    // m-blocks.  Cold, M = 40 / 64: 4096 x 6144 12.1 / 15.0 -> 11.3 / 11.4 us, 4096 x 8192 13.2 / 16.1 -> 12.0 / 12.2 us, 4096 x 4096
+    // 9.8 / 12.7 against 10.8 / 10.8 us (the tiles from 49 rows on), 3072 x 3072 7.6 / 9.6 against 9.1 / 9.1 us, 2048 x 2048
+    // 5.5 / 7.0 against 7.4 / 7.4 us (this kernel).
+    const int64_t cols = (N + 63) / 64;
+    if (tuning().exp[13] != 1 && tuning().fp8_tile_cfg <= 0 && K % 128 == 0 && 2 * cols <= (int64_t)num_cus_current_device() &&
+        (K * N >= ((int64_t)20 << 20) || (M > 48 && K * N >= ((int64_t)8 << 20))))
+      return 0;
     return (fits && (M <= 48 || (M <= 64 && N / 16 <= 2 * num_cus_current_device()))) ? 4 : 0;
   }
   if (steps <= 8 * 4) return 4;
