@@ -509,7 +509,7 @@ def vendor_ceiling_section(dev):
 
 
 def vendor_small_m_section(dev):
-    """The same two vendor GEMMs beside this library's at M = 16 / 256 / 1024 with cold weights (distinct copies cycle
+    """The same two vendor GEMMs beside this library's at M = 16 / 64 / 128 / 256 / 1024 with cold weights (distinct copies cycle
     through the graph, as in the decode section): where the weight bytes and the launch matter more than the matrix
     core.  The W4A16 GEMM stands beside the vendor's bf16 GEMM, which reads four times its weight bytes."""
     import vllm_amd._custom_ops as ops
@@ -522,7 +522,7 @@ def vendor_small_m_section(dev):
         w16 = [(torch.randn(n, k, device=dev, generator=gen) * 0.05).to(torch.bfloat16) for _ in range(n16)]
         layers = [W4Layer(k, n, dev, gen, asym=True) for _ in range(max(2, int(600e6 // (k * n // 2))))]
         sb = torch.rand(n, 1, device=dev, generator=gen) + 0.5
-        for m in (16, 256, 1024):
+        for m in (16, 64, 128, 256, 1024):
             a8 = torch.randn(m, k, device=dev, generator=gen).to(torch.float8_e4m3fn)
             a16 = torch.randn(m, k, device=dev, generator=gen).to(torch.bfloat16)
             sa = torch.rand(m, 1, device=dev, generator=gen) + 0.5
