@@ -504,12 +504,14 @@ def test_scaled_mm_rotated_k_loop_exact(device, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(64, 4096, 4096), (50, 6144, 4096), (33, 8192, 4096), (100, 4096, 2048), (192, 4096, 1024),
-                                   (384, 6144, 512), (130, 2048, 2048), (70, 5120, 5120), (190, 2048, 6656)])
+                                   (384, 6144, 512), (130, 2048, 2048), (70, 5120, 5120), (190, 2048, 6656),
+                                   (64, 2048, 7168), (190, 1024, 8192), (100, 2048, 8192 + 64)])
 def test_scaled_mm_tile_row_past_m_exact(device, m, n, k):
     """Up to three tile rows with compute units to spare: one more row of workgroups runs past M beside them (it reads the
     same weights, its activation rows do not exist, it stores nothing).  Small-integer operands: the result must equal
-    the integer GEMM, rows next to the output (a taller buffer, M rows of it handed in) must stay untouched, and two
-    runs must agree."""
+    the integer GEMM and two runs must agree (the activations come as the first M rows of a taller buffer whose other
+    rows are not zero).  The last three cases split K over workgroups as well: the extra row's workgroups take no part
+    in the hand-over, and the arrival counters return to zero."""
     import vllm_amd._custom_ops as ops
     g = torch.Generator().manual_seed(m * 7 + k)
     a = torch.randint(-2, 3, (m, k), generator=g).float()
@@ -523,6 +525,7 @@ def test_scaled_mm_tile_row_past_m_exact(device, m, n, k):
     assert out.shape == (m, n)
     assert torch.equal(out.cpu().float(), a @ w.t())
     assert torch.equal(out, ops.cutlass_scaled_mm(*args))
+    assert all(bool((t == 0).all()) for t in ops._FP8_COUNTERS.values()), "arrival counters not restored to zero"
 
 
 def test_scaled_mm_split_k_exact_and_deterministic(device):

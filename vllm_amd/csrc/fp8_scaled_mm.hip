@@ -1034,8 +1034,9 @@ struct Fp8TilePlan {
   int cfg, sk, bm, bn, nw;
   int64_t tiles;
   int64_t tail_first = 0;      // > 0: only the tiles from this position on are split (tile_handover.h)
+  int64_t extra_tiles = 0;     // split K: the tiles of a tile row past M that runs beside the real ones (see m_tiles_extra in dispatch_tile)
   // scratch of the K split: partial tiles and arrival counters of the tiles that are split
-  int64_t split_tiles() const { return sk > 1 ? tiles - tail_first : 0; }
+  int64_t split_tiles() const { return sk > 1 ? tiles + extra_tiles - tail_first : 0; }
   int64_t tmp_bytes() const { return (int64_t)sk * split_tiles() * bm * bn * 4; }
   int64_t counter_ints() const { return split_tiles() * nw; }
 };
@@ -1227,6 +1228,14 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   while (sk > 1 && (uint64_t)sk * (uint64_t)(pl.tiles - pl.tail_first) * pl.bm * pl.bn * 4 >= (1ull << 32)) --sk;   // 32-bit buffer offsets
   pl.sk = sk;
   if (sk == 1) pl.tail_first = 0;
+  // A split K with compute units left for the parts of one more tile row: that row runs past M beside the real ones, as
+  // with an unsplit K (see m_tiles_extra in dispatch_tile); its workgroups take no part in the hand-over, but tile
+  // positions -- and with them the places in the scratch -- count it.  Cold: 7168 x 2048 at M = 40 / 64 / 192 12.1 / 13.6 /
+  // 18.0 -> 10.3 / 10.4 / 12.8 us, 8192 x 1024 at M = 40 .. 192 12.4 .. 13.2 -> 10.7 .. 11.0 us.
+  if (sk > 1 && pl.tail_first == 0 && tuning().exp[13] != 1) {
+    const int64_t rows = (M + pl.bm - 1) / pl.bm, cols = pl.tiles / rows;
+    if (rows <= 3 && (pl.tiles + cols) * sk <= (int64_t)cus) pl.extra_tiles = cols;
+  }
   return pl;
 }
 
@@ -1274,7 +1283,7 @@ static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t c
       // 2048 x 2048 at M = 128 8.6 -> 7.3 us; 128 x 128 tiles: 4096 x 6144 at M = 384 25.8 -> 23.5 us, 8192 x 8192 at M = 384
       // 46.7 -> 41.7 us.  The real rows then start together (rotated they lose the gain); from four tile rows on the
       // rotation alone is level or ahead (3072 x 3072 at M = 384 14.8 against 16.0 us) and stays.
-      p.m_tiles_extra = 0;
+      p.m_tiles_extra = pl.extra_tiles > 0 && pl.sk > 1 ? 1 : 0;
       if (pl.sk == 1 && pl.tail_first == 0 && tiles_m <= 3 && pl.tiles + pl.tiles / tiles_m <= cus && tuning().exp[13] != 1) {
         p.m_tiles_extra = 1;
         p.rotate_k = 0;
