@@ -436,7 +436,7 @@ def test_scaled_mm_into_a_view_of_a_wider_buffer(device, offset):
         assert bool((got[:, :offset] == 7).all()) and bool((got[:, offset + n:] == 7).all()), "wrote outside the view"
 
 
-@pytest.mark.parametrize("cfg", [1, 8, 2, 10, 11, 3, 4, 5, 7, 9, 13, 23, 14, 24, 15, 17])
+@pytest.mark.parametrize("cfg", [1, 8, 2, 10, 11, 3, 4, 5, 7, 9, 13, 23, 14, 24, 15, 16, 17])
 def test_scaled_mm_every_tile_shape_exact(device, cfg):
     """Every shape of the multi-stage tile kernel, forced through a per-call tuning override (the automatic choice only reaches
     some of them at any one problem size), including the ones that take two k-slices per step: small-integer operands
@@ -505,12 +505,15 @@ def test_scaled_mm_rotated_k_loop_exact(device, m, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(64, 4096, 4096), (50, 6144, 4096), (33, 8192, 4096), (100, 4096, 2048), (192, 4096, 1024),
                                    (384, 6144, 512), (130, 2048, 2048), (70, 5120, 5120), (190, 2048, 6656),
+                                   (320, 4096, 4096), (136, 6144, 4096), (264, 4608, 3584),
                                    (64, 2048, 7168), (190, 1024, 8192), (100, 2048, 8192 + 64)])
 def test_scaled_mm_tile_row_past_m_exact(device, m, n, k):
     """Up to three tile rows with compute units to spare: one more row of workgroups runs past M beside them (it reads the
     same weights, its activation rows do not exist, it stores nothing).  Small-integer operands: the result must equal
     the integer GEMM and two runs must agree (the activations come as the first M rows of a taller buffer whose other
-    rows are not zero).  The last three cases split K over workgroups as well: the extra row's workgroups take no part
+    rows are not zero).  Three cases run 128 x 64 tiles, which the planner takes where such a row fits beside them and beside
+    64 x 64 tiles it would not (the second of them without the extra row: too many tile columns).  The last three cases
+    split K over workgroups as well: the extra row's workgroups take no part
     in the hand-over, and the arrival counters return to zero."""
     import vllm_amd._custom_ops as ops
     g = torch.Generator().manual_seed(m * 7 + k)

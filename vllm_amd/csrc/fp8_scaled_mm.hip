@@ -1114,6 +1114,18 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
   // (cold weights: 4096 x 6144 at M = 128 21.8 -> 15.0 us, 4096 x 4096 at M = 192 19.8 -> 13.8 us; 14336 x 4096 at
   // M = 128 30.0 -> 34.0 us, and slower as soon as the tiles need a second round)
   if (tuning().fp8_tile_cfg <= 0 && pl.cfg == 14 && tiles(64, 64) <= cus) pl.cfg = 15;
+  // 128 x 64 tiles where the 64 x 64 ones need a second round: up to three tile rows, each weight row read by one workgroup
+  // per tile row as with the 64 x 64 tiles, when they leave compute units for one more row of workgroups past M (see
+  // m_tiles_extra in dispatch_tile), or are more workgroups than the 64 x 128 tiles while the last tile row holds at most
+  // 32 rows of M.  Cold: 4096 x 4096 at M = 264 .. 384 18.0 .. 18.6 -> 15.2 .. 15.5 us, 5120 x 5120 at M = 200 .. 288 22.5 .. 24.2
+  // -> 19.6 .. 20.3 us, 3584 x 4608 at M = 200 / 256 16.7 / 16.9 -> 13.9 / 14.0 us, 6656 x 6656 at M = 136 31.0 -> 24.4 us,
+  // 4096 x 6144 at M = 136 / 160 19.0 -> 15.4 / 16.3 us and at M = 176 / 192, 48 / 64 rows in the last tile row, 19.1 -> 20.0 us;
+  // with as many workgroups as the 64 x 128 tiles and no room for the row past M they lose 6 % (4096 x 6144 at M = 256).
+  if (tuning().fp8_tile_cfg <= 0 && pl.cfg == 14 && K <= 6656 && M <= 384 && tiles(128, 64) <= cus && tuning().exp[14] != 1) {
+    const int64_t t = tiles(128, 64), cols = (N + 63) / 64;
+    const int last_rows = M - (M - 1) / 128 * 128;
+    if (t + cols <= (int64_t)cus || (t > tiles(64, 128) && last_rows <= 32)) pl.cfg = 16;
+  }
   if (pl.cfg >= 10 && K % 128 != 0) pl.cfg %= 10;      // two k-slices per step need K % 128 == 0
   int sk = 1;
   const int steps = K / 64;
@@ -1124,6 +1136,7 @@ static Fp8TilePlan plan_tile3(int M, int N, int K) {
     case 3: case 13: case 23: pl.bm = 128; pl.bn = 128; pl.nw = 4; break;
     case 4: case 14: case 24: pl.bm = 64; pl.bn = 128; pl.nw = 4; break;
     case 5: case 15: pl.bm = 64; pl.bn = 64; pl.nw = 4; break;
+    case 16: pl.bm = 128; pl.bn = 64; pl.nw = 4; break;
     case 7: case 17: pl.bm = 128; pl.bn = 256; pl.nw = 8; break;
     case 9: pl.bm = 256; pl.bn = 128; pl.nw = 8; break;
     case 2: pl.bm = 256; pl.bn = 256; pl.nw = 4; break;
@@ -1306,6 +1319,7 @@ static int dispatch_tile(const Fp8MMParams& p_in, int64_t c_tmp_bytes, int64_t c
       case 24: return launch_tile3<BF16_OUT, 64, 128, 2, 2, 3, 2>(p, s);
       case 15: return launch_tile3<BF16_OUT, 64, 64, 2, 2, 5, 2>(p, s);
       case 5: return launch_tile3<BF16_OUT, 64, 64, 2, 2, 5>(p, s);
+      case 16: return launch_tile3<BF16_OUT, 128, 64, 2, 2, 5, 2>(p, s);
       case 17: return launch_tile3<BF16_OUT, 128, 256, 2, 4, 3, 2>(p, s);
       case 9: return launch_tile3<BF16_OUT, 256, 128, 4, 2, 5>(p, s);
       default: break;
