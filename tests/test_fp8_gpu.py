@@ -531,6 +531,31 @@ def test_scaled_mm_tile_row_past_m_exact(device, m, n, k):
     assert all(bool((t == 0).all()) for t in ops._FP8_COUNTERS.values()), "arrival counters not restored to zero"
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_scaled_mm_random_mid_m_exact(device, seed):
+    """Seeded sweep through the tile planner's middle: 33 .. 420 rows on layers of 1024 .. 8320 columns and K = 512 .. 8320
+    (some not a multiple of 64 or 128), where the automatic choice moves between tile shapes, K parts, rotated K loops and
+    the tile row past M.  Small-integer operands, power-of-two scales and an integer bias keep every step exact: the
+    result must equal the scaled integer GEMM, whichever plan ran, and the arrival counters must be back at zero."""
+    import vllm_amd._custom_ops as ops
+    rng = np.random.default_rng(7000 + seed)
+    g = torch.Generator().manual_seed(7000 + seed)
+    for _ in range(5):
+        m = int(rng.integers(33, 421))
+        n = 16 * int(rng.integers(64, 521))
+        k = 64 * int(rng.integers(8, 131)) + int(rng.choice([0, 0, 0, 16, 32]))
+        a = torch.randint(-2, 3, (m, k), generator=g).float()
+        w = torch.randint(-1, 2, (n, k), generator=g).float()
+        sa = torch.tensor(rng.choice([0.5, 1.0], size=(m, 1)), dtype=torch.float32)
+        sb = torch.tensor(rng.choice([0.5, 1.0], size=(n, 1)), dtype=torch.float32)
+        bias = torch.randint(-3, 4, (n,), generator=g).to(torch.float16) if rng.integers(0, 2) else None
+        ref = (a @ w.t()) * sa * sb.t() + (0 if bias is None else bias.float())
+        out = ops.cutlass_scaled_mm(a.to(torch.float8_e4m3fn).to(device), w.to(torch.float8_e4m3fn).to(device).t(),
+                                    sa.to(device), sb.to(device), torch.float16, None if bias is None else bias.to(device))
+        assert torch.equal(out.cpu().float(), ref), (m, n, k, bias is not None)
+    assert all(bool((t == 0).all()) for t in ops._FP8_COUNTERS.values()), "arrival counters not restored to zero"
+
+
 def test_scaled_mm_split_k_exact_and_deterministic(device):
     """Few output tiles and a long K: the tile kernel splits K over workgroups (fp32 partial tiles through the op's
     scratch, arrival counters left zero).  Small-integer operands make every partial sum exact, so the split result
