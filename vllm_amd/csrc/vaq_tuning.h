@@ -45,7 +45,8 @@ typedef struct VaqTuning {
                         /*   [9] = 1 both tile kernels: 256-row tiles also when M fills them poorly; [10] = 1 both tile     */
                         /*   kernels: never split only the tiles of a half-empty last round; [11] = 1 W4A16 tile kernel:  */
                         /*   no 128 x 256 tiles; [12] = 1 FP8 tile kernel: every tile starts at the first K step;       */
-                        /*   [13] = 1 FP8 tile kernel: no tile row past M; [14] = 1 FP8 tile kernel: no 128 x 64 tiles   */
+                        /*   [13] = 1 FP8 tile kernel: no tile row past M; [14] = 1 FP8 tile kernel: no 128 x 64 tiles;  */
+                        /*   [7] = 1 LDS-staged decode kernel: n-tiles in launch order, not grouped by XCD             */
 } VaqTuning;
 
 /* The entry points of the same name without `_tuned`, with `tuning` (may be NULL) applied to this call. */

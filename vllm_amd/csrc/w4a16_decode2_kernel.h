@@ -51,6 +51,7 @@ struct Decode2Params {
   // k-octets of the staged slab; both exact in those ranges); step_m, step_ko = (threads / KO, threads % KO).
   uint32_t wn_magic, ko_magic;
   int step_m, step_ko;
+  int gx8;                 // see the kernel's n-tile order
   uint32_t b_bytes, s_bytes, z_bytes, a_bytes;   // extents of the buffer descriptors (saturated to 4 GiB - 1)
 };
 
@@ -128,7 +129,11 @@ __global__ __launch_bounds__(D2_WAVES * 64) void w4a16_decode2_kernel(const Deco
   const int sk = blockIdx.y;
   const int slab_groups = WKS * GS;                 // tiles in this workgroup's K slab
   const int slab_g0 = sk * slab_groups;             // first tile of the slab
-  const int nt_raw = blockIdx.x * WN + wn;
+  // Workgroups go to the XCDs round robin, and an n-tile's scales, zero points and output are 32-byte pieces of lines that
+  // it shares with its neighbours: workgroups of one XCD take neighbouring n-tiles, so that an L2 fetches those lines once
+  // instead of once per XCD (gx8 = workgroups along N / 8 where that is a whole number, else 0).
+  const int bx = p.gx8 > 0 ? (int)(blockIdx.x & 7u) * p.gx8 + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+  const int nt_raw = bx * WN + wn;
   const bool nt_ok = nt_raw < p.NT;
   const int nt = nt_ok ? nt_raw : p.NT - 1;
   const int g_first = slab_g0 + wks * GS;           // this wavefront's first group
@@ -587,6 +592,11 @@ static int launch_decode2(const Decode2Params& p_in, hipStream_t s) {
   static size_t reserved[VAQ_MAX_DEVICES];
   if (const int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds, reserved, "w4a16_gemm(decode)"); rc != VAQ_OK) return rc;
   const int gx = (p.NT + WN - 1) / WN;
+  // n-tiles grouped by XCD (see the kernel) on layers of up to 1.5 n-tiles per compute unit whose K is not split over
+  // workgroups.  Cold, M = 1 / 4 / 16: 4096 x 6144 5.35 / 5.75 / 6.59 -> 5.16 / 5.55 / 6.32 us, 4096 x 4096 4.44 / 4.55 / 5.42 -> 4.23 /
+  // 4.42 / 5.27 us, 14336 x 4096 at M = 1 / 4 8.16 / 9.09 -> 7.78 / 8.76 us; with K parts and their hand-over it costs 4 % (14336 x
+  // 4096 at M = 16 / 32), wider layers show nothing either way (4096 x 28672, 4096 x 14336) or lose (8192 x 8192 at M = 1 +9 %).
+  p.gx8 = (gx % 8 == 0 && p.SK == 1 && p.NT * 2 <= num_cus_current_device() * 3 && tuning().exp[7] != 1) ? gx / 8 : 0;
   hipLaunchKernelGGL(kern, dim3(gx, p.SK, MSP ? (p.M + 15) / 16 : 1), dim3(64, p.WKS * WN), lds, s, p);
   return VAQ_OK;
 }
