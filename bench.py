@@ -37,11 +37,12 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes moved per algorithmic byte over the 12 headline GEMMs, from two hardware-counter runs of
 # `bench.py --counter-pass` (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same counter reads for the 256 MiB
 # copy in that run (FETCH_SIZE reads 131083.5 for 262144 KiB -> x2.000, WRITE_SIZE reads 262144.0 -> x1.000):
-# fetch 361.73 MB + write 2.90 MB = 364.62 MB against 340.30 MB algorithmic.  The excess is about 10 % on the fetch
-# side of every small layer (its size matches a 128-byte line of a scale row, which spans four 16-column tiles, being
-# fetched by each of the four XCDs those tiles' workgroups run on), the fp32 split-K partials of the K=14336, M=16 case, and activation re-reads at M=16.
+# fetch 351.15 MB + write 2.90 MB = 354.04 MB against 340.30 MB algorithmic.  The excess is the fp32 split-K partials and
+# scale rows of the K=14336, M=16 case (1.18x there), activation re-reads by every XCD at M=16, and 3-6 % on the fetch side of the
+# small layers (it was 10 % -- a 128-byte line of a scale row spans four 16-column tiles and was fetched by each XCD those
+# tiles' workgroups ran on -- before the workgroups of one XCD took neighbouring tiles).
 STEPS_PER_GRAPH = 10      # consecutive steps captured into one HIP graph (see headline())
-MEASURED_TRAFFIC_PER_ALGORITHMIC_BYTE = 364.62 / 340.30
+MEASURED_TRAFFIC_PER_ALGORITHMIC_BYTE = 354.04 / 340.30
 BF16_PEAK_TFLOPS = 2500.0
 FP8_PEAK_TFLOPS = 5000.0
 GROUP = 128
