@@ -538,6 +538,25 @@ def test_rows_over_workgroups_beyond_four_m_blocks(device, k, n, m, dtype):
         assert torch.equal(layer(hot.to(device)).cpu(), w_ref[rows]), "one-hot rows must return the dequantised weights exactly"
 
 
+@pytest.mark.parametrize("k,n", [(4096, 4096), (4096, 6144), (1024, 1472), (2048, 1984), (4096, 3008), (2048, 2048), (14336, 4096)])
+def test_decode_n_tiles_grouped_by_xcd_same_bits(device, k, n):
+    """On narrow layers the decode kernel hands the workgroups of one XCD neighbouring n-tiles (a permutation of which
+    workgroup computes which columns, nothing else): with the grouping switched off for one call the output must be the
+    same bits, for 1 .. 48 rows (one m-block, two, and rows over workgroups), with zero points, also on column counts
+    that are no power of two."""
+    from vllm_amd import _tuning
+    case = o.make_w4a16_case(k, n, 128, asym=True, dtype=torch.bfloat16, seed=k + n)
+    layer = W4A16Layer(case, device, torch.bfloat16)
+    w_ref = o.case_w_ref(case)
+    for m in (1, 4, 16, 32, 48):
+        a = _acts(m, k, device, seed=m)
+        out = layer(a)
+        with _tuning.override(exp=[0] * 7 + [1]):
+            plain = layer(a)
+        assert torch.equal(out, plain), (k, n, m)
+        check_gemm_close(out, o.gemm_ref(a.cpu(), w_ref), f"k={k} n={n} m={m}")
+
+
 # layer shapes of other models on which the planners take branches that the Llama-3-8B shapes do not reach: K slabs that
 # would come out uneven (9216 x 4608, 10240 x 2560), a ragged single slab on a narrow layer (5120 x 5120), a short K on
 # few tiles (1536 x 1536), an odd number of 64-row blocks on a wide short-K layer (2560 x 10240), long K parts on few
