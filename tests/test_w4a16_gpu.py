@@ -518,8 +518,9 @@ def test_decode_three_and_four_m_blocks(device, k, n, m):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_rows_over_workgroups_beyond_four_m_blocks(device, k, n, m, dtype):
     """65 .. 256 rows on a narrow layer: where workgroups of 16 rows each make one round, the decode kernel takes the rows
-    as five to sixteen m-blocks with workgroups of their own (a ragged last block among them); elsewhere -- the last
-    case, 258 workgroups -- and with act_order the tile kernel does.  Same answer either way: symmetric and with zero
+    as five to sixteen m-blocks with workgroups of their own (a ragged last block among them; the last case with eight
+    n-tiles per workgroup, because six would need a second round and seven lose to eight); with act_order the tile kernel
+    does.  Same answer either way: symmetric and with zero
     points against the fp64 oracle, one-hot rows bit for bit, no scratch used, deterministic."""
     for asym, act_order in ((False, False), (True, False), (True, True)):
         case = o.make_w4a16_case(k, n, 128, asym=asym, act_order=act_order, dtype=dtype, seed=k + n + m)

@@ -258,17 +258,25 @@ static bool row_split_config(int M, int N, int K, int sub, int wt, bool has_perm
   // wavefronts on a compute unit.  Cold: 4096 x 4096 at M = 128 16.2 -> 13.4 us, 4096 x 6144 at M = 80 18.8 -> 13.5 us,
   // 4096 x 2048 at M = 128 / 256 14.8 / 16.0 -> 8.8 / 13.2 us, 2048 x 2048 at M = 128 / 256 11.5 / 12.5 -> 6.3 / 8.3 us; grids
   // of a second round lose (4096 x 4096 at M = 96 with 258 workgroups: 16.1 -> 22.3 us), ten wavefronts too (M = 80: 20.2 us).
+  // (An odd number of n-tiles gives way to the next even one where that grid passes too: seven n-tiles -- 14 wavefronts and
+  // a ragged last workgroup -- measured 15-20 % behind eight, 4096 x 4096 at M = 96 15.6 against 13.3 us, 4096 x 2048 at
+  // M = 192 / 208 15.4 / 15.7 against 13.1 us, and five behind six, 2048 x 2048 at M = 144 9.0 against 7.6 us.)
   const long lds_slots = (long)((size_t)(160 * 1024) / decode2_lds_bytes(c.wks, c.gs, c.mr, 1));
-  for (int wn = 1; wn * c.wks <= D2_WAVES; ++wn) {
+  auto passes = [&](int wn) {
+    if (wn * c.wks > D2_WAVES) return false;
     long slots = D2_WAVES / (c.wks * wn);
     if (slots > lds_slots) slots = lds_slots;
     if (slots < 1) slots = 1;
     const long wgs = (long)((NT + wn - 1) / wn) * MB;
     const long per_cu = (wgs + cus - 1) / cus;
-    if (per_cu <= slots && per_cu * c.wks * wn >= 12) {
-      out->wn = wn;
-      return true;
-    }
+    return per_cu <= slots && per_cu * c.wks * wn >= 12;
+  };
+  for (int wn = 1; wn * c.wks <= D2_WAVES; ++wn) {
+    if (tuning().decode2_wn > 0 && wn != tuning().decode2_wn) continue;
+    if (!passes(wn)) continue;
+    if (tuning().decode2_wn <= 0 && wn >= 3 && (wn & 1) && passes(wn + 1)) continue;
+    out->wn = wn;
+    return true;
   }
   return false;
 }
